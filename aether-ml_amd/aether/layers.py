@@ -1,0 +1,569 @@
+"""Layer, loss and optimizer classes with the reference's names, constructor
+signatures and attributes (CNN/models/CNN_classes_cupy.py), running on
+libaether_hip.so.  ``forward(inputs, training)`` sets ``.output``,
+``backward(dvalues)`` sets ``.dinputs`` (+ ``.dweights`` / ``.dbiases``); all of
+these are DeviceTensors in MI355X HBM.  Inputs may be NumPy arrays (uploaded) or
+DeviceTensors.
+
+Departures from the reference, each deliberate:
+  * everything is float32 on the device (the reference's Dense weights are
+    float64 by accident of ``cp.random.randn``);
+  * ``Conv_Layer.dinputs`` is the full gradient also when the pad is 0 under
+    "same" (the reference slices ``[:, 0:-0]`` to an empty array, :149-151);
+  * ``Conv_Layer.set_parameters`` refreshes the ``weights`` alias (:159-161 does not);
+  * ``Pooling(padding="same")`` raises ValueError (the reference reads ``H_out``
+    before assigning it, :226-228).
+"""
+import os
+
+import numpy as np
+
+from . import _lib
+from .tensor import DeviceTensor, as_device
+
+_F32 = np.float32
+
+
+def _L():
+    return _lib.lib()
+
+
+def _ck(rc):
+    _lib.check(rc)
+
+
+# ----------------------------------------------------------------------------------
+# Conv_Layer  (CNN_classes_cupy.py:37-161)
+# ----------------------------------------------------------------------------------
+class Conv_Layer:
+    def __init__(self, input_shape, num_filters=1, filter_size=(3, 3), strides=(1, 1), padding="same"):
+        self.input_shape = input_shape
+        self.num_filters = num_filters
+        self.filter_size = filter_size
+        self.strides = strides
+        self.padding = padding
+        self.biases = DeviceTensor.zeros(self.num_filters)
+        self.weight_regularizer_l1 = 0
+        self.weight_regularizer_l2 = 0
+        self.bias_regularizer_l1 = 0
+        self.bias_regularizer_l2 = 0
+        input_depth = input_shape[-1]
+        n = self.filter_size[0] * self.filter_size[1] * input_depth
+        std = np.sqrt(_F32(2.0 / n))
+        # He initialisation from the legacy global RNG, as the reference (:61-66)
+        w = np.random.randn(filter_size[0], filter_size[1], input_depth, num_filters).astype(_F32) * std
+        self.filter_weights = DeviceTensor.from_numpy(w, _F32)
+        self.weights = self.filter_weights
+        # "fp32" (reference arithmetic) or "bf16" (bf16 inputs, fp32 accumulate)
+        self.precision = os.environ.get("AETHER_PRECISION", "fp32")
+
+    def _geometry(self, H_in, W_in):
+        fH, fW = self.filter_size
+        sH, sW = self.strides
+        P = (fH - 1) // 2 if self.padding == "same" else 0
+        H_out = int((H_in + 2 * P - fH) / sH + 1)
+        W_out = int((W_in + 2 * P - fW) / sW + 1)
+        return P, H_out, W_out
+
+    def _dims(self, S, H, W, C):
+        fH, fW = self.filter_size
+        sH, sW = self.strides
+        P = (fH - 1) // 2 if self.padding == "same" else 0
+        return (S, H, W, C, self.num_filters, fH, fW, sH, sW, P, P)
+
+    @staticmethod
+    def _bf16(t):
+        out = DeviceTensor(t.shape, np.uint16)
+        _ck(_L().aeth_cast_f32_to_bf16(t.ptr, out.ptr, t.size))
+        return out
+
+    def forward(self, inputs, training):
+        inputs = as_device(inputs, _F32)
+        if inputs.ndim != 4:
+            raise ValueError(f"Expected a 4D tensor, got {inputs.ndim} instead.")
+        S, H_in, W_in, D_in = inputs.shape
+        if D_in != self.filter_weights.shape[2]:
+            raise ValueError(f"Expected {self.filter_weights.shape[2]} input channels, got {D_in}.")
+        P, H_out, W_out = self._geometry(H_in, W_in)
+        self.output = DeviceTensor((S, H_out, W_out, self.num_filters), _F32)
+        dims = self._dims(S, H_in, W_in, D_in)
+        if self.precision == "bf16":
+            self._x_bf16 = self._bf16(inputs)
+            w16 = self._bf16(self.filter_weights)
+            _ck(_L().aeth_conv_fprop_bf16(self._x_bf16.ptr, w16.ptr, self.biases.ptr, self.output.ptr, *dims))
+        else:
+            _ck(_L().aeth_conv_fprop_f32(inputs.ptr, self.filter_weights.ptr, self.biases.ptr,
+                                         self.output.ptr, *dims))
+        self.inputs = inputs
+        return self.output
+
+    def backward(self, dvalues):
+        dvalues = as_device(dvalues, _F32)
+        S, H_in, W_in, C_in = self.inputs.shape
+        dims = self._dims(S, H_in, W_in, C_in)
+        self.dbiases = DeviceTensor(self.biases.shape, _F32)
+        self.dweights = DeviceTensor(self.filter_weights.shape, _F32)
+        self.dinputs = DeviceTensor(self.inputs.shape, _F32)
+        if self.precision == "bf16":
+            dy16 = self._bf16(dvalues)
+            w16 = self._bf16(self.filter_weights)
+            _ck(_L().aeth_conv_wgrad_bf16(self._x_bf16.ptr, dy16.ptr, self.dweights.ptr, self.dbiases.ptr, *dims))
+            _ck(_L().aeth_conv_dgrad_bf16(dy16.ptr, w16.ptr, self.dinputs.ptr, *dims))
+        else:
+            _ck(_L().aeth_conv_wgrad_f32(self.inputs.ptr, dvalues.ptr, self.dweights.ptr, self.dbiases.ptr, *dims))
+            _ck(_L().aeth_conv_dgrad_f32(dvalues.ptr, self.filter_weights.ptr, self.dinputs.ptr, *dims))
+        return self.dinputs
+
+    def get_parameters(self):
+        return self.filter_weights, self.biases
+
+    def set_parameters(self, weights, biases):
+        self.filter_weights = as_device(weights, _F32)
+        self.biases = as_device(biases, _F32).reshape(-1)
+        self.weights = self.filter_weights
+
+
+# ----------------------------------------------------------------------------------
+# Pooling  (CNN_classes_cupy.py:204-312)
+# ----------------------------------------------------------------------------------
+class Pooling:
+    def __init__(self, filter_size=(2, 2), strides=(2, 2), padding="valid", pooling_type="max"):
+        self.filter_size = filter_size
+        self.strides = strides
+        self.padding = padding
+        self.pooling_type = pooling_type
+
+    def forward(self, inputs, training):
+        inputs = as_device(inputs, _F32)
+        if inputs.ndim != 4:
+            raise ValueError(f"Expected a 4D tensor, got {inputs.ndim} instead.")
+        S, H_in, W_in, C = inputs.shape
+        fH, fW = self.filter_size
+        sH, sW = self.strides
+        if self.padding == "valid":
+            H_out = int(np.floor((H_in - fH) / sH + 1))
+            W_out = int(np.floor((W_in - fW) / sW + 1))
+        elif self.padding == "same":
+            raise ValueError("Pooling with padding == same is not supported")
+        else:
+            raise ValueError(f"Expected padding == valid or same, recieved {self.padding} instead")
+        self.inputs = inputs
+        self.output = DeviceTensor((S, H_out, W_out, C), _F32)
+        if self.pooling_type == "max":
+            self.max_indicies = DeviceTensor((S, H_out, W_out, C), np.uint8)
+            _ck(_L().aeth_maxpool_fwd_f32(inputs.ptr, self.output.ptr, self.max_indicies.ptr,
+                                          S, H_in, W_in, C, fH, fW, sH, sW))
+        elif self.pooling_type == "average":
+            _ck(_L().aeth_avgpool_fwd_f32(inputs.ptr, self.output.ptr, S, H_in, W_in, C, fH, fW, sH, sW))
+        else:
+            raise ValueError(f"Expected pooling_type == max or average, recieved {self.pooling_type} instead")
+        return self.output
+
+    def backward(self, dvalues):
+        dvalues = as_device(dvalues, _F32)
+        S, H_in, W_in, C = self.inputs.shape
+        fH, fW = self.filter_size
+        sH, sW = self.strides
+        self.dinputs = DeviceTensor(self.inputs.shape, _F32)
+        if self.pooling_type == "max":
+            _ck(_L().aeth_maxpool_bwd_f32(dvalues.ptr, self.max_indicies.ptr, self.dinputs.ptr,
+                                          S, H_in, W_in, C, fH, fW, sH, sW))
+        elif self.pooling_type == "average":
+            _ck(_L().aeth_avgpool_bwd_f32(dvalues.ptr, self.dinputs.ptr, S, H_in, W_in, C, fH, fW, sH, sW))
+        return self.dinputs
+
+
+# ----------------------------------------------------------------------------------
+# Layer_Dense  (CNN_classes_cupy.py:315-362)
+# ----------------------------------------------------------------------------------
+class Layer_Dense:
+    def __init__(self, n_inputs, n_neurons, weight_regularizer_l1=0, bias_regularizer_l1=0,
+                 weight_regularizer_l2=0, bias_regularizer_l2=0):
+        w = .01 * np.random.randn(n_inputs, n_neurons) * np.sqrt(2.0 / n_inputs)
+        self.weights = DeviceTensor.from_numpy(w, _F32)
+        self.biases = DeviceTensor.zeros((1, n_neurons))
+        self.weight_regularizer_l1 = weight_regularizer_l1
+        self.weight_regularizer_l2 = weight_regularizer_l2
+        self.bias_regularizer_l1 = bias_regularizer_l1
+        self.bias_regularizer_l2 = bias_regularizer_l2
+
+    def forward(self, inputs, training):
+        inputs = as_device(inputs, _F32)
+        if inputs.ndim != 2 or inputs.shape[1] != self.weights.shape[0]:
+            raise ValueError(f"shapes {inputs.shape} and {self.weights.shape} not aligned")
+        self.inputs = inputs
+        M = inputs.shape[0]
+        n_in, n_out = self.weights.shape
+        self.output = DeviceTensor((M, n_out), _F32)
+        _ck(_L().aeth_dense_fprop_f32(inputs.ptr, self.weights.ptr, self.biases.ptr, self.output.ptr,
+                                      M, n_in, n_out))
+        return self.output
+
+    def backward(self, dvalues):
+        dvalues = as_device(dvalues, _F32)
+        M = self.inputs.shape[0]
+        n_in, n_out = self.weights.shape
+        self.dweights = DeviceTensor(self.weights.shape, _F32)
+        self.dbiases = DeviceTensor((1, n_out), _F32)
+        _ck(_L().aeth_dense_wgrad_f32(self.inputs.ptr, dvalues.ptr, self.dweights.ptr, self.dbiases.ptr,
+                                      M, n_in, n_out))
+        if self.weight_regularizer_l1 > 0:
+            _ck(_L().aeth_l1_grad_f32(self.weight_regularizer_l1, self.weights.ptr, self.dweights.ptr,
+                                      self.weights.size))
+        if self.weight_regularizer_l2 > 0:
+            _ck(_L().aeth_axpy_f32(2 * self.weight_regularizer_l2, self.weights.ptr, self.dweights.ptr,
+                                   self.weights.size))
+        if self.bias_regularizer_l1 > 0:
+            _ck(_L().aeth_l1_grad_f32(self.bias_regularizer_l1, self.biases.ptr, self.dbiases.ptr,
+                                      self.biases.size))
+        if self.bias_regularizer_l2 > 0:
+            _ck(_L().aeth_axpy_f32(2 * self.bias_regularizer_l2, self.biases.ptr, self.dbiases.ptr,
+                                   self.biases.size))
+        self.dinputs = DeviceTensor(self.inputs.shape, _F32)
+        _ck(_L().aeth_dense_dgrad_f32(dvalues.ptr, self.weights.ptr, self.dinputs.ptr, M, n_in, n_out))
+
+    def get_parameters(self):
+        return self.weights, self.biases
+
+    def set_parameters(self, weights, biases):
+        self.weights = as_device(weights, _F32)
+        b = as_device(biases, _F32)
+        self.biases = b.reshape(1, b.size)
+
+
+# ----------------------------------------------------------------------------------
+# Dropout  (CNN_classes_cupy.py:364-404).  Masks are drawn on the host from the
+# legacy global RNG, exactly as the reference draws them, and multiplied on the GPU.
+# Assigning ``fixed_mask`` (already divided by the keep probability) replaces the draw.
+# ----------------------------------------------------------------------------------
+class Layer_Dropout:
+    def __init__(self, rate):
+        self.rate = 1 - rate
+        self.fixed_mask = None
+
+    def forward(self, inputs, training):
+        inputs = as_device(inputs, _F32)
+        self.inputs = inputs
+        if not training:
+            self.output = inputs.copy()
+            return self.output
+        if self.fixed_mask is not None:
+            mask = np.asarray(self.fixed_mask, dtype=_F32)
+        else:
+            mask = (np.random.binomial(1, self.rate, size=inputs.shape) / self.rate).astype(_F32)
+        self.binary_mask = DeviceTensor.from_numpy(np.broadcast_to(mask, inputs.shape), _F32)
+        self.output = DeviceTensor(inputs.shape, _F32)
+        _ck(_L().aeth_mul_mask_f32(inputs.ptr, self.binary_mask.ptr, self.output.ptr, inputs.size, inputs.size))
+        return self.output
+
+    def backward(self, dvalues):
+        dvalues = as_device(dvalues, _F32)
+        self.dinputs = DeviceTensor(dvalues.shape, _F32)
+        _ck(_L().aeth_mul_mask_f32(dvalues.ptr, self.binary_mask.ptr, self.dinputs.ptr, dvalues.size, dvalues.size))
+
+
+class Layer_Dropout_Spatial:
+    def __init__(self, rate):
+        self.rate = rate
+        self.keep_prob = 1 - rate
+        self.fixed_mask = None
+
+    def forward(self, inputs, training):
+        inputs = as_device(inputs, _F32)
+        self.inputs = inputs
+        if not training:
+            self.output = inputs.copy()
+            return self.output
+        C = inputs.shape[-1]
+        if self.fixed_mask is not None:
+            mask = np.asarray(self.fixed_mask, dtype=_F32).reshape(1, 1, 1, C)
+        else:
+            mask = (np.random.binomial(1, self.keep_prob, size=(1, 1, 1, C)) / self.keep_prob).astype(_F32)
+        self.channel_mask = DeviceTensor.from_numpy(mask, _F32)
+        self.output = DeviceTensor(inputs.shape, _F32)
+        _ck(_L().aeth_mul_mask_f32(inputs.ptr, self.channel_mask.ptr, self.output.ptr, inputs.size, C))
+        return self.output
+
+    def backward(self, dvalues):
+        dvalues = as_device(dvalues, _F32)
+        self.dinputs = DeviceTensor(dvalues.shape, _F32)
+        _ck(_L().aeth_mul_mask_f32(dvalues.ptr, self.channel_mask.ptr, self.dinputs.ptr, dvalues.size,
+                                   self.channel_mask.size))
+
+
+# ----------------------------------------------------------------------------------
+# ReLU / Leaky_ReLU  (CNN_classes_cupy.py:406-428)
+# ----------------------------------------------------------------------------------
+class ReLU:
+    def forward(self, inputs, training):
+        inputs = as_device(inputs, _F32)
+        self.inputs = inputs
+        self.output = DeviceTensor(inputs.shape, _F32)
+        _ck(_L().aeth_relu_fwd_f32(inputs.ptr, self.output.ptr, 0.0, inputs.size))
+        return self.output
+
+    def backward(self, dvalues):
+        dvalues = as_device(dvalues, _F32)
+        self.dinputs = DeviceTensor(dvalues.shape, _F32)
+        _ck(_L().aeth_relu_bwd_f32(self.inputs.ptr, dvalues.ptr, self.dinputs.ptr, 0.0, dvalues.size))
+
+
+class Leaky_ReLU:
+    def __init__(self, alpha=0.01):
+        self.alpha = alpha
+
+    def forward(self, inputs, training):
+        inputs = as_device(inputs, _F32)
+        self.inputs = inputs
+        self.output = DeviceTensor(inputs.shape, _F32)
+        _ck(_L().aeth_relu_fwd_f32(inputs.ptr, self.output.ptr, self.alpha, inputs.size))
+        return self.output
+
+    def backward(self, dvalues):
+        dvalues = as_device(dvalues, _F32)
+        self.dinputs = DeviceTensor(dvalues.shape, _F32)
+        _ck(_L().aeth_relu_bwd_f32(self.inputs.ptr, dvalues.ptr, self.dinputs.ptr, self.alpha, dvalues.size))
+
+
+# ----------------------------------------------------------------------------------
+# Batch_Norm  (CNN_classes_cupy.py:430-526)
+# ----------------------------------------------------------------------------------
+class Batch_Norm:
+    def __init__(self, epsilon=1e-5, momentum=0.9, n_features=None):
+        self.epsilon = epsilon
+        self.momentum = momentum
+        if n_features is not None:
+            self.gamma = DeviceTensor.full(n_features, 1.0)
+            self.beta = DeviceTensor.zeros(n_features)
+        else:
+            self.gamma = None
+            self.beta = None
+        self.weights = self.gamma
+        self.biases = self.beta
+        self.running_mean = None
+        self.running_var = None
+        self.weight_regularizer_l1 = 0
+        self.weight_regularizer_l2 = 0
+        self.bias_regularizer_l1 = 0
+        self.bias_regularizer_l2 = 0
+
+    def _lazy_init(self, C):
+        if self.gamma is None:
+            self.gamma = DeviceTensor.full(C, 1.0)
+            self.beta = DeviceTensor.zeros(C)
+            self.weights = self.gamma
+            self.biases = self.beta
+        if self.running_mean is None:
+            self.running_mean = DeviceTensor.zeros(C)
+            self.running_var = DeviceTensor.full(C, 1.0)
+
+    def forward(self, inputs, training):
+        inputs = as_device(inputs, _F32)
+        self.inputs = inputs
+        C = inputs.shape[-1]
+        self._lazy_init(C)
+        rows = inputs.size // C
+        self.output = DeviceTensor(inputs.shape, _F32)
+        if training:
+            self.batch_mean = DeviceTensor(C, _F32)
+            self.batch_invstd = DeviceTensor(C, _F32)
+            _ck(_L().aeth_bn_fwd_train_f32(inputs.ptr, self.gamma.ptr, self.beta.ptr, self.running_mean.ptr,
+                                           self.running_var.ptr, self.batch_mean.ptr, self.batch_invstd.ptr,
+                                           self.output.ptr, rows, C, self.epsilon, self.momentum))
+            # the reference's running statistics take the keepdims shape after a
+            # training step (:475-476); keep that shape for get_parameters()
+            keep = (1,) * (inputs.ndim - 1) + (C,)
+            if self.running_mean.shape != keep:
+                self.running_mean = self.running_mean.reshape(keep)
+                self.running_var = self.running_var.reshape(keep)
+        else:
+            _ck(_L().aeth_bn_fwd_infer_f32(inputs.ptr, self.gamma.ptr, self.beta.ptr, self.running_mean.ptr,
+                                           self.running_var.ptr, self.output.ptr, rows, C, self.epsilon))
+        return self.output
+
+    def backward(self, dvalues):
+        dvalues = as_device(dvalues, _F32)
+        C = self.inputs.shape[-1]
+        rows = self.inputs.size // C
+        self.dinputs = DeviceTensor(self.inputs.shape, _F32)
+        self.dweights = DeviceTensor(C, _F32)
+        self.dbiases = DeviceTensor(C, _F32)
+        _ck(_L().aeth_bn_bwd_f32(self.inputs.ptr, dvalues.ptr, self.gamma.ptr, self.batch_mean.ptr,
+                                 self.batch_invstd.ptr, self.dinputs.ptr, self.dweights.ptr, self.dbiases.ptr,
+                                 rows, C))
+        return self.dinputs
+
+    def get_parameters(self):
+        return (self.gamma, self.beta, self.running_mean, self.running_var)
+
+    def set_parameters(self, gamma, beta, running_mean, running_var):
+        self.gamma = as_device(gamma, _F32).reshape(-1)
+        self.beta = as_device(beta, _F32).reshape(-1)
+        self.running_mean = as_device(running_mean, _F32)
+        self.running_var = as_device(running_var, _F32)
+        self.weights = self.gamma
+        self.biases = self.beta
+
+
+# ----------------------------------------------------------------------------------
+# Flatten / SoftMax  (CNN_classes_cupy.py:528-563)
+# ----------------------------------------------------------------------------------
+class Flatten:
+    def forward(self, inputs, training):
+        inputs = as_device(inputs, _F32)
+        self.inputs_shape = inputs.shape
+        self.output = inputs.reshape(inputs.shape[0], -1)
+        return self.output
+
+    def backward(self, dvalues):
+        self.dinputs = as_device(dvalues, _F32).reshape(self.inputs_shape)
+
+
+class SoftMax:
+    def forward(self, inputs, training=None):
+        inputs = as_device(inputs, _F32)
+        rows, K = inputs.shape
+        self.output = DeviceTensor(inputs.shape, _F32)
+        _ck(_L().aeth_softmax_f32(inputs.ptr, self.output.ptr, rows, K))
+        return self.output
+
+    def backward(self, dvalues):
+        dvalues = as_device(dvalues, _F32)
+        rows, K = dvalues.shape
+        self.dinputs = DeviceTensor(dvalues.shape, _F32)
+        _ck(_L().aeth_softmax_bwd_f32(self.output.ptr, dvalues.ptr, self.dinputs.ptr, rows, K))
+
+    def predictions(self, outputs):
+        return np.argmax(np.asarray(outputs), axis=1)
+
+
+# ----------------------------------------------------------------------------------
+# Loss  (CNN_classes_cupy.py:565-680)
+# ----------------------------------------------------------------------------------
+def _sparse_labels(y_true):
+    """int32 class indices; one-hot rows are reduced with argmax."""
+    y = np.asarray(y_true)
+    if y.ndim == 2:
+        y = np.argmax(y, axis=1)
+    return np.ascontiguousarray(y, dtype=np.int32)
+
+
+class Loss:
+    def remember_trainable_layers(self, trainable_layers):
+        self.trainable_layers = trainable_layers
+
+    def calculate(self, output, y, *, include_regularization=False, training=True):
+        sample_losses = self.forward(output, y, training)
+        data_loss = np.mean(sample_losses)
+        self.accumulated_sum += np.sum(sample_losses)
+        self.accumulated_count += len(sample_losses)
+        if not include_regularization:
+            return data_loss
+        return data_loss, self.regularization_loss()
+
+    def calculate_accumulated(self, *, include_regularization=False):
+        data_loss = self.accumulated_sum / self.accumulated_count
+        if not include_regularization:
+            return data_loss
+        return data_loss, self.regularization_loss()
+
+    def new_pass(self):
+        self.accumulated_sum = 0
+        self.accumulated_count = 0
+
+    def _device_sum(self, t, mode):
+        out = DeviceTensor(1, _F32)
+        _ck(_L().aeth_reduce_f32(t.ptr, t.size, mode, out.ptr))
+        return float(out.get()[0])
+
+    def regularization_loss(self):
+        regularization_loss = 0
+        for layer in self.trainable_layers:
+            if layer.weight_regularizer_l1 > 0:
+                regularization_loss += layer.weight_regularizer_l1 * self._device_sum(layer.weights, 0)
+            if layer.weight_regularizer_l2 > 0:
+                regularization_loss += layer.weight_regularizer_l2 * self._device_sum(layer.weights, 1)
+            if layer.bias_regularizer_l1 > 0:
+                regularization_loss += layer.bias_regularizer_l1 * self._device_sum(layer.biases, 0)
+            if layer.bias_regularizer_l2 > 0:
+                regularization_loss += layer.bias_regularizer_l2 * self._device_sum(layer.biases, 1)
+        return regularization_loss
+
+
+class Loss_CategoricalCrossEntropy(Loss):
+    def __init__(self, label_smoothing=0.0):
+        self.label_smoothing = label_smoothing
+
+    def forward(self, y_pred, y_true, training=True):
+        y_pred = as_device(y_pred, _F32)
+        rows, K = y_pred.shape
+        labels = DeviceTensor.from_numpy(_sparse_labels(y_true), np.int32)
+        ls = self.label_smoothing if (self.label_smoothing > 0 and training) else 0.0
+        loss = DeviceTensor(rows, _F32)
+        correct = DeviceTensor(rows, np.int32)
+        _ck(_L().aeth_cce_fwd_f32(y_pred.ptr, labels.ptr, ls, loss.ptr, correct.ptr, rows, K))
+        self.correct = correct
+        return loss.get()
+
+    def backward(self, dvalues, y_true):
+        dvalues = as_device(dvalues, _F32)
+        rows, K = dvalues.shape
+        labels = DeviceTensor.from_numpy(_sparse_labels(y_true), np.int32)
+        self.dinputs = DeviceTensor(dvalues.shape, _F32)
+        _ck(_L().aeth_softmax_cce_bwd_f32(dvalues.ptr, labels.ptr, self.label_smoothing, self.dinputs.ptr, rows, K))
+
+
+class Activation_Softmax_Loss_CategoricalCrossEntropy():
+    def __init__(self, label_smoothing=0.0):
+        self.activation = SoftMax()
+        self.loss = Loss_CategoricalCrossEntropy(label_smoothing)
+        self.loss.new_pass()
+        self.label_smoothing = label_smoothing
+
+    def forward(self, inputs, y_true, training=True):
+        self.activation.forward(inputs)
+        self.output = self.activation.output
+        return self.loss.calculate(self.output, y_true, training=training)
+
+    def backward(self, dvalues, y_true, training=True):
+        dvalues = as_device(dvalues, _F32)
+        rows, K = dvalues.shape
+        labels = DeviceTensor.from_numpy(_sparse_labels(y_true), np.int32)
+        ls = self.label_smoothing if (self.label_smoothing > 0 and training) else 0.0
+        self.dinputs = DeviceTensor(dvalues.shape, _F32)
+        _ck(_L().aeth_softmax_cce_bwd_f32(dvalues.ptr, labels.ptr, ls, self.dinputs.ptr, rows, K))
+
+
+# ----------------------------------------------------------------------------------
+# Optimizer_Adam  (CNN_classes_cupy.py:685-736)
+# ----------------------------------------------------------------------------------
+class Optimizer_Adam:
+    def __init__(self, learning_rate=.001, decay=0., epsilon=1e-7, beta_1=0.9, beta_2=.999):
+        self.learning_rate = learning_rate
+        self.current_learning_rate = learning_rate
+        self.decay = decay
+        self.iterations = 0
+        self.epsilon = epsilon
+        self.beta_1 = beta_1
+        self.beta_2 = beta_2
+
+    def pre_update_parameters(self):
+        if self.decay:
+            self.current_learning_rate = self.learning_rate * (1. / (1. + self.decay * self.iterations))
+
+    def update_parameters(self, layer):
+        if not hasattr(layer, "weight_cache"):
+            layer.weight_momentums = DeviceTensor.zeros(layer.weights.shape)
+            layer.weight_cache = DeviceTensor.zeros(layer.weights.shape)
+            layer.bias_momentums = DeviceTensor.zeros(layer.biases.shape)
+            layer.bias_cache = DeviceTensor.zeros(layer.biases.shape)
+        L = _L()
+        _ck(L.aeth_adam_f32(layer.weights.ptr, layer.dweights.ptr, layer.weight_momentums.ptr,
+                            layer.weight_cache.ptr, layer.weights.size, self.current_learning_rate,
+                            self.beta_1, self.beta_2, self.epsilon, self.iterations))
+        _ck(L.aeth_adam_f32(layer.biases.ptr, layer.dbiases.ptr, layer.bias_momentums.ptr,
+                            layer.bias_cache.ptr, layer.biases.size, self.current_learning_rate,
+                            self.beta_1, self.beta_2, self.epsilon, self.iterations))
+
+    def post_update_parameters(self):
+        self.iterations += 1

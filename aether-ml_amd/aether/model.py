@@ -1,0 +1,292 @@
+"""Model orchestrator with the reference's method names and behaviour
+(CNN/models/CNN_model_cupy.py:5-392): layer chain, batching loop, loss/accuracy
+bookkeeping and the printed progress lines.  Batches are sliced on the host and
+uploaded once; every activation then stays in HBM until the three printed
+scalars are read back.
+
+Parameter files written by ``save_parameters`` hold plain NumPy arrays (a list
+of per-layer tuples, the reference's structure).  ``load_parameters`` reads them
+with a restricted unpickler that only rebuilds NumPy arrays; the wrapper the
+reference's CuPy pickles use (``cupy._core.core.array``) is mapped to
+``numpy.asarray`` so such a file loads without CuPy and without executing
+anything else from it.
+"""
+import io
+import pickle
+
+import numpy as np
+
+from .layers import (Activation_Softmax_Loss_CategoricalCrossEntropy, Loss_CategoricalCrossEntropy, SoftMax)
+
+
+class _ArrayOnlyUnpickler(pickle.Unpickler):
+    _ALLOWED = {
+        ("numpy.core.multiarray", "_reconstruct"),
+        ("numpy._core.multiarray", "_reconstruct"),
+        ("numpy", "ndarray"),
+        ("numpy", "dtype"),
+        ("numpy.core.multiarray", "scalar"),
+        ("numpy._core.multiarray", "scalar"),
+    }
+
+    def find_class(self, module, name):
+        if (module, name) in self._ALLOWED:
+            return super().find_class(module, name)
+        if module.startswith("cupy") and name == "array":
+            return np.asarray
+        raise pickle.UnpicklingError("parameter files may only contain NumPy arrays (found %s.%s)" % (module, name))
+
+
+class Model:
+    def __init__(self):
+        self.layers = []
+        self.softmax_classifier_output = None
+
+    def add(self, layer):
+        self.layers.append(layer)
+
+    def set(self, *, loss=None, optimizer=None, accuracy=None):
+        if loss is not None:
+            self.loss = loss
+        if optimizer is not None:
+            self.optimizer = optimizer
+        if accuracy is not None:
+            self.accuracy = accuracy
+
+    def finalize(self):
+        self.input_layer = Layer_Input()
+        layer_count = len(self.layers)
+        self.trainable_layers = []
+        for i in range(layer_count):
+            if i == 0:
+                self.layers[i].prev = self.input_layer
+                self.layers[i].next = self.layers[i + 1]
+            elif i < layer_count - 1:
+                self.layers[i].prev = self.layers[i - 1]
+                self.layers[i].next = self.layers[i + 1]
+            else:
+                self.layers[i].prev = self.layers[i - 1]
+                self.layers[i].next = self.loss
+                self.output_layer_activation = self.layers[i]
+            if hasattr(self.layers[i], 'weights'):
+                self.trainable_layers.append(self.layers[i])
+        if self.loss is not None:
+            self.loss.remember_trainable_layers(self.trainable_layers)
+        if isinstance(self.layers[-1], SoftMax) and isinstance(self.loss, Loss_CategoricalCrossEntropy):
+            self.softmax_classifier_output = \
+                Activation_Softmax_Loss_CategoricalCrossEntropy(self.loss.label_smoothing)
+
+    def train(self, X, y, *, epochs=1, batch_size=None, print_every=1, validation_data=None):
+        self.accuracy.init(y)
+        train_steps = 1
+        if validation_data is not None:
+            X_val, y_val = validation_data
+        if batch_size is not None:
+            train_steps = len(X) // batch_size
+            if train_steps * batch_size < len(X):
+                train_steps += 1
+        print("Training")
+        for epoch in range(1, epochs + 1):
+            print(f' epoch: {epoch}')
+            self.loss.new_pass()
+            self.accuracy.new_pass()
+            for step in range(train_steps):
+                if batch_size is None:
+                    batch_X = X
+                    batch_y = y
+                else:
+                    batch_X = X[step * batch_size:(step + 1) * batch_size]
+                    batch_y = y[step * batch_size:(step + 1) * batch_size]
+                loss, data_loss, regularization_loss, accuracy = self.train_step(batch_X, batch_y)
+                if not step % print_every or step == train_steps - 1:
+                    print(f'epoch: {epoch}, ' +
+                          f'acc: {accuracy:.3f}, ' +
+                          f'loss: {loss:.3f} (' +
+                          f'data_loss: {data_loss:.3f}, ' +
+                          f'reg_loss: {regularization_loss:.3f}, ' +
+                          f'lr:: {self.optimizer.current_learning_rate}')
+        epoch_data_loss, epoch_regularization_loss = \
+            self.loss.calculate_accumulated(include_regularization=True)
+        epoch_loss = epoch_data_loss + epoch_regularization_loss
+        epoch_accuracy = self.accuracy.calculate_accumulated()
+        print(f' training, ' +
+              f'acc: {epoch_accuracy:.3f}, ' +
+              f'loss: {epoch_loss:.3f} (' +
+              f'data_loss: {epoch_data_loss:.3f}, ' +
+              f'reg_loss: {epoch_regularization_loss:.3f}, ' +
+              f'lr:: {self.optimizer.current_learning_rate}')
+        if validation_data is not None:
+            self.evaluate(*validation_data, batch_size=batch_size)
+
+    def train_step(self, batch_X, batch_y):
+        """One iteration of the loop body of ``train`` (CNN_model_cupy.py:107-126):
+        forward, loss, accuracy, backward, Adam.  Returns (loss, data_loss,
+        regularization_loss, accuracy)."""
+        output = self.forward(batch_X, training=True)
+        data_loss, regularization_loss = self.loss.calculate(output, batch_y, include_regularization=True,
+                                                             training=True)
+        loss = data_loss + regularization_loss
+        predictions = self.output_layer_activation.predictions(output)
+        accuracy = self.accuracy.calculate(predictions, batch_y)
+        self.backward(output, batch_y)
+        self.optimizer.pre_update_parameters()
+        for layer in self.trainable_layers:
+            self.optimizer.update_parameters(layer)
+        self.optimizer.post_update_parameters()
+        return loss, data_loss, regularization_loss, accuracy
+
+    def forward(self, X, training):
+        self.input_layer.forward(X, training)
+        for layer in self.layers:
+            layer.forward(layer.prev.output, training)
+        return layer.output
+
+    def backward(self, output, y):
+        if self.softmax_classifier_output is not None:
+            self.softmax_classifier_output.backward(output, y, training=True)
+            self.layers[-1].dinputs = self.softmax_classifier_output.dinputs
+            for layer in reversed(self.layers[:-1]):
+                layer.backward(layer.next.dinputs)
+            return
+        self.loss.backward(output, y)
+        for layer in reversed(self.layers):
+            layer.backward(layer.next.dinputs)
+
+    def backward_debug(self, X, y):
+        out = X
+        print("Forward pass:")
+        for i, layer in enumerate(self.layers):
+            layer.forward(out, training=True)
+            out = layer.output
+            print(f"Layer {i} ({layer.__class__.__name__}) output: {out.shape}")
+        print("\nBackward pass:")
+        if self.softmax_classifier_output is not None:
+            self.softmax_classifier_output.backward(out, y)
+            self.layers[-1].dinputs = self.softmax_classifier_output.dinputs
+            chain = list(enumerate(reversed(self.layers[:-1])))
+            first = -2
+        else:
+            self.loss.backward(out, y)
+            chain = list(enumerate(reversed(self.layers)))
+            first = -1
+        for i, layer in chain:
+            layer.backward(layer.next.dinputs)
+            print(f"Layer {first - i} ({layer.__class__.__name__}) dinputs: {layer.dinputs.shape}")
+            if hasattr(layer, 'dweights'):
+                print(f"             dweights: {layer.dweights.shape}")
+            if hasattr(layer, 'dbiases'):
+                print(f"             dbiases: {layer.dbiases.shape}")
+
+    def evaluate(self, X_val, y_val, *, batch_size=None):
+        validation_steps = 1
+        if batch_size is not None:
+            validation_steps = len(X_val) // batch_size
+            if validation_steps * batch_size < len(X_val):
+                validation_steps += 1
+        self.loss.new_pass()
+        self.accuracy.new_pass()
+        for step in range(validation_steps):
+            if batch_size is None:
+                batch_X = X_val
+                batch_y = y_val
+            else:
+                batch_X = X_val[step * batch_size:(step + 1) * batch_size]
+                batch_y = y_val[step * batch_size:(step + 1) * batch_size]
+            output = self.forward(batch_X, training=False)
+            self.loss.calculate(output, batch_y, training=False)
+            predictions = self.output_layer_activation.predictions(output)
+            self.accuracy.calculate(predictions, batch_y)
+        validation_loss = self.loss.calculate_accumulated()
+        validation_accuracy = self.accuracy.calculate_accumulated()
+        print(f'Valdiation, ' +
+              f'acc: {validation_accuracy:.3f}, ' +
+              f'loss: {validation_loss:.3f}')
+
+    def get_parameters(self):
+        parameters = []
+        for layer in self.trainable_layers:
+            parameters.append(layer.get_parameters())
+        return parameters
+
+    def set_parameters(self, parameters):
+        for parameter_set, layer in zip(parameters, self.trainable_layers):
+            layer.set_parameters(*parameter_set)
+
+    def save_parameters(self, path):
+        host = [tuple(np.asarray(a) for a in tup) for tup in self.get_parameters()]
+        with open(path, 'wb') as f:
+            pickle.dump(host, f)
+
+    def load_parameters(self, path):
+        with open(path, 'rb') as f:
+            self.set_parameters(_ArrayOnlyUnpickler(io.BytesIO(f.read())).load())
+
+    def save(self, path):
+        raise NotImplementedError(
+            "whole-model pickles are not supported (device buffers cannot be pickled); use save_parameters")
+
+    @staticmethod
+    def load(path):
+        raise NotImplementedError(
+            "whole-model pickles are not supported (device buffers cannot be pickled); use load_parameters")
+
+    def predict(self, X, *, batch_size=None):
+        prediction_steps = 1
+        if batch_size is not None:
+            prediction_steps = len(X) // batch_size
+            if prediction_steps * batch_size < len(X):
+                prediction_steps += 1
+        output = []
+        for step in range(prediction_steps):
+            if batch_size is None:
+                batch_X = X
+            else:
+                batch_X = X[step * batch_size:(step + 1) * batch_size]
+            batch_output = self.forward(batch_X, training=False)
+            output.append(np.asarray(batch_output))
+        return np.vstack(output)
+
+
+class Accuracy:
+    def calculate(self, predictions, y):
+        comparisons = self.compare(predictions, y)
+        accuracy = np.mean(comparisons)
+        self.accumulated_sum += np.sum(comparisons)
+        self.accumulated_count += len(comparisons)
+        return accuracy
+
+    def calculate_accumulated(self):
+        accuracy = self.accumulated_sum / self.accumulated_count
+        return accuracy
+
+    def new_pass(self):
+        self.accumulated_sum = 0
+        self.accumulated_count = 0
+
+
+class Accuracy_Regression(Accuracy):
+    def __init__(self):
+        self.precision = None
+
+    def init(self, y, reinit=False):
+        if self.precision is None or reinit:
+            self.precision = np.std(np.asarray(y)) / 250
+
+    def compare(self, predictions, y):
+        return np.absolute(np.asarray(predictions) - np.asarray(y)) < self.precision
+
+
+class Accuracy_Categorical(Accuracy):
+    def init(self, y):
+        pass
+
+    def compare(self, predictions, y):
+        y = np.asarray(y)
+        if len(y.shape) == 2:
+            y = np.argmax(y, axis=1)
+        return np.asarray(predictions) == y
+
+
+class Layer_Input:
+    def forward(self, inputs, training):
+        self.output = inputs

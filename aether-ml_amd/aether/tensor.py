@@ -1,0 +1,142 @@
+"""DeviceTensor: a dense C-contiguous array living in MI355X HBM, owned through
+aeth_malloc / aeth_free.  It plays the role the CuPy ndarray plays in the
+reference (CNN/models/CNN_classes_cupy.py): layers keep activations and
+parameters in it between forward and backward, and ``np.asarray(t)`` / ``t.get()``
+bring a copy to the host."""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+
+
+class DeviceTensor:
+    __slots__ = ("ptr", "shape", "dtype", "_base", "__weakref__")
+
+    def __init__(self, shape, dtype=np.float32, _ptr=None, _base=None):
+        if isinstance(shape, (int, np.integer)):
+            shape = (int(shape),)
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = np.dtype(dtype)
+        self._base = _base
+        if _ptr is None:
+            p = C.c_void_p()
+            _lib.check(_lib.lib().aeth_malloc(C.byref(p), self.nbytes))
+            self.ptr = p.value
+        else:
+            self.ptr = _ptr
+
+    # -- construction ---------------------------------------------------------------
+    @classmethod
+    def from_numpy(cls, a, dtype=None):
+        a = np.ascontiguousarray(a, dtype=dtype if dtype is not None else None)
+        t = cls(a.shape, a.dtype)
+        if a.nbytes:
+            _lib.check(_lib.lib().aeth_memcpy_h2d(t.ptr, a.ctypes.data, a.nbytes))
+        return t
+
+    @classmethod
+    def zeros(cls, shape, dtype=np.float32):
+        t = cls(shape, dtype)
+        t.fill(0)
+        return t
+
+    @classmethod
+    def full(cls, shape, value, dtype=np.float32):
+        t = cls(shape, dtype)
+        t.fill(value)
+        return t
+
+    # -- properties -------------------------------------------------------------------
+    @property
+    def size(self):
+        n = 1
+        for s in self.shape:
+            n *= s
+        return n
+
+    @property
+    def nbytes(self):
+        return self.size * self.dtype.itemsize
+
+    @property
+    def ndim(self):
+        return len(self.shape)
+
+    def __len__(self):
+        return self.shape[0]
+
+    # -- host transfer ------------------------------------------------------------------
+    def get(self):
+        out = np.empty(self.shape, dtype=self.dtype)
+        if out.nbytes:
+            _lib.check(_lib.lib().aeth_memcpy_d2h(out.ctypes.data, self.ptr, out.nbytes))
+        return out
+
+    numpy = get
+
+    def __array__(self, dtype=None, copy=None):
+        a = self.get()
+        return a if dtype is None else a.astype(dtype, copy=False)
+
+    def set(self, a):
+        a = np.ascontiguousarray(a, dtype=self.dtype)
+        if a.shape != self.shape:
+            if a.size != self.size:
+                raise ValueError("cannot set shape %s from %s" % (self.shape, a.shape))
+            a = a.reshape(self.shape)
+        if a.nbytes:
+            _lib.check(_lib.lib().aeth_memcpy_h2d(self.ptr, a.ctypes.data, a.nbytes))
+        return self
+
+    # -- device ops -----------------------------------------------------------------------
+    def fill(self, value):
+        if self.size == 0:
+            return self
+        if self.dtype == np.float32:
+            _lib.check(_lib.lib().aeth_fill_f32(self.ptr, float(value), self.size))
+        else:
+            self.set(np.full(self.shape, value, dtype=self.dtype))
+        return self
+
+    def copy(self):
+        t = DeviceTensor(self.shape, self.dtype)
+        if self.nbytes:
+            _lib.check(_lib.lib().aeth_memcpy_d2d(t.ptr, self.ptr, self.nbytes))
+        return t
+
+    def reshape(self, *shape):
+        if len(shape) == 1 and isinstance(shape[0], (tuple, list)):
+            shape = tuple(shape[0])
+        shape = list(int(s) for s in shape)
+        if -1 in shape:
+            known = 1
+            for s in shape:
+                if s != -1:
+                    known *= s
+            shape[shape.index(-1)] = self.size // known if known else 0
+        n = 1
+        for s in shape:
+            n *= s
+        if n != self.size:
+            raise ValueError("cannot reshape %s into %s" % (self.shape, tuple(shape)))
+        return DeviceTensor(shape, self.dtype, _ptr=self.ptr, _base=self._base if self._base is not None else self)
+
+    def __repr__(self):
+        return "DeviceTensor(shape=%s, dtype=%s)" % (self.shape, self.dtype)
+
+    def __del__(self):
+        try:
+            if self._base is None and self.ptr and _lib._lib is not None and _lib._initialised:
+                _lib._lib.aeth_free(self.ptr)
+        except Exception:
+            pass
+
+
+def as_device(a, dtype=np.float32):
+    """Pass a DeviceTensor through; upload anything array-like as ``dtype``."""
+    if isinstance(a, DeviceTensor):
+        if a.dtype != np.dtype(dtype):
+            return DeviceTensor.from_numpy(a.get().astype(dtype))
+        return a
+    return DeviceTensor.from_numpy(np.asarray(a), dtype=dtype)

@@ -1,0 +1,87 @@
+// Shared host-side plumbing of libaether_hip.so: the process-wide context,
+// error reporting, the scratch workspace and small device helpers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/aether_hip.h"
+
+namespace aeth {
+
+struct Context {
+    bool ready = false;
+    int device = -1;
+    hipStream_t stream = nullptr;
+    hipDeviceProp_t prop;
+    // scratch owned by the library (packed filters, split partial sums)
+    void* ws = nullptr;
+    int64_t ws_bytes = 0;
+    // small always-present buffer for counters used by single-pass reductions
+    unsigned int* counters = nullptr;
+};
+
+Context& ctx();
+int fail(int code, const char* fmt, ...);
+// Returns a pointer to at least `bytes` of scratch; grows the buffer when
+// needed (synchronises the stream before freeing the old one).
+int workspace(int64_t bytes, void** out);
+
+#define AETH_REQUIRE_INIT()                                                     \
+    do {                                                                        \
+        if (!aeth::ctx().ready) return aeth::fail(AETH_E_STATE, "%s: aeth_init has not been called", __func__); \
+    } while (0)
+
+#define AETH_CHECK_ARG(cond)                                                    \
+    do {                                                                        \
+        if (!(cond)) return aeth::fail(AETH_E_INVALID, "%s: argument check failed: %s", __func__, #cond); \
+    } while (0)
+
+#define AETH_HIP(call)                                                          \
+    do {                                                                        \
+        hipError_t e__ = (call);                                                \
+        if (e__ != hipSuccess)                                                  \
+            return aeth::fail(e__ == hipErrorOutOfMemory ? AETH_E_NOMEM : AETH_E_HIP, \
+                              "%s: %s -> %s", __func__, #call, hipGetErrorString(e__)); \
+    } while (0)
+
+#define AETH_LAUNCH_CHECK()                                                     \
+    do {                                                                        \
+        hipError_t e__ = hipGetLastError();                                     \
+        if (e__ != hipSuccess)                                                  \
+            return aeth::fail(AETH_E_HIP, "%s: kernel launch -> %s", __func__, hipGetErrorString(e__)); \
+    } while (0)
+
+// Division by a runtime-constant positive divisor for 0 <= n < 2^31:
+// q = umulhi(n, mul) >> shr (d == 1 is passed through).
+struct FastDiv {
+    unsigned int d, mul, shr;
+    FastDiv() : d(1), mul(0), shr(0) {}
+    explicit FastDiv(int div) : d((unsigned)div), mul(0), shr(0) {
+        if (div > 1) {
+            unsigned l = 0;
+            while ((1u << l) < (unsigned)div) ++l;           // ceil(log2 d)
+            unsigned p = 31 + l;
+            mul = (unsigned)(((1ull << p) + (unsigned)div - 1) / (unsigned)div);
+            shr = p - 32;
+        }
+    }
+    __host__ __device__ __forceinline__ unsigned div(unsigned n) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+        return d == 1 ? n : (__umulhi(n, mul) >> shr);
+#else
+        return d == 1 ? n : (unsigned)(((unsigned long long)n * mul) >> 32) >> shr;
+#endif
+    }
+    __host__ __device__ __forceinline__ void divmod(unsigned n, unsigned& q, unsigned& r) const {
+        q = div(n);
+        r = n - q * d;
+    }
+};
+
+static inline int cdiv(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+static inline int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
+
+}  // namespace aeth

@@ -1,0 +1,678 @@
+// Coalesced helper kernels for the layers either side of the convolution path:
+// batch norm, ReLU / leaky ReLU, pooling, dropout masks, softmax + cross entropy,
+// Adam, regulariser terms.  All tensors are row-major with the channel (or
+// class) axis last, so consecutive lanes touch consecutive addresses.
+#include "common.h"
+
+namespace aeth {
+
+constexpr int kEwThreads = 256;
+
+static inline int ew_blocks(int64_t n, int per_thread = 1) {
+    int64_t b = (n + (int64_t)kEwThreads * per_thread - 1) / ((int64_t)kEwThreads * per_thread);
+    if (b > 8192) b = 8192;
+    if (b < 1) b = 1;
+    return (int)b;
+}
+
+// ------------------------------------------------------------------------------
+// column reductions over a [rows, C] matrix
+// Lane layout: when C < 64 divides 64 a wave covers 64/C rows per step, otherwise
+// columns are tiled by 64 (blockIdx.y).  Each block reduces `rows_per_block` rows
+// and writes NV partial values per column to part[(v*nblk + blockIdx.x)*C + c];
+// a second kernel finishes in block order, so results do not depend on timing.
+// ------------------------------------------------------------------------------
+__device__ __forceinline__ void col_layout(int C, int& lanes_c, int& sub_rows) {
+    lanes_c = (C < 64 && (64 % C) == 0) ? C : 64;
+    sub_rows = 64 / lanes_c;
+}
+
+template <int NV, typename F>
+__device__ __forceinline__ void column_partials(int rows, int C, int rows_per_block, float* __restrict__ part, F f) {
+    __shared__ float red[NV][kEwThreads];
+    int lanes_c, sub_rows;
+    col_layout(C, lanes_c, sub_rows);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int c = blockIdx.y * 64 + (lane % lanes_c);
+    const int rl = wave * sub_rows + lane / lanes_c;   // row lane inside the block
+    const int nrl = 4 * sub_rows;
+    const int rbeg = blockIdx.x * rows_per_block;
+    int rend = rbeg + rows_per_block;
+    if (rend > rows) rend = rows;
+    float acc[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[v] = 0.f;
+    if (c < C) {
+        for (int r = rbeg + rl; r < rend; r += nrl) f((size_t)r * C + c, c, acc);
+    }
+#pragma unroll
+    for (int v = 0; v < NV; ++v) red[v][tid] = acc[v];
+    __syncthreads();
+    // thread with rl == 0 owns column c: sum the nrl row lanes in fixed order
+    if (rl == 0 && c < C) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            float s = 0.f;
+            for (int w = 0; w < 4; ++w)
+                for (int sr = 0; sr < sub_rows; ++sr) s += red[v][w * 64 + sr * lanes_c + (lane % lanes_c)];
+            part[((size_t)v * gridDim.x + blockIdx.x) * C + c] = s;
+        }
+    }
+}
+
+static void col_grid(int rows, int C, int* nblk, int* rows_per_block, dim3* grid) {
+    int nb = cdiv(rows, 256);
+    if (nb > 512) nb = 512;
+    if (nb < 1) nb = 1;
+    int rpb = cdiv(rows, nb);
+    nb = cdiv(rows, rpb);
+    *nblk = nb;
+    *rows_per_block = rpb;
+    *grid = dim3(nb, cdiv(C, 64));
+}
+
+// ---- batch norm ------------------------------------------------------------------
+// Statistics use sums of (x - shift) and (x - shift)^2 with shift = x[0][c]: the
+// variance then comes from numbers of the size of the spread, not of the mean.
+__global__ __launch_bounds__(kEwThreads) void bn_stats_partial(const float* __restrict__ x, int rows, int C,
+                                                              int rpb, float* __restrict__ part) {
+    column_partials<2>(rows, C, rpb, part, [&](size_t i, int c, float* acc) {
+        float d = x[i] - x[c];
+        acc[0] += d;
+        acc[1] += d * d;
+    });
+}
+
+__global__ void bn_stats_final(const float* __restrict__ x, const float* __restrict__ part, int nblk, int rows, int C,
+                               float eps, float momentum, float* __restrict__ running_mean,
+                               float* __restrict__ running_var, float* __restrict__ save_mean,
+                               float* __restrict__ save_invstd) {
+    int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    float s1 = 0.f, s2 = 0.f;
+    for (int b = 0; b < nblk; ++b) {
+        s1 += part[(size_t)b * C + c];
+        s2 += part[((size_t)nblk + b) * C + c];
+    }
+    const float inv_n = 1.0f / (float)rows;
+    const float dm = s1 * inv_n;
+    const float mean = x[c] + dm;
+    float var = s2 * inv_n - dm * dm;
+    if (var < 0.f) var = 0.f;
+    save_mean[c] = mean;
+    save_invstd[c] = 1.0f / sqrtf(var + eps);
+    running_mean[c] = momentum * running_mean[c] + (1.0f - momentum) * mean;
+    running_var[c] = momentum * running_var[c] + (1.0f - momentum) * var;
+}
+
+// y = gamma * (x - mean) * invstd + beta
+__global__ void bn_apply(const float* __restrict__ x, const float* __restrict__ gamma, const float* __restrict__ beta,
+                         const float* __restrict__ mean, const float* __restrict__ invstd, float* __restrict__ y,
+                         int64_t n, int C) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        int c = (int)(i % C);
+        y[i] = gamma[c] * ((x[i] - mean[c]) * invstd[c]) + beta[c];
+    }
+}
+
+__global__ void bn_apply_infer(const float* __restrict__ x, const float* __restrict__ gamma,
+                               const float* __restrict__ beta, const float* __restrict__ rm,
+                               const float* __restrict__ rv, float* __restrict__ y, int64_t n, int C, float eps) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        int c = (int)(i % C);
+        y[i] = gamma[c] * ((x[i] - rm[c]) / sqrtf(rv[c] + eps)) + beta[c];
+    }
+}
+
+__global__ __launch_bounds__(kEwThreads) void bn_bwd_partial(const float* __restrict__ x, const float* __restrict__ dy,
+                                                            const float* __restrict__ mean, int rows, int C, int rpb,
+                                                            float* __restrict__ part) {
+    column_partials<2>(rows, C, rpb, part, [&](size_t i, int c, float* acc) {
+        float g = dy[i];
+        acc[0] += g;
+        acc[1] += g * (x[i] - mean[c]);
+    });
+}
+
+// coef[0*C+c] = gamma*invstd ; coef[1*C+c] = A ; coef[2*C+c] = B  with
+// dx = coef0*dy + A*(x-mean) + B,  A = -gamma*s2*invstd^3/N,  B = -gamma*invstd*s1/N
+__global__ void bn_bwd_final(const float* __restrict__ part, int nblk, int rows, int C,
+                             const float* __restrict__ gamma, const float* __restrict__ invstd,
+                             float* __restrict__ dgamma, float* __restrict__ dbeta, float* __restrict__ coef) {
+    int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    float s1 = 0.f, s2 = 0.f;
+    for (int b = 0; b < nblk; ++b) {
+        s1 += part[(size_t)b * C + c];
+        s2 += part[((size_t)nblk + b) * C + c];
+    }
+    const float is = invstd[c], g = gamma[c];
+    const float inv_n = 1.0f / (float)rows;
+    dgamma[c] = s2 * is;
+    dbeta[c] = s1;
+    coef[c] = g * is;
+    coef[C + c] = -g * s2 * is * is * is * inv_n;
+    coef[2 * C + c] = -g * is * s1 * inv_n;
+}
+
+__global__ void bn_bwd_apply(const float* __restrict__ x, const float* __restrict__ dy, const float* __restrict__ mean,
+                             const float* __restrict__ coef, float* __restrict__ dx, int64_t n, int C) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        int c = (int)(i % C);
+        dx[i] = coef[c] * dy[i] + coef[C + c] * (x[i] - mean[c]) + coef[2 * C + c];
+    }
+}
+
+// ---- elementwise ---------------------------------------------------------------------
+__global__ void relu_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, float alpha, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        float v = x[i];
+        y[i] = v > 0.f ? v : alpha * v;
+    }
+}
+
+__global__ void relu_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy, float* __restrict__ dx,
+                                float alpha, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) dx[i] = x[i] < 0.f ? alpha * dy[i] : dy[i];
+}
+
+__global__ void mul_mask_kernel(const float* __restrict__ x, const float* __restrict__ mask, float* __restrict__ y,
+                                int64_t n, int64_t mask_n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) y[i] = x[i] * mask[i % mask_n];
+}
+
+__global__ void axpy_kernel(float alpha, const float* __restrict__ x, float* __restrict__ y, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) y[i] += alpha * x[i];
+}
+
+__global__ void l1_grad_kernel(float lambda, const float* __restrict__ w, float* __restrict__ dw, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) dw[i] += w[i] < 0.f ? -lambda : lambda;
+}
+
+__global__ void cast_bf16_kernel(const float* __restrict__ src, uint16_t* __restrict__ dst, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        unsigned u = __float_as_uint(src[i]);
+        unsigned r;
+        if ((u & 0x7fffffffu) > 0x7f800000u) r = (u >> 16) | 0x40u;   // NaN stays NaN
+        else r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+        dst[i] = (uint16_t)r;
+    }
+}
+
+__global__ void adam_kernel(float* __restrict__ theta, const float* __restrict__ g, float* __restrict__ m,
+                            float* __restrict__ v, int64_t n, float lr, float b1, float b2, float eps, float c1,
+                            float c2) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        float gi = g[i];
+        float mi = b1 * m[i] + (1.0f - b1) * gi;
+        float vi = b2 * v[i] + (1.0f - b2) * (gi * gi);
+        m[i] = mi;
+        v[i] = vi;
+        float mh = mi / c1;
+        float vh = vi / c2;
+        theta[i] += -lr * mh / (sqrtf(vh) + eps);
+    }
+}
+
+// single block: out[0] = sum |x| or sum x^2, summed in a fixed tree
+__global__ __launch_bounds__(1024) void reduce_kernel(const float* __restrict__ x, int64_t n, int mode,
+                                                      float* __restrict__ out) {
+    __shared__ float red[1024];
+    float s = 0.f;
+    for (int64_t i = threadIdx.x; i < n; i += 1024) {
+        float v = x[i];
+        s += mode == 0 ? fabsf(v) : v * v;
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 512; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[0] = red[0];
+}
+
+// ---- pooling ---------------------------------------------------------------------------
+struct PoolParams {
+    int S, H, W, C, Ho, Wo, fH, fW, sH, sW;
+};
+
+__global__ void maxpool_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, uint8_t* __restrict__ idx,
+                                   PoolParams p, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        int c = (int)(i % p.C);
+        int64_t t = i / p.C;
+        int wo = (int)(t % p.Wo);
+        t /= p.Wo;
+        int ho = (int)(t % p.Ho);
+        int s = (int)(t / p.Ho);
+        const float* base = x + (((size_t)s * p.H + (size_t)ho * p.sH) * p.W + (size_t)wo * p.sW) * p.C + c;
+        float best = base[0];
+        int bi = 0;
+        for (int fh = 0; fh < p.fH; ++fh)
+            for (int fw = 0; fw < p.fW; ++fw) {
+                float v = base[((size_t)fh * p.W + fw) * p.C];
+                if (v > best) {          // strict: the first maximum keeps its place
+                    best = v;
+                    bi = fh * p.fW + fw;
+                }
+            }
+        y[i] = best;
+        idx[i] = (uint8_t)bi;
+    }
+}
+
+// gather form of the scatter-add: every input element sums, in (h,w) order, the
+// windows that contain it and whose argmax points at it
+__global__ void maxpool_bwd_kernel(const float* __restrict__ dy, const uint8_t* __restrict__ idx,
+                                   float* __restrict__ dx, PoolParams p, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        int c = (int)(i % p.C);
+        int64_t t = i / p.C;
+        int col = (int)(t % p.W);
+        t /= p.W;
+        int row = (int)(t % p.H);
+        int s = (int)(t / p.H);
+        int h_lo = row - p.fH + 1;
+        h_lo = h_lo <= 0 ? 0 : (h_lo + p.sH - 1) / p.sH;
+        int h_hi = row / p.sH;
+        if (h_hi > p.Ho - 1) h_hi = p.Ho - 1;
+        int w_lo = col - p.fW + 1;
+        w_lo = w_lo <= 0 ? 0 : (w_lo + p.sW - 1) / p.sW;
+        int w_hi = col / p.sW;
+        if (w_hi > p.Wo - 1) w_hi = p.Wo - 1;
+        float acc = 0.f;
+        for (int h = h_lo; h <= h_hi; ++h)
+            for (int w = w_lo; w <= w_hi; ++w) {
+                size_t o = (((size_t)s * p.Ho + h) * p.Wo + w) * p.C + c;
+                int want = (row - h * p.sH) * p.fW + (col - w * p.sW);
+                if ((int)idx[o] == want) acc += dy[o];
+            }
+        dx[i] = acc;
+    }
+}
+
+__global__ void avgpool_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, PoolParams p, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const float inv = 1.0f / (float)(p.fH * p.fW);
+    for (; i < n; i += stride) {
+        int c = (int)(i % p.C);
+        int64_t t = i / p.C;
+        int wo = (int)(t % p.Wo);
+        t /= p.Wo;
+        int ho = (int)(t % p.Ho);
+        int s = (int)(t / p.Ho);
+        const float* base = x + (((size_t)s * p.H + (size_t)ho * p.sH) * p.W + (size_t)wo * p.sW) * p.C + c;
+        float acc = 0.f;
+        for (int fh = 0; fh < p.fH; ++fh)
+            for (int fw = 0; fw < p.fW; ++fw) acc += base[((size_t)fh * p.W + fw) * p.C];
+        y[i] = acc * inv;
+    }
+}
+
+__global__ void avgpool_bwd_kernel(const float* __restrict__ dy, float* __restrict__ dx, PoolParams p, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const float div = (float)(p.fH * p.fW);
+    for (; i < n; i += stride) {
+        int c = (int)(i % p.C);
+        int64_t t = i / p.C;
+        int col = (int)(t % p.W);
+        t /= p.W;
+        int row = (int)(t % p.H);
+        int s = (int)(t / p.H);
+        int h_lo = row - p.fH + 1;
+        h_lo = h_lo <= 0 ? 0 : (h_lo + p.sH - 1) / p.sH;
+        int h_hi = row / p.sH;
+        if (h_hi > p.Ho - 1) h_hi = p.Ho - 1;
+        int w_lo = col - p.fW + 1;
+        w_lo = w_lo <= 0 ? 0 : (w_lo + p.sW - 1) / p.sW;
+        int w_hi = col / p.sW;
+        if (w_hi > p.Wo - 1) w_hi = p.Wo - 1;
+        float acc = 0.f;
+        for (int h = h_lo; h <= h_hi; ++h)
+            for (int w = w_lo; w <= w_hi; ++w) acc += dy[(((size_t)s * p.Ho + h) * p.Wo + w) * p.C + c] / div;
+        dx[i] = acc;
+    }
+}
+
+// ---- softmax / cross entropy (one thread per row; K is the class count) -----------------
+__global__ void softmax_kernel(const float* __restrict__ logits, float* __restrict__ probs, int rows, int K) {
+    int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= rows) return;
+    const float* in = logits + (size_t)r * K;
+    float* out = probs + (size_t)r * K;
+    float mx = in[0];
+    for (int k = 1; k < K; ++k) mx = fmaxf(mx, in[k]);
+    float sum = 0.f;
+    for (int k = 0; k < K; ++k) {
+        float e = expf(in[k] - mx);
+        out[k] = e;
+        sum += e;
+    }
+    for (int k = 0; k < K; ++k) out[k] = out[k] / sum;
+}
+
+__global__ void softmax_bwd_kernel(const float* __restrict__ probs, const float* __restrict__ dy,
+                                   float* __restrict__ dx, int rows, int K) {
+    int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= rows) return;
+    const float* p = probs + (size_t)r * K;
+    const float* g = dy + (size_t)r * K;
+    float dot = 0.f;
+    for (int k = 0; k < K; ++k) dot += p[k] * g[k];
+    for (int k = 0; k < K; ++k) dx[(size_t)r * K + k] = p[k] * (g[k] - dot);
+}
+
+__global__ void cce_fwd_kernel(const float* __restrict__ probs, const int32_t* __restrict__ labels, float ls,
+                               float* __restrict__ loss, int32_t* __restrict__ correct, int rows, int K) {
+    int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= rows) return;
+    const float* p = probs + (size_t)r * K;
+    const int y = labels[r];
+    const float t_off = ls / (float)K;
+    const float t_on = (1.0f - ls) + t_off;
+    float acc = 0.f;
+    float best = p[0];
+    int bi = 0;
+    for (int k = 0; k < K; ++k) {
+        float v = p[k];
+        if (v > best) {
+            best = v;
+            bi = k;
+        }
+        float pc = fminf(fmaxf(v, 1e-7f), 1.0f - 1e-7f);
+        float t = (k == y) ? t_on : t_off;
+        acc += t * logf(pc);
+    }
+    loss[r] = -acc;
+    correct[r] = (bi == y) ? 1 : 0;
+}
+
+__global__ void softmax_cce_bwd_kernel(const float* __restrict__ probs, const int32_t* __restrict__ labels, float ls,
+                                       float* __restrict__ dlogits, int rows, int K) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= rows * K) return;
+    int r = i / K, k = i - r * K;
+    const float t_off = ls / (float)K;
+    float t = (k == labels[r]) ? (1.0f - ls) + t_off : t_off;
+    dlogits[i] = (probs[i] - t) / (float)rows;
+}
+
+static int pool_dims(const char* fn, int S, int H, int W, int C, int fH, int fW, int sH, int sW, PoolParams* p) {
+    if (S <= 0 || H <= 0 || W <= 0 || C <= 0 || fH <= 0 || fW <= 0 || sH <= 0 || sW <= 0)
+        return fail(AETH_E_INVALID, "%s: non-positive dimension", fn);
+    if (fH > H || fW > W) return fail(AETH_E_INVALID, "%s: window larger than input", fn);
+    if (fH * fW > 256) return fail(AETH_E_INVALID, "%s: window larger than 256 elements", fn);
+    p->S = S; p->H = H; p->W = W; p->C = C; p->fH = fH; p->fW = fW; p->sH = sH; p->sW = sW;
+    p->Ho = (H - fH) / sH + 1;
+    p->Wo = (W - fW) / sW + 1;
+    if ((int64_t)S * H * W * C >= ((int64_t)1 << 31)) return fail(AETH_E_INVALID, "%s: tensor too large", fn);
+    return AETH_OK;
+}
+
+}  // namespace aeth
+
+using namespace aeth;
+
+#define EW_LAUNCH(kernel, n, ...)                                                          \
+    do {                                                                                   \
+        hipLaunchKernelGGL(kernel, dim3(ew_blocks(n)), dim3(kEwThreads), 0, ctx().stream, __VA_ARGS__); \
+        AETH_LAUNCH_CHECK();                                                               \
+    } while (0)
+
+extern "C" {
+
+int aeth_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, float* running_mean,
+                          float* running_var, float* save_mean, float* save_invstd, float* y, int rows, int C,
+                          float eps, float momentum) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(x && gamma && beta && running_mean && running_var && save_mean && save_invstd && y);
+    AETH_CHECK_ARG(rows > 0 && C > 0 && (int64_t)rows * C < ((int64_t)1 << 31));
+    int nblk, rpb;
+    dim3 grid;
+    col_grid(rows, C, &nblk, &rpb, &grid);
+    void* ws;
+    int rc = workspace((int64_t)2 * nblk * C * sizeof(float), &ws);
+    if (rc) return rc;
+    float* part = (float*)ws;
+    hipStream_t st = ctx().stream;
+    hipLaunchKernelGGL(bn_stats_partial, grid, dim3(kEwThreads), 0, st, x, rows, C, rpb, part);
+    AETH_LAUNCH_CHECK();
+    hipLaunchKernelGGL(bn_stats_final, dim3(cdiv(C, 64)), dim3(64), 0, st, x, part, nblk, rows, C, eps, momentum,
+                       running_mean, running_var, save_mean, save_invstd);
+    AETH_LAUNCH_CHECK();
+    int64_t n = (int64_t)rows * C;
+    EW_LAUNCH(bn_apply, n, x, gamma, beta, save_mean, save_invstd, y, n, C);
+    return AETH_OK;
+}
+
+int aeth_bn_fwd_infer_f32(const float* x, const float* gamma, const float* beta, const float* running_mean,
+                          const float* running_var, float* y, int rows, int C, float eps) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(x && gamma && beta && running_mean && running_var && y);
+    AETH_CHECK_ARG(rows > 0 && C > 0 && (int64_t)rows * C < ((int64_t)1 << 31));
+    int64_t n = (int64_t)rows * C;
+    EW_LAUNCH(bn_apply_infer, n, x, gamma, beta, running_mean, running_var, y, n, C, eps);
+    return AETH_OK;
+}
+
+int aeth_bn_bwd_f32(const float* x, const float* dy, const float* gamma, const float* save_mean,
+                    const float* save_invstd, float* dx, float* dgamma, float* dbeta, int rows, int C) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(x && dy && gamma && save_mean && save_invstd && dx && dgamma && dbeta);
+    AETH_CHECK_ARG(rows > 0 && C > 0 && (int64_t)rows * C < ((int64_t)1 << 31));
+    int nblk, rpb;
+    dim3 grid;
+    col_grid(rows, C, &nblk, &rpb, &grid);
+    void* ws;
+    int rc = workspace(((int64_t)2 * nblk * C + 3 * C) * sizeof(float), &ws);
+    if (rc) return rc;
+    float* part = (float*)ws;
+    float* coef = part + (int64_t)2 * nblk * C;
+    hipStream_t st = ctx().stream;
+    hipLaunchKernelGGL(bn_bwd_partial, grid, dim3(kEwThreads), 0, st, x, dy, save_mean, rows, C, rpb, part);
+    AETH_LAUNCH_CHECK();
+    hipLaunchKernelGGL(bn_bwd_final, dim3(cdiv(C, 64)), dim3(64), 0, st, part, nblk, rows, C, gamma, save_invstd,
+                       dgamma, dbeta, coef);
+    AETH_LAUNCH_CHECK();
+    int64_t n = (int64_t)rows * C;
+    EW_LAUNCH(bn_bwd_apply, n, x, dy, save_mean, coef, dx, n, C);
+    return AETH_OK;
+}
+
+int aeth_relu_fwd_f32(const float* x, float* y, float alpha, int64_t n) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(n >= 0);
+    if (n == 0) return AETH_OK;
+    AETH_CHECK_ARG(x && y);
+    EW_LAUNCH(relu_fwd_kernel, n, x, y, alpha, n);
+    return AETH_OK;
+}
+
+int aeth_relu_bwd_f32(const float* x, const float* dy, float* dx, float alpha, int64_t n) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(n >= 0);
+    if (n == 0) return AETH_OK;
+    AETH_CHECK_ARG(x && dy && dx);
+    EW_LAUNCH(relu_bwd_kernel, n, x, dy, dx, alpha, n);
+    return AETH_OK;
+}
+
+int aeth_maxpool_fwd_f32(const float* x, float* y, uint8_t* idx, int S, int H, int W, int C, int fH, int fW, int sH,
+                         int sW) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(x && y && idx);
+    PoolParams p;
+    int rc = pool_dims(__func__, S, H, W, C, fH, fW, sH, sW, &p);
+    if (rc) return rc;
+    int64_t n = (int64_t)S * p.Ho * p.Wo * C;
+    EW_LAUNCH(maxpool_fwd_kernel, n, x, y, idx, p, n);
+    return AETH_OK;
+}
+
+int aeth_maxpool_bwd_f32(const float* dy, const uint8_t* idx, float* dx, int S, int H, int W, int C, int fH, int fW,
+                         int sH, int sW) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(dy && idx && dx);
+    PoolParams p;
+    int rc = pool_dims(__func__, S, H, W, C, fH, fW, sH, sW, &p);
+    if (rc) return rc;
+    int64_t n = (int64_t)S * H * W * C;
+    EW_LAUNCH(maxpool_bwd_kernel, n, dy, idx, dx, p, n);
+    return AETH_OK;
+}
+
+int aeth_avgpool_fwd_f32(const float* x, float* y, int S, int H, int W, int C, int fH, int fW, int sH, int sW) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(x && y);
+    PoolParams p;
+    int rc = pool_dims(__func__, S, H, W, C, fH, fW, sH, sW, &p);
+    if (rc) return rc;
+    int64_t n = (int64_t)S * p.Ho * p.Wo * C;
+    EW_LAUNCH(avgpool_fwd_kernel, n, x, y, p, n);
+    return AETH_OK;
+}
+
+int aeth_avgpool_bwd_f32(const float* dy, float* dx, int S, int H, int W, int C, int fH, int fW, int sH, int sW) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(dy && dx);
+    PoolParams p;
+    int rc = pool_dims(__func__, S, H, W, C, fH, fW, sH, sW, &p);
+    if (rc) return rc;
+    int64_t n = (int64_t)S * H * W * C;
+    EW_LAUNCH(avgpool_bwd_kernel, n, dy, dx, p, n);
+    return AETH_OK;
+}
+
+int aeth_mul_mask_f32(const float* x, const float* mask, float* y, int64_t n, int64_t mask_n) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(n >= 0 && mask_n > 0);
+    if (n == 0) return AETH_OK;
+    AETH_CHECK_ARG(x && mask && y);
+    EW_LAUNCH(mul_mask_kernel, n, x, mask, y, n, mask_n);
+    return AETH_OK;
+}
+
+int aeth_softmax_f32(const float* logits, float* probs, int rows, int K) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(logits && probs && rows > 0 && K > 0);
+    hipLaunchKernelGGL(softmax_kernel, dim3(cdiv(rows, 64)), dim3(64), 0, ctx().stream, logits, probs, rows, K);
+    AETH_LAUNCH_CHECK();
+    return AETH_OK;
+}
+
+int aeth_softmax_bwd_f32(const float* probs, const float* dy, float* dx, int rows, int K) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(probs && dy && dx && rows > 0 && K > 0);
+    hipLaunchKernelGGL(softmax_bwd_kernel, dim3(cdiv(rows, 64)), dim3(64), 0, ctx().stream, probs, dy, dx, rows, K);
+    AETH_LAUNCH_CHECK();
+    return AETH_OK;
+}
+
+int aeth_cce_fwd_f32(const float* probs, const int32_t* labels, float label_smoothing, float* sample_loss,
+                     int32_t* correct, int rows, int K) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(probs && labels && sample_loss && correct && rows > 0 && K > 0);
+    hipLaunchKernelGGL(cce_fwd_kernel, dim3(cdiv(rows, 64)), dim3(64), 0, ctx().stream, probs, labels,
+                       label_smoothing, sample_loss, correct, rows, K);
+    AETH_LAUNCH_CHECK();
+    return AETH_OK;
+}
+
+int aeth_softmax_cce_bwd_f32(const float* probs, const int32_t* labels, float label_smoothing, float* dlogits,
+                             int rows, int K) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(probs && labels && dlogits && rows > 0 && K > 0);
+    AETH_CHECK_ARG((int64_t)rows * K < ((int64_t)1 << 31));
+    hipLaunchKernelGGL(softmax_cce_bwd_kernel, dim3(cdiv((int64_t)rows * K, 256)), dim3(256), 0, ctx().stream, probs,
+                       labels, label_smoothing, dlogits, rows, K);
+    AETH_LAUNCH_CHECK();
+    return AETH_OK;
+}
+
+int aeth_adam_f32(float* theta, const float* grad, float* m, float* v, int64_t n, float lr, float beta1, float beta2,
+                  float eps, int t) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(n >= 0 && t >= 0);
+    if (n == 0) return AETH_OK;
+    AETH_CHECK_ARG(theta && grad && m && v);
+    double c1 = 1.0, c2 = 1.0;
+    {
+        double p1 = 1.0, p2 = 1.0;
+        // beta^(t+1) by repeated squaring in double
+        double b1 = beta1, b2 = beta2;
+        for (unsigned e = (unsigned)t + 1; e; e >>= 1) {
+            if (e & 1) { p1 *= b1; p2 *= b2; }
+            b1 *= b1; b2 *= b2;
+        }
+        c1 = 1.0 - p1;
+        c2 = 1.0 - p2;
+    }
+    EW_LAUNCH(adam_kernel, n, theta, grad, m, v, n, lr, beta1, beta2, eps, (float)c1, (float)c2);
+    return AETH_OK;
+}
+
+int aeth_axpy_f32(float alpha, const float* x, float* y, int64_t n) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(n >= 0);
+    if (n == 0) return AETH_OK;
+    AETH_CHECK_ARG(x && y);
+    EW_LAUNCH(axpy_kernel, n, alpha, x, y, n);
+    return AETH_OK;
+}
+
+int aeth_l1_grad_f32(float lambda, const float* w, float* dw, int64_t n) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(n >= 0);
+    if (n == 0) return AETH_OK;
+    AETH_CHECK_ARG(w && dw);
+    EW_LAUNCH(l1_grad_kernel, n, lambda, w, dw, n);
+    return AETH_OK;
+}
+
+int aeth_reduce_f32(const float* x, int64_t n, int mode, float* out) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(n >= 0 && (mode == 0 || mode == 1) && out);
+    AETH_CHECK_ARG(n == 0 || x);
+    hipLaunchKernelGGL(reduce_kernel, dim3(1), dim3(1024), 0, ctx().stream, x, n, mode, out);
+    AETH_LAUNCH_CHECK();
+    return AETH_OK;
+}
+
+int aeth_cast_f32_to_bf16(const float* src, uint16_t* dst, int64_t n) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(n >= 0);
+    if (n == 0) return AETH_OK;
+    AETH_CHECK_ARG(src && dst);
+    EW_LAUNCH(cast_bf16_kernel, n, src, dst, n);
+    return AETH_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,255 @@
+// Context, memory, copies, events: the part of the C ABI that owns device state.
+#include "common.h"
+
+#include <string.h>
+#include <map>
+#include <unordered_map>
+#include <vector>
+
+namespace aeth {
+
+static thread_local char g_err[512] = "";
+
+Context& ctx() {
+    static Context c;
+    return c;
+}
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int workspace(int64_t bytes, void** out) {
+    Context& c = ctx();
+    if (bytes > c.ws_bytes) {
+        int64_t want = round_up(bytes + bytes / 4, 1 << 20);
+        if (c.ws) {
+            AETH_HIP(hipStreamSynchronize(c.stream));
+            AETH_HIP(hipFree(c.ws));
+            c.ws = nullptr;
+            c.ws_bytes = 0;
+        }
+        AETH_HIP(hipMalloc(&c.ws, (size_t)want));
+        c.ws_bytes = want;
+    }
+    *out = c.ws;
+    return AETH_OK;
+}
+
+// Caching allocator.  Every kernel and copy runs on the one library stream, so a
+// block handed back by the caller can be reused by a later allocation without a
+// synchronisation: anything still reading it was queued earlier on that stream.
+struct Pool {
+    std::unordered_map<void*, size_t> live;            // pointer -> rounded size
+    std::map<size_t, std::vector<void*>> free_blocks;  // rounded size -> idle blocks
+    size_t cached_bytes = 0;
+
+    static size_t rounded(int64_t bytes) {
+        size_t b = bytes <= 0 ? 256 : (size_t)bytes;
+        return (b + 255) & ~(size_t)255;
+    }
+    hipError_t release_cached() {
+        hipError_t st = hipStreamSynchronize(ctx().stream);
+        for (auto& kv : free_blocks)
+            for (void* p : kv.second) (void)hipFree(p);
+        free_blocks.clear();
+        cached_bytes = 0;
+        return st;
+    }
+};
+static Pool g_pool;
+
+__global__ void fill_f32_kernel(float* __restrict__ dst, float v, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) dst[i] = v;
+}
+
+__global__ void fill_u32_kernel(unsigned int* __restrict__ dst, unsigned int v, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = v;
+}
+
+}  // namespace aeth
+
+using namespace aeth;
+
+extern "C" {
+
+const char* aeth_last_error(void) { return g_err; }
+
+int aeth_init(int device) {
+    Context& c = ctx();
+    if (c.ready) {
+        if (c.device == device) return AETH_OK;
+        return fail(AETH_E_STATE, "aeth_init: already bound to device %d", c.device);
+    }
+    int n = 0;
+    AETH_HIP(hipGetDeviceCount(&n));
+    if (device < 0 || device >= n) return fail(AETH_E_INVALID, "aeth_init: device %d out of range (%d present)", device, n);
+    AETH_HIP(hipSetDevice(device));
+    AETH_HIP(hipGetDeviceProperties(&c.prop, device));
+    if (strncmp(c.prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(AETH_E_STATE, "aeth_init: built for gfx950, device is %s", c.prop.gcnArchName);
+    AETH_HIP(hipStreamCreateWithFlags(&c.stream, hipStreamNonBlocking));
+    AETH_HIP(hipMalloc((void**)&c.counters, 256 * sizeof(unsigned int)));
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(256), 0, c.stream, c.counters, 0u, 256);
+    AETH_LAUNCH_CHECK();
+    AETH_HIP(hipStreamSynchronize(c.stream));
+    c.device = device;
+    c.ready = true;
+    return AETH_OK;
+}
+
+int aeth_shutdown(void) {
+    Context& c = ctx();
+    if (!c.ready) return AETH_OK;
+    g_pool.release_cached();
+    for (auto& kv : g_pool.live) (void)hipFree(kv.first);
+    g_pool.live.clear();
+    if (c.ws) hipFree(c.ws);
+    if (c.counters) hipFree(c.counters);
+    hipStreamDestroy(c.stream);
+    c = Context();
+    return AETH_OK;
+}
+
+int aeth_device_info(char* host_buf, int n) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(host_buf != nullptr && n > 0);
+    Context& c = ctx();
+    snprintf(host_buf, (size_t)n, "arch=%s;cus=%d;clock_mhz=%d;mem_clock_mhz=%d;mem_bus_bits=%d;hbm_bytes=%lld;lds_bytes=%lld;l2_bytes=%d",
+             c.prop.gcnArchName, c.prop.multiProcessorCount, c.prop.clockRate / 1000,
+             c.prop.memoryClockRate / 1000, c.prop.memoryBusWidth,
+             (long long)c.prop.totalGlobalMem, (long long)c.prop.sharedMemPerBlock, c.prop.l2CacheSize);
+    return AETH_OK;
+}
+
+int aeth_malloc(void** host_out_ptr, int64_t bytes) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(host_out_ptr != nullptr);
+    AETH_CHECK_ARG(bytes >= 0);
+    *host_out_ptr = nullptr;
+    size_t sz = Pool::rounded(bytes);
+    auto it = g_pool.free_blocks.find(sz);
+    if (it != g_pool.free_blocks.end() && !it->second.empty()) {
+        void* p = it->second.back();
+        it->second.pop_back();
+        g_pool.cached_bytes -= sz;
+        g_pool.live[p] = sz;
+        *host_out_ptr = p;
+        return AETH_OK;
+    }
+    void* p = nullptr;
+    hipError_t e = hipMalloc(&p, sz);
+    if (e == hipErrorOutOfMemory && g_pool.cached_bytes > 0) {
+        (void)hipGetLastError();
+        g_pool.release_cached();
+        e = hipMalloc(&p, sz);
+    }
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(e == hipErrorOutOfMemory ? AETH_E_NOMEM : AETH_E_HIP,
+                    "aeth_malloc: hipMalloc(%lld bytes) -> %s", (long long)bytes, hipGetErrorString(e));
+    }
+    g_pool.live[p] = sz;
+    *host_out_ptr = p;
+    return AETH_OK;
+}
+
+int aeth_free(void* p) {
+    AETH_REQUIRE_INIT();
+    if (!p) return AETH_OK;
+    auto it = g_pool.live.find(p);
+    if (it == g_pool.live.end()) return fail(AETH_E_INVALID, "aeth_free: %p was not returned by aeth_malloc", p);
+    size_t sz = it->second;
+    g_pool.live.erase(it);
+    g_pool.free_blocks[sz].push_back(p);
+    g_pool.cached_bytes += sz;
+    return AETH_OK;
+}
+
+int aeth_memcpy_h2d(void* dst, const void* host_src, int64_t bytes) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(bytes >= 0);
+    if (bytes == 0) return AETH_OK;
+    AETH_CHECK_ARG(dst != nullptr && host_src != nullptr);
+    // pageable source: the call returns once the source has been staged
+    AETH_HIP(hipMemcpyAsync(dst, host_src, (size_t)bytes, hipMemcpyHostToDevice, ctx().stream));
+    AETH_HIP(hipStreamSynchronize(ctx().stream));
+    return AETH_OK;
+}
+
+int aeth_memcpy_d2h(void* host_dst, const void* src, int64_t bytes) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(bytes >= 0);
+    if (bytes == 0) return AETH_OK;
+    AETH_CHECK_ARG(host_dst != nullptr && src != nullptr);
+    AETH_HIP(hipMemcpyAsync(host_dst, src, (size_t)bytes, hipMemcpyDeviceToHost, ctx().stream));
+    AETH_HIP(hipStreamSynchronize(ctx().stream));
+    return AETH_OK;
+}
+
+int aeth_memcpy_d2d(void* dst, const void* src, int64_t bytes) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(bytes >= 0);
+    if (bytes == 0) return AETH_OK;
+    AETH_CHECK_ARG(dst != nullptr && src != nullptr);
+    AETH_HIP(hipMemcpyAsync(dst, src, (size_t)bytes, hipMemcpyDeviceToDevice, ctx().stream));
+    return AETH_OK;
+}
+
+int aeth_fill_f32(float* dst, float value, int64_t n) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(n >= 0);
+    if (n == 0) return AETH_OK;
+    AETH_CHECK_ARG(dst != nullptr);
+    int blocks = (int)((n + 255) / 256);
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(fill_f32_kernel, dim3(blocks), dim3(256), 0, ctx().stream, dst, value, n);
+    AETH_LAUNCH_CHECK();
+    return AETH_OK;
+}
+
+int aeth_sync(void) {
+    AETH_REQUIRE_INIT();
+    AETH_HIP(hipStreamSynchronize(ctx().stream));
+    return AETH_OK;
+}
+
+int aeth_event_create(void** host_out_event) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(host_out_event != nullptr);
+    hipEvent_t ev;
+    AETH_HIP(hipEventCreate(&ev));
+    *host_out_event = (void*)ev;
+    return AETH_OK;
+}
+
+int aeth_event_destroy(void* event) {
+    AETH_REQUIRE_INIT();
+    if (!event) return AETH_OK;
+    AETH_HIP(hipEventDestroy((hipEvent_t)event));
+    return AETH_OK;
+}
+
+int aeth_event_record(void* event) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(event != nullptr);
+    AETH_HIP(hipEventRecord((hipEvent_t)event, ctx().stream));
+    return AETH_OK;
+}
+
+int aeth_event_elapsed_ms(void* start, void* stop, float* host_out_ms) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(start != nullptr && stop != nullptr && host_out_ms != nullptr);
+    AETH_HIP(hipEventSynchronize((hipEvent_t)stop));
+    AETH_HIP(hipEventElapsedTime(host_out_ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return AETH_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,193 @@
+"""Headline benchmark: fp32 convolution throughput (fprop + dgrad + wgrad) on one
+MI355X, on the ResNet-style shape input NHWC [256,56,56,64], 64 filters 3x3,
+stride 1, "same" padding.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one pass of the hot path over one batch: Conv_Layer's three
+contractions (fprop with fused bias, dgrad, wgrad with dbias) through the C ABI,
+inputs already resident in HBM.  Prints ONE JSON line.  `value` is the
+algorithmic TFLOP/s of the whole step (3 * 2*M*N*K flops / step time); the
+per-direction figures, the bf16 variant and the training-step images/sec are
+reported under "extra".  The CPU baseline is the NumPy einsum oracle timed on a
+bounded sample (a smaller batch of the same layer) on this machine's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "aether-ml_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+import numpy as np
+
+FP32_MFMA_PEAK_TFLOPS = 157.3
+BF16_MFMA_PEAK_TFLOPS = 2500.0
+HBM_PEAK_GBS = 8000.0
+
+
+def conv_flops(S, Ho, Wo, fH, fW, C, D):
+    return 2.0 * S * Ho * Wo * fH * fW * C * D
+
+
+def time_loop(fn, steps, warmup):
+    """Average ms per call from HIP events on the library's stream."""
+    from aether import _lib
+    for _ in range(warmup):
+        fn()
+    _lib.sync()
+    e0, e1 = _lib.Event(), _lib.Event()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    return e0.elapsed_ms(e1) / steps
+
+
+def cpu_baseline(S_small, H, W, C, D):
+    """NumPy einsum oracle (single-threaded by construction) on a reduced batch."""
+    from oracle import oracle as O
+    r = np.random.RandomState(1)
+    x = r.randn(S_small, H, W, C).astype(np.float32)
+    w = (r.randn(3, 3, C, D) * np.sqrt(2.0 / (9 * C))).astype(np.float32)
+    b = np.zeros(D, np.float32)
+    dy = r.randn(S_small, H, W, D).astype(np.float32)
+    t0 = time.perf_counter()
+    O.conv_fprop(x, w, b, (1, 1), "same")
+    t1 = time.perf_counter()
+    O.conv_dgrad(dy, w, (H, W), (1, 1), "same")
+    t2 = time.perf_counter()
+    O.conv_wgrad(x, dy, (3, 3), (1, 1), "same")
+    O.conv_dbias(dy)
+    t3 = time.perf_counter()
+    fl = conv_flops(S_small, H, W, 3, 3, C, D)
+    return {
+        "value": 3 * fl / (t3 - t0) / 1e12,
+        "unit": "TFLOP/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": "same layer, batch %d instead of 256 (fprop %.2fs, dgrad %.2fs, wgrad %.2fs); np.einsum is single-threaded; host has %d cores"
+                  % (S_small, t1 - t0, t2 - t1, t3 - t2, os.cpu_count()),
+        "per_direction_gflops": {"fprop": fl / (t1 - t0) / 1e9, "dgrad": fl / (t2 - t1) / 1e9,
+                                 "wgrad": fl / (t3 - t2) / 1e9},
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the bf16 / train-step extras")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    from aether import _lib
+    from aether.tensor import DeviceTensor
+    L = _lib.lib()
+    info = _lib.device_info()
+
+    S, H, W, C, D = 256, 56, 56, 64, 64
+    dims = (S, H, W, C, D, 3, 3, 1, 1, 1, 1)
+    np.random.seed(0)
+    x_h = np.random.randn(S, H, W, C).astype(np.float32)
+    w_h = (np.random.randn(3, 3, C, D).astype(np.float32) * np.float32(np.sqrt(2.0 / (9 * C))))
+    dy_h = np.random.randn(S, H, W, D).astype(np.float32)
+    x, w, dy = (DeviceTensor.from_numpy(a) for a in (x_h, w_h, dy_h))
+    bias = DeviceTensor.zeros(D)
+    y, dx = DeviceTensor((S, H, W, D)), DeviceTensor((S, H, W, C))
+    dw, db = DeviceTensor((3, 3, C, D)), DeviceTensor(D)
+    del x_h, dy_h
+
+    def fprop():
+        _lib.check(L.aeth_conv_fprop_f32(x.ptr, w.ptr, bias.ptr, y.ptr, *dims))
+
+    def dgrad():
+        _lib.check(L.aeth_conv_dgrad_f32(dy.ptr, w.ptr, dx.ptr, *dims))
+
+    def wgrad():
+        _lib.check(L.aeth_conv_wgrad_f32(x.ptr, dy.ptr, dw.ptr, db.ptr, *dims))
+
+    def step():
+        fprop()
+        wgrad()
+        dgrad()
+
+    fl = conv_flops(S, H, W, 3, 3, C, D)
+
+    # ---- the timed region: exactly K steps between two synchronisations --------
+    for _ in range(args.warmup):
+        step()
+    _lib.sync()
+    t0 = time.perf_counter()
+    e0, e1 = _lib.Event(), _lib.Event()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    _lib.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = e0.elapsed_ms(e1) / args.steps
+    ms_per_step = max(ms_per_step, 0.0)
+    value = 3 * fl / (ms_per_step * 1e-3) / 1e12
+
+    # ---- per-direction kernel times (HIP events on the launch stream) -----------
+    per = {}
+    for name, fn in (("fprop", fprop), ("dgrad", dgrad), ("wgrad", wgrad)):
+        ms = time_loop(fn, args.steps, 2)
+        per[name] = {"ms": ms, "tflops": fl / (ms * 1e-3) / 1e12,
+                     "frac_fp32_mfma_peak": fl / (ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS}
+    slowest = max(per, key=lambda k: per[k]["ms"])
+    roofline = {
+        "bound": "mfma",
+        "kernel": {"fprop": "gather_gemm_f32", "dgrad": "gather_gemm_f32", "wgrad": "wgrad_gemm_f32"}[slowest],
+        "direction": slowest,
+        "achieved": per[slowest]["tflops"],
+        "peak": FP32_MFMA_PEAK_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": per[slowest]["tflops"] / FP32_MFMA_PEAK_TFLOPS,
+        "traffic": None,
+    }
+
+    extra = {"per_direction_fp32": per, "wall_ms_per_step": wall_ms,
+             "device": {k: info[k] for k in ("arch", "cus", "clock_mhz")}}
+    if not args.no_extra:
+        try:
+            import bench_extra
+            extra.update(bench_extra.run(args.steps, args.warmup))
+        except Exception as e:   # extras never hide the headline number
+            extra["extra_error"] = "%s: %s" % (type(e).__name__, e)
+
+    out = {
+        "metric": "conv TFLOP/s (fprop+dgrad+wgrad), fp32 MFMA",
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "Conv_Layer fwd+bwd, input NHWC [256,56,56,64], 64 filters 3x3 stride 1 same pad, "
+                               "He-normal weights, N(0,1) input and upstream gradient, seed 0",
+                   "frac_fp32_mfma_peak": value / FP32_MFMA_PEAK_TFLOPS},
+        "roofline": roofline,
+        "extra": extra,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(32, H, W, C, D)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

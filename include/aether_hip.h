@@ -1,0 +1,174 @@
+/*
+ * libaether_hip.so -- C ABI of the MI355X (gfx950) convolution hot path.
+ *
+ * The reference framework has no FFI: its boundary is the duck-typed layer
+ * protocol that Model drives (CNN/models/CNN_model_cupy.py:153-193).  Each entry
+ * point below replaces the array-library calls one reference method makes, and
+ * cites that method.  The Python classes in aether/layers.py keep the reference
+ * class API and call these through ctypes.
+ *
+ * Conventions
+ *   - every function returns 0 on success or a negative AETH_E_* code;
+ *     aeth_last_error() returns a thread-local message for the last failure.
+ *     Nothing aborts the process.
+ *   - every pointer is a DEVICE pointer obtained from aeth_malloc unless its
+ *     name starts with host_.
+ *   - tensors are dense, C-contiguous: activations NHWC [S,H,W,C], filters
+ *     [fH,fW,C,D] (the reference's filter_weights layout), dense weights
+ *     [n_in,n_out] row-major, all float32 unless the name says bf16 (uint16_t
+ *     holding the upper 16 bits of a float32, rounded to nearest even).
+ *   - element counts fit int32; byte counts are int64.
+ *   - one process-wide context bound to one GPU with one stream; calls are
+ *     asynchronous on that stream, aeth_sync() and the d2h copy are the sync
+ *     points.  Not re-entrant: one caller thread at a time.
+ *   - convolution geometry: Ho = (H + 2*pH - fH)/sH + 1, Wo likewise, the caller
+ *     passes pH = pW = P where P = (fH-1)/2 for "same" and 0 for "valid"
+ *     (CNN/models/CNN_classes_cupy.py:78-85).
+ */
+#ifndef AETHER_HIP_H
+#define AETHER_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AETH_OK          0
+#define AETH_E_INVALID  -1   /* bad shape / NULL pointer / unsupported argument */
+#define AETH_E_HIP      -2   /* a HIP runtime call failed                       */
+#define AETH_E_NOMEM    -3   /* device allocation failed                        */
+#define AETH_E_STATE    -4   /* aeth_init not called, or called twice on different devices */
+
+/* ---- lifetime -------------------------------------------------------------- */
+int aeth_init(int device);
+int aeth_shutdown(void);
+const char* aeth_last_error(void);
+/* "arch=gfx950;cus=256;clock_mhz=2400;mem_clock_mhz=...;hbm_bytes=...;lds_bytes=..." */
+int aeth_device_info(char* host_buf, int n);
+
+/* ---- memory (replaces cp.zeros / cp.asarray / .get(), cupy array ownership) - */
+int aeth_malloc(void** host_out_ptr, int64_t bytes);
+int aeth_free(void* p);
+int aeth_memcpy_h2d(void* dst, const void* host_src, int64_t bytes);
+int aeth_memcpy_d2h(void* host_dst, const void* src, int64_t bytes);   /* synchronises */
+int aeth_memcpy_d2d(void* dst, const void* src, int64_t bytes);
+int aeth_fill_f32(float* dst, float value, int64_t n);
+int aeth_sync(void);
+
+/* ---- timing on the library's own stream (used by the benchmark) ------------ */
+int aeth_event_create(void** host_out_event);
+int aeth_event_destroy(void* event);
+int aeth_event_record(void* event);
+int aeth_event_elapsed_ms(void* start, void* stop, float* host_out_ms);  /* synchronises on stop */
+
+/* ---- convolution, fp32 in / fp32 accumulate on MFMA ----------------------------
+ * fprop  : Conv_Layer.forward, CNN/models/CNN_classes_cupy.py:70-120
+ *          (cp.pad :92, as_strided :101, einsum 'shwxyc,xycd->shwd' :115, bias :116)
+ *          y[s,h,w,d] = bias[d] + sum_{x,y,c} xpad[s,h*sH+x,w*sW+y,c] * w[x,y,c,d]
+ *          bias may be NULL.
+ * dgrad  : Conv_Layer.backward, :136-153 (einsum 'shwd,xycd->shwxyc' :138 and the
+ *          atomicAdd scatter kernel :4-35, :141-146, crop :149-153).  Writes every
+ *          element of the UNPADDED dx [S,H,W,C]; positions no tap reaches get 0.
+ * wgrad  : Conv_Layer.backward, :132 (dbiases = sum over s,h,w) and :134
+ *          (einsum 'shwxyc,shwd->xycd').  dbias may be NULL.  Deterministic.
+ */
+int aeth_conv_fprop_f32(const float* x, const float* w, const float* bias, float* y,
+                        int S, int H, int W, int C, int D,
+                        int fH, int fW, int sH, int sW, int pH, int pW);
+int aeth_conv_dgrad_f32(const float* dy, const float* w, float* dx,
+                        int S, int H, int W, int C, int D,
+                        int fH, int fW, int sH, int sW, int pH, int pW);
+int aeth_conv_wgrad_f32(const float* x, const float* dy, float* dw, float* dbias,
+                        int S, int H, int W, int C, int D,
+                        int fH, int fW, int sH, int sW, int pH, int pW);
+
+/* ---- convolution, bf16 in / fp32 accumulate / fp32 out --------------------------
+ * Same three contractions with x, w, dy given as bf16.  No reference counterpart
+ * (the reference is fp32 only); the inputs are produced by aeth_cast_f32_to_bf16.
+ */
+int aeth_cast_f32_to_bf16(const float* src, uint16_t* dst, int64_t n);
+int aeth_conv_fprop_bf16(const uint16_t* x, const uint16_t* w, const float* bias, float* y,
+                         int S, int H, int W, int C, int D,
+                         int fH, int fW, int sH, int sW, int pH, int pW);
+int aeth_conv_dgrad_bf16(const uint16_t* dy, const uint16_t* w, float* dx,
+                         int S, int H, int W, int C, int D,
+                         int fH, int fW, int sH, int sW, int pH, int pW);
+int aeth_conv_wgrad_bf16(const uint16_t* x, const uint16_t* dy, float* dw, float* dbias,
+                         int S, int H, int W, int C, int D,
+                         int fH, int fW, int sH, int sW, int pH, int pW);
+
+/* ---- dense layer ------------------------------------------------------------------
+ * fprop : Layer_Dense.forward, CNN_classes_cupy.py:328-331   y = x.w + bias
+ * dgrad : Layer_Dense.backward :354                           dx = dy.w^T
+ * wgrad : Layer_Dense.backward :334-335                       dw = x^T.dy, dbias = sum_rows dy
+ * x [M,n_in], w [n_in,n_out], bias [n_out], y/dy [M,n_out].  bias/dbias may be NULL.
+ * axpy and l1_grad implement the regulariser terms of :337-351
+ * (y += alpha*x ;  dw += lambda * (w < 0 ? -1 : +1)).
+ */
+int aeth_dense_fprop_f32(const float* x, const float* w, const float* bias, float* y,
+                         int M, int n_in, int n_out);
+int aeth_dense_dgrad_f32(const float* dy, const float* w, float* dx,
+                         int M, int n_in, int n_out);
+int aeth_dense_wgrad_f32(const float* x, const float* dy, float* dw, float* dbias,
+                         int M, int n_in, int n_out);
+int aeth_axpy_f32(float alpha, const float* x, float* y, int64_t n);
+int aeth_l1_grad_f32(float lambda, const float* w, float* dw, int64_t n);
+/* out[0] = sum |x| (mode 0) or sum x*x (mode 1): Loss.regularization_loss :593-609 */
+int aeth_reduce_f32(const float* x, int64_t n, int mode, float* out);
+
+/* ---- layers either side of the path (so activations stay on the GPU) -------------
+ * rows = product of the leading axes, C = channels (last axis).
+ * bn_fwd_train : Batch_Norm.forward training branch :467-476 (biased variance,
+ *                running = momentum*running + (1-momentum)*batch).  Saves batch mean
+ *                and 1/sqrt(var+eps) for the backward pass.
+ * bn_fwd_infer : :478-480.       bn_bwd : Batch_Norm.backward :484-508.
+ */
+int aeth_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta,
+                          float* running_mean, float* running_var,
+                          float* save_mean, float* save_invstd, float* y,
+                          int rows, int C, float eps, float momentum);
+int aeth_bn_fwd_infer_f32(const float* x, const float* gamma, const float* beta,
+                          const float* running_mean, const float* running_var, float* y,
+                          int rows, int C, float eps);
+int aeth_bn_bwd_f32(const float* x, const float* dy, const float* gamma,
+                    const float* save_mean, const float* save_invstd,
+                    float* dx, float* dgamma, float* dbeta, int rows, int C);
+/* ReLU (alpha = 0) :406-415 and Leaky_ReLU :417-428.
+ * fwd: y = x > 0 ? x : alpha*x ;  bwd: dx = x < 0 ? alpha*dy : dy  (strict <). */
+int aeth_relu_fwd_f32(const float* x, float* y, float alpha, int64_t n);
+int aeth_relu_bwd_f32(const float* x, const float* dy, float* dx, float alpha, int64_t n);
+/* Pooling "max"/"valid" :212-273 and :275-300.  idx holds the flat window index
+ * fh*fW+fw of the FIRST maximum in row-major window order. */
+int aeth_maxpool_fwd_f32(const float* x, float* y, uint8_t* idx,
+                         int S, int H, int W, int C, int fH, int fW, int sH, int sW);
+int aeth_maxpool_bwd_f32(const float* dy, const uint8_t* idx, float* dx,
+                         int S, int H, int W, int C, int fH, int fW, int sH, int sW);
+/* Pooling "average" :267-268 and the scatter kernel :163-202. */
+int aeth_avgpool_fwd_f32(const float* x, float* y,
+                         int S, int H, int W, int C, int fH, int fW, int sH, int sW);
+int aeth_avgpool_bwd_f32(const float* dy, float* dx,
+                         int S, int H, int W, int C, int fH, int fW, int sH, int sW);
+/* Dropout masks :375-377, :397-399: y[i] = x[i] * mask[i % mask_n]
+ * (mask_n = n for Layer_Dropout, = C for Layer_Dropout_Spatial). */
+int aeth_mul_mask_f32(const float* x, const float* mask, float* y, int64_t n, int64_t mask_n);
+/* SoftMax.forward :542-547 and SoftMax.backward :549-560
+ * (dx = (diag(p) - p p^T) dy per row = p * (dy - sum_j p_j dy_j)). */
+int aeth_softmax_f32(const float* logits, float* probs, int rows, int K);
+int aeth_softmax_bwd_f32(const float* probs, const float* dy, float* dx, int rows, int K);
+/* Loss_CategoricalCrossEntropy.forward :615-632 on probabilities (clip to
+ * [1e-7, 1-1e-7], label smoothing) -> per-sample loss; correct[i] = argmax == label. */
+int aeth_cce_fwd_f32(const float* probs, const int32_t* labels, float label_smoothing,
+                     float* sample_loss, int32_t* correct, int rows, int K);
+/* Activation_Softmax_Loss_CategoricalCrossEntropy.backward :666-680:
+ * dlogits = (probs - smooth(onehot)) / rows. */
+int aeth_softmax_cce_bwd_f32(const float* probs, const int32_t* labels, float label_smoothing,
+                             float* dlogits, int rows, int K);
+/* Optimizer_Adam.update_parameters for one tensor :702-734; t = iterations (0-based). */
+int aeth_adam_f32(float* theta, const float* grad, float* m, float* v, int64_t n,
+                  float lr, float beta1, float beta2, float eps, int t);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AETHER_HIP_H */

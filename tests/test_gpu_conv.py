@@ -1,0 +1,126 @@
+"""Parity of the fp32 HIP convolution (through the C ABI) with the CPU oracle.
+Tolerance (fp32): |gpu - oracle| <= 1e-5 + 1e-4*|oracle| per element, oracle
+evaluated in float64 on the float32 inputs."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+# S, H, W, C, D, fH, fW, sH, sW, padding
+CASES = [
+    (2, 5, 5, 1, 1, 3, 3, 1, 1, "valid"),
+    (2, 6, 7, 3, 4, 3, 3, 1, 1, "same"),
+    (3, 8, 8, 4, 5, 3, 3, 2, 2, "valid"),
+    (2, 9, 7, 2, 3, 3, 3, 2, 2, "same"),
+    (2, 7, 7, 4, 6, 1, 1, 1, 1, "valid"),
+    (1, 8, 9, 3, 2, 5, 3, 1, 2, "same"),
+    (2, 6, 6, 2, 2, 2, 2, 2, 2, "valid"),
+    (1, 10, 10, 2, 3, 3, 3, 3, 3, "valid"),
+    (4, 12, 12, 8, 16, 3, 3, 1, 1, "same"),
+    (3, 16, 16, 32, 64, 3, 3, 1, 1, "same"),     # config-2a channel counts
+    (2, 8, 8, 64, 128, 3, 3, 1, 1, "same"),      # config-2b channel counts
+    (2, 14, 14, 64, 64, 3, 3, 1, 1, "same"),     # config-4 channel counts, ragged M
+    (2, 14, 14, 64, 256, 1, 1, 1, 1, "valid"),   # config-4 1x1
+    (3, 13, 13, 128, 256, 3, 3, 2, 2, "valid"),  # config-5 channel counts
+    (5, 9, 9, 20, 36, 3, 3, 1, 1, "same"),       # C,D multiples of 4 but not of 32
+    (2, 9, 9, 6, 10, 3, 3, 1, 1, "same"),        # C,D not multiples of 4
+    (2, 9, 9, 5, 7, 1, 1, 2, 2, "same"),         # 1x1 stride 2: dgrad classes without taps
+    (40, 16, 16, 3, 32, 3, 3, 1, 1, "same"),     # config-1 channel counts
+]
+
+
+def _case(case, seed):
+    from tests import abi
+    S, H, W, C, D, fH, fW, sH, sW, pad = case
+    r = np.random.RandomState(seed)
+    x = r.randn(S, H, W, C).astype(np.float32)
+    w = (r.randn(fH, fW, C, D) * np.sqrt(2.0 / (fH * fW * C))).astype(np.float32)
+    b = r.randn(D).astype(np.float32)
+    _, yshape = abi.conv_dims(x.shape, w.shape, (sH, sW), pad)
+    dy = r.randn(*yshape).astype(np.float32)
+    return x, w, b, dy
+
+
+def test_library_reports_gfx950():
+    from aether import _lib
+    info = _lib.device_info()
+    assert str(info["arch"]).startswith("gfx950")
+    assert info["cus"] > 0
+
+
+def test_notebook_known_answers_on_gpu():
+    from tests import abi
+    # CNN/notebooks/CNN_Implementation.ipynb:421-472 -> :411-414
+    img = np.array([[1, 2, 3, 0], [0, 1, 2, 3], [3, 0, 1, 2], [2, 3, 0, 1]], dtype=np.float32)
+    k = np.array([[1, 0, -1]] * 3, dtype=np.float32)
+    y = abi.fprop(img[None, :, :, None], k[:, :, None, None], None, (1, 1), "same")
+    want = np.array([[-3, -4, 0, 5], [-3, -2, -2, 6], [-4, 2, -2, 3], [-3, 4, 0, 1]], dtype=np.float32)
+    assert np.array_equal(y[0, :, :, 0], want)
+    # :747-752, :774-779, :803-811
+    y = abi.fprop(np.ones((1, 5, 5, 1), np.float32), np.ones((3, 3, 1, 1), np.float32), np.zeros(1, np.float32),
+                  (1, 1), "valid")
+    assert y.shape == (1, 3, 3, 1) and np.all(y == 9)
+    y = abi.fprop(np.ones((1, 5, 5, 3), np.float32), np.ones((3, 3, 3, 1), np.float32), np.zeros(1, np.float32),
+                  (1, 1), "valid")
+    assert np.all(y == 27)
+    w = np.ones((3, 3, 1, 2), np.float32)
+    w[..., 1] = 2
+    y = abi.fprop(np.ones((1, 5, 5, 1), np.float32), w, np.zeros(2, np.float32), (1, 1), "valid")
+    assert np.all(y[..., 0] == 9) and np.all(y[..., 1] == 18)
+    # CNN/notebooks/Backpropagation_Conv.ipynb:84-110: taps accumulate
+    dy = np.zeros((1, 4, 4, 1), np.float32)
+    dy[0, 0, :, 0] = [1, 2, 3, 0]
+    dx = abi.dgrad(dy, np.ones((3, 3, 1, 1), np.float32), (1, 4, 4, 1), (1, 1), "same")
+    assert np.array_equal(dx[0, 0, :, 0], [3, 6, 5, 3])
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_fprop_parity(case):
+    from tests import abi
+    x, w, b, dy = _case(case, 0)
+    stride, pad = (case[7], case[8]), case[9]
+    want = O.conv_fprop(x, w, b, stride, pad, dtype=np.float64)
+    abi.close(abi.fprop(x, w, b, stride, pad), want)
+    abi.close(abi.fprop(x, w, None, stride, pad), O.conv_fprop(x, w, None, stride, pad, dtype=np.float64))
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_dgrad_parity(case):
+    from tests import abi
+    x, w, b, dy = _case(case, 1)
+    stride, pad = (case[7], case[8]), case[9]
+    want = O.conv_dgrad(dy, w, x.shape[1:3], stride, pad, dtype=np.float64)
+    abi.close(abi.dgrad(dy, w, x.shape, stride, pad), want)
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_wgrad_parity(case):
+    from tests import abi
+    x, w, b, dy = _case(case, 2)
+    stride, pad = (case[7], case[8]), case[9]
+    dw, db = abi.wgrad(x, dy, w.shape, stride, pad)
+    want = O.conv_wgrad(x, dy, w.shape[:2], stride, pad, dtype=np.float64)
+    abi.close(dw, want, rms_scaled=True)
+    abi.close(db, O.conv_dbias(dy, dtype=np.float64), rms_scaled=True)
+    # and no less accurate than the reference arithmetic run in float32
+    ref32 = O.conv_wgrad(x, dy, w.shape[:2], stride, pad, dtype=np.float32)
+    assert np.abs(dw - want).max() <= 2.0 * np.abs(ref32 - want).max() + 1e-6
+    dw2, none = abi.wgrad(x, dy, w.shape, stride, pad, want_dbias=False)
+    assert none is None and np.array_equal(dw, dw2)       # deterministic
+
+
+def test_bad_arguments_are_errors_not_crashes():
+    from aether import _lib
+    from aether.tensor import DeviceTensor
+    L = _lib.lib()
+    t = DeviceTensor.zeros(16)
+    assert L.aeth_conv_fprop_f32(None, t.ptr, None, t.ptr, 1, 2, 2, 1, 1, 1, 1, 1, 1, 0, 0) == _lib.AETH_E_INVALID
+    assert L.aeth_conv_fprop_f32(t.ptr, t.ptr, None, t.ptr, 1, 2, 2, 1, 1, 3, 3, 1, 1, 0, 0) == _lib.AETH_E_INVALID
+    assert L.aeth_conv_fprop_f32(t.ptr, t.ptr, None, t.ptr, 0, 2, 2, 1, 1, 1, 1, 1, 1, 0, 0) == _lib.AETH_E_INVALID
+    assert b"aeth_conv_fprop_f32" in L.aeth_last_error()
+    with pytest.raises(ValueError):
+        _lib.check(L.aeth_conv_wgrad_f32(t.ptr, t.ptr, t.ptr, None, 1, 2, 2, 1, 1, 1, 1, 0, 1, 0, 0))
+    with pytest.raises(ValueError):
+        _lib.check(L.aeth_free(12345))
