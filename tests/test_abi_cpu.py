@@ -1,0 +1,94 @@
+"""CPU-side checks of the C ABI: the library loads, exports every function the
+header declares, the ctypes table matches the header, and calls made before
+aeth_init fail with a status code instead of touching a GPU."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "aether_hip.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    decls = re.findall(r"\b(?:int|const char\*)\s+(aeth_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S)
+    return {name: [a.strip() for a in args.split(",")] if args.strip() not in ("", "void") else []
+            for name, args in decls}
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from aether import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        import __graft_entry__
+        __graft_entry__.build()
+    return _lib.load()
+
+
+def test_header_declares_the_hot_path():
+    d = _declared()
+    for name in ("aeth_conv_fprop_f32", "aeth_conv_dgrad_f32", "aeth_conv_wgrad_f32",
+                 "aeth_conv_fprop_bf16", "aeth_conv_dgrad_bf16", "aeth_conv_wgrad_bf16",
+                 "aeth_dense_fprop_f32", "aeth_dense_dgrad_f32", "aeth_dense_wgrad_f32",
+                 "aeth_init", "aeth_malloc", "aeth_last_error"):
+        assert name in d
+    assert len(d) >= 40
+
+
+def test_library_exports_every_declared_symbol(lib):
+    for name in _declared():
+        assert hasattr(lib, name), name
+
+
+def test_ctypes_table_matches_header(lib):
+    from aether import _lib
+    d = _declared()
+    d.pop("aeth_last_error")
+    assert set(d) == set(_lib.SIGNATURES)
+    for name, args in d.items():
+        assert len(args) == len(_lib.SIGNATURES[name]), name
+        for decl, ct in zip(args, _lib.SIGNATURES[name]):
+            if "*" in decl:
+                assert ct in (ctypes.c_void_p, ctypes.c_char_p) or hasattr(ct, "contents"), (name, decl)
+            elif decl.startswith("float"):
+                assert ct is ctypes.c_float, (name, decl)
+            elif decl.startswith("int64_t"):
+                assert ct is ctypes.c_int64, (name, decl)
+            else:
+                assert decl.startswith("int") and ct is ctypes.c_int, (name, decl)
+
+
+def test_no_torch_or_python_types_in_the_abi():
+    text = open(HEADER).read()
+    assert "torch" not in text.lower() and "PyObject" not in text and "#include <hip" not in text
+    out = subprocess.run(["nm", "-D", "--defined-only", os.path.join(ROOT, "aether-ml_amd", "aether", "lib",
+                                                                    "libaether_hip.so")],
+                         capture_output=True, text=True).stdout
+    exported = {l.split()[-1] for l in out.splitlines() if " T " in l}
+    assert set(_declared()) <= exported
+
+
+def test_calls_before_init_report_state_error(lib):
+    if os.path.exists("/dev/kfd"):
+        pytest.skip("a GPU is present: the context may already be initialised by other tests")
+    assert lib.aeth_sync() == -4
+    assert b"aeth_init" in lib.aeth_last_error()
+    p = ctypes.c_void_p()
+    assert lib.aeth_malloc(ctypes.byref(p), 16) == -4
+    assert lib.aeth_conv_fprop_f32(None, None, None, None, 1, 1, 1, 1, 1, 1, 1, 1, 1, 0, 0) == -4
+    # without a GPU aeth_init fails with a HIP error and a message, it does not abort
+    assert lib.aeth_init(0) == -2
+    assert b"aeth_init" in lib.aeth_last_error()
+
+
+def test_product_package_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "aether-ml_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, os.path.join(dirpath, f)

@@ -1,0 +1,85 @@
+"""The benchmark's full-size shapes on the GPU, checked without a full-size CPU
+run: convolution is independent per sample, so fprop/dgrad of individual samples
+of the big batch are compared with the oracle directly; wgrad is linear in the
+upstream gradient, so a gradient that is zero outside one sample must reproduce
+the oracle's wgrad of that sample; and the adjoint identities
+<y - b, dy> = <x, dx> = <W, dW> tie the three full-size results together."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+FULL = [
+    # name, S, H, W, C, D, fH, fW, stride, padding
+    ("resnet3x3", 256, 56, 56, 64, 64, 3, 3, 1, "same"),
+    ("resnet1x1", 256, 56, 56, 64, 256, 1, 1, 1, "valid"),
+    ("wide_s2", 1024, 28, 28, 128, 256, 3, 3, 2, "valid"),
+]
+
+
+@pytest.mark.parametrize("cfg", FULL, ids=lambda c: c[0])
+def test_full_size_conv(cfg):
+    from aether import _lib
+    from aether.tensor import DeviceTensor
+    from tests import abi
+    name, S, H, W, C, D, fH, fW, st, pad = cfg
+    stride = (st, st)
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((S, H, W, C), dtype=np.float32)
+    w = (rng.standard_normal((fH, fW, C, D), dtype=np.float32) * np.float32(np.sqrt(2.0 / (fH * fW * C))))
+    b = rng.standard_normal(D, dtype=np.float32)
+    dims, yshape = abi.conv_dims(x.shape, w.shape, stride, pad)
+    dy = rng.standard_normal(yshape, dtype=np.float32)
+    L = _lib.lib()
+    xd, wd, bd, dyd = (DeviceTensor.from_numpy(a) for a in (x, w, b, dy))
+    y = DeviceTensor.full(yshape, np.nan)
+    dx = DeviceTensor.full(x.shape, np.nan)
+    dw = DeviceTensor.full(w.shape, np.nan)
+    db = DeviceTensor.full(D, np.nan)
+    _lib.check(L.aeth_conv_fprop_f32(xd.ptr, wd.ptr, bd.ptr, y.ptr, *dims))
+    _lib.check(L.aeth_conv_dgrad_f32(dyd.ptr, wd.ptr, dx.ptr, *dims))
+    _lib.check(L.aeth_conv_wgrad_f32(xd.ptr, dyd.ptr, dw.ptr, db.ptr, *dims))
+    y_h, dx_h, dw_h, db_h = y.get(), dx.get(), dw.get(), db.get()
+    assert np.all(np.isfinite(y_h)) and np.all(np.isfinite(dx_h))
+
+    # per-sample parity at the real launch geometry (first, middle, last sample)
+    for s in (0, S // 2 + 1, S - 1):
+        abi.close(y_h[s:s + 1], O.conv_fprop(x[s:s + 1], w, b, stride, pad, dtype=np.float64))
+        abi.close(dx_h[s:s + 1], O.conv_dgrad(dy[s:s + 1], w, (H, W), stride, pad, dtype=np.float64))
+    if name == "wide_s2":
+        # 28x28, 3x3 stride 2 valid: row/column 27 is never read, so its gradient is exactly 0
+        assert np.all(dx_h[:, 27] == 0) and np.all(dx_h[:, :, 27] == 0)
+
+    # adjoint identities in float64 on the full tensors
+    lhs = float(np.sum((y_h.astype(np.float64) - b.astype(np.float64)) * dy))
+    rhs_x = float(np.sum(x.astype(np.float64) * dx_h))
+    rhs_w = float(np.sum(w.astype(np.float64) * dw_h))
+    scale = float(np.sqrt(np.sum(y_h.astype(np.float64) ** 2)) * np.sqrt(np.sum(dy.astype(np.float64) ** 2)))
+    assert abs(lhs - rhs_x) <= 1e-6 * scale, (lhs, rhs_x)
+    assert abs(lhs - rhs_w) <= 1e-6 * scale, (lhs, rhs_w)
+    abi.close(db_h, np.sum(dy.astype(np.float64), axis=(0, 1, 2)), rms_scaled=True)
+
+    # wgrad of a gradient supported on one sample == the oracle's wgrad of that sample
+    for s in (0, S - 1):
+        dy1 = np.zeros_like(dy)
+        dy1[s] = dy[s]
+        dyd.set(dy1)
+        _lib.check(L.aeth_conv_wgrad_f32(xd.ptr, dyd.ptr, dw.ptr, db.ptr, *dims))
+        want = O.conv_wgrad(x[s:s + 1], dy[s:s + 1], (fH, fW), stride, pad, dtype=np.float64)
+        abi.close(dw.get(), want, rms_scaled=True)
+        abi.close(db.get(), np.sum(dy[s].astype(np.float64), axis=(0, 1)), rms_scaled=True)
+
+    # wgrad is additive over the batch: halves sum to the whole
+    half = S // 2
+    dy1 = dy.copy()
+    dy1[half:] = 0
+    dyd.set(dy1)
+    _lib.check(L.aeth_conv_wgrad_f32(xd.ptr, dyd.ptr, dw.ptr, None, *dims))
+    first = dw.get().astype(np.float64)
+    dy1 = dy.copy()
+    dy1[:half] = 0
+    dyd.set(dy1)
+    _lib.check(L.aeth_conv_wgrad_f32(xd.ptr, dyd.ptr, dw.ptr, None, *dims))
+    abi.close(dw_h, first + dw.get().astype(np.float64), rms_scaled=True)

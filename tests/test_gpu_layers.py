@@ -1,0 +1,304 @@
+"""Parity of the layer classes (reference API, HIP underneath) with the CPU
+oracle.  fp32 tolerance 1e-5 + 1e-4*|oracle| unless a test says otherwise;
+index / mask / selection work (pooling argmax, ReLU masks) is bit-exact."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _close(got, want, **kw):
+    from tests import abi
+    return abi.close(np.asarray(got), want, **kw)
+
+
+# ---- Conv_Layer class API ---------------------------------------------------------
+def test_conv_layer_api_and_parity():
+    import aether
+    np.random.seed(0)
+    layer = aether.Conv_Layer((12, 12, 8), num_filters=16, filter_size=(3, 3), strides=(1, 1), padding="same")
+    assert layer.weights is layer.filter_weights
+    assert layer.filter_weights.shape == (3, 3, 8, 16) and layer.biases.shape == (16,)
+    assert layer.weight_regularizer_l2 == 0 and layer.bias_regularizer_l1 == 0
+    # He-normal draw from the legacy global RNG in the reference's order
+    np.random.seed(0)
+    want_w = np.random.randn(3, 3, 8, 16).astype(np.float32) * np.sqrt(np.float32(2.0 / 72))
+    assert np.array_equal(layer.filter_weights.get(), want_w)
+    assert np.all(layer.biases.get() == 0)
+    x = np.random.randn(4, 12, 12, 8).astype(np.float32)
+    dy = np.random.randn(4, 12, 12, 16).astype(np.float32)
+    b = np.random.randn(16).astype(np.float32)
+    layer.set_parameters(want_w, b)
+    assert layer.weights is layer.filter_weights            # alias refreshed
+    out = layer.forward(x, training=True)
+    assert out is layer.output and out.shape == (4, 12, 12, 16)
+    _close(out, O.conv_fprop(x, want_w, b, (1, 1), "same", dtype=np.float64))
+    ret = layer.backward(dy)
+    assert ret is layer.dinputs and ret.shape == x.shape
+    _close(layer.dinputs, O.conv_dgrad(dy, want_w, (12, 12), (1, 1), "same", dtype=np.float64))
+    _close(layer.dweights, O.conv_wgrad(x, dy, (3, 3), (1, 1), "same", dtype=np.float64), rms_scaled=True)
+    _close(layer.dbiases, O.conv_dbias(dy, dtype=np.float64), rms_scaled=True)
+    w2, b2 = layer.get_parameters()
+    assert w2 is layer.filter_weights and b2 is layer.biases
+    with pytest.raises(ValueError):
+        layer.forward(np.zeros((4, 12, 12), np.float32), training=True)
+
+
+def test_conv_layer_same_with_1x1_returns_full_gradient():
+    import aether
+    np.random.seed(1)
+    layer = aether.Conv_Layer((6, 6, 4), num_filters=8, filter_size=(1, 1), strides=(1, 1), padding="same")
+    x = np.random.randn(2, 6, 6, 4).astype(np.float32)
+    dy = np.random.randn(2, 6, 6, 8).astype(np.float32)
+    layer.forward(x, True)
+    layer.backward(dy)
+    assert layer.dinputs.shape == (2, 6, 6, 4)
+    w = layer.filter_weights.get()
+    _close(layer.dinputs, (dy.reshape(-1, 8).astype(np.float64) @ w.reshape(4, 8).T.astype(np.float64)).reshape(2, 6, 6, 4))
+
+
+# ---- dense ------------------------------------------------------------------------------
+@pytest.mark.parametrize("M,n_in,n_out", [(128, 2048, 256), (128, 256, 10), (7, 5, 3), (33, 100, 64)])
+def test_dense_parity(M, n_in, n_out):
+    import aether
+    np.random.seed(2)
+    layer = aether.Layer_Dense(n_in, n_out, weight_regularizer_l1=1e-3, bias_regularizer_l1=2e-3,
+                               weight_regularizer_l2=3e-3, bias_regularizer_l2=4e-3)
+    assert layer.weights.shape == (n_in, n_out) and layer.biases.shape == (1, n_out)
+    w = (np.random.randn(n_in, n_out) * 0.1).astype(np.float32)
+    w[0, 0] = 0.0                                         # sign(0) = +1 in the L1 term
+    b = np.random.randn(1, n_out).astype(np.float32)
+    layer.set_parameters(w, b)
+    x = np.random.randn(M, n_in).astype(np.float32)
+    dy = np.random.randn(M, n_out).astype(np.float32)
+    layer.forward(x, training=True)
+    # outputs here have rms ~ 0.1*sqrt(n_in) > 1: the absolute part of the
+    # tolerance is scaled by that rms (see tests/abi.py)
+    _close(layer.output, O.dense_forward(x, w, b, dtype=np.float64), rms_scaled=True)
+    assert layer.backward(dy) is None
+    dw, db, dx = O.dense_backward(x, w, b, dy, wl1=1e-3, wl2=3e-3, bl1=2e-3, bl2=4e-3, dtype=np.float64)
+    _close(layer.dweights, dw, rms_scaled=True)
+    _close(layer.dbiases, db, rms_scaled=True)
+    _close(layer.dinputs, dx, rms_scaled=True)
+    assert layer.dbiases.shape == (1, n_out)
+
+
+# ---- activations ---------------------------------------------------------------------------
+def test_relu_and_leaky_relu_bit_exact():
+    import aether
+    r = np.random.RandomState(3)
+    x = r.randn(5, 7, 3, 9).astype(np.float32)
+    x[0, 0, 0, :3] = [0.0, -0.0, 1e-30]
+    dy = r.randn(*x.shape).astype(np.float32)
+    relu = aether.ReLU()
+    relu.forward(x, True)
+    relu.backward(dy)
+    assert np.array_equal(relu.output.get(), O.relu_forward(x))
+    assert np.array_equal(relu.dinputs.get(), O.relu_backward(x, dy))
+    lk = aether.Leaky_ReLU(0.01)
+    lk.forward(x, True)
+    lk.backward(dy)
+    assert np.array_equal(lk.output.get(), O.leaky_relu_forward(x, 0.01))
+    assert np.array_equal(lk.dinputs.get(), O.leaky_relu_backward(x, dy, 0.01))
+    assert aether.Leaky_ReLU().alpha == 0.01
+
+
+# ---- pooling -----------------------------------------------------------------------------------
+def test_maxpool_notebook_example_and_ties():
+    import aether
+    # CNN/notebooks/Backpropagation_Pooling.ipynb:103-128
+    a = np.array([[1, 2, 3, 4], [4, 5, 6, 5], [7, 8, 9, 6], [8, 7, 6, 5]], dtype=np.float32)
+    pool = aether.Pooling()
+    out = pool.forward(a[None, :, :, None], True)
+    assert np.array_equal(out.get()[0, :, :, 0], [[5, 6], [8, 9]])
+    pool.backward(out)
+    want = np.zeros((4, 4), np.float32)
+    want[1, 1], want[1, 2], want[2, 1], want[2, 2] = 5, 6, 8, 9
+    assert np.array_equal(pool.dinputs.get()[0, :, :, 0], want)
+    # all-zero window (post-ReLU) routes to the top-left element
+    z = np.zeros((1, 2, 2, 1), np.float32)
+    pool.forward(z, True)
+    pool.backward(np.ones((1, 1, 1, 1), np.float32))
+    assert np.array_equal(pool.dinputs.get()[0, :, :, 0], [[1, 0], [0, 0]])
+
+
+@pytest.mark.parametrize("shape,f,s", [((4, 16, 16, 32), (2, 2), (2, 2)), ((2, 7, 6, 3), (2, 2), (2, 2)),
+                                       ((2, 9, 9, 5), (3, 3), (2, 2)), ((2, 8, 8, 4), (2, 2), (1, 1)),
+                                       ((3, 10, 7, 6), (3, 2), (1, 2))])
+def test_maxpool_bit_exact(shape, f, s):
+    import aether
+    r = np.random.RandomState(4)
+    x = r.randint(0, 5, shape).astype(np.float32)          # many ties
+    pool = aether.Pooling(filter_size=f, strides=s)
+    pool.forward(x, True)
+    pooled, idx = O.maxpool_forward(x, f, s)
+    assert np.array_equal(pool.output.get(), pooled)
+    assert np.array_equal(pool.max_indicies.get(), idx.astype(np.uint8))
+    dy = r.randn(*pooled.shape).astype(np.float32)
+    pool.backward(dy)
+    want = O.maxpool_backward(dy, idx, x.shape, f, s)
+    if s[0] >= f[0] and s[1] >= f[1]:
+        assert np.array_equal(pool.dinputs.get(), want)
+    else:
+        _close(pool.dinputs, want)
+
+
+def test_avgpool_and_pooling_errors():
+    import aether
+    a = np.array([[1, 2, 3, 4], [4, 5, 6, 5], [7, 8, 9, 6], [8, 7, 6, 5]], dtype=np.float32)
+    pool = aether.Pooling(pooling_type="average")
+    out = pool.forward(a[None, :, :, None], True)
+    assert np.array_equal(out.get()[0, :, :, 0], [[3, 4.5], [7.5, 6.5]])      # nb :483-516
+    pool.backward(out)
+    assert np.array_equal(pool.dinputs.get()[0, :2, 2:, 0], np.full((2, 2), 1.125))
+    r = np.random.RandomState(5)
+    x = r.randn(2, 9, 8, 3).astype(np.float32)
+    pool = aether.Pooling((3, 3), (2, 1), pooling_type="average")
+    pool.forward(x, True)
+    _close(pool.output, O.avgpool_forward(x, (3, 3), (2, 1)))
+    dy = r.randn(*pool.output.shape).astype(np.float32)
+    pool.backward(dy)
+    _close(pool.dinputs, O.avgpool_backward(dy, x.shape, (3, 3), (2, 1)))
+    with pytest.raises(ValueError):
+        aether.Pooling().forward(np.zeros((2, 4, 4), np.float32), True)
+    with pytest.raises(ValueError):
+        aether.Pooling(padding="full").forward(np.zeros((2, 4, 4, 1), np.float32), True)
+
+
+# ---- batch norm ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(128, 32, 32, 32), (16, 8, 8, 128), (6, 5, 5, 3), (64, 40), (3, 4, 4, 70)])
+def test_batch_norm_parity(shape):
+    import aether
+    r = np.random.RandomState(6)
+    C = shape[-1]
+    x = (r.randn(*shape) * 2 + 5).astype(np.float32)       # mean >> 0 stresses the variance
+    dy = r.randn(*shape).astype(np.float32)
+    g = (r.rand(C) + 0.5).astype(np.float32)
+    be = r.randn(C).astype(np.float32)
+    bn = aether.Batch_Norm()
+    assert bn.gamma is None and bn.running_mean is None
+    bn.forward(x, training=True)                            # lazy init: gamma 1, beta 0
+    assert np.all(bn.gamma.get() == 1) and np.all(bn.beta.get() == 0)
+    assert bn.weights is bn.gamma and bn.biases is bn.beta
+    bn.set_parameters(g, be, np.zeros(C, np.float32), np.ones(C, np.float32))
+    bn.forward(x, training=True)
+    x64 = x.astype(np.float64)
+    y, xhat, mu, var, rm, rv = O.bn_forward_train(x64, g.astype(np.float64), be.astype(np.float64),
+                                                  np.zeros(C), np.ones(C), 1e-5, 0.9)
+    _close(bn.output, y)
+    assert bn.running_mean.shape == rm.shape               # keepdims shape, as saved by the reference
+    _close(bn.running_mean, rm)
+    _close(bn.running_var, rv)
+    bn.backward(dy)
+    dx, dg, db = O.bn_backward(x64, dy.astype(np.float64), g.astype(np.float64), mu, var, 1e-5)
+    _close(bn.dinputs, dx)
+    _close(bn.dweights, dg, rms_scaled=True)
+    _close(bn.dbiases, db, rms_scaled=True)
+    bn.forward(x, training=False)
+    _close(bn.output, O.bn_forward_infer(x64, g.astype(np.float64), be.astype(np.float64), rm, rv, 1e-5))
+    assert len(bn.get_parameters()) == 4
+
+
+# ---- dropout -------------------------------------------------------------------------------------
+def test_dropout_layers_with_reference_shaped_masks():
+    import aether
+    r = np.random.RandomState(7)
+    x = r.randn(4, 6, 6, 8).astype(np.float32)
+    dy = r.randn(*x.shape).astype(np.float32)
+    d = aether.Layer_Dropout(0.25)
+    assert d.rate == 0.75
+    np.random.seed(11)
+    d.forward(x, training=True)
+    np.random.seed(11)
+    mask = (np.random.binomial(1, 0.75, size=x.shape) / 0.75).astype(np.float32)
+    assert np.array_equal(d.output.get(), mask * x)
+    d.backward(dy)
+    assert np.array_equal(d.dinputs.get(), dy * mask)
+    d.forward(x, training=False)
+    assert np.array_equal(d.output.get(), x)
+    sp = aether.Layer_Dropout_Spatial(0.5)
+    np.random.seed(12)
+    sp.forward(x, training=True)
+    np.random.seed(12)
+    cmask = (np.random.binomial(1, 0.5, size=(1, 1, 1, 8)) / 0.5).astype(np.float32)
+    assert np.array_equal(sp.output.get(), x * cmask)
+    sp.backward(dy)
+    assert np.array_equal(sp.dinputs.get(), dy * cmask)
+    d0 = aether.Layer_Dropout(0.0)                           # rate 0: identity
+    d0.forward(x, training=True)
+    assert np.array_equal(d0.output.get(), x)
+
+
+# ---- flatten / softmax / loss / adam ------------------------------------------------------------------
+def test_flatten_softmax_loss():
+    import aether
+    r = np.random.RandomState(8)
+    x = r.randn(4, 3, 2, 5).astype(np.float32)
+    fl = aether.Flatten()
+    fl.forward(x, True)
+    assert np.array_equal(fl.output.get(), x.reshape(4, -1))
+    fl.backward(fl.output)
+    assert fl.dinputs.shape == x.shape
+    logits = (r.randn(128, 10) * 3).astype(np.float32)
+    y = r.randint(0, 10, 128)
+    sm = aether.SoftMax()
+    sm.forward(logits, True)
+    p64 = O.softmax(logits.astype(np.float64))
+    _close(sm.output, p64)
+    assert np.array_equal(sm.predictions(sm.output), np.argmax(p64, axis=1))
+    dv = r.randn(128, 10).astype(np.float32)
+    sm.backward(dv)
+    jac = np.stack([(np.diagflat(p) - np.outer(p, p)) @ d for p, d in zip(p64, dv.astype(np.float64))])
+    _close(sm.dinputs, jac)
+    for ls in (0.0, 0.01):
+        loss = aether.Loss_CategoricalCrossEntropy(label_smoothing=ls)
+        loss.new_pass()
+        loss.remember_trainable_layers([])
+        data_loss, reg = loss.calculate(sm.output, y, include_regularization=True, training=True)
+        want = O.cce_forward(p64, y, ls, training=True)
+        assert abs(data_loss - want.mean()) <= 1e-5 + 1e-4 * abs(want.mean()) and reg == 0
+        ev = loss.calculate(sm.output, y, training=False)
+        assert abs(ev - O.cce_forward(p64, y, ls, training=False).mean()) <= 1e-4
+        assert abs(loss.calculate_accumulated() - (want.sum() + O.cce_forward(p64, y, 0.0).sum()) / 256) <= 1e-4
+        comb = aether.Activation_Softmax_Loss_CategoricalCrossEntropy(ls)
+        comb.backward(sm.output, y, training=True)
+        _close(comb.dinputs, O.softmax_cce_backward(p64, y, ls))
+        comb.backward(sm.output, np.eye(10)[y], training=True)        # one-hot labels
+        _close(comb.dinputs, O.softmax_cce_backward(p64, y, ls))
+
+
+def test_regularization_loss_and_adam():
+    import aether
+    np.random.seed(9)
+    dense = aether.Layer_Dense(20, 30, weight_regularizer_l1=0.1, bias_regularizer_l1=0.2,
+                               weight_regularizer_l2=0.3, bias_regularizer_l2=0.4)
+    w = np.random.randn(20, 30).astype(np.float32)
+    b = np.random.randn(1, 30).astype(np.float32)
+    dense.set_parameters(w, b)
+    loss = aether.Loss_CategoricalCrossEntropy()
+    loss.remember_trainable_layers([dense])
+    want = 0.1 * np.abs(w).sum() + 0.3 * (w * w).sum() + 0.2 * np.abs(b).sum() + 0.4 * (b * b).sum()
+    assert abs(loss.regularization_loss() - want) <= 1e-4 * want
+    opt = aether.Optimizer_Adam(learning_rate=1e-3, decay=1e-2)
+    th, bb = w.astype(np.float64), b.astype(np.float64)
+    m = [np.zeros_like(th), np.zeros_like(bb)]
+    v = [np.zeros_like(th), np.zeros_like(bb)]
+    for it in range(4):
+        gw = np.random.randn(20, 30).astype(np.float32)
+        gb = np.random.randn(1, 30).astype(np.float32)
+        dense.dweights = aether.DeviceTensor.from_numpy(gw)
+        dense.dbiases = aether.DeviceTensor.from_numpy(gb)
+        opt.pre_update_parameters()
+        opt.update_parameters(dense)
+        opt.post_update_parameters()
+        lr = 1e-3 / (1 + 1e-2 * it)
+        assert abs(opt.current_learning_rate - lr) < 1e-12
+        th, m[0], v[0] = O.adam_update(th, gw.astype(np.float64), m[0], v[0], lr, it)
+        bb, m[1], v[1] = O.adam_update(bb, gb.astype(np.float64), m[1], v[1], lr, it)
+        _close(dense.weights, th)
+        _close(dense.biases, bb)
+    assert opt.iterations == 4
+    _close(dense.weight_momentums, m[0])
+    _close(dense.weight_cache, v[0], atol=1e-7)

@@ -1,0 +1,236 @@
+"""Whole training step of the three-block CNN (batch 128, 32x32x3 synthetic
+images) through the reference's Model API on the GPU, against the float64 CPU
+oracle started from the same float32 parameters.
+
+Tolerances.  Scalars and per-tensor parameter gradients: 1e-5*max(1,rms) +
+1e-4*|oracle| (the rms scaling is explained in tests/abi.py), applied to the
+first step.  Activations' gradients pass through ReLU / max-pool selections,
+where a float32 and a float64 evaluation may pick differently for values within
+rounding of a tie; those tensors are compared by relative L2 error <= 1e-4 and by
+the share of elements outside tolerance <= 1e-4.  After three Adam steps the
+parameters are compared with rtol 1e-3: Adam's m/sqrt(v) amplifies rounding of
+tiny gradients (|g| ~ eps) into O(lr) differences, so the updated parameters get
+an absolute allowance of 2*lr per step."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def build_model(aether, label_smoothing=0.01, hw=32, in_ch=3):
+    m = aether.Model()
+    c = in_ch
+    size = hw
+    for d in (32, 64, 128):
+        m.add(aether.Conv_Layer((size, size, c), num_filters=d, filter_size=(3, 3), strides=(1, 1), padding="same"))
+        m.add(aether.Batch_Norm())
+        m.add(aether.ReLU())
+        m.add(aether.Pooling(filter_size=(2, 2), strides=(2, 2), padding="valid", pooling_type="max"))
+        c = d
+        size //= 2
+    m.add(aether.Flatten())
+    m.add(aether.Layer_Dense(size * size * 128, 256))
+    m.add(aether.Leaky_ReLU(alpha=0.01))
+    m.add(aether.Layer_Dense(256, 10))
+    m.add(aether.SoftMax())
+    m.set(loss=aether.Loss_CategoricalCrossEntropy(label_smoothing=label_smoothing),
+          optimizer=aether.Optimizer_Adam(learning_rate=1e-3),
+          accuracy=aether.Accuracy_Categorical())
+    m.finalize()
+    return m
+
+
+def host_params(model):
+    """Parameter tuples as float32 NumPy arrays; BN running stats that do not exist
+    yet (lazy init) are the reference's initial values."""
+    out = []
+    for layer in model.trainable_layers:
+        tup = layer.get_parameters()
+        if len(tup) == 4 and tup[0] is None:
+            C = layer.prev.filter_weights.shape[3]
+            out.append((np.ones(C, np.float32), np.zeros(C, np.float32), np.zeros(C, np.float32),
+                        np.ones(C, np.float32)))
+        else:
+            out.append(tuple(np.asarray(a) for a in tup))
+    return out
+
+
+def rel_l2(got, want):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    return float(np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30))
+
+
+def outside_share(got, want, rtol=1e-4, atol=1e-5):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    scale = max(1.0, float(np.sqrt(np.mean(want * want))))
+    return float(np.mean(np.abs(got - want) > atol * scale + rtol * np.abs(want)))
+
+
+def test_three_block_cnn_training_steps_match_oracle(capsys):
+    import aether
+    from tests import abi
+    np.random.seed(0)
+    X = np.random.rand(128, 32, 32, 3).astype(np.float32)
+    y = np.random.randint(0, 10, 128)
+    model = build_model(aether)
+    assert [type(l).__name__ for l in model.trainable_layers] == \
+        ["Conv_Layer", "Batch_Norm"] * 3 + ["Layer_Dense", "Layer_Dense"]
+    assert model.softmax_classifier_output is not None
+    params = host_params(model)
+    n_params = sum(int(np.prod(a.shape)) for tup in params for a in tup[:2])
+    assert n_params == 620810
+    net = O.OracleCNN(params, label_smoothing=0.01, lr=1e-3, dtype=np.float64)
+
+    model.loss.new_pass()
+    model.accuracy.new_pass()
+    for step in range(3):
+        ref = net.step(X, y)
+        loss, data_loss, reg_loss, acc = model.train_step(X, y)
+        assert reg_loss == 0
+        assert abs(loss - ref["loss"]) <= 1e-5 + 1e-4 * abs(ref["loss"]), (step, loss, ref["loss"])
+        assert abs(acc - ref["acc"]) <= 1.0 / 128 + 1e-9
+        probs = model.layers[-1].output.get()
+        assert rel_l2(probs, ref["probs"]) <= (1e-4 if step == 0 else 2e-3)
+        if step == 0:
+            abi.close(probs, ref["probs"])
+            for i, layer in enumerate(model.trainable_layers):
+                gw, gb = ref["grads"][i]
+                name = "%d:%s" % (i, type(layer).__name__)
+                assert rel_l2(layer.dweights.get(), gw.reshape(layer.dweights.shape)) <= 2e-4, name
+                assert outside_share(layer.dweights.get(), gw.reshape(layer.dweights.shape)) <= 1e-3, name
+                if np.linalg.norm(gb) > 1e-12:          # conv biases feed a batch norm: gradient is 0
+                    assert rel_l2(layer.dbiases.get(), gb.reshape(layer.dbiases.shape)) <= 2e-4, name
+                else:
+                    assert np.abs(layer.dbiases.get()).max() <= 1e-5, name
+            convs = [l for l in model.layers if isinstance(l, aether.Conv_Layer)]
+            for blk, conv in enumerate(convs):
+                want = ref["dinputs"]["conv%d" % blk]
+                assert conv.dinputs.shape == want.shape
+                assert rel_l2(conv.dinputs.get(), want) <= 2e-4, blk
+                assert outside_share(conv.dinputs.get(), want) <= 1e-3, blk
+        lr_allow = 2e-3 * (step + 1)
+        for i, layer in enumerate(model.trainable_layers):
+            got = [np.asarray(a) for a in layer.get_parameters()]
+            for j, want in enumerate(net.p[i]):
+                g = got[j].reshape(want.shape)
+                if j < 2:
+                    assert np.all(np.abs(g - want) <= lr_allow + 1e-3 * np.abs(want)), (step, i, j)
+                else:                                      # BN running statistics
+                    assert np.all(np.abs(g - want) <= 1e-5 + 1e-3 * np.abs(want)), (step, i, j)
+    assert model.optimizer.iterations == 3
+    assert model.loss.accumulated_count == 3 * 128
+
+    # evaluation path (running statistics, no smoothing) and predict()
+    probs_eval, _ = net.forward(X, training=False)
+    pred = model.predict(X, batch_size=50)                  # ragged last batch
+    assert pred.shape == (128, 10)
+    assert rel_l2(pred, probs_eval) <= 5e-3
+    model.evaluate(X, y, batch_size=64)
+    out = capsys.readouterr().out
+    assert "Valdiation, acc:" in out
+    want_loss = float(np.mean(O.cce_forward(probs_eval, y, 0.01, training=False)))
+    assert abs(float(model.loss.calculate_accumulated()) - want_loss) <= 5e-3 * max(1.0, want_loss)
+
+
+def test_train_prints_reference_format_and_parameters_round_trip(tmp_path, capsys):
+    import aether
+    np.random.seed(3)
+    X = np.random.rand(48, 16, 16, 3).astype(np.float32)
+    y = np.random.randint(0, 10, 48)
+    model = build_model(aether, hw=16)
+    model.train(X, y, epochs=2, batch_size=20, print_every=2, validation_data=(X, y))
+    out = capsys.readouterr().out.splitlines()
+    assert out[0] == "Training" and out[1] == " epoch: 1"
+    step_lines = [l for l in out if l.startswith("epoch: ")]
+    assert len(step_lines) == 4                              # steps 0 and 2 of each epoch
+    assert step_lines[0].startswith("epoch: 1, acc: 0.") and ", loss: " in step_lines[0]
+    assert "(data_loss: " in step_lines[0] and "reg_loss: 0.000, lr:: 0.001" in step_lines[0]
+    assert any(l.startswith(" training, acc: ") for l in out)
+    assert any(l.startswith("Valdiation, acc: ") for l in out)
+
+    path = str(tmp_path / "params.pkl")
+    model.save_parameters(path)
+    before = model.predict(X)
+    np.random.seed(4)
+    other = build_model(aether, hw=16)
+    other.forward(X[:4], training=False)                     # lazily creates the BN tensors
+    other.load_parameters(path)
+    assert other.layers[0].weights is other.layers[0].filter_weights
+    after = other.predict(X)
+    assert np.array_equal(before, after)
+    with pytest.raises(Exception):
+        bad = tmp_path / "bad.pkl"
+        import pickle
+        bad.write_bytes(pickle.dumps([(__import__("os").getcwd,)]))
+        other.load_parameters(str(bad))
+
+
+def test_load_parameters_accepts_cupy_wrapped_float64_checkpoints(tmp_path):
+    """The reference's CuPy checkpoints pickle every array as
+    cupy._core.core.array(ndarray), dense weights in float64 and BN running stats
+    with shape (1,1,1,C).  A file with that structure (written here, synthetic
+    values) loads without CuPy."""
+    import pickle
+    import aether
+
+    class _Wrapped:                                           # pickles as cupy._core.core.array(ndarray)
+        def __init__(self, a):
+            self.a = a
+
+        def __reduce__(self):
+            return (_FakeCupyArray, (self.a,))
+
+    class _FakeCupyArray:
+        pass
+    _FakeCupyArray.__module__ = "cupy._core.core"
+    _FakeCupyArray.__qualname__ = _FakeCupyArray.__name__ = "array"
+
+    import sys
+    import types
+    mods = {}
+    for name in ("cupy", "cupy._core", "cupy._core.core"):
+        mods[name] = types.ModuleType(name)
+    mods["cupy._core.core"].array = _FakeCupyArray
+    sys.modules.update(mods)
+    try:
+        r = np.random.RandomState(5)
+        params = [
+            (r.randn(3, 3, 1, 32).astype(np.float32), r.randn(32).astype(np.float32)),
+            (r.rand(32).astype(np.float32) + 0.5, r.randn(32).astype(np.float32),
+             r.randn(1, 1, 1, 32).astype(np.float32), r.rand(1, 1, 1, 32).astype(np.float32) + 0.5),
+            (r.randn(6272, 10) * 0.01, r.randn(1, 10)),       # float64 dense
+        ]
+        blob = pickle.dumps([tuple(_Wrapped(a) for a in tup) for tup in params], protocol=4)
+    finally:
+        for name in mods:
+            sys.modules.pop(name, None)
+    assert b"cupy._core.core" in blob
+    path = tmp_path / "cupy_style"
+    path.write_bytes(blob)
+
+    m = aether.Model()
+    m.add(aether.Conv_Layer((28, 28, 1), num_filters=32))
+    m.add(aether.Batch_Norm())
+    m.add(aether.ReLU())
+    m.add(aether.Pooling())
+    m.add(aether.Flatten())
+    m.add(aether.Layer_Dense(6272, 10))
+    m.add(aether.SoftMax())
+    m.set(loss=aether.Loss_CategoricalCrossEntropy(), optimizer=aether.Optimizer_Adam(),
+          accuracy=aether.Accuracy_Categorical())
+    m.finalize()
+    m.load_parameters(str(path))
+    x = r.rand(5, 28, 28, 1).astype(np.float32)
+    got = m.predict(x)
+    W, b = params[0]
+    a = O.conv_fprop(x, W, b, (1, 1), "same", dtype=np.float64)
+    g, be, rm, rv = (p.astype(np.float64) for p in params[1])
+    a = O.relu_forward(O.bn_forward_infer(a, g, be, rm, rv, 1e-5))
+    a, _ = O.maxpool_forward(a, dtype=np.float64)
+    want = O.softmax(O.dense_forward(a.reshape(5, -1), params[2][0], params[2][1], dtype=np.float64))
+    from tests import abi
+    abi.close(got, want, rtol=1e-3)
