@@ -1,0 +1,765 @@
+// Implicit-GEMM convolution kernels for gfx950, shared by the fp32 and the
+// bf16-input entry points (T = float or uint16_t holding bf16 bits).
+//
+// GEMM view (M = S*Ho*Wo, N = D, K = fH*fW*C):
+//   fprop : Y[M,N]  = A[M,K] . W[K,N] + bias      A gathered from x on the fly
+//   dgrad : dX[M',C] = A'[M',K'] . W'[K',C]        A' gathered from dy; one launch
+//           per stride-parity class so that no tap multiplies a structural zero
+//   wgrad : dW[K,N] = A[M,K]^T . dY[M,N]           reduction over M split across
+//           workgroups, partial sums reduced in a fixed order
+//
+// "gather" kernel (fprop, dgrad, dense fprop/dgrad)
+//   workgroup = 256 threads = 4 waves, tile BM x BN; K is consumed in slabs of
+//   128 bytes per row (32 floats or 64 bf16).  An A slab is read with one 128-bit
+//   load per thread per chunk (NHWC: channels are contiguous), zero where the tap
+//   falls in the padding, and stored to LDS row-major with a row pitch of 144
+//   bytes; the B slab comes from a pre-packed [N][K] copy of the filter and uses
+//   the same pitch.  With that pitch the 128-bit stores and the 128-bit operand
+//   reads both touch 32 distinct banks per 8 lanes.
+//   fp32: each lane feeds the 4 floats of its chunk to 4 successive
+//   v_mfma_f32_32x32x2_f32; the k order inside a slab is permuted identically for
+//   A and B, which leaves the sum unchanged.
+//   bf16: a chunk is exactly the 8 k-values one lane supplies to
+//   v_mfma_f32_32x32x16_bf16.
+#pragma once
+
+#include "common.h"
+
+#include <limits.h>
+#include <vector>
+
+namespace aeth {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kThreads = 256;
+constexpr int kChunksPerRow = 8;   // 16-byte chunks per slab row
+constexpr int kLDC = 9;            // LDS row pitch in chunks (8 data + 1 pad)
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static constexpr int CE = 4;   // elements per 16-byte chunk
+    static constexpr int BK = 32;  // elements per slab row
+    static __device__ __forceinline__ float to_f32(float v) { return v; }
+};
+template <> struct Elem<uint16_t> {
+    static constexpr int CE = 8;
+    static constexpr int BK = 64;
+    static __device__ __forceinline__ float to_f32(uint16_t v) { return __uint_as_float((unsigned)v << 16); }
+};
+
+template <typename T>
+__device__ __forceinline__ void mma_chunk(const f4& a, const f4& b, f16v& acc);
+
+template <>
+__device__ __forceinline__ void mma_chunk<float>(const f4& a, const f4& b, f16v& acc) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b[t], acc, 0, 0, 0);
+}
+
+template <>
+__device__ __forceinline__ void mma_chunk<uint16_t>(const f4& a, const f4& b, f16v& acc) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc,
+                                                  0, 0, 0);
+}
+
+// ------------------------------------------------------------------------------
+// gather-GEMM
+// ------------------------------------------------------------------------------
+struct GatherParams {
+    const void* src;     // [S, Hs, Ws, Cs] of T
+    const void* bt;      // packed filter [Npad][Kpad] of T, zero filled
+    const float* bias;   // [N] or nullptr
+    float* out;
+    int S, Hs, Ws, Cs;
+    int Hg, Wg;          // output pixel grid of this launch
+    int M, N, K, Kpad;   // M = S*Hg*Wg, K = Th*Tw*Cs
+    int Tw;              // taps per filter row
+    int sh, sw;          // source step per output pixel
+    int rh0, rw0;        // source offset of tap (0,0)
+    // output element (s,i,j,n) lives at ((s*Hof + oh0 + i*ohs)*Wof + ow0 + j*ows)*N + n
+    int Hof, Wof, oh0, ow0, ohs, ows;
+    int dense_out;       // 1: row m is stored at out + m*N
+    FastDiv div_hw, div_w, div_c, div_tw;
+};
+
+constexpr int kInvalidRow = -16384;
+
+template <typename T, int BM, int BN, int WM, int WN, int VEC>
+__global__ __launch_bounds__(kThreads) void gather_gemm(const GatherParams p) {
+    static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "32x32 MFMA tiles");
+    constexpr int CE = Elem<T>::CE;
+    constexpr int BK = Elem<T>::BK;
+    constexpr int AL = BM / 32;          // 128-bit A loads per thread per slab
+    constexpr int BL = BN / 32;
+    constexpr int TM = WM / 32;
+    constexpr int TN = WN / 32;
+
+    __shared__ f4 lds_a[BM * kLDC];
+    __shared__ f4 lds_b[BN * kLDC];
+
+    const T* __restrict__ src = static_cast<const T*>(p.src);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int l32 = lane & 31;
+    const int lh = lane >> 5;
+    const int wm0 = (wave % (BM / WM)) * WM;
+    const int wn0 = (wave / (BM / WM)) * WN;
+
+    const int m0 = blockIdx.x * BM;
+    const int n0 = blockIdx.y * BN;
+
+    // ---- per-thread row bookkeeping for the A gather --------------------------
+    const int k4 = tid & 7;              // which chunk of the slab row
+    const int r0 = tid >> 3;             // first row handled (then +32 each)
+    int base_off[AL];
+    int base_rc[AL];                     // (row << 16) | (col & 0xffff) of tap (0,0)
+#pragma unroll
+    for (int i = 0; i < AL; ++i) {
+        int m = m0 + r0 + 32 * i;
+        if (m < p.M) {
+            unsigned s, rem, ii, jj;
+            p.div_hw.divmod((unsigned)m, s, rem);
+            p.div_w.divmod(rem, ii, jj);
+            int br = (int)ii * p.sh + p.rh0;
+            int bc = (int)jj * p.sw + p.rw0;
+            base_off[i] = (((int)s * p.Hs + br) * p.Ws + bc) * p.Cs;
+            base_rc[i] = (int)(((unsigned)br << 16) | ((unsigned)bc & 0xffffu));
+        } else {
+            base_off[i] = 0;
+            base_rc[i] = (int)((unsigned)kInvalidRow << 16);
+        }
+    }
+    const T* bt_row = static_cast<const T*>(p.bt) + (size_t)(n0 + r0) * p.Kpad + CE * k4;
+
+    f4 areg[AL];
+    f4 breg[BL];
+
+    auto load_slab = [&](int k0) {
+        if (VEC == CE) {
+            int kk = k0 + CE * k4;
+            unsigned tap, c, th, tw;
+            p.div_c.divmod((unsigned)kk, tap, c);
+            p.div_tw.divmod(tap, th, tw);
+            bool kvalid = kk < p.K;
+            int tap_off = ((int)th * p.Ws + (int)tw) * p.Cs + (int)c;
+#pragma unroll
+            for (int i = 0; i < AL; ++i) {
+                int r = (base_rc[i] >> 16) + (int)th;
+                int cc = ((int)((unsigned)base_rc[i] << 16) >> 16) + (int)tw;
+                bool ok = kvalid && (unsigned)r < (unsigned)p.Hs && (unsigned)cc < (unsigned)p.Ws;
+                f4 v = {0.f, 0.f, 0.f, 0.f};
+                if (ok) v = *reinterpret_cast<const f4*>(src + (base_off[i] + tap_off));
+                areg[i] = v;
+            }
+        } else {
+            struct Chunk { T e[CE]; } tmp[AL];
+#pragma unroll
+            for (int e = 0; e < CE; ++e) {
+                int kk = k0 + CE * k4 + e;
+                unsigned tap, c, th, tw;
+                p.div_c.divmod((unsigned)kk, tap, c);
+                p.div_tw.divmod(tap, th, tw);
+                bool kvalid = kk < p.K;
+                int tap_off = ((int)th * p.Ws + (int)tw) * p.Cs + (int)c;
+#pragma unroll
+                for (int i = 0; i < AL; ++i) {
+                    int r = (base_rc[i] >> 16) + (int)th;
+                    int cc = ((int)((unsigned)base_rc[i] << 16) >> 16) + (int)tw;
+                    bool ok = kvalid && (unsigned)r < (unsigned)p.Hs && (unsigned)cc < (unsigned)p.Ws;
+                    T v = (T)0;
+                    if (ok) v = src[base_off[i] + tap_off];
+                    tmp[i].e[e] = v;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < AL; ++i) areg[i] = __builtin_bit_cast(f4, tmp[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < BL; ++i)
+            breg[i] = *reinterpret_cast<const f4*>(bt_row + (size_t)(32 * i) * p.Kpad + k0);
+    };
+
+    auto store_slab = [&]() {
+#pragma unroll
+        for (int i = 0; i < AL; ++i) lds_a[(r0 + 32 * i) * kLDC + k4] = areg[i];
+#pragma unroll
+        for (int i = 0; i < BL; ++i) lds_b[(r0 + 32 * i) * kLDC + k4] = breg[i];
+    };
+
+    f16v acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    if (p.Kpad > 0) {
+        load_slab(0);
+        store_slab();
+        __syncthreads();
+    }
+
+    for (int k0 = 0; k0 < p.Kpad; k0 += BK) {
+        const bool more = k0 + BK < p.Kpad;
+        if (more) load_slab(k0 + BK);
+
+#pragma unroll
+        for (int g = 0; g < kChunksPerRow / 2; ++g) {
+            f4 a[TM], b[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) a[i] = lds_a[(wm0 + 32 * i + l32) * kLDC + 2 * g + lh];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) b[j] = lds_b[(wn0 + 32 * j + l32) * kLDC + 2 * g + lh];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) mma_chunk<T>(a[i], b[j], acc[i][j]);
+        }
+        __syncthreads();
+        if (more) {
+            store_slab();
+            __syncthreads();
+        }
+    }
+
+    // ---- epilogue: bias add and store -------------------------------------------
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int n = n0 + wn0 + 32 * j + l32;
+        const bool nok = n < p.N;
+        const float bv = (p.bias != nullptr && nok) ? p.bias[n] : 0.f;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + wm0 + 32 * i + 8 * (v >> 2) + 4 * lh + (v & 3);
+                if (nok && m < p.M) {
+                    size_t row;
+                    if (p.dense_out) {
+                        row = (size_t)m;
+                    } else {
+                        unsigned s, rem, ii, jj;
+                        p.div_hw.divmod((unsigned)m, s, rem);
+                        p.div_w.divmod(rem, ii, jj);
+                        row = ((size_t)s * p.Hof + p.oh0 + (size_t)ii * p.ohs) * p.Wof + p.ow0 + (size_t)jj * p.ows;
+                    }
+                    p.out[row * p.N + n] = acc[i][j][v] + bv;
+                }
+            }
+        }
+    }
+}
+
+// Packs the filter w[fH][fW][C][D] into bt[Npad][Kpad] (k contiguous) for one
+// gather-GEMM launch.  k = (th*Tw + tw)*Ck + kc ; filter tap x = xa + xs*th,
+// y = ya + ys*tw.  transposed == 0: n is the output channel d and kc the input
+// channel c (fprop).  transposed == 1: n is c and kc is d (dgrad).
+struct PackParams {
+    const void* w;
+    void* bt;
+    int fW, C, D;
+    int Tw, Ck;
+    int xa, xs, ya, ys;
+    int transposed;
+    int N, K, Npad, Kpad;
+};
+
+template <typename T>
+__global__ void pack_filter(const PackParams p) {
+    int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    int total = p.Npad * p.Kpad;
+    if (idx >= total) return;
+    int n = idx / p.Kpad;
+    int k = idx - n * p.Kpad;
+    T v = (T)0;
+    if (n < p.N && k < p.K) {
+        int tap = k / p.Ck;
+        int kc = k - tap * p.Ck;
+        int th = tap / p.Tw;
+        int tw = tap - th * p.Tw;
+        int x = p.xa + p.xs * th;
+        int y = p.ya + p.ys * tw;
+        int c = p.transposed ? n : kc;
+        int d = p.transposed ? kc : n;
+        v = static_cast<const T*>(p.w)[((size_t)(x * p.fW + y) * p.C + c) * p.D + d];
+    }
+    static_cast<T*>(p.bt)[idx] = v;
+}
+
+template <typename T, int BM, int BN, int WM, int WN>
+static void launch_gather_cfg(const GatherParams& gp, bool vec, hipStream_t st) {
+    dim3 grid(cdiv(gp.M, BM), cdiv(gp.N, BN));
+    if (vec)
+        hipLaunchKernelGGL((gather_gemm<T, BM, BN, WM, WN, Elem<T>::CE>), grid, dim3(kThreads), 0, st, gp);
+    else
+        hipLaunchKernelGGL((gather_gemm<T, BM, BN, WM, WN, 1>), grid, dim3(kThreads), 0, st, gp);
+}
+
+static inline int gather_bn(int N) { return N <= 32 ? 32 : 64; }
+
+static inline int gather_bm(int M, int N, int cus) {
+    const int bn = gather_bn(N);
+    const int ntiles = cdiv(N, bn);
+    const int want = 2 * cus;
+    const int cands[3] = {256, 128, 64};
+    for (int i = 0; i < 3; ++i) {
+        int bm = cands[i];
+        if (bn == 32 && bm == 64) break;
+        if ((int64_t)cdiv(M, bm) * ntiles >= want) return bm;
+    }
+    return bn == 32 ? 128 : 64;
+}
+
+template <typename T>
+static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t st) {
+    const int bn = gather_bn(gp.N);
+    const int bm = gather_bm(gp.M, gp.N, cus);
+    if (bn == 32) {
+        if (bm == 256) launch_gather_cfg<T, 256, 32, 64, 32>(gp, vec, st);
+        else launch_gather_cfg<T, 128, 32, 32, 32>(gp, vec, st);
+    } else {
+        if (bm == 256) launch_gather_cfg<T, 256, 64, 64, 64>(gp, vec, st);
+        else if (bm == 128) launch_gather_cfg<T, 128, 64, 32, 64>(gp, vec, st);
+        else launch_gather_cfg<T, 64, 64, 32, 32>(gp, vec, st);
+    }
+}
+
+// One gather-GEMM problem: pack the filter into the workspace at `ws_off`, launch.
+struct GatherSetup {
+    GatherParams gp;
+    PackParams pp;
+    int64_t bt_bytes;
+};
+
+template <typename T>
+static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
+    Context& c = ctx();
+    void* bt = ws + ws_off;
+    gs.gp.bt = bt;
+    gs.pp.bt = bt;
+    int total = gs.pp.Npad * gs.pp.Kpad;
+    if (total > 0) {
+        hipLaunchKernelGGL(pack_filter<T>, dim3(cdiv(total, 256)), dim3(256), 0, c.stream, gs.pp);
+        AETH_LAUNCH_CHECK();
+    }
+    if (gs.gp.M > 0 && gs.gp.N > 0) {
+        launch_gather<T>(gs.gp, vec, c.prop.multiProcessorCount, c.stream);
+        AETH_LAUNCH_CHECK();
+    }
+    return AETH_OK;
+}
+
+static inline int check_conv_dims(const char* fn, int S, int H, int W, int C, int D, int fH, int fW,
+                                  int sH, int sW, int pH, int pW, int* Ho, int* Wo) {
+    if (S <= 0 || H <= 0 || W <= 0 || C <= 0 || D <= 0 || fH <= 0 || fW <= 0 || sH <= 0 || sW <= 0 ||
+        pH < 0 || pW < 0)
+        return fail(AETH_E_INVALID, "%s: non-positive dimension", fn);
+    if (H + 2 * pH < fH || W + 2 * pW < fW) return fail(AETH_E_INVALID, "%s: filter larger than padded input", fn);
+    if (H >= 8192 || W >= 8192 || fH > 64 || fW > 64 || pH >= 64 || pW >= 64)
+        return fail(AETH_E_INVALID, "%s: spatial extent out of supported range", fn);
+    *Ho = (H + 2 * pH - fH) / sH + 1;
+    *Wo = (W + 2 * pW - fW) / sW + 1;
+    const int64_t lim = (int64_t)INT_MAX - (1 << 24);
+    if ((int64_t)S * (H + 2 * pH + fH) * (W + 2 * pW + fW) * C >= lim || (int64_t)S * *Ho * *Wo * D >= lim ||
+        (int64_t)fH * fW * C * D >= lim)
+        return fail(AETH_E_INVALID, "%s: tensor has 2^31 elements or more", fn);
+    return AETH_OK;
+}
+
+static inline void set_out_divs(GatherParams& g) {
+    g.div_hw = FastDiv(g.Hg * g.Wg > 0 ? g.Hg * g.Wg : 1);
+    g.div_w = FastDiv(g.Wg > 0 ? g.Wg : 1);
+    g.div_c = FastDiv(g.Cs);
+    g.div_tw = FastDiv(g.Tw > 0 ? g.Tw : 1);
+}
+
+template <typename T>
+int conv_fprop_impl(const char* fn, const T* x, const T* w, const float* bias, float* y,
+                    int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW) {
+    int Ho, Wo;
+    int rc = check_conv_dims(fn, S, H, W, C, D, fH, fW, sH, sW, pH, pW, &Ho, &Wo);
+    if (rc) return rc;
+    constexpr int BK = Elem<T>::BK;
+    GatherSetup gs;
+    GatherParams& g = gs.gp;
+    g.src = x; g.bias = bias; g.out = y;
+    g.S = S; g.Hs = H; g.Ws = W; g.Cs = C;
+    g.Hg = Ho; g.Wg = Wo; g.M = S * Ho * Wo; g.N = D; g.K = fH * fW * C;
+    g.Kpad = (int)round_up(g.K, BK);
+    g.Tw = fW; g.sh = sH; g.sw = sW; g.rh0 = -pH; g.rw0 = -pW;
+    g.Hof = Ho; g.Wof = Wo; g.oh0 = 0; g.ow0 = 0; g.ohs = 1; g.ows = 1; g.dense_out = 1;
+    set_out_divs(g);
+    PackParams& pk = gs.pp;
+    pk.w = w; pk.fW = fW; pk.C = C; pk.D = D; pk.Tw = fW; pk.Ck = C;
+    pk.xa = 0; pk.xs = 1; pk.ya = 0; pk.ys = 1; pk.transposed = 0;
+    pk.N = D; pk.K = g.K; pk.Npad = (int)round_up(D, 64); pk.Kpad = g.Kpad;
+    gs.bt_bytes = (int64_t)pk.Npad * pk.Kpad * sizeof(T);
+    void* ws;
+    rc = workspace(gs.bt_bytes, &ws);
+    if (rc) return rc;
+    return run_gather<T>(gs, (char*)ws, 0, C % Elem<T>::CE == 0);
+}
+
+// dgrad: for input row i the contributing taps are x with (i + pH - x) % sH == 0 and
+// 0 <= (i + pH - x)/sH < Ho.  Rows are split by a = i % sH; inside a class the taps
+// are x_t = xmax - sH*t (xmax = largest x < fH with x == (a+pH) mod sH), and the
+// source row for class-row i' (i = a + sH*i') and tap t is i' + (a + pH - xmax)/sH + t:
+// a unit-stride gather over dy with Th = number of such taps.
+template <typename T>
+int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
+                    int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW) {
+    int Ho, Wo;
+    int rc = check_conv_dims(fn, S, H, W, C, D, fH, fW, sH, sW, pH, pW, &Ho, &Wo);
+    if (rc) return rc;
+    constexpr int BK = Elem<T>::BK;
+    const int nclass = sH * sW;
+    if (nclass > 64) return fail(AETH_E_INVALID, "%s: stride too large", fn);
+    std::vector<GatherSetup> sets;
+    int64_t total_bytes = 0;
+    for (int a = 0; a < sH; ++a) {
+        if (a >= H) continue;
+        int ra = (a + pH) % sH;
+        int Th = ra < fH ? (fH - 1 - ra) / sH + 1 : 0;
+        int xmax = ra + (Th - 1) * sH;
+        int offh = Th > 0 ? (a + pH - xmax) / sH : 0;   // exact: (a+pH-xmax) is a multiple of sH
+        int Hg = (H - a + sH - 1) / sH;
+        for (int b = 0; b < sW; ++b) {
+            if (b >= W) continue;
+            int rb = (b + pW) % sW;
+            int Tw = rb < fW ? (fW - 1 - rb) / sW + 1 : 0;
+            int ymax = rb + (Tw - 1) * sW;
+            int offw = Tw > 0 ? (b + pW - ymax) / sW : 0;
+            int Wg = (W - b + sW - 1) / sW;
+            GatherSetup gs;
+            GatherParams& g = gs.gp;
+            g.src = dy; g.bias = nullptr; g.out = dx;
+            g.S = S; g.Hs = Ho; g.Ws = Wo; g.Cs = D;
+            g.Hg = Hg; g.Wg = Wg; g.M = S * Hg * Wg; g.N = C;
+            g.K = Th * Tw * D;
+            g.Kpad = (int)round_up(g.K, BK);
+            g.Tw = Tw; g.sh = 1; g.sw = 1; g.rh0 = offh; g.rw0 = offw;
+            g.Hof = H; g.Wof = W; g.oh0 = a; g.ow0 = b; g.ohs = sH; g.ows = sW;
+            g.dense_out = (nclass == 1);
+            set_out_divs(g);
+            PackParams& pk = gs.pp;
+            pk.w = w; pk.fW = fW; pk.C = C; pk.D = D; pk.Tw = Tw > 0 ? Tw : 1; pk.Ck = D;
+            pk.xa = xmax; pk.xs = -sH; pk.ya = ymax; pk.ys = -sW; pk.transposed = 1;
+            pk.N = C; pk.K = g.K; pk.Npad = (int)round_up(C, 64); pk.Kpad = g.Kpad;
+            gs.bt_bytes = round_up((int64_t)pk.Npad * pk.Kpad * sizeof(T), 256);
+            total_bytes += gs.bt_bytes;
+            sets.push_back(gs);
+        }
+    }
+    void* ws;
+    rc = workspace(total_bytes > 0 ? total_bytes : 256, &ws);
+    if (rc) return rc;
+    int64_t off = 0;
+    for (auto& gs : sets) {
+        rc = run_gather<T>(gs, (char*)ws, off, D % Elem<T>::CE == 0);
+        if (rc) return rc;
+        off += gs.bt_bytes;
+    }
+    return AETH_OK;
+}
+
+// ------------------------------------------------------------------------------
+// wgrad: out[k][n] = sum_m A[m][k] * dy[m][n], k = (fx*fW + fy)*C + c
+// Workgroup tile 128 (k) x 64 (n); each of the 4 waves owns 32 k-rows x 64 n.
+// The M range of a workgroup (blockIdx.z) is walked in slabs of 32 rows which are
+// kept in LDS as fp32 (bf16 inputs are widened on the way in: products of bf16
+// values are exact in fp32, so this is bf16-in / fp32-accumulate arithmetic on
+// v_mfma_f32_32x32x2_f32).  The partial tile of split z goes to
+// out + z*(K*D + D); the trailing D floats of each split hold the dbias partial.
+// ------------------------------------------------------------------------------
+struct WgradParams {
+    const void* x;       // [S,H,W,C] of T
+    const void* dy;      // [S,Ho,Wo,D] = [M,D] of T
+    float* out;          // [splits][K*D + D]
+    int want_dbias;
+    int S, H, W, C, Ho, Wo, D;
+    int M, K;
+    int fW, sH, sW, pH, pW;
+    int m_per_split;     // multiple of 32
+    FastDiv div_howo, div_wo, div_c, div_fw;
+};
+
+constexpr int kWgBK = 128;   // k rows per workgroup
+constexpr int kWgBN = 64;
+constexpr int kWgBR = 32;    // m rows per slab
+constexpr int kWgLDA = kWgBK + 32;
+constexpr int kWgLDY = kWgBN + 32;
+
+template <typename T, int VECA, int VECY>
+__global__ __launch_bounds__(kThreads) void wgrad_gemm(const WgradParams p) {
+    constexpr int CE = Elem<T>::CE;
+    constexpr int A_CPR = kWgBK / CE;              // A chunks per slab row
+    constexpr int A_RPP = kThreads / A_CPR;        // rows covered per pass
+    constexpr int A_PASSES = kWgBR / A_RPP;
+    constexpr int Y_CPR = kWgBN / CE;
+    constexpr int Y_RPP = kThreads / Y_CPR;
+    constexpr int Y_PASSES = kWgBR / Y_RPP;
+    constexpr int NE = VECA == CE ? 1 : CE;        // tap decodes per thread
+
+    __shared__ float lds_a[kWgBR * kWgLDA];
+    __shared__ float lds_y[kWgBR * kWgLDY];
+    __shared__ float lds_db[Y_RPP * 64];
+
+    const T* __restrict__ xs = static_cast<const T*>(p.x);
+    const T* __restrict__ dys = static_cast<const T*>(p.dy);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int l32 = lane & 31;
+    const int lh = lane >> 5;
+
+    const int kt0 = blockIdx.x * kWgBK;
+    const int n0 = blockIdx.y * kWgBN;
+    const int m_begin = blockIdx.z * p.m_per_split;
+    int m_end = m_begin + p.m_per_split;
+    if (m_end > p.M) m_end = p.M;
+
+    // A chunk owned by this thread: CE consecutive k starting at kt0 + CE*ka
+    const int ka = tid % A_CPR;
+    const int ra0 = tid / A_CPR;
+    int a_tap_off[NE];
+    int a_fx[NE];
+    int a_fy[NE];
+    bool a_kok[NE];
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+        int kk = kt0 + CE * ka + e;
+        unsigned tap, c, fx, fy;
+        p.div_c.divmod((unsigned)kk, tap, c);
+        p.div_fw.divmod(tap, fx, fy);
+        a_kok[e] = kk < p.K;
+        a_fx[e] = (int)fx - p.pH;
+        a_fy[e] = (int)fy - p.pW;
+        a_tap_off[e] = (a_fx[e] * p.W + a_fy[e]) * p.C + (int)c;
+    }
+    // dy chunk: CE consecutive n starting at n0 + CE*ky
+    const int ky = tid % Y_CPR;
+    const int ry0 = tid / Y_CPR;
+    const bool do_db = p.want_dbias && (blockIdx.x == 0);
+
+    float areg[A_PASSES][CE];
+    float yreg[Y_PASSES][CE];
+    float dbsum[CE];
+#pragma unroll
+    for (int e = 0; e < CE; ++e) dbsum[e] = 0.f;
+
+    auto load_slab = [&](int mb) {
+#pragma unroll
+        for (int i = 0; i < A_PASSES; ++i) {
+            int m = mb + ra0 + A_RPP * i;
+            T raw[CE];
+#pragma unroll
+            for (int e = 0; e < CE; ++e) raw[e] = (T)0;
+            if (m < m_end) {
+                unsigned s, rem, ho, wo;
+                p.div_howo.divmod((unsigned)m, s, rem);
+                p.div_wo.divmod(rem, ho, wo);
+                int r0 = (int)ho * p.sH;
+                int c0 = (int)wo * p.sW;
+                int pix = (((int)s * p.H + r0) * p.W + c0) * p.C;
+                if (VECA == CE) {
+                    bool ok = a_kok[0] && (unsigned)(r0 + a_fx[0]) < (unsigned)p.H &&
+                              (unsigned)(c0 + a_fy[0]) < (unsigned)p.W;
+                    if (ok) {
+                        f4 v = *reinterpret_cast<const f4*>(xs + (pix + a_tap_off[0]));
+                        __builtin_memcpy(raw, &v, 16);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < CE; ++e) {
+                        const int ee = NE == 1 ? 0 : e;
+                        bool ok = a_kok[ee] && (unsigned)(r0 + a_fx[ee]) < (unsigned)p.H &&
+                                  (unsigned)(c0 + a_fy[ee]) < (unsigned)p.W;
+                        if (ok) raw[e] = xs[pix + a_tap_off[ee]];
+                    }
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < CE; ++e) areg[i][e] = Elem<T>::to_f32(raw[e]);
+        }
+#pragma unroll
+        for (int i = 0; i < Y_PASSES; ++i) {
+            int m = mb + ry0 + Y_RPP * i;
+            T raw[CE];
+#pragma unroll
+            for (int e = 0; e < CE; ++e) raw[e] = (T)0;
+            int n = n0 + CE * ky;
+            if (m < m_end) {
+                if (VECY == CE) {
+                    if (n < p.D) {
+                        f4 v = *reinterpret_cast<const f4*>(dys + ((size_t)m * p.D + n));
+                        __builtin_memcpy(raw, &v, 16);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < CE; ++e)
+                        if (n + e < p.D) raw[e] = dys[(size_t)m * p.D + n + e];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < CE; ++e) yreg[i][e] = Elem<T>::to_f32(raw[e]);
+        }
+    };
+
+    auto store_slab = [&]() {
+#pragma unroll
+        for (int i = 0; i < A_PASSES; ++i)
+#pragma unroll
+            for (int q = 0; q < CE / 4; ++q)
+                *reinterpret_cast<f4*>(&lds_a[(ra0 + A_RPP * i) * kWgLDA + CE * ka + 4 * q]) =
+                    f4{areg[i][4 * q], areg[i][4 * q + 1], areg[i][4 * q + 2], areg[i][4 * q + 3]};
+#pragma unroll
+        for (int i = 0; i < Y_PASSES; ++i) {
+#pragma unroll
+            for (int q = 0; q < CE / 4; ++q)
+                *reinterpret_cast<f4*>(&lds_y[(ry0 + Y_RPP * i) * kWgLDY + CE * ky + 4 * q]) =
+                    f4{yreg[i][4 * q], yreg[i][4 * q + 1], yreg[i][4 * q + 2], yreg[i][4 * q + 3]};
+            if (do_db) {
+#pragma unroll
+                for (int e = 0; e < CE; ++e) dbsum[e] += yreg[i][e];
+            }
+        }
+    };
+
+    f16v acc[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+
+    if (m_begin < m_end) {
+        load_slab(m_begin);
+        store_slab();
+        __syncthreads();
+    }
+    for (int mb = m_begin; mb < m_end; mb += kWgBR) {
+        const bool more = mb + kWgBR < m_end;
+        if (more) load_slab(mb + kWgBR);
+        const int wk0 = wave * 32;
+#pragma unroll
+        for (int t2 = 0; t2 < kWgBR / 2; ++t2) {
+            float a = lds_a[(2 * t2 + lh) * kWgLDA + wk0 + l32];
+            float b0 = lds_y[(2 * t2 + lh) * kWgLDY + l32];
+            float b1 = lds_y[(2 * t2 + lh) * kWgLDY + 32 + l32];
+            acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b0, acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b1, acc[1], 0, 0, 0);
+        }
+        __syncthreads();
+        if (more) {
+            store_slab();
+            __syncthreads();
+        }
+    }
+
+    const size_t split_stride = (size_t)p.K * p.D + p.D;
+    float* outp = p.out + (size_t)blockIdx.z * split_stride;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int n = n0 + 32 * j + l32;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int k = kt0 + wave * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            if (k < p.K && n < p.D) outp[(size_t)k * p.D + n] = acc[j][v];
+        }
+    }
+
+    if (do_db) {
+        // Y_RPP row lanes each hold a partial of the same CE columns: fixed-order sum
+#pragma unroll
+        for (int e = 0; e < CE; ++e) lds_db[ry0 * 64 + CE * ky + e] = dbsum[e];
+        __syncthreads();
+        if (tid < 64) {
+            float s = 0.f;
+#pragma unroll
+            for (int r = 0; r < Y_RPP; ++r) s += lds_db[r * 64 + tid];
+            if (n0 + tid < p.D) outp[(size_t)p.K * p.D + n0 + tid] = s;
+        }
+    }
+}
+
+// out[i] = sum_s part[s*stride + i] for i < n, in a fixed order: 4 split lanes per
+// output (splits s, s+4, ...), then the 4 lanes in order.  i < n_dw goes to dw,
+// the rest to dbias.
+static __global__ __launch_bounds__(kThreads) void reduce_splits(const float* __restrict__ part, float* __restrict__ dw,
+                                                         float* __restrict__ dbias, int n_dw, int n, int stride,
+                                                         int splits) {
+    __shared__ float red[4][64];
+    const int col = threadIdx.x & 63;
+    const int sl = threadIdx.x >> 6;
+    const int i = blockIdx.x * 64 + col;
+    float s = 0.f;
+    if (i < n) {
+        const float* q = part + i;
+        int k = sl;
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        for (; k + 12 < splits; k += 16) {
+            s0 += q[(size_t)k * stride];
+            s1 += q[(size_t)(k + 4) * stride];
+            s2 += q[(size_t)(k + 8) * stride];
+            s3 += q[(size_t)(k + 12) * stride];
+        }
+        for (; k < splits; k += 4) s0 += q[(size_t)k * stride];
+        s = (s0 + s1) + (s2 + s3);
+    }
+    red[sl][col] = s;
+    __syncthreads();
+    if (sl == 0 && i < n) {
+        float t = (red[0][col] + red[1][col]) + (red[2][col] + red[3][col]);
+        if (i < n_dw) dw[i] = t;
+        else if (dbias != nullptr) dbias[i - n_dw] = t;
+    }
+}
+
+template <typename T>
+int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* dbias,
+                    int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW) {
+    int Ho, Wo;
+    int rc = check_conv_dims(fn, S, H, W, C, D, fH, fW, sH, sW, pH, pW, &Ho, &Wo);
+    if (rc) return rc;
+    Context& c = ctx();
+    WgradParams p;
+    p.x = x; p.dy = dy;
+    p.S = S; p.H = H; p.W = W; p.C = C; p.Ho = Ho; p.Wo = Wo; p.D = D;
+    p.M = S * Ho * Wo; p.K = fH * fW * C;
+    p.fW = fW; p.sH = sH; p.sW = sW; p.pH = pH; p.pW = pW;
+    p.want_dbias = dbias != nullptr;
+    p.div_howo = FastDiv(Ho * Wo); p.div_wo = FastDiv(Wo); p.div_c = FastDiv(C); p.div_fw = FastDiv(fW);
+    const int kt = cdiv(p.K, kWgBK), nt = cdiv(D, kWgBN);
+    const int slabs = cdiv(p.M, kWgBR);
+    int splits = cdiv(4 * c.prop.multiProcessorCount, kt * nt);
+    if (splits > slabs) splits = slabs;
+    if (splits < 1) splits = 1;
+    int slabs_per = cdiv(slabs, splits);
+    splits = cdiv(slabs, slabs_per);
+    p.m_per_split = slabs_per * kWgBR;
+    const int64_t kd = (int64_t)p.K * D;
+    void* ws;
+    rc = workspace((int64_t)splits * (kd + D) * sizeof(float), &ws);
+    if (rc) return rc;
+    p.out = (float*)ws;
+    dim3 grid(kt, nt, splits);
+    constexpr int CE = Elem<T>::CE;
+    const bool va = (C % CE == 0), vy = (D % CE == 0);
+    if (va && vy) hipLaunchKernelGGL((wgrad_gemm<T, CE, CE>), grid, dim3(kThreads), 0, c.stream, p);
+    else if (va) hipLaunchKernelGGL((wgrad_gemm<T, CE, 1>), grid, dim3(kThreads), 0, c.stream, p);
+    else if (vy) hipLaunchKernelGGL((wgrad_gemm<T, 1, CE>), grid, dim3(kThreads), 0, c.stream, p);
+    else hipLaunchKernelGGL((wgrad_gemm<T, 1, 1>), grid, dim3(kThreads), 0, c.stream, p);
+    AETH_LAUNCH_CHECK();
+    const int n = (int)(kd + (dbias ? D : 0));
+    hipLaunchKernelGGL(reduce_splits, dim3(cdiv(n, 64)), dim3(kThreads), 0, c.stream, (const float*)ws, dw, dbias,
+                       (int)kd, n, (int)(kd + D), splits);
+    AETH_LAUNCH_CHECK();
+    return AETH_OK;
+}
+
+}  // namespace aeth

@@ -84,6 +84,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the bf16 / train-step extras")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch relu_fwd_kernel with alpha=1 (a plain copy) over 64 Mi floats three times: "
+                         "256 MiB read + 256 MiB written per launch, the yardstick for FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported" % args.gpus, file=sys.stderr)
@@ -121,6 +124,14 @@ def main():
         dgrad()
 
     fl = conv_flops(S, H, W, 3, 3, C, D)
+
+    if args.copy_probe:
+        n = 64 * 1024 * 1024
+        src, dst = DeviceTensor.zeros(n), DeviceTensor(n)
+        for _ in range(3):
+            _lib.check(L.aeth_relu_fwd_f32(src.ptr, dst.ptr, 1.0, n))
+        _lib.sync()
+        del src, dst
 
     # ---- the timed region: exactly K steps between two synchronisations --------
     for _ in range(args.warmup):

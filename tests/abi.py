@@ -63,3 +63,37 @@ def close(got, want, rtol=1e-4, atol=1e-5, rms_scaled=False):
     worst = float(np.max(err / tol)) if err.size else 0.0
     assert worst <= 1.0, "max err/tol = %.3g (max abs err %.3g)" % (worst, float(err.max()))
     return worst
+
+
+# ---- bf16-input variants: inputs are cast on the device by aeth_cast_f32_to_bf16 ----
+def to_bf16_device(a):
+    src = DeviceTensor.from_numpy(a, np.float32)
+    dst = DeviceTensor(a.shape, np.uint16)
+    _lib.check(_lib.lib().aeth_cast_f32_to_bf16(src.ptr, dst.ptr, src.size))
+    return dst
+
+
+def fprop_bf16(x, w, b, strides, padding):
+    dims, yshape = conv_dims(x.shape, w.shape, strides, padding)
+    xd, wd = to_bf16_device(x), to_bf16_device(w)
+    bd = DeviceTensor.from_numpy(b, np.float32) if b is not None else None
+    y = DeviceTensor.full(yshape, np.nan)
+    _lib.check(_lib.lib().aeth_conv_fprop_bf16(xd.ptr, wd.ptr, bd.ptr if bd else None, y.ptr, *dims))
+    return y.get()
+
+
+def dgrad_bf16(dy, w, x_shape, strides, padding):
+    dims, yshape = conv_dims(x_shape, w.shape, strides, padding)
+    dyd, wd = to_bf16_device(dy), to_bf16_device(w)
+    dx = DeviceTensor.full(x_shape, np.nan)
+    _lib.check(_lib.lib().aeth_conv_dgrad_bf16(dyd.ptr, wd.ptr, dx.ptr, *dims))
+    return dx.get()
+
+
+def wgrad_bf16(x, dy, w_shape, strides, padding):
+    dims, yshape = conv_dims(x.shape, w_shape, strides, padding)
+    xd, dyd = to_bf16_device(x), to_bf16_device(dy)
+    dw = DeviceTensor.full(w_shape, np.nan)
+    db = DeviceTensor.full(w_shape[3], np.nan)
+    _lib.check(_lib.lib().aeth_conv_wgrad_bf16(xd.ptr, dyd.ptr, dw.ptr, db.ptr, *dims))
+    return dw.get(), db.get()

@@ -1,0 +1,95 @@
+"""bf16-input / fp32-accumulate convolution against the oracle.
+
+Two comparisons per case:
+  * exact-input: the oracle (float64) evaluated on the bf16-rounded x, w, dy.
+    Products of bf16 values are exact in fp32 and accumulation is fp32, so the
+    fp32 tolerance applies: 1e-5 + 1e-4*|oracle| (rms-scaled for wgrad/dbias).
+  * the stated bf16 tolerance against the unrounded fp32 oracle: relative 2e-2,
+    measured against the rms of the output tensor (elements near zero carry the
+    rounding noise of the whole dot product)."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    (2, 6, 7, 3, 4, 3, 3, 1, 1, "same"),          # scalar-gather path (C, D not multiples of 8)
+    (2, 9, 7, 4, 12, 3, 3, 2, 2, "same"),
+    (4, 12, 12, 8, 16, 3, 3, 1, 1, "same"),
+    (3, 16, 16, 32, 64, 3, 3, 1, 1, "same"),
+    (2, 8, 8, 64, 128, 3, 3, 1, 1, "same"),
+    (2, 14, 14, 64, 64, 3, 3, 1, 1, "same"),
+    (2, 14, 14, 64, 256, 1, 1, 1, 1, "valid"),
+    (3, 13, 13, 128, 256, 3, 3, 2, 2, "valid"),
+    (5, 9, 9, 24, 40, 3, 3, 1, 1, "same"),
+    (40, 16, 16, 3, 32, 3, 3, 1, 1, "same"),
+]
+
+
+def _case(case, seed):
+    from tests import abi
+    S, H, W, C, D, fH, fW, sH, sW, pad = case
+    r = np.random.RandomState(seed)
+    x = r.randn(S, H, W, C).astype(np.float32)
+    w = (r.randn(fH, fW, C, D) * np.sqrt(2.0 / (fH * fW * C))).astype(np.float32)
+    b = r.randn(D).astype(np.float32)
+    _, yshape = abi.conv_dims(x.shape, w.shape, (sH, sW), pad)
+    dy = r.randn(*yshape).astype(np.float32)
+    return x, w, b, dy
+
+
+def _loose(got, want, rel=2e-2):
+    want = np.asarray(want, np.float64)
+    rms = max(float(np.sqrt(np.mean(want * want))), 1e-30)
+    assert np.max(np.abs(got - want)) <= rel * (np.abs(want).max() + rms), np.max(np.abs(got - want)) / rms
+    assert np.sqrt(np.mean((got - want) ** 2)) <= rel * rms
+
+
+def test_cast_is_round_to_nearest_even_bit_exact():
+    from tests import abi
+    r = np.random.RandomState(0)
+    a = (r.randn(100000) * 10.0 ** r.randint(-8, 8, 100000)).astype(np.float32)
+    a[:6] = [0.0, -0.0, np.inf, -np.inf, 1.00390625, 1.01171875]     # the last two are ties
+    got = abi.to_bf16_device(a).get()
+    assert np.array_equal(got, O.bf16_bits(a))
+    nan = abi.to_bf16_device(np.array([np.nan], np.float32)).get()
+    assert (nan[0] & 0x7F80) == 0x7F80 and (nan[0] & 0x7F) != 0
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_bf16_fprop_dgrad_wgrad(case):
+    from tests import abi
+    x, w, b, dy = _case(case, 3)
+    stride, pad = (case[7], case[8]), case[9]
+    xr, wr, dyr = O.round_to_bf16(x), O.round_to_bf16(w), O.round_to_bf16(dy)
+
+    y = abi.fprop_bf16(x, w, b, stride, pad)
+    abi.close(y, O.conv_fprop(xr, wr, b, stride, pad, dtype=np.float64))
+    _loose(y, O.conv_fprop(x, w, b, stride, pad, dtype=np.float64))
+
+    dx = abi.dgrad_bf16(dy, w, x.shape, stride, pad)
+    abi.close(dx, O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
+    _loose(dx, O.conv_dgrad(dy, w, x.shape[1:3], stride, pad, dtype=np.float64))
+
+    dw, db = abi.wgrad_bf16(x, dy, w.shape, stride, pad)
+    abi.close(dw, O.conv_wgrad(xr, dyr, w.shape[:2], stride, pad, dtype=np.float64), rms_scaled=True)
+    abi.close(db, O.conv_dbias(dyr, dtype=np.float64), rms_scaled=True)
+    _loose(dw, O.conv_wgrad(x, dy, w.shape[:2], stride, pad, dtype=np.float64))
+
+
+def test_conv_layer_bf16_precision_switch():
+    import aether
+    np.random.seed(5)
+    layer = aether.Conv_Layer((10, 10, 16), num_filters=32)
+    layer.precision = "bf16"
+    x = np.random.randn(3, 10, 10, 16).astype(np.float32)
+    dy = np.random.randn(3, 10, 10, 32).astype(np.float32)
+    w, b = layer.filter_weights.get(), layer.biases.get()
+    layer.forward(x, True)
+    layer.backward(dy)
+    _loose(layer.output.get(), O.conv_fprop(x, w, b, (1, 1), "same", dtype=np.float64))
+    _loose(layer.dinputs.get(), O.conv_dgrad(dy, w, (10, 10), (1, 1), "same", dtype=np.float64))
+    _loose(layer.dweights.get(), O.conv_wgrad(x, dy, (3, 3), (1, 1), "same", dtype=np.float64))
+    _loose(layer.dbiases.get(), O.conv_dbias(dy, dtype=np.float64))
