@@ -1,0 +1,147 @@
+"""Secondary measurements printed under "extra" by bench.py: every convolution
+shape of the benchmark list in fp32 (and bf16-input where the list asks for it),
+per direction, and the three-block CNN training step in images/sec."""
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "aether-ml_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+FP32_PEAK = 157.3
+BF16_PEAK = 2500.0
+HBM_GBS = 8000.0
+
+# name, S, H, W, C, D, f, stride, pad P, bf16 too?
+SHAPES = [
+    ("cfg1_32x32x3_to32", 128, 32, 32, 3, 32, 3, 1, 1, False),
+    ("cfg2a_16x16x32_to64", 128, 16, 16, 32, 64, 3, 1, 1, False),
+    ("cfg2b_8x8x64_to128", 128, 8, 8, 64, 128, 3, 1, 1, False),
+    ("cfg4_56x56x64_to64", 256, 56, 56, 64, 64, 3, 1, 1, True),
+    ("cfg4_1x1_64_to256", 256, 56, 56, 64, 256, 1, 1, 0, True),
+    ("cfg5_28x28x128_to256_s2", 1024, 28, 28, 128, 256, 3, 2, 0, True),
+]
+
+
+def _time(fn, steps, warmup):
+    from aether import _lib
+    for _ in range(warmup):
+        fn()
+    _lib.sync()
+    e0, e1 = _lib.Event(), _lib.Event()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    return e0.elapsed_ms(e1) / steps
+
+
+def conv_table(steps, warmup):
+    from aether import _lib
+    from aether.tensor import DeviceTensor
+    L = _lib.lib()
+    rng = np.random.default_rng(0)
+    out = {}
+    for name, S, H, W, C, D, f, st, P, with_bf16 in SHAPES:
+        Ho = (H + 2 * P - f) // st + 1
+        Wo = (W + 2 * P - f) // st + 1
+        dims = (S, H, W, C, D, f, f, st, st, P, P)
+        x = DeviceTensor.from_numpy(rng.standard_normal((S, H, W, C), dtype=np.float32))
+        w = DeviceTensor.from_numpy(rng.standard_normal((f, f, C, D), dtype=np.float32) *
+                                    np.float32(np.sqrt(2.0 / (f * f * C))))
+        dy = DeviceTensor.from_numpy(rng.standard_normal((S, Ho, Wo, D), dtype=np.float32))
+        b = DeviceTensor.zeros(D)
+        y, dx = DeviceTensor((S, Ho, Wo, D)), DeviceTensor((S, H, W, C))
+        dw, db = DeviceTensor((f, f, C, D)), DeviceTensor(D)
+        flops = 2.0 * S * Ho * Wo * f * f * C * D
+        nx, ny, nw = S * H * W * C, S * Ho * Wo * D, f * f * C * D
+        row = {"gflop_per_direction": flops / 1e9}
+        calls = {
+            "fprop": lambda: _lib.check(L.aeth_conv_fprop_f32(x.ptr, w.ptr, b.ptr, y.ptr, *dims)),
+            "dgrad": lambda: _lib.check(L.aeth_conv_dgrad_f32(dy.ptr, w.ptr, dx.ptr, *dims)),
+            "wgrad": lambda: _lib.check(L.aeth_conv_wgrad_f32(x.ptr, dy.ptr, dw.ptr, db.ptr, *dims)),
+        }
+        byts = {"fprop": 4 * (nx + nw + D + ny), "dgrad": 4 * (ny + nw + nx), "wgrad": 4 * (nx + ny + nw + D)}
+        for k, fn in calls.items():
+            ms = _time(fn, steps, warmup)
+            row["f32_" + k] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 3),
+                               "frac_mfma_peak": round(flops / ms / 1e9 / FP32_PEAK, 4),
+                               "frac_hbm_peak": round(byts[k] / ms / 1e6 / HBM_GBS, 4)}
+        if with_bf16:
+            x16, w16, dy16 = (DeviceTensor(t.shape, np.uint16) for t in (x, w, dy))
+            for src, dst in ((x, x16), (w, w16), (dy, dy16)):
+                _lib.check(L.aeth_cast_f32_to_bf16(src.ptr, dst.ptr, src.size))
+            calls = {
+                "fprop": lambda: _lib.check(L.aeth_conv_fprop_bf16(x16.ptr, w16.ptr, b.ptr, y.ptr, *dims)),
+                "dgrad": lambda: _lib.check(L.aeth_conv_dgrad_bf16(dy16.ptr, w16.ptr, dx.ptr, *dims)),
+                "wgrad": lambda: _lib.check(L.aeth_conv_wgrad_bf16(x16.ptr, dy16.ptr, dw.ptr, db.ptr, *dims)),
+            }
+            byts = {"fprop": 2 * (nx + nw) + 4 * (D + ny), "dgrad": 2 * (ny + nw) + 4 * nx,
+                    "wgrad": 2 * (nx + ny) + 4 * (nw + D)}
+            for k, fn in calls.items():
+                ms = _time(fn, steps, warmup)
+                row["bf16_" + k] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 3),
+                                    "frac_mfma_peak": round(flops / ms / 1e9 / BF16_PEAK, 4),
+                                    "frac_hbm_peak": round(byts[k] / ms / 1e6 / HBM_GBS, 4)}
+        out[name] = row
+        del x, w, dy, y, dx
+    return out
+
+
+def build_cnn(aether):
+    """Conv(32)-BN-ReLU-Pool, Conv(64)-BN-ReLU-Pool, Conv(128)-BN-ReLU-Pool, Flatten,
+    Dense 2048->256, LeakyReLU(0.01), Dense 256->10, softmax CCE(ls 0.01), Adam 1e-3."""
+    m = aether.Model()
+    c, size = 3, 32
+    for d in (32, 64, 128):
+        m.add(aether.Conv_Layer((size, size, c), num_filters=d, filter_size=(3, 3), strides=(1, 1), padding="same"))
+        m.add(aether.Batch_Norm())
+        m.add(aether.ReLU())
+        m.add(aether.Pooling(filter_size=(2, 2), strides=(2, 2), padding="valid", pooling_type="max"))
+        c, size = d, size // 2
+    m.add(aether.Flatten())
+    m.add(aether.Layer_Dense(size * size * 128, 256))
+    m.add(aether.Leaky_ReLU(alpha=0.01))
+    m.add(aether.Layer_Dense(256, 10))
+    m.add(aether.SoftMax())
+    m.set(loss=aether.Loss_CategoricalCrossEntropy(label_smoothing=0.01),
+          optimizer=aether.Optimizer_Adam(learning_rate=1e-3), accuracy=aether.Accuracy_Categorical())
+    m.finalize()
+    return m
+
+
+def train_step(steps, warmup):
+    import aether
+    from aether import _lib
+    np.random.seed(0)
+    X = aether.DeviceTensor.from_numpy(np.random.rand(128, 32, 32, 3).astype(np.float32))
+    y = np.random.randint(0, 10, 128)
+    model = build_cnn(aether)
+    model.loss.new_pass()
+    model.accuracy.new_pass()
+    for _ in range(warmup):
+        model.train_step(X, y)
+    _lib.sync()
+    times = []
+    for _ in range(steps):
+        t0 = time.perf_counter()
+        loss, data_loss, reg, acc = model.train_step(X, y)
+        _lib.sync()
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    return {"ms_per_step_median": med * 1e3, "images_per_sec": 128.0 / med, "batch": 128,
+            "last_loss": float(loss), "note": "forward + loss + accuracy + backward + Adam, batch resident in HBM, "
+                                              "includes the per-step scalar read-backs"}
+
+
+def run(steps, warmup):
+    return {"conv_shapes": conv_table(max(5, steps // 2), 2), "train_step_cnn3": train_step(max(steps, 20), warmup)}
+
+
+if __name__ == "__main__":
+    import json
+    print(json.dumps(run(20, 5), indent=1))
