@@ -19,6 +19,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wno-unused-command-line-argument",
 ]
 
@@ -26,6 +27,7 @@ FLAGS = [
 def _headers():
     out = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
     out.append(os.path.join(HERE, "..", "include", "aether_hip.h"))
+    out.append(os.path.abspath(__file__))       # the flags live here
     return out
 
 

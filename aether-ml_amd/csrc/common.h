@@ -55,11 +55,12 @@ int workspace(int64_t bytes, void** out);
     } while (0)
 
 // Division by a runtime-constant positive divisor for 0 <= n < 2^31:
-// q = umulhi(n, mul) >> shr (d == 1 is passed through).
+// q = umulhi(n, mul) >> shr.  d == 1 has no 32-bit multiplier; it is handled by a
+// bit mask instead of a branch so that callers stay straight-line code.
 struct FastDiv {
-    unsigned int d, mul, shr;
-    FastDiv() : d(1), mul(0), shr(0) {}
-    explicit FastDiv(int div) : d((unsigned)div), mul(0), shr(0) {
+    unsigned int d, mul, shr, one;   // one = ~0u when d == 1
+    FastDiv() : d(1), mul(0), shr(0), one(~0u) {}
+    explicit FastDiv(int div) : d((unsigned)div), mul(0), shr(0), one(div == 1 ? ~0u : 0u) {
         if (div > 1) {
             unsigned l = 0;
             while ((1u << l) < (unsigned)div) ++l;           // ceil(log2 d)
@@ -70,10 +71,11 @@ struct FastDiv {
     }
     __host__ __device__ __forceinline__ unsigned div(unsigned n) const {
 #if defined(__HIP_DEVICE_COMPILE__)
-        return d == 1 ? n : (__umulhi(n, mul) >> shr);
+        unsigned q = __umulhi(n, mul) >> shr;
 #else
-        return d == 1 ? n : (unsigned)(((unsigned long long)n * mul) >> 32) >> shr;
+        unsigned q = (unsigned)(((unsigned long long)n * mul) >> 32) >> shr;
 #endif
+        return (q & ~one) | (n & one);
     }
     __host__ __device__ __forceinline__ void divmod(unsigned n, unsigned& q, unsigned& r) const {
         q = div(n);

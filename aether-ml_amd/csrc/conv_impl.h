@@ -26,6 +26,7 @@
 #include "common.h"
 
 #include <limits.h>
+#include <stdlib.h>
 #include <vector>
 
 namespace aeth {
@@ -82,13 +83,60 @@ struct GatherParams {
     // output element (s,i,j,n) lives at ((s*Hof + oh0 + i*ohs)*Wof + ow0 + j*ows)*N + n
     int Hof, Wof, oh0, ow0, ohs, ows;
     int dense_out;       // 1: row m is stored at out + m*N
+    unsigned src_bytes;  // extent of src / bt for the buffer descriptors (0: too large, not used)
+    unsigned bt_bytes;
     FastDiv div_hw, div_w, div_c, div_tw;
 };
 
 constexpr int kInvalidRow = -16384;
+constexpr int kXcds = 8;
+
+// Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has its
+// own L2.  This maps the hardware id to a logical id such that every XCD works on
+// one contiguous range of logical ids: tiles that share operands (the N tiles of
+// one M tile, the k tiles of one wgrad split, neighbouring M tiles with their
+// common halo rows) then hit the same L2 at about the same time.
+__device__ __forceinline__ int xcd_contiguous_id(int wg, int total) {
+    const int per = total / kXcds, rem = total % kXcds;
+    const int xcd = wg % kXcds, idx = wg / kXcds;
+    return xcd * per + (xcd < rem ? xcd : rem) + idx;
+}
+
+// Bias add and store of a wave's TM x TN accumulator tiles.  acc[i][j][v] holds row
+// 32*i + 8*(v/4) + 4*(lane/32) + v%4, column 32*j + lane%32 of the wave tile.
+template <int TM, int TN>
+__device__ __forceinline__ void store_tile(const GatherParams& p, const f16v (&acc)[TM][TN], int mw0, int nw0,
+                                           int l32, int lh) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int n = nw0 + 32 * j + l32;
+        const bool nok = n < p.N;
+        const float bv = (p.bias != nullptr && nok) ? p.bias[n] : 0.f;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = mw0 + 32 * i + 8 * (v >> 2) + 4 * lh + (v & 3);
+                if (nok && m < p.M) {
+                    size_t row;
+                    if (p.dense_out) {
+                        row = (size_t)m;
+                    } else {
+                        unsigned s, rem, ii, jj;
+                        p.div_hw.divmod((unsigned)m, s, rem);
+                        p.div_w.divmod(rem, ii, jj);
+                        row = ((size_t)s * p.Hof + p.oh0 + (size_t)ii * p.ohs) * p.Wof + p.ow0 + (size_t)jj * p.ows;
+                    }
+                    p.out[row * p.N + n] = acc[i][j][v] + bv;
+                }
+            }
+        }
+    }
+}
+
 
 template <typename T, int BM, int BN, int WM, int WN, int VEC>
-__global__ __launch_bounds__(kThreads) void gather_gemm(const GatherParams p) {
+__global__ __launch_bounds__(kThreads, 3) void gather_gemm(const GatherParams p) {
     static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
     static_assert(WM % 32 == 0 && WN % 32 == 0, "32x32 MFMA tiles");
     constexpr int CE = Elem<T>::CE;
@@ -110,8 +158,10 @@ __global__ __launch_bounds__(kThreads) void gather_gemm(const GatherParams p) {
     const int wm0 = (wave % (BM / WM)) * WM;
     const int wn0 = (wave / (BM / WM)) * WN;
 
-    const int m0 = blockIdx.x * BM;
-    const int n0 = blockIdx.y * BN;
+    const int ntile = (p.N + BN - 1) / BN;
+    const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
+    const int m0 = (lid / ntile) * BM;
+    const int n0 = (lid % ntile) * BN;
 
     // ---- per-thread row bookkeeping for the A gather --------------------------
     const int k4 = tid & 7;              // which chunk of the slab row
@@ -228,32 +278,155 @@ __global__ __launch_bounds__(kThreads) void gather_gemm(const GatherParams p) {
         }
     }
 
-    // ---- epilogue: bias add and store -------------------------------------------
+    store_tile<TM, TN>(p, acc, m0 + wm0, n0 + wn0, l32, lh);
+}
+
+// ------------------------------------------------------------------------------
+// gather-GEMM, LDS-direct variant (the fast path whenever channels come in whole
+// 16-byte chunks).  Same tiling and MFMA schedule as gather_gemm, but the slabs go
+// from memory straight into LDS with `buffer_load_dwordx4 ... lds`: no staging
+// registers, no ds_write, and two LDS buffers so the loads of slab k+1 are in
+// flight while slab k is multiplied (one barrier per slab).
+//   * One wave-level load writes 64 consecutive 16-byte chunks = 8 slab rows, so
+//     rows are unpadded (128 B) and bank conflicts are avoided by an XOR swizzle:
+//     logical chunk c of row r lives at chunk position c ^ (r & 7).  The swizzle is
+//     applied on the global side (lane l of a load fetches logical chunk
+//     (l & 7) ^ (l >> 3) of row l >> 3) and undone by the operand reads.
+//   * Padding taps and rows past M use a byte offset of 2^31, which is outside the
+//     buffer descriptor's extent: the load returns zeros.
+// ------------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+template <typename T, int BM, int BN, int WM, int WN, int MINW>
+__global__ __launch_bounds__(kThreads, MINW) void gather_gemm_dma(const GatherParams p) {
+    static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
+    constexpr int CE = Elem<T>::CE;
+    constexpr int BK = Elem<T>::BK;
+    constexpr int AL = BM / 32;          // wave-level A loads per wave per slab (8 rows each)
+    constexpr int BL = BN / 32;
+    constexpr int TM = WM / 32;
+    constexpr int TN = WN / 32;
+
+    __shared__ f4 lds_a0[BM * 8];
+    __shared__ f4 lds_a1[BM * 8];
+    __shared__ f4 lds_b0[BN * 8];
+    __shared__ f4 lds_b1[BN * 8];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int l32 = lane & 31;
+    const int lh = lane >> 5;
+    const int wm0 = (wave % (BM / WM)) * WM;
+    const int wn0 = (wave / (BM / WM)) * WN;
+    const int ntile = (p.N + BN - 1) / BN;
+    const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
+    const int m0 = (lid / ntile) * BM;
+    const int n0 = (lid % ntile) * BN;
+
+    const int lr = lane >> 3;                  // row inside an 8-row load block
+    const int k4 = (lane & 7) ^ lr;            // logical chunk this lane fetches
+    int base_off[AL];
+    int base_rc[AL];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int n = n0 + wn0 + 32 * j + l32;
-        const bool nok = n < p.N;
-        const float bv = (p.bias != nullptr && nok) ? p.bias[n] : 0.f;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int m = m0 + wm0 + 32 * i + 8 * (v >> 2) + 4 * lh + (v & 3);
-                if (nok && m < p.M) {
-                    size_t row;
-                    if (p.dense_out) {
-                        row = (size_t)m;
-                    } else {
-                        unsigned s, rem, ii, jj;
-                        p.div_hw.divmod((unsigned)m, s, rem);
-                        p.div_w.divmod(rem, ii, jj);
-                        row = ((size_t)s * p.Hof + p.oh0 + (size_t)ii * p.ohs) * p.Wof + p.ow0 + (size_t)jj * p.ows;
-                    }
-                    p.out[row * p.N + n] = acc[i][j][v] + bv;
-                }
-            }
+    for (int i = 0; i < AL; ++i) {
+        int m = m0 + (wave * AL + i) * 8 + lr;
+        if (m < p.M) {
+            unsigned s, rem, ii, jj;
+            p.div_hw.divmod((unsigned)m, s, rem);
+            p.div_w.divmod(rem, ii, jj);
+            int br = (int)ii * p.sh + p.rh0;
+            int bc = (int)jj * p.sw + p.rw0;
+            base_off[i] = (((int)s * p.Hs + br) * p.Ws + bc) * p.Cs;
+            base_rc[i] = (int)(((unsigned)br << 16) | ((unsigned)bc & 0xffffu));
+        } else {
+            base_off[i] = 0;
+            base_rc[i] = (int)((unsigned)kInvalidRow << 16);
         }
     }
+    unsigned b_off[BL];
+#pragma unroll
+    for (int i = 0; i < BL; ++i)
+        b_off[i] = (unsigned)(((n0 + (wave * BL + i) * 8 + lr) * p.Kpad + CE * k4) * (int)sizeof(T));
+
+    const __amdgpu_buffer_rsrc_t rsrc_a =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.src), 0, (int)p.src_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.bt), 0, (int)p.bt_bytes, 0x00020000);
+
+    auto issue = [&](int k0, f4* la, f4* lb) {
+        int kk = k0 + CE * k4;
+        unsigned tap, c, th, tw;
+        p.div_c.divmod((unsigned)kk, tap, c);
+        p.div_tw.divmod(tap, th, tw);
+        bool kvalid = kk < p.K;
+        int tap_off = ((int)th * p.Ws + (int)tw) * p.Cs + (int)c;
+#pragma unroll
+        for (int i = 0; i < AL; ++i) {
+            int r = (base_rc[i] >> 16) + (int)th;
+            int cc = ((int)((unsigned)base_rc[i] << 16) >> 16) + (int)tw;
+            // bitwise, not short-circuit: keeps the slab issue free of branches
+            const unsigned bad = (unsigned)!(kvalid & ((unsigned)r < (unsigned)p.Hs) & ((unsigned)cc < (unsigned)p.Ws));
+            const unsigned voff = ((unsigned)(base_off[i] + tap_off) * (unsigned)sizeof(T)) | (bad << 31);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(la + (wave * AL + i) * 64), 16, (int)voff, 0,
+                                                     0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < BL; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(lb + (wave * BL + i) * 64), 16,
+                                                     (int)(b_off[i] + (unsigned)k0 * (unsigned)sizeof(T)), 0, 0, 0);
+    };
+
+    f16v acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    const int sw7 = l32 & 7;                   // row & 7 of every operand row this lane reads
+    f4 fa[2][TM], fb[2][TN];                   // operand fragments, double buffered across k groups
+    auto read_frags = [&](const f4* la, const f4* lb, int g, int slot) {
+        const int pc = (2 * g + lh) ^ sw7;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[slot][i] = la[(wm0 + 32 * i + l32) * 8 + pc];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[slot][j] = lb[(wn0 + 32 * j + l32) * 8 + pc];
+    };
+    auto mma_group = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) mma_chunk<T>(fa[slot][i], fb[slot][j], acc[i][j]);
+    };
+    // One slab: the first operand reads go out right after the barrier, then the
+    // loads of the next slab are issued (their address arithmetic overlaps the LDS
+    // latency), then each k group's MFMAs run while the next group's operands load.
+    auto slab = [&](const f4* la, const f4* lb, f4* na, f4* nb, int next_k0, bool has_next) {
+        __builtin_amdgcn_s_waitcnt(0);         // this wave's loads of the slab have landed
+        __syncthreads();                       // everyone's have; everyone is done reading the other buffer
+        read_frags(la, lb, 0, 0);
+        if (has_next) issue(next_k0, na, nb);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            if (g < 3) read_frags(la, lb, g + 1, (g + 1) & 1);
+            // keep the prefetch ahead of the MFMAs (the scheduler would otherwise sink
+            // the reads next to their first use and expose the LDS latency)
+            __builtin_amdgcn_sched_barrier(0);
+            mma_group(g & 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    const int nslabs = p.Kpad / BK;
+    if (nslabs > 0) issue(0, lds_a0, lds_b0);
+    for (int s = 0; s < nslabs; s += 2) {
+        slab(lds_a0, lds_b0, lds_a1, lds_b1, (s + 1) * BK, s + 1 < nslabs);
+        if (s + 1 < nslabs) slab(lds_a1, lds_b1, lds_a0, lds_b0, (s + 2) * BK, s + 2 < nslabs);
+    }
+
+    store_tile<TM, TN>(p, acc, m0 + wm0, n0 + wn0, l32, lh);
 }
 
 // Packs the filter w[fH][fW][C][D] into bt[Npad][Kpad] (k contiguous) for one
@@ -294,8 +467,10 @@ __global__ void pack_filter(const PackParams p) {
 
 template <typename T, int BM, int BN, int WM, int WN>
 static void launch_gather_cfg(const GatherParams& gp, bool vec, hipStream_t st) {
-    dim3 grid(cdiv(gp.M, BM), cdiv(gp.N, BN));
-    if (vec)
+    dim3 grid(cdiv(gp.M, BM) * cdiv(gp.N, BN));
+    if (vec && gp.src_bytes != 0 && gp.bt_bytes != 0)
+        hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, 1>), grid, dim3(kThreads), 0, st, gp);
+    else if (vec)
         hipLaunchKernelGGL((gather_gemm<T, BM, BN, WM, WN, Elem<T>::CE>), grid, dim3(kThreads), 0, st, gp);
     else
         hipLaunchKernelGGL((gather_gemm<T, BM, BN, WM, WN, 1>), grid, dim3(kThreads), 0, st, gp);
@@ -303,12 +478,20 @@ static void launch_gather_cfg(const GatherParams& gp, bool vec, hipStream_t st) 
 
 static inline int gather_bn(int N) { return N <= 32 ? 32 : 64; }
 
-static inline int gather_bm(int M, int N, int cus) {
+// Tile height.  The LDS-direct kernel keeps two slabs per operand in LDS, so a
+// 128-row tile (48 KB) lets three workgroups share a CU where a 256-row tile
+// (80 KB) allows one or two; measured on the 56x56x64 shape, 128 rows is 11 %
+// faster.  The register-staged kernel prefers 256 rows.
+static inline int gather_bm(int M, int N, int cus, bool dma) {
     const int bn = gather_bn(N);
+    if (const char* f = getenv("AETHER_GATHER_BM")) {       // tuning override: 256, 128 or 64
+        int v = atoi(f);
+        if (v == 256 || v == 128 || (v == 64 && bn == 64)) return v;
+    }
     const int ntiles = cdiv(N, bn);
     const int want = 2 * cus;
     const int cands[3] = {256, 128, 64};
-    for (int i = 0; i < 3; ++i) {
+    for (int i = dma ? 1 : 0; i < 3; ++i) {
         int bm = cands[i];
         if (bn == 32 && bm == 64) break;
         if ((int64_t)cdiv(M, bm) * ntiles >= want) return bm;
@@ -319,7 +502,8 @@ static inline int gather_bm(int M, int N, int cus) {
 template <typename T>
 static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t st) {
     const int bn = gather_bn(gp.N);
-    const int bm = gather_bm(gp.M, gp.N, cus);
+    const bool dma = vec && gp.src_bytes != 0 && gp.bt_bytes != 0;
+    const int bm = gather_bm(gp.M, gp.N, cus, dma);
     if (bn == 32) {
         if (bm == 256) launch_gather_cfg<T, 256, 32, 64, 32>(gp, vec, st);
         else launch_gather_cfg<T, 128, 32, 32, 32>(gp, vec, st);
@@ -344,6 +528,14 @@ static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
     gs.gp.bt = bt;
     gs.pp.bt = bt;
     int total = gs.pp.Npad * gs.pp.Kpad;
+    {
+        const GatherParams& g = gs.gp;
+        int64_t sb = (int64_t)g.S * g.Hs * g.Ws * g.Cs * (int64_t)sizeof(T);
+        int64_t bb = (int64_t)total * (int64_t)sizeof(T);
+        const int64_t lim = (int64_t)1 << 31;
+        gs.gp.src_bytes = (sb < lim && bb < lim) ? (unsigned)sb : 0u;
+        gs.gp.bt_bytes = (sb < lim && bb < lim) ? (unsigned)bb : 0u;
+    }
     if (total > 0) {
         hipLaunchKernelGGL(pack_filter<T>, dim3(cdiv(total, 256)), dim3(256), 0, c.stream, gs.pp);
         AETH_LAUNCH_CHECK();
@@ -486,6 +678,8 @@ struct WgradParams {
     int M, K;
     int fW, sH, sW, pH, pW;
     int m_per_split;     // multiple of 32
+    int kt, nt;          // output tiles along k and n
+    unsigned x_bytes, dy_bytes;   // extents for the buffer descriptors (LDS-direct kernel)
     FastDiv div_howo, div_wo, div_c, div_fw;
 };
 
@@ -518,9 +712,14 @@ __global__ __launch_bounds__(kThreads) void wgrad_gemm(const WgradParams p) {
     const int l32 = lane & 31;
     const int lh = lane >> 5;
 
-    const int kt0 = blockIdx.x * kWgBK;
-    const int n0 = blockIdx.y * kWgBN;
-    const int m_begin = blockIdx.z * p.m_per_split;
+    const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
+    const int tiles = p.kt * p.nt;
+    const int split = lid / tiles;
+    const int tile = lid - split * tiles;
+    const int ktile = tile % p.kt;
+    const int kt0 = ktile * kWgBK;
+    const int n0 = (tile / p.kt) * kWgBN;
+    const int m_begin = split * p.m_per_split;
     int m_end = m_begin + p.m_per_split;
     if (m_end > p.M) m_end = p.M;
 
@@ -545,7 +744,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_gemm(const WgradParams p) {
     // dy chunk: CE consecutive n starting at n0 + CE*ky
     const int ky = tid % Y_CPR;
     const int ry0 = tid / Y_CPR;
-    const bool do_db = p.want_dbias && (blockIdx.x == 0);
+    const bool do_db = p.want_dbias && (ktile == 0);
 
     float areg[A_PASSES][CE];
     float yreg[Y_PASSES][CE];
@@ -662,7 +861,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_gemm(const WgradParams p) {
     }
 
     const size_t split_stride = (size_t)p.K * p.D + p.D;
-    float* outp = p.out + (size_t)blockIdx.z * split_stride;
+    float* outp = p.out + (size_t)split * split_stride;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int n = n0 + 32 * j + l32;
@@ -683,6 +882,161 @@ __global__ __launch_bounds__(kThreads) void wgrad_gemm(const WgradParams p) {
 #pragma unroll
             for (int r = 0; r < Y_RPP; ++r) s += lds_db[r * 64 + tid];
             if (n0 + tid < p.D) outp[(size_t)p.K * p.D + n0 + tid] = s;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------
+// wgrad, LDS-direct variant (fp32, C and D multiples of 4).  Same 128 (k) x 64 (n)
+// tile and split over M as wgrad_gemm, with:
+//   * x and dy slabs loaded straight into LDS (`buffer_load_dwordx4 ... lds`), two
+//     buffers, one barrier per 32-row slab, operand reads of step t+1 issued before
+//     the MFMAs of step t;
+//   * rows unpadded (512 B / 256 B); odd slab rows store their 32-float halves
+//     swapped, so the two half-waves of an operand read (rows m and m+1) fall into
+//     different halves of the banks;
+//   * dbias for free: when it is wanted, row K of the A operand is set to 1 for
+//     every valid m, so row K of the product is sum_m dy[m][n];
+//   * waves whose 32 k-rows lie entirely past the last row issue no MFMAs.
+// ------------------------------------------------------------------------------
+static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma(const WgradParams p) {
+    __shared__ float lds_a0[kWgBR * kWgBK];
+    __shared__ float lds_a1[kWgBR * kWgBK];
+    __shared__ float lds_y0[kWgBR * kWgBN];
+    __shared__ float lds_y1[kWgBR * kWgBN];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int l32 = lane & 31;
+    const int lh = lane >> 5;
+
+    const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
+    const int tiles = p.kt * p.nt;
+    const int split = lid / tiles;
+    const int tile = lid - split * tiles;
+    const int ktile = tile % p.kt;
+    const int kt0 = ktile * kWgBK;
+    const int n0 = (tile / p.kt) * kWgBN;
+    const int m_begin = split * p.m_per_split;
+    int m_end = m_begin + p.m_per_split;
+    if (m_end > p.M) m_end = p.M;
+    const int Kout = p.K + (p.want_dbias ? 1 : 0);      // row K carries dbias
+
+    // ---- A: one wave-level load = 2 slab rows x 32 chunks; 4 loads per wave ------
+    const int a_row = lane >> 5;                         // row inside the 2-row block
+    const int a_lc = (lane & 31) ^ (a_row << 3);         // logical chunk fetched (odd rows: halves swapped)
+    int a_tap_off, a_fx, a_fy;
+    bool a_kok;
+    {
+        int kk = kt0 + 4 * a_lc;
+        unsigned tap, c, fx, fy;
+        p.div_c.divmod((unsigned)kk, tap, c);
+        p.div_fw.divmod(tap, fx, fy);
+        a_kok = kk < p.K;
+        a_fx = (int)fx - p.pH;
+        a_fy = (int)fy - p.pW;
+        a_tap_off = (a_fx * p.W + a_fy) * p.C + (int)c;
+    }
+    // the lane whose chunk contains row K plants the ones (after its own load landed)
+    const int one_k = p.K - kt0;                         // tile-local row of the ones
+    const bool plant = p.want_dbias && one_k >= 4 * a_lc && one_k < 4 * a_lc + 4;
+    // ---- dy: one wave-level load = 4 slab rows x 16 chunks; 2 loads per wave -----
+    const int y_row = lane >> 4;
+    const int y_lc = (lane & 15) ^ ((y_row & 1) << 3);
+    const int y_n = n0 + 4 * y_lc;
+    const bool y_nok = y_n < p.D;
+
+    const __amdgpu_buffer_rsrc_t rsrc_x =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.x), 0, (int)p.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_y =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.dy), 0, (int)p.dy_bytes, 0x00020000);
+
+    auto issue = [&](int mb, float* la, float* ly) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int ml = (wave * 4 + i) * 2 + a_row;
+            const int m = mb + ml;
+            unsigned s, rem, ho, wo;
+            p.div_howo.divmod((unsigned)m, s, rem);
+            p.div_wo.divmod(rem, ho, wo);
+            const int r0 = (int)ho * p.sH, c0 = (int)wo * p.sW;
+            const int pix = (((int)s * p.H + r0) * p.W + c0) * p.C;
+            const unsigned bad = (unsigned)!((m < m_end) & a_kok & ((unsigned)(r0 + a_fx) < (unsigned)p.H) &
+                                             ((unsigned)(c0 + a_fy) < (unsigned)p.W));
+            const unsigned voff = ((unsigned)(pix + a_tap_off) * 4u) | (bad << 31);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + (wave * 4 + i) * 256), 16, (int)voff, 0,
+                                                     0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int m = mb + (wave * 2 + i) * 4 + y_row;
+            const unsigned bad = (unsigned)!((m < m_end) & y_nok);
+            const unsigned voff = ((unsigned)(m * p.D + y_n) * 4u) | (bad << 31);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_y, (lds_ptr_t)(ly + (wave * 2 + i) * 256), 16, (int)voff, 0,
+                                                     0, 0);
+        }
+    };
+    auto plant_ones = [&](int mb, float* la) {
+        if (plant) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int ml = (wave * 4 + i) * 2 + a_row;
+                if (mb + ml < m_end) la[ml * kWgBK + (one_k ^ (a_row << 5))] = 1.0f;
+            }
+        }
+    };
+
+    f16v acc[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+
+    const bool active = kt0 + wave * 32 < Kout;          // wave-uniform
+    const int a_rd = ((wave * 32) ^ (lh << 5)) + l32;    // physical float of this lane's k, rows m = 2t + lh
+    const int y_rd0 = l32 + (lh << 5);                   // logical n = l32
+    const int y_rd1 = l32 + ((lh ^ 1) << 5);             // logical n = 32 + l32
+    auto slab = [&](int mb, const float* la, const float* ly, float* na, float* ny, bool has_next) {
+        __builtin_amdgcn_s_waitcnt(0);                   // this wave's loads of the slab have landed
+        plant_ones(mb, const_cast<float*>(la));
+        __syncthreads();
+        if (has_next) issue(mb + kWgBR, na, ny);
+        if (active) {
+            float fa[2], fb0[2], fb1[2];
+            fa[0] = la[lh * kWgBK + a_rd];
+            fb0[0] = ly[lh * kWgBN + y_rd0];
+            fb1[0] = ly[lh * kWgBN + y_rd1];
+#pragma unroll
+            for (int t = 0; t < kWgBR / 2; ++t) {
+                if (t + 1 < kWgBR / 2) {
+                    fa[(t + 1) & 1] = la[(2 * t + 2 + lh) * kWgBK + a_rd];
+                    fb0[(t + 1) & 1] = ly[(2 * t + 2 + lh) * kWgBN + y_rd0];
+                    fb1[(t + 1) & 1] = ly[(2 * t + 2 + lh) * kWgBN + y_rd1];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[t & 1], fb0[t & 1], acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[t & 1], fb1[t & 1], acc[1], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+
+    if (m_begin < m_end) issue(m_begin, lds_a0, lds_y0);
+    for (int mb = m_begin; mb < m_end; mb += 2 * kWgBR) {
+        slab(mb, lds_a0, lds_y0, lds_a1, lds_y1, mb + kWgBR < m_end);
+        if (mb + kWgBR < m_end) slab(mb + kWgBR, lds_a1, lds_y1, lds_a0, lds_y0, mb + 2 * kWgBR < m_end);
+    }
+
+    const size_t split_stride = (size_t)p.K * p.D + p.D;
+    float* outp = p.out + (size_t)split * split_stride;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int n = n0 + 32 * j + l32;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int k = kt0 + wave * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            if (k < Kout && n < p.D) outp[(size_t)k * p.D + n] = acc[j][v];
         }
     }
 }
@@ -734,9 +1088,18 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     p.fW = fW; p.sH = sH; p.sW = sW; p.pH = pH; p.pW = pW;
     p.want_dbias = dbias != nullptr;
     p.div_howo = FastDiv(Ho * Wo); p.div_wo = FastDiv(Wo); p.div_c = FastDiv(C); p.div_fw = FastDiv(fW);
-    const int kt = cdiv(p.K, kWgBK), nt = cdiv(D, kWgBN);
+    constexpr int CE = Elem<T>::CE;
+    const bool va = (C % CE == 0), vy = (D % CE == 0);
+    const int64_t xb = (int64_t)S * H * W * C * (int64_t)sizeof(T), yb = (int64_t)p.M * D * (int64_t)sizeof(T);
+    const bool dma = sizeof(T) == 4 && va && vy && xb < ((int64_t)1 << 31) && yb < ((int64_t)1 << 31);
+    p.x_bytes = dma ? (unsigned)xb : 0u;
+    p.dy_bytes = dma ? (unsigned)yb : 0u;
+    // the LDS-direct kernel gets dbias from an extra row K of the product
+    const int krows = p.K + ((dma && dbias) ? 1 : 0);
+    const int kt = cdiv(krows, kWgBK), nt = cdiv(D, kWgBN);
     const int slabs = cdiv(p.M, kWgBR);
-    int splits = cdiv(4 * c.prop.multiProcessorCount, kt * nt);
+    // about two rounds of resident workgroups (3 per CU for the LDS-direct kernel)
+    int splits = cdiv((dma ? 6 : 4) * c.prop.multiProcessorCount, kt * nt);
     if (splits > slabs) splits = slabs;
     if (splits < 1) splits = 1;
     int slabs_per = cdiv(slabs, splits);
@@ -747,10 +1110,10 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     rc = workspace((int64_t)splits * (kd + D) * sizeof(float), &ws);
     if (rc) return rc;
     p.out = (float*)ws;
-    dim3 grid(kt, nt, splits);
-    constexpr int CE = Elem<T>::CE;
-    const bool va = (C % CE == 0), vy = (D % CE == 0);
-    if (va && vy) hipLaunchKernelGGL((wgrad_gemm<T, CE, CE>), grid, dim3(kThreads), 0, c.stream, p);
+    p.kt = kt; p.nt = nt;
+    dim3 grid(kt * nt * splits);
+    if (dma) hipLaunchKernelGGL(wgrad_gemm_dma, grid, dim3(kThreads), 0, c.stream, p);
+    else if (va && vy) hipLaunchKernelGGL((wgrad_gemm<T, CE, CE>), grid, dim3(kThreads), 0, c.stream, p);
     else if (va) hipLaunchKernelGGL((wgrad_gemm<T, CE, 1>), grid, dim3(kThreads), 0, c.stream, p);
     else if (vy) hipLaunchKernelGGL((wgrad_gemm<T, 1, CE>), grid, dim3(kThreads), 0, c.stream, p);
     else hipLaunchKernelGGL((wgrad_gemm<T, 1, 1>), grid, dim3(kThreads), 0, c.stream, p);
