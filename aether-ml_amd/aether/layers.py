@@ -434,6 +434,10 @@ class SoftMax:
         _ck(_L().aeth_softmax_bwd_f32(self.output.ptr, dvalues.ptr, self.dinputs.ptr, rows, K))
 
     def predictions(self, outputs):
+        # the loss kernel already produced the row argmax of these probabilities
+        cached = getattr(outputs, "_cache", None)
+        if cached is not None and "argmax" in cached:
+            return cached["argmax"]
         return np.argmax(np.asarray(outputs), axis=1)
 
 
@@ -446,6 +450,19 @@ def _sparse_labels(y_true):
     if y.ndim == 2:
         y = np.argmax(y, axis=1)
     return np.ascontiguousarray(y, dtype=np.int32)
+
+
+_label_cache = [None, None]     # (bytes of the last label batch, its device copy)
+
+
+def _device_labels(y_true):
+    """Labels on the device; the forward and backward pass of one step share the upload."""
+    y = _sparse_labels(y_true)
+    key = y.tobytes()
+    if _label_cache[0] != key:
+        _label_cache[0] = key
+        _label_cache[1] = DeviceTensor.from_numpy(y, np.int32)
+    return _label_cache[1]
 
 
 class Loss:
@@ -497,18 +514,19 @@ class Loss_CategoricalCrossEntropy(Loss):
     def forward(self, y_pred, y_true, training=True):
         y_pred = as_device(y_pred, _F32)
         rows, K = y_pred.shape
-        labels = DeviceTensor.from_numpy(_sparse_labels(y_true), np.int32)
+        labels = _device_labels(y_true)
         ls = self.label_smoothing if (self.label_smoothing > 0 and training) else 0.0
-        loss = DeviceTensor(rows, _F32)
-        correct = DeviceTensor(rows, np.int32)
-        _ck(_L().aeth_cce_fwd_f32(y_pred.ptr, labels.ptr, ls, loss.ptr, correct.ptr, rows, K))
-        self.correct = correct
-        return loss.get()
+        # per-sample loss and row argmax side by side: one read-back for both
+        buf = DeviceTensor(2 * rows, _F32)
+        _ck(_L().aeth_cce_fwd_f32(y_pred.ptr, labels.ptr, ls, buf.ptr, buf.ptr + 4 * rows, rows, K))
+        host = buf.get()
+        y_pred._cache = {"argmax": host[rows:].view(np.int32)}
+        return host[:rows]
 
     def backward(self, dvalues, y_true):
         dvalues = as_device(dvalues, _F32)
         rows, K = dvalues.shape
-        labels = DeviceTensor.from_numpy(_sparse_labels(y_true), np.int32)
+        labels = _device_labels(y_true)
         self.dinputs = DeviceTensor(dvalues.shape, _F32)
         _ck(_L().aeth_softmax_cce_bwd_f32(dvalues.ptr, labels.ptr, self.label_smoothing, self.dinputs.ptr, rows, K))
 
@@ -528,7 +546,7 @@ class Activation_Softmax_Loss_CategoricalCrossEntropy():
     def backward(self, dvalues, y_true, training=True):
         dvalues = as_device(dvalues, _F32)
         rows, K = dvalues.shape
-        labels = DeviceTensor.from_numpy(_sparse_labels(y_true), np.int32)
+        labels = _device_labels(y_true)
         ls = self.label_smoothing if (self.label_smoothing > 0 and training) else 0.0
         self.dinputs = DeviceTensor(dvalues.shape, _F32)
         _ck(_L().aeth_softmax_cce_bwd_f32(dvalues.ptr, labels.ptr, ls, self.dinputs.ptr, rows, K))
@@ -546,6 +564,7 @@ class Optimizer_Adam:
         self.epsilon = epsilon
         self.beta_1 = beta_1
         self.beta_2 = beta_2
+        self._pending = []
 
     def pre_update_parameters(self):
         if self.decay:
@@ -557,13 +576,26 @@ class Optimizer_Adam:
             layer.weight_cache = DeviceTensor.zeros(layer.weights.shape)
             layer.bias_momentums = DeviceTensor.zeros(layer.biases.shape)
             layer.bias_cache = DeviceTensor.zeros(layer.biases.shape)
-        L = _L()
-        _ck(L.aeth_adam_f32(layer.weights.ptr, layer.dweights.ptr, layer.weight_momentums.ptr,
-                            layer.weight_cache.ptr, layer.weights.size, self.current_learning_rate,
-                            self.beta_1, self.beta_2, self.epsilon, self.iterations))
-        _ck(L.aeth_adam_f32(layer.biases.ptr, layer.dbiases.ptr, layer.bias_momentums.ptr,
-                            layer.bias_cache.ptr, layer.biases.size, self.current_learning_rate,
-                            self.beta_1, self.beta_2, self.epsilon, self.iterations))
+        # The updates of all layers of a step go out as one launch: they are queued
+        # here and issued by post_update_parameters (or when 32 tensors are waiting).
+        self._pending.append((layer.weights, layer.dweights, layer.weight_momentums, layer.weight_cache))
+        self._pending.append((layer.biases, layer.dbiases, layer.bias_momentums, layer.bias_cache))
+        if len(self._pending) >= 32:
+            self._flush()
+
+    def _flush(self):
+        import ctypes as C
+        while self._pending:
+            batch, self._pending = self._pending[:32], self._pending[32:]
+            n = len(batch)
+            arr = lambda k: (C.c_void_p * n)(*[t[k].ptr for t in batch])
+            sizes = (C.c_int64 * n)(*[t[0].size for t in batch])
+            for t in batch:
+                if t[1].size != t[0].size:
+                    raise ValueError("gradient shape %s does not match parameter shape %s" % (t[1].shape, t[0].shape))
+            _ck(_L().aeth_adam_multi_f32(n, arr(0), arr(1), arr(2), arr(3), sizes, self.current_learning_rate,
+                                         self.beta_1, self.beta_2, self.epsilon, self.iterations))
 
     def post_update_parameters(self):
+        self._flush()
         self.iterations += 1

@@ -11,7 +11,7 @@ from . import _lib
 
 
 class DeviceTensor:
-    __slots__ = ("ptr", "shape", "dtype", "_base", "__weakref__")
+    __slots__ = ("ptr", "shape", "dtype", "_base", "_cache", "__weakref__")
 
     def __init__(self, shape, dtype=np.float32, _ptr=None, _base=None):
         if isinstance(shape, (int, np.integer)):
@@ -19,6 +19,7 @@ class DeviceTensor:
         self.shape = tuple(int(s) for s in shape)
         self.dtype = np.dtype(dtype)
         self._base = _base
+        self._cache = None      # host-side values derived from this tensor by a kernel (e.g. row argmax)
         if _ptr is None:
             p = C.c_void_p()
             _lib.check(_lib.lib().aeth_malloc(C.byref(p), self.nbytes))

@@ -63,7 +63,7 @@ __device__ __forceinline__ void column_partials(int rows, int C, int rows_per_bl
 
 static void col_grid(int rows, int C, int* nblk, int* rows_per_block, dim3* grid) {
     int nb = cdiv(rows, 256);
-    if (nb > 512) nb = 512;
+    if (nb > 256) nb = 256;
     if (nb < 1) nb = 1;
     int rpb = cdiv(rows, nb);
     nb = cdiv(rows, rpb);
@@ -73,6 +73,37 @@ static void col_grid(int rows, int C, int* nblk, int* rows_per_block, dim3* grid
 }
 
 // ---- batch norm ------------------------------------------------------------------
+// Sums part[v][b][c] over the blocks b for v = 0, 1.  Launched with 256 threads =
+// 64 channels x 4 block lanes; lane j adds blocks j, j+4, ... with four independent
+// accumulators, then the lanes are added in order.  Returns true for the thread
+// that holds the result (lane 0 of a valid channel).
+__device__ __forceinline__ bool sum_partials2(const float* __restrict__ part, int nblk, int C, int c, float& s1,
+                                              float& s2) {
+    __shared__ float red[2][4][64];
+    const int col = threadIdx.x & 63, bl = threadIdx.x >> 6;
+    float a[4] = {0.f, 0.f, 0.f, 0.f}, q[4] = {0.f, 0.f, 0.f, 0.f};
+    if (c < C) {
+        int b = bl;
+        for (; b + 12 < nblk; b += 16) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                a[u] += part[(size_t)(b + 4 * u) * C + c];
+                q[u] += part[((size_t)nblk + b + 4 * u) * C + c];
+            }
+        }
+        for (; b < nblk; b += 4) {
+            a[0] += part[(size_t)b * C + c];
+            q[0] += part[((size_t)nblk + b) * C + c];
+        }
+    }
+    red[0][bl][col] = (a[0] + a[1]) + (a[2] + a[3]);
+    red[1][bl][col] = (q[0] + q[1]) + (q[2] + q[3]);
+    __syncthreads();
+    s1 = (red[0][0][col] + red[0][1][col]) + (red[0][2][col] + red[0][3][col]);
+    s2 = (red[1][0][col] + red[1][1][col]) + (red[1][2][col] + red[1][3][col]);
+    return bl == 0 && c < C;
+}
+
 // Statistics use sums of (x - shift) and (x - shift)^2 with shift = x[0][c]: the
 // variance then comes from numbers of the size of the spread, not of the mean.
 __global__ __launch_bounds__(kEwThreads) void bn_stats_partial(const float* __restrict__ x, int rows, int C,
@@ -88,13 +119,9 @@ __global__ void bn_stats_final(const float* __restrict__ x, const float* __restr
                                float eps, float momentum, float* __restrict__ running_mean,
                                float* __restrict__ running_var, float* __restrict__ save_mean,
                                float* __restrict__ save_invstd) {
-    int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= C) return;
-    float s1 = 0.f, s2 = 0.f;
-    for (int b = 0; b < nblk; ++b) {
-        s1 += part[(size_t)b * C + c];
-        s2 += part[((size_t)nblk + b) * C + c];
-    }
+    const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+    float s1, s2;
+    if (!sum_partials2(part, nblk, C, c, s1, s2)) return;
     const float inv_n = 1.0f / (float)rows;
     const float dm = s1 * inv_n;
     const float mean = x[c] + dm;
@@ -144,13 +171,9 @@ __global__ __launch_bounds__(kEwThreads) void bn_bwd_partial(const float* __rest
 __global__ void bn_bwd_final(const float* __restrict__ part, int nblk, int rows, int C,
                              const float* __restrict__ gamma, const float* __restrict__ invstd,
                              float* __restrict__ dgamma, float* __restrict__ dbeta, float* __restrict__ coef) {
-    int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= C) return;
-    float s1 = 0.f, s2 = 0.f;
-    for (int b = 0; b < nblk; ++b) {
-        s1 += part[(size_t)b * C + c];
-        s2 += part[((size_t)nblk + b) * C + c];
-    }
+    const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+    float s1, s2;
+    if (!sum_partials2(part, nblk, C, c, s1, s2)) return;
     const float is = invstd[c], g = gamma[c];
     const float inv_n = 1.0f / (float)rows;
     dgamma[c] = s2 * is;
@@ -221,6 +244,37 @@ __global__ void cast_bf16_kernel(const float* __restrict__ src, uint16_t* __rest
 __global__ void adam_kernel(float* __restrict__ theta, const float* __restrict__ g, float* __restrict__ m,
                             float* __restrict__ v, int64_t n, float lr, float b1, float b2, float eps, float c1,
                             float c2) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        float gi = g[i];
+        float mi = b1 * m[i] + (1.0f - b1) * gi;
+        float vi = b2 * v[i] + (1.0f - b2) * (gi * gi);
+        m[i] = mi;
+        v[i] = vi;
+        float mh = mi / c1;
+        float vh = vi / c2;
+        theta[i] += -lr * mh / (sqrtf(vh) + eps);
+    }
+}
+
+constexpr int kAdamMax = 32;
+struct AdamTable {
+    float* theta[kAdamMax];
+    const float* grad[kAdamMax];
+    float* m[kAdamMax];
+    float* v[kAdamMax];
+    int64_t n[kAdamMax];
+};
+
+// blockIdx.y selects the tensor, blockIdx.x strides over its elements
+__global__ void adam_multi_kernel(const AdamTable tb, float lr, float b1, float b2, float eps, float c1, float c2) {
+    const int t = blockIdx.y;
+    float* __restrict__ theta = tb.theta[t];
+    const float* __restrict__ g = tb.grad[t];
+    float* __restrict__ m = tb.m[t];
+    float* __restrict__ v = tb.v[t];
+    const int64_t n = tb.n[t];
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (; i < n; i += stride) {
@@ -391,7 +445,7 @@ __global__ void softmax_bwd_kernel(const float* __restrict__ probs, const float*
 }
 
 __global__ void cce_fwd_kernel(const float* __restrict__ probs, const int32_t* __restrict__ labels, float ls,
-                               float* __restrict__ loss, int32_t* __restrict__ correct, int rows, int K) {
+                               float* __restrict__ loss, int32_t* __restrict__ pred, int rows, int K) {
     int r = blockIdx.x * blockDim.x + threadIdx.x;
     if (r >= rows) return;
     const float* p = probs + (size_t)r * K;
@@ -412,7 +466,7 @@ __global__ void cce_fwd_kernel(const float* __restrict__ probs, const int32_t* _
         acc += t * logf(pc);
     }
     loss[r] = -acc;
-    correct[r] = (bi == y) ? 1 : 0;
+    pred[r] = bi;
 }
 
 __global__ void softmax_cce_bwd_kernel(const float* __restrict__ probs, const int32_t* __restrict__ labels, float ls,
@@ -435,6 +489,17 @@ static int pool_dims(const char* fn, int S, int H, int W, int C, int fH, int fW,
     p->Wo = (W - fW) / sW + 1;
     if ((int64_t)S * H * W * C >= ((int64_t)1 << 31)) return fail(AETH_E_INVALID, "%s: tensor too large", fn);
     return AETH_OK;
+}
+
+static void adam_corrections(float beta1, float beta2, int t, float* c1, float* c2) {
+    // 1 - beta^(t+1) by repeated squaring in double
+    double p1 = 1.0, p2 = 1.0, b1 = beta1, b2 = beta2;
+    for (unsigned e = (unsigned)t + 1; e; e >>= 1) {
+        if (e & 1) { p1 *= b1; p2 *= b2; }
+        b1 *= b1; b2 *= b2;
+    }
+    *c1 = (float)(1.0 - p1);
+    *c2 = (float)(1.0 - p2);
 }
 
 }  // namespace aeth
@@ -465,7 +530,7 @@ int aeth_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta,
     hipStream_t st = ctx().stream;
     hipLaunchKernelGGL(bn_stats_partial, grid, dim3(kEwThreads), 0, st, x, rows, C, rpb, part);
     AETH_LAUNCH_CHECK();
-    hipLaunchKernelGGL(bn_stats_final, dim3(cdiv(C, 64)), dim3(64), 0, st, x, part, nblk, rows, C, eps, momentum,
+    hipLaunchKernelGGL(bn_stats_final, dim3(cdiv(C, 64)), dim3(256), 0, st, x, part, nblk, rows, C, eps, momentum,
                        running_mean, running_var, save_mean, save_invstd);
     AETH_LAUNCH_CHECK();
     int64_t n = (int64_t)rows * C;
@@ -499,7 +564,7 @@ int aeth_bn_bwd_f32(const float* x, const float* dy, const float* gamma, const f
     hipStream_t st = ctx().stream;
     hipLaunchKernelGGL(bn_bwd_partial, grid, dim3(kEwThreads), 0, st, x, dy, save_mean, rows, C, rpb, part);
     AETH_LAUNCH_CHECK();
-    hipLaunchKernelGGL(bn_bwd_final, dim3(cdiv(C, 64)), dim3(64), 0, st, part, nblk, rows, C, gamma, save_invstd,
+    hipLaunchKernelGGL(bn_bwd_final, dim3(cdiv(C, 64)), dim3(256), 0, st, part, nblk, rows, C, gamma, save_invstd,
                        dgamma, dbeta, coef);
     AETH_LAUNCH_CHECK();
     int64_t n = (int64_t)rows * C;
@@ -597,11 +662,11 @@ int aeth_softmax_bwd_f32(const float* probs, const float* dy, float* dx, int row
 }
 
 int aeth_cce_fwd_f32(const float* probs, const int32_t* labels, float label_smoothing, float* sample_loss,
-                     int32_t* correct, int rows, int K) {
+                     int32_t* pred, int rows, int K) {
     AETH_REQUIRE_INIT();
-    AETH_CHECK_ARG(probs && labels && sample_loss && correct && rows > 0 && K > 0);
+    AETH_CHECK_ARG(probs && labels && sample_loss && pred && rows > 0 && K > 0);
     hipLaunchKernelGGL(cce_fwd_kernel, dim3(cdiv(rows, 64)), dim3(64), 0, ctx().stream, probs, labels,
-                       label_smoothing, sample_loss, correct, rows, K);
+                       label_smoothing, sample_loss, pred, rows, K);
     AETH_LAUNCH_CHECK();
     return AETH_OK;
 }
@@ -623,19 +688,36 @@ int aeth_adam_f32(float* theta, const float* grad, float* m, float* v, int64_t n
     AETH_CHECK_ARG(n >= 0 && t >= 0);
     if (n == 0) return AETH_OK;
     AETH_CHECK_ARG(theta && grad && m && v);
-    double c1 = 1.0, c2 = 1.0;
-    {
-        double p1 = 1.0, p2 = 1.0;
-        // beta^(t+1) by repeated squaring in double
-        double b1 = beta1, b2 = beta2;
-        for (unsigned e = (unsigned)t + 1; e; e >>= 1) {
-            if (e & 1) { p1 *= b1; p2 *= b2; }
-            b1 *= b1; b2 *= b2;
-        }
-        c1 = 1.0 - p1;
-        c2 = 1.0 - p2;
+    float c1, c2;
+    adam_corrections(beta1, beta2, t, &c1, &c2);
+    EW_LAUNCH(adam_kernel, n, theta, grad, m, v, n, lr, beta1, beta2, eps, c1, c2);
+    return AETH_OK;
+}
+
+int aeth_adam_multi_f32(int count, float* const* host_theta, const float* const* host_grad, float* const* host_m,
+                        float* const* host_v, const int64_t* host_n, float lr, float beta1, float beta2, float eps,
+                        int t) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(count >= 1 && count <= kAdamMax && t >= 0);
+    AETH_CHECK_ARG(host_theta && host_grad && host_m && host_v && host_n);
+    AdamTable tb;
+    int64_t nmax = 0;
+    for (int i = 0; i < kAdamMax; ++i) {
+        const int j = i < count ? i : 0;
+        AETH_CHECK_ARG(host_n[j] >= 0);
+        AETH_CHECK_ARG(host_n[j] == 0 || (host_theta[j] && host_grad[j] && host_m[j] && host_v[j]));
+        tb.theta[i] = host_theta[j]; tb.grad[i] = host_grad[j]; tb.m[i] = host_m[j]; tb.v[i] = host_v[j];
+        tb.n[i] = i < count ? host_n[j] : 0;
+        if (tb.n[i] > nmax) nmax = tb.n[i];
     }
-    EW_LAUNCH(adam_kernel, n, theta, grad, m, v, n, lr, beta1, beta2, eps, (float)c1, (float)c2);
+    if (nmax == 0) return AETH_OK;
+    float c1, c2;
+    adam_corrections(beta1, beta2, t, &c1, &c2);
+    int bx = (int)((nmax + 4 * kEwThreads - 1) / (4 * kEwThreads));
+    if (bx > 256) bx = 256;
+    hipLaunchKernelGGL(adam_multi_kernel, dim3(bx, count), dim3(kEwThreads), 0, ctx().stream, tb, lr, beta1, beta2,
+                       eps, c1, c2);
+    AETH_LAUNCH_CHECK();
     return AETH_OK;
 }
 

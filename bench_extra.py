@@ -28,9 +28,16 @@ SHAPES = [
 
 
 def _time(fn, steps, warmup):
+    """Average ms per call over `steps` calls, after at least `warmup` calls and
+    40 ms of back-to-back work (so clocks have ramped after the host-side setup)."""
     from aether import _lib
-    for _ in range(warmup):
+    t0 = time.perf_counter()
+    n = 0
+    while n < warmup or time.perf_counter() - t0 < 0.04:
         fn()
+        n += 1
+        if n % 8 == 0:
+            _lib.sync()
     _lib.sync()
     e0, e1 = _lib.Event(), _lib.Event()
     e0.record()
@@ -144,4 +151,7 @@ def run(steps, warmup):
 
 if __name__ == "__main__":
     import json
-    print(json.dumps(run(20, 5), indent=1))
+    if "--train-only" in sys.argv:
+        print(json.dumps(train_step(50, 10), indent=1))
+    else:
+        print(json.dumps(run(20, 5), indent=1))

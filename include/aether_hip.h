@@ -157,9 +157,10 @@ int aeth_mul_mask_f32(const float* x, const float* mask, float* y, int64_t n, in
 int aeth_softmax_f32(const float* logits, float* probs, int rows, int K);
 int aeth_softmax_bwd_f32(const float* probs, const float* dy, float* dx, int rows, int K);
 /* Loss_CategoricalCrossEntropy.forward :615-632 on probabilities (clip to
- * [1e-7, 1-1e-7], label smoothing) -> per-sample loss; correct[i] = argmax == label. */
+ * [1e-7, 1-1e-7], label smoothing) -> per-sample loss; pred[i] = argmax_k probs[i][k]
+ * (first maximum), which is what SoftMax.predictions :562-563 returns. */
 int aeth_cce_fwd_f32(const float* probs, const int32_t* labels, float label_smoothing,
-                     float* sample_loss, int32_t* correct, int rows, int K);
+                     float* sample_loss, int32_t* pred, int rows, int K);
 /* Activation_Softmax_Loss_CategoricalCrossEntropy.backward :666-680:
  * dlogits = (probs - smooth(onehot)) / rows. */
 int aeth_softmax_cce_bwd_f32(const float* probs, const int32_t* labels, float label_smoothing,
@@ -167,6 +168,13 @@ int aeth_softmax_cce_bwd_f32(const float* probs, const int32_t* labels, float la
 /* Optimizer_Adam.update_parameters for one tensor :702-734; t = iterations (0-based). */
 int aeth_adam_f32(float* theta, const float* grad, float* m, float* v, int64_t n,
                   float lr, float beta1, float beta2, float eps, int t);
+/* The same update for `count` (1..32) tensors in ONE launch: the loop over
+ * trainable layers of Model.train (CNN_model_cupy.py:124-125) with each layer's
+ * weights and biases as separate entries.  The five host_ arrays have `count`
+ * entries; the pointers they hold are device pointers. */
+int aeth_adam_multi_f32(int count, float* const* host_theta, const float* const* host_grad,
+                        float* const* host_m, float* const* host_v, const int64_t* host_n,
+                        float lr, float beta1, float beta2, float eps, int t);
 
 #ifdef __cplusplus
 }
