@@ -289,17 +289,26 @@ __global__ __launch_bounds__(kThreads, 3) void gather_gemm(const GatherParams p)
 // flight while slab k is multiplied (one barrier per slab).
 //   * One wave-level load writes 64 consecutive 16-byte chunks = 8 slab rows, so
 //     rows are unpadded (128 B) and bank conflicts are avoided by an XOR swizzle:
-//     logical chunk c of row r lives at chunk position c ^ (r & 7).  The swizzle is
-//     applied on the global side (lane l of a load fetches logical chunk
-//     (l & 7) ^ (l >> 3) of row l >> 3) and undone by the operand reads.
+//     logical chunk c of row r lives at chunk position c ^ ((r >> 1) & 7).  A
+//     128-bit operand read is served 16 lanes (= 16 consecutive rows) at a time
+//     from 64 banks; rows r and r+1 differ in address bit 7 and the 8 row pairs get
+//     8 different chunk positions, so the 16 lanes cover the 64 banks exactly once.
+//     The swizzle is applied on the global side (each lane of a load fetches the
+//     logical chunk that belongs at its LDS position) and undone by the operand reads.
 //   * Padding taps and rows past M use a byte offset of 2^31, which is outside the
 //     buffer descriptor's extent: the load returns zeros.
 // ------------------------------------------------------------------------------
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
-template <typename T, int BM, int BN, int WM, int WN, int MINW>
-__global__ __launch_bounds__(kThreads, MINW) void gather_gemm_dma(const GatherParams p) {
+//   * UT ("uniform tap"): when the channel count is a multiple of the slab width and
+//     the filter has at most 32 taps, a slab lies inside one tap.  fp32 MFMA shares
+//     the FP32 lanes with ordinary vector instructions, so every address instruction
+//     costs MFMA time; in this mode the tap decode runs on the scalar unit and each
+//     row's per-tap validity is a precomputed bit mask: 3 vector instructions per load.
+template <typename T, int BM, int BN, int WM, int WN, bool UT>
+__global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p) {
     static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
+    static_assert((BM / 32) % 2 == 0, "8-row load blocks of a wave alternate even/odd");
     constexpr int CE = Elem<T>::CE;
     constexpr int BK = Elem<T>::BK;
     constexpr int AL = BM / 32;          // wave-level A loads per wave per slab (8 rows each)
@@ -325,7 +334,9 @@ __global__ __launch_bounds__(kThreads, MINW) void gather_gemm_dma(const GatherPa
     const int n0 = (lid % ntile) * BN;
 
     const int lr = lane >> 3;                  // row inside an 8-row load block
-    const int k4 = (lane & 7) ^ lr;            // logical chunk this lane fetches
+    // logical chunk this lane fetches: (lane & 7) ^ ((row >> 1) & 7); the 8-row blocks
+    // alternate between row bits (0,lane>>4) and (4 | lane>>4)
+    const int k4e = (lane & 7) ^ (lane >> 4);  // even 8-row blocks; odd blocks use k4e ^ 4
     int base_off[AL];
     int base_rc[AL];
 #pragma unroll
@@ -344,10 +355,33 @@ __global__ __launch_bounds__(kThreads, MINW) void gather_gemm_dma(const GatherPa
             base_rc[i] = (int)((unsigned)kInvalidRow << 16);
         }
     }
+    // uniform-tap mode: byte offset of this lane's chunk at tap (0,0), and one bit per
+    // tap that says "outside the image" (all ones for rows past M)
+    unsigned a_byte[AL], a_inv[AL];
+    if (UT) {
+        const int ntaps = p.K / p.Cs;
+#pragma unroll
+        for (int i = 0; i < AL; ++i) {
+            const int br = base_rc[i] >> 16;
+            const int bc = (int)((unsigned)base_rc[i] << 16) >> 16;
+            unsigned inv = 0;
+            int th = 0, tw = 0;
+            for (int t = 0; t < ntaps; ++t) {
+                const unsigned bad =
+                    (unsigned)!(((unsigned)(br + th) < (unsigned)p.Hs) & ((unsigned)(bc + tw) < (unsigned)p.Ws));
+                inv |= bad << t;
+                if (++tw == p.Tw) { tw = 0; ++th; }
+            }
+            a_inv[i] = inv;
+            a_byte[i] = (unsigned)(base_off[i] + CE * (k4e ^ ((i & 1) << 2))) * (unsigned)sizeof(T);
+        }
+    }
     unsigned b_off[BL];
 #pragma unroll
-    for (int i = 0; i < BL; ++i)
+    for (int i = 0; i < BL; ++i) {
+        const int k4 = k4e ^ (((wave * BL + i) & 1) << 2);
         b_off[i] = (unsigned)(((n0 + (wave * BL + i) * 8 + lr) * p.Kpad + CE * k4) * (int)sizeof(T));
+    }
 
     const __amdgpu_buffer_rsrc_t rsrc_a =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.src), 0, (int)p.src_bytes, 0x00020000);
@@ -355,19 +389,48 @@ __global__ __launch_bounds__(kThreads, MINW) void gather_gemm_dma(const GatherPa
         __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.bt), 0, (int)p.bt_bytes, 0x00020000);
 
     auto issue = [&](int k0, f4* la, f4* lb) {
-        int kk = k0 + CE * k4;
-        unsigned tap, c, th, tw;
-        p.div_c.divmod((unsigned)kk, tap, c);
-        p.div_tw.divmod(tap, th, tw);
-        bool kvalid = kk < p.K;
-        int tap_off = ((int)th * p.Ws + (int)tw) * p.Cs + (int)c;
+        if (UT) {
+            // k0 is wave-uniform: this arithmetic runs on the scalar unit
+            unsigned tap, c0, th, tw;
+            p.div_c.divmod((unsigned)k0, tap, c0);
+            p.div_tw.divmod(tap, th, tw);
+            const unsigned tap_bytes = (unsigned)(((int)th * p.Ws + (int)tw) * p.Cs + (int)c0) * (unsigned)sizeof(T);
+#pragma unroll
+            for (int i = 0; i < AL; ++i) {
+                const unsigned bad = (a_inv[i] >> tap) & 1u;
+                const unsigned voff = (a_byte[i] + tap_bytes) | (bad << 31);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(la + (wave * AL + i) * 64), 16,
+                                                         (int)voff, 0, 0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < BL; ++i)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(lb + (wave * BL + i) * 64), 16,
+                                                         (int)(b_off[i] + (unsigned)k0 * (unsigned)sizeof(T)), 0, 0, 0);
+            return;
+        }
+        // tap decode for the two chunk columns a lane serves (even / odd 8-row blocks)
+        int tap_off[2], tap_h[2], tap_w[2];
+        bool kvalid[2];
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            int kk = k0 + CE * (k4e ^ (q << 2));
+            unsigned tap, c, th, tw;
+            p.div_c.divmod((unsigned)kk, tap, c);
+            p.div_tw.divmod(tap, th, tw);
+            kvalid[q] = kk < p.K;
+            tap_h[q] = (int)th;
+            tap_w[q] = (int)tw;
+            tap_off[q] = ((int)th * p.Ws + (int)tw) * p.Cs + (int)c;
+        }
 #pragma unroll
         for (int i = 0; i < AL; ++i) {
-            int r = (base_rc[i] >> 16) + (int)th;
-            int cc = ((int)((unsigned)base_rc[i] << 16) >> 16) + (int)tw;
+            const int q = i & 1;                    // AL is even: block parity = i & 1
+            int r = (base_rc[i] >> 16) + tap_h[q];
+            int cc = ((int)((unsigned)base_rc[i] << 16) >> 16) + tap_w[q];
             // bitwise, not short-circuit: keeps the slab issue free of branches
-            const unsigned bad = (unsigned)!(kvalid & ((unsigned)r < (unsigned)p.Hs) & ((unsigned)cc < (unsigned)p.Ws));
-            const unsigned voff = ((unsigned)(base_off[i] + tap_off) * (unsigned)sizeof(T)) | (bad << 31);
+            const unsigned bad =
+                (unsigned)!(kvalid[q] & ((unsigned)r < (unsigned)p.Hs) & ((unsigned)cc < (unsigned)p.Ws));
+            const unsigned voff = ((unsigned)(base_off[i] + tap_off[q]) * (unsigned)sizeof(T)) | (bad << 31);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(la + (wave * AL + i) * 64), 16, (int)voff, 0,
                                                      0, 0);
         }
@@ -385,7 +448,7 @@ __global__ __launch_bounds__(kThreads, MINW) void gather_gemm_dma(const GatherPa
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    const int sw7 = l32 & 7;                   // row & 7 of every operand row this lane reads
+    const int sw7 = (l32 >> 1) & 7;            // (row >> 1) & 7 of every operand row this lane reads
     f4 fa[2][TM], fb[2][TN];                   // operand fragments, double buffered across k groups
     auto read_frags = [&](const f4* la, const f4* lb, int g, int slot) {
         const int pc = (2 * g + lh) ^ sw7;
@@ -468,8 +531,11 @@ __global__ void pack_filter(const PackParams p) {
 template <typename T, int BM, int BN, int WM, int WN>
 static void launch_gather_cfg(const GatherParams& gp, bool vec, hipStream_t st) {
     dim3 grid(cdiv(gp.M, BM) * cdiv(gp.N, BN));
-    if (vec && gp.src_bytes != 0 && gp.bt_bytes != 0)
-        hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, 1>), grid, dim3(kThreads), 0, st, gp);
+    if (vec && gp.src_bytes != 0 && gp.bt_bytes != 0) {
+        const bool ut = gp.Cs % Elem<T>::BK == 0 && gp.K == gp.Kpad && gp.K / gp.Cs <= 32;
+        if (ut) hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true>), grid, dim3(kThreads), 0, st, gp);
+        else hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, false>), grid, dim3(kThreads), 0, st, gp);
+    }
     else if (vec)
         hipLaunchKernelGGL((gather_gemm<T, BM, BN, WM, WN, Elem<T>::CE>), grid, dim3(kThreads), 0, st, gp);
     else
@@ -895,8 +961,8 @@ __global__ __launch_bounds__(kThreads) void wgrad_gemm(const WgradParams p) {
 //   * rows unpadded (512 B / 256 B); odd slab rows store their 32-float halves
 //     swapped, so the two half-waves of an operand read (rows m and m+1) fall into
 //     different halves of the banks;
-//   * dbias for free: when it is wanted, row K of the A operand is set to 1 for
-//     every valid m, so row K of the product is sum_m dy[m][n];
+//   * dbias fused: the workgroups of k tile 0 also add up the columns of every dy
+//     slab they hold in LDS (8 reads + adds per thread per slab);
 //   * waves whose 32 k-rows lie entirely past the last row issue no MFMAs.
 // ------------------------------------------------------------------------------
 static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma(const WgradParams p) {
@@ -921,7 +987,8 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma(const WgradPar
     const int m_begin = split * p.m_per_split;
     int m_end = m_begin + p.m_per_split;
     if (m_end > p.M) m_end = p.M;
-    const int Kout = p.K + (p.want_dbias ? 1 : 0);      // row K carries dbias
+    const int Kout = p.K;
+    const bool do_db = p.want_dbias && (ktile == 0);
 
     // ---- A: one wave-level load = 2 slab rows x 32 chunks; 4 loads per wave ------
     const int a_row = lane >> 5;                         // row inside the 2-row block
@@ -938,9 +1005,6 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma(const WgradPar
         a_fy = (int)fy - p.pW;
         a_tap_off = (a_fx * p.W + a_fy) * p.C + (int)c;
     }
-    // the lane whose chunk contains row K plants the ones (after its own load landed)
-    const int one_k = p.K - kt0;                         // tile-local row of the ones
-    const bool plant = p.want_dbias && one_k >= 4 * a_lc && one_k < 4 * a_lc + 4;
     // ---- dy: one wave-level load = 4 slab rows x 16 chunks; 2 loads per wave -----
     const int y_row = lane >> 4;
     const int y_lc = (lane & 15) ^ ((y_row & 1) << 3);
@@ -977,14 +1041,13 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma(const WgradPar
                                                      0, 0);
         }
     };
-    auto plant_ones = [&](int mb, float* la) {
-        if (plant) {
+    // dbias: thread (column tid & 63, row group tid >> 6) adds 8 rows of each dy slab;
+    // odd rows keep their 32-float halves swapped
+    float dbsum = 0.f;
+    const int db_col = tid & 63, db_rg = tid >> 6;
+    auto add_columns = [&](const float* ly) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int ml = (wave * 4 + i) * 2 + a_row;
-                if (mb + ml < m_end) la[ml * kWgBK + (one_k ^ (a_row << 5))] = 1.0f;
-            }
-        }
+        for (int j = 0; j < 8; ++j) dbsum += ly[(db_rg * 8 + j) * kWgBN + (db_col ^ ((j & 1) << 5))];
     };
 
     f16v acc[2];
@@ -993,15 +1056,18 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma(const WgradPar
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
 
-    const bool active = kt0 + wave * 32 < Kout;          // wave-uniform
-    const int a_rd = ((wave * 32) ^ (lh << 5)) + l32;    // physical float of this lane's k, rows m = 2t + lh
+    // Which 32 k-rows this wave multiplies.  Rotated by the split index so that the
+    // idle row blocks of a partly filled last k tile do not always land on the same SIMDs.
+    const int kblk = (wave + split) & 3;
+    const bool active = kt0 + kblk * 32 < Kout;          // wave-uniform
+    const int a_rd = ((kblk * 32) ^ (lh << 5)) + l32;    // physical float of this lane's k, rows m = 2t + lh
     const int y_rd0 = l32 + (lh << 5);                   // logical n = l32
     const int y_rd1 = l32 + ((lh ^ 1) << 5);             // logical n = 32 + l32
     auto slab = [&](int mb, const float* la, const float* ly, float* na, float* ny, bool has_next) {
         __builtin_amdgcn_s_waitcnt(0);                   // this wave's loads of the slab have landed
-        plant_ones(mb, const_cast<float*>(la));
         __syncthreads();
         if (has_next) issue(mb + kWgBR, na, ny);
+        if (do_db) add_columns(ly);
         if (active) {
             float fa[2], fb0[2], fb1[2];
             fa[0] = la[lh * kWgBK + a_rd];
@@ -1035,9 +1101,16 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma(const WgradPar
         const int n = n0 + 32 * j + l32;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            const int k = kt0 + wave * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            const int k = kt0 + kblk * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
             if (k < Kout && n < p.D) outp[(size_t)k * p.D + n] = acc[j][v];
         }
+    }
+    if (do_db) {
+        __syncthreads();                                 // the slab buffers are free: reuse one for the 4 row groups
+        lds_y0[db_rg * 64 + db_col] = dbsum;
+        __syncthreads();
+        if (tid < 64 && n0 + tid < p.D)
+            outp[(size_t)p.K * p.D + n0 + tid] = (lds_y0[tid] + lds_y0[64 + tid]) + (lds_y0[128 + tid] + lds_y0[192 + tid]);
     }
 }
 
@@ -1094,9 +1167,7 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     const bool dma = sizeof(T) == 4 && va && vy && xb < ((int64_t)1 << 31) && yb < ((int64_t)1 << 31);
     p.x_bytes = dma ? (unsigned)xb : 0u;
     p.dy_bytes = dma ? (unsigned)yb : 0u;
-    // the LDS-direct kernel gets dbias from an extra row K of the product
-    const int krows = p.K + ((dma && dbias) ? 1 : 0);
-    const int kt = cdiv(krows, kWgBK), nt = cdiv(D, kWgBN);
+    const int kt = cdiv(p.K, kWgBK), nt = cdiv(D, kWgBN);
     const int slabs = cdiv(p.M, kWgBR);
     // about two rounds of resident workgroups (3 per CU for the LDS-direct kernel)
     int splits = cdiv((dma ? 6 : 4) * c.prop.multiProcessorCount, kt * nt);
