@@ -953,23 +953,220 @@ __global__ __launch_bounds__(kThreads) void wgrad_gemm(const WgradParams p) {
 }
 
 // ------------------------------------------------------------------------------
-// wgrad, LDS-direct variant (fp32, C and D multiples of 4).  Same 128 (k) x 64 (n)
-// tile and split over M as wgrad_gemm, with:
+// wgrad, LDS-direct variant (fp32, C and D multiples of 4).  Output tile
+// (128*WKB) k x 64 n per workgroup, each wave owns WKB blocks of 32 k-rows x 64 n;
+// the M range of a split is walked in slabs of 32/WKB rows:
 //   * x and dy slabs loaded straight into LDS (`buffer_load_dwordx4 ... lds`), two
-//     buffers, one barrier per 32-row slab, operand reads of step t+1 issued before
-//     the MFMAs of step t;
-//   * rows unpadded (512 B / 256 B); odd slab rows store their 32-float halves
-//     swapped, so the two half-waves of an operand read (rows m and m+1) fall into
-//     different halves of the banks;
+//     buffers, one barrier per slab, operand reads of step t+1 issued before the
+//     MFMAs of step t;
+//   * slab rows are unpadded; odd rows store the 32-float halves of every 64-float
+//     group swapped, so the two half-waves of an operand read (rows m and m+1) fall
+//     into different halves of the 64 banks;
+//   * WKB = 2 moves half the bytes per flop through L2 and LDS and issues one LDS
+//     read per MFMA instead of 1.5; it is used when K fills at least one 256-row tile;
 //   * dbias fused: the workgroups of k tile 0 also add up the columns of every dy
-//     slab they hold in LDS (8 reads + adds per thread per slab);
-//   * waves whose 32 k-rows lie entirely past the last row issue no MFMAs.
+//     slab they hold in LDS;
+//   * wave blocks whose 32 k-rows lie entirely past K issue no MFMAs; which wave
+//     gets which block rotates with the split index.
 // ------------------------------------------------------------------------------
+template <int WKB>
 static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma(const WgradParams p) {
-    __shared__ float lds_a0[kWgBR * kWgBK];
-    __shared__ float lds_a1[kWgBR * kWgBK];
-    __shared__ float lds_y0[kWgBR * kWgBN];
-    __shared__ float lds_y1[kWgBR * kWgBN];
+    constexpr int TK = kWgBK * WKB;          // k rows per workgroup tile
+    constexpr int BR = kWgBR / WKB;          // m rows per slab
+    constexpr int RPL = 256 / TK;            // A rows per wave-level load (1024 B): 2 or 1
+    constexpr int CPR = TK / 4;              // chunks per A row
+    constexpr int YL = BR / 16;              // dy loads per wave per slab (4 rows each)
+    __shared__ float lds_a0[BR * TK];
+    __shared__ float lds_a1[BR * TK];
+    __shared__ float lds_y0[kWgBR * kWgBN];  // BR rows used; sized for the dbias epilogue too
+    __shared__ float lds_y1[BR * kWgBN];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int l32 = lane & 31;
+    const int lh = lane >> 5;
+
+    const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
+    const int tiles = p.kt * p.nt;
+    const int split = lid / tiles;
+    const int tile = lid - split * tiles;
+    const int ktile = tile % p.kt;
+    const int kt0 = ktile * TK;
+    const int n0 = (tile / p.kt) * kWgBN;
+    const int m_begin = split * p.m_per_split;
+    int m_end = m_begin + p.m_per_split;
+    if (m_end > p.M) m_end = p.M;
+    const bool do_db = p.want_dbias && (ktile == 0);
+
+    // ---- A: a wave-level load covers RPL slab rows; 4 loads per wave per slab --------
+    const int a_row = lane / CPR;                        // row inside the load block (0 when RPL == 1)
+    const int a_pc = lane % CPR;                         // chunk position written by this lane
+    int a_tap_off[2], a_fx[2], a_fy[2];                  // tap of the chunk fetched for even / odd slab rows
+    bool a_kok[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        int kk = kt0 + 4 * (a_pc ^ (q << 3));
+        unsigned tap, c, fx, fy;
+        p.div_c.divmod((unsigned)kk, tap, c);
+        p.div_fw.divmod(tap, fx, fy);
+        a_kok[q] = kk < p.K;
+        a_fx[q] = (int)fx - p.pH;
+        a_fy[q] = (int)fy - p.pW;
+        a_tap_off[q] = (a_fx[q] * p.W + a_fy[q]) * p.C + (int)c;
+    }
+    // ---- dy: one wave-level load = 4 slab rows x 16 chunks ---------------------------
+    const int y_row = lane >> 4;
+    const int y_lc = (lane & 15) ^ ((y_row & 1) << 3);
+    const int y_n = n0 + 4 * y_lc;
+    const bool y_nok = y_n < p.D;
+
+    const __amdgpu_buffer_rsrc_t rsrc_x =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.x), 0, (int)p.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_y =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.dy), 0, (int)p.dy_bytes, 0x00020000);
+
+    auto issue = [&](int mb, float* la, float* ly) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int ml = (wave * 4 + i) * RPL + a_row;
+            const int q = RPL == 2 ? a_row : (i & 1);    // row parity
+            const int m = mb + ml;
+            unsigned s, rem, ho, wo;
+            p.div_howo.divmod((unsigned)m, s, rem);
+            p.div_wo.divmod(rem, ho, wo);
+            const int r0 = (int)ho * p.sH, c0 = (int)wo * p.sW;
+            const int pix = (((int)s * p.H + r0) * p.W + c0) * p.C;
+            const unsigned bad = (unsigned)!((m < m_end) & a_kok[q] & ((unsigned)(r0 + a_fx[q]) < (unsigned)p.H) &
+                                             ((unsigned)(c0 + a_fy[q]) < (unsigned)p.W));
+            const unsigned voff = ((unsigned)(pix + a_tap_off[q]) * 4u) | (bad << 31);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + (wave * 4 + i) * 256), 16, (int)voff, 0,
+                                                     0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < YL; ++i) {
+            const int m = mb + (wave * YL + i) * 4 + y_row;
+            const unsigned bad = (unsigned)!((m < m_end) & y_nok);
+            const unsigned voff = ((unsigned)(m * p.D + y_n) * 4u) | (bad << 31);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_y, (lds_ptr_t)(ly + (wave * YL + i) * 256), 16, (int)voff,
+                                                     0, 0, 0);
+        }
+    };
+
+    // dbias: thread (column tid & 63, row group tid >> 6) adds BR/4 rows of each dy slab;
+    // odd rows keep their 32-float halves swapped
+    float dbsum = 0.f;
+    const int db_col = tid & 63, db_rg = tid >> 6;
+    auto add_columns = [&](const float* ly) {
+#pragma unroll
+        for (int j = 0; j < BR / 4; ++j) dbsum += ly[(db_rg * (BR / 4) + j) * kWgBN + (db_col ^ ((j & 1) << 5))];
+    };
+
+    f16v acc[WKB][2];
+#pragma unroll
+    for (int b = 0; b < WKB; ++b)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[b][j][v] = 0.f;
+
+    // Which k-row blocks this wave multiplies.  Rotated by the split index so that the
+    // idle blocks of a partly filled last k tile do not always land on the same SIMDs.
+    const int wv = (wave + split) & 3;
+    bool active[WKB];
+    int a_rd[WKB];                                       // physical float of this lane's k, rows m = 2t + lh
+#pragma unroll
+    for (int b = 0; b < WKB; ++b) {
+        const int kblk = wv * WKB + b;
+        active[b] = kt0 + kblk * 32 < p.K;               // wave-uniform
+        a_rd[b] = ((kblk * 32) ^ (lh << 5)) + l32;
+    }
+    const int y_rd0 = l32 + (lh << 5);                   // logical n = l32
+    const int y_rd1 = l32 + ((lh ^ 1) << 5);             // logical n = 32 + l32
+    auto slab = [&](int mb, const float* la, const float* ly, float* na, float* ny, bool has_next) {
+        __builtin_amdgcn_s_waitcnt(0);                   // this wave's loads of the slab have landed
+        __syncthreads();
+        if (has_next) issue(mb + BR, na, ny);
+        if (do_db) add_columns(ly);
+        if (active[0]) {
+            float fa[2][WKB], fb0[2], fb1[2];
+#pragma unroll
+            for (int b = 0; b < WKB; ++b) fa[0][b] = la[lh * TK + a_rd[b]];
+            fb0[0] = ly[lh * kWgBN + y_rd0];
+            fb1[0] = ly[lh * kWgBN + y_rd1];
+#pragma unroll
+            for (int t = 0; t < BR / 2; ++t) {
+                if (t + 1 < BR / 2) {
+#pragma unroll
+                    for (int b = 0; b < WKB; ++b) fa[(t + 1) & 1][b] = la[(2 * t + 2 + lh) * TK + a_rd[b]];
+                    fb0[(t + 1) & 1] = ly[(2 * t + 2 + lh) * kWgBN + y_rd0];
+                    fb1[(t + 1) & 1] = ly[(2 * t + 2 + lh) * kWgBN + y_rd1];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int b = 0; b < WKB; ++b) {
+                    if (b == 0 || active[b]) {
+                        acc[b][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[t & 1][b], fb0[t & 1], acc[b][0], 0, 0, 0);
+                        acc[b][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[t & 1][b], fb1[t & 1], acc[b][1], 0, 0, 0);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+
+    if (m_begin < m_end) issue(m_begin, lds_a0, lds_y0);
+    for (int mb = m_begin; mb < m_end; mb += 2 * BR) {
+        slab(mb, lds_a0, lds_y0, lds_a1, lds_y1, mb + BR < m_end);
+        if (mb + BR < m_end) slab(mb + BR, lds_a1, lds_y1, lds_a0, lds_y0, mb + 2 * BR < m_end);
+    }
+
+    const size_t split_stride = (size_t)p.K * p.D + p.D;
+    float* outp = p.out + (size_t)split * split_stride;
+#pragma unroll
+    for (int b = 0; b < WKB; ++b)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int n = n0 + 32 * j + l32;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int k = kt0 + (wv * WKB + b) * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+                if (k < p.K && n < p.D) outp[(size_t)k * p.D + n] = acc[b][j][v];
+            }
+        }
+    if (do_db) {
+        __syncthreads();                                 // the slab buffers are free: reuse one for the 4 row groups
+        lds_y0[db_rg * 64 + db_col] = dbsum;
+        __syncthreads();
+        if (tid < 64 && n0 + tid < p.D)
+            outp[(size_t)p.K * p.D + n0 + tid] = (lds_y0[tid] + lds_y0[64 + tid]) + (lds_y0[128 + tid] + lds_y0[192 + tid]);
+    }
+}
+
+// ------------------------------------------------------------------------------
+// wgrad for bf16 inputs on v_mfma_f32_32x32x16_bf16 (C and D multiples of 8).
+// The MFMA reduces over m, so each lane needs 8 consecutive m of ONE k (or n)
+// column, while the slabs arrive m-major ([m][k], k contiguous) straight from
+// memory.  `ds_read_b64_tr_b16` does the transposition inside LDS reads: in every
+// group of 16 lanes, lane j supplies the address of 4 consecutive elements of row
+// j/4 and lane i receives element i%4 of the rows 4r + i/4, r = 0..3 -- i.e. four
+// consecutive m of column i.  Two such reads give one MFMA operand.
+//   tile 128 k x 64 n per workgroup, wave = 32 k x 64 n, slab = 64 rows of m,
+//   two LDS buffers filled by `buffer_load_dwordx4 ... lds`, one barrier per slab.
+//   Rows are unpadded (x: 256 B, dy: 128 B); 16-byte chunk c of row m is stored at
+//   c ^ ((m & 3) << 1) for x and c ^ (((m >> 1) & 1) << 2) for dy, which spreads the
+//   4 rows x 32 B touched by a 16-lane group (and its neighbour group) over all banks.
+// ------------------------------------------------------------------------------
+typedef short s4v __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) s4v* lds_s4_ptr_t;
+
+static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma_bf16(const WgradParams p) {
+    constexpr int BR = 64;                               // m rows per slab
+    __shared__ uint16_t lds_a0[BR * kWgBK];
+    __shared__ uint16_t lds_a1[BR * kWgBK];
+    __shared__ uint16_t lds_y0[BR * kWgBN];
+    __shared__ uint16_t lds_y1[BR * kWgBN];
+    __shared__ float lds_db[4 * 64];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -987,16 +1184,15 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma(const WgradPar
     const int m_begin = split * p.m_per_split;
     int m_end = m_begin + p.m_per_split;
     if (m_end > p.M) m_end = p.M;
-    const int Kout = p.K;
     const bool do_db = p.want_dbias && (ktile == 0);
 
-    // ---- A: one wave-level load = 2 slab rows x 32 chunks; 4 loads per wave ------
-    const int a_row = lane >> 5;                         // row inside the 2-row block
-    const int a_lc = (lane & 31) ^ (a_row << 3);         // logical chunk fetched (odd rows: halves swapped)
+    // ---- x: one wave-level load = 4 slab rows x 16 chunks (8 bf16 each); 4 per wave ---
+    const int a_row = lane >> 4;
+    const int a_lc = (lane & 15) ^ ((a_row & 3) << 1);   // logical chunk fetched
     int a_tap_off, a_fx, a_fy;
     bool a_kok;
     {
-        int kk = kt0 + 4 * a_lc;
+        int kk = kt0 + 8 * a_lc;
         unsigned tap, c, fx, fy;
         p.div_c.divmod((unsigned)kk, tap, c);
         p.div_fw.divmod(tap, fx, fy);
@@ -1005,10 +1201,10 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma(const WgradPar
         a_fy = (int)fy - p.pW;
         a_tap_off = (a_fx * p.W + a_fy) * p.C + (int)c;
     }
-    // ---- dy: one wave-level load = 4 slab rows x 16 chunks; 2 loads per wave -----
-    const int y_row = lane >> 4;
-    const int y_lc = (lane & 15) ^ ((y_row & 1) << 3);
-    const int y_n = n0 + 4 * y_lc;
+    // ---- dy: one wave-level load = 8 slab rows x 8 chunks; 2 per wave -----------------
+    const int y_row = lane >> 3;
+    const int y_lc = (lane & 7) ^ (((y_row >> 1) & 1) << 2);
+    const int y_n = n0 + 8 * y_lc;
     const bool y_nok = y_n < p.D;
 
     const __amdgpu_buffer_rsrc_t rsrc_x =
@@ -1016,11 +1212,10 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma(const WgradPar
     const __amdgpu_buffer_rsrc_t rsrc_y =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.dy), 0, (int)p.dy_bytes, 0x00020000);
 
-    auto issue = [&](int mb, float* la, float* ly) {
+    auto issue = [&](int mb, uint16_t* la, uint16_t* ly) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int ml = (wave * 4 + i) * 2 + a_row;
-            const int m = mb + ml;
+            const int m = mb + (wave * 4 + i) * 4 + a_row;
             unsigned s, rem, ho, wo;
             p.div_howo.divmod((unsigned)m, s, rem);
             p.div_wo.divmod(rem, ho, wo);
@@ -1028,89 +1223,102 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma(const WgradPar
             const int pix = (((int)s * p.H + r0) * p.W + c0) * p.C;
             const unsigned bad = (unsigned)!((m < m_end) & a_kok & ((unsigned)(r0 + a_fx) < (unsigned)p.H) &
                                              ((unsigned)(c0 + a_fy) < (unsigned)p.W));
-            const unsigned voff = ((unsigned)(pix + a_tap_off) * 4u) | (bad << 31);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + (wave * 4 + i) * 256), 16, (int)voff, 0,
+            const unsigned voff = ((unsigned)(pix + a_tap_off) * 2u) | (bad << 31);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + (wave * 4 + i) * 512), 16, (int)voff, 0,
                                                      0, 0);
         }
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const int m = mb + (wave * 2 + i) * 4 + y_row;
+            const int m = mb + (wave * 2 + i) * 8 + y_row;
             const unsigned bad = (unsigned)!((m < m_end) & y_nok);
-            const unsigned voff = ((unsigned)(m * p.D + y_n) * 4u) | (bad << 31);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_y, (lds_ptr_t)(ly + (wave * 2 + i) * 256), 16, (int)voff, 0,
+            const unsigned voff = ((unsigned)(m * p.D + y_n) * 2u) | (bad << 31);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_y, (lds_ptr_t)(ly + (wave * 2 + i) * 512), 16, (int)voff, 0,
                                                      0, 0);
         }
     };
-    // dbias: thread (column tid & 63, row group tid >> 6) adds 8 rows of each dy slab;
-    // odd rows keep their 32-float halves swapped
-    float dbsum = 0.f;
-    const int db_col = tid & 63, db_rg = tid >> 6;
-    auto add_columns = [&](const float* ly) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) dbsum += ly[(db_rg * 8 + j) * kWgBN + (db_col ^ ((j & 1) << 5))];
+
+    // ---- transposing operand reads -------------------------------------------------------
+    // 16-lane group G: columns 16*(G&1).., rows 8*(G>>1)..; lane j of the group points at
+    // row j>>2, elements 4*(j&3)..+3.
+    const int G = lane >> 4, j16 = lane & 15;
+    const int t_row = 8 * (G >> 1) + (j16 >> 2);         // row inside a 16-row step, first read (+4: second)
+    const int a_col = wave * 32 + 16 * (G & 1) + 4 * (j16 & 3);      // first k element addressed
+    const int y_col = 16 * (G & 1) + 4 * (j16 & 3);                  // first n element (n tile 0; +32: tile 1)
+    // element offsets (in bf16) inside a slab row, swizzle applied; row & 3 == j16 >> 2, (row >> 1) & 1 == j16 >> 3
+    const int a_eo = (((a_col >> 3) ^ ((j16 >> 2) << 1)) << 3) + (a_col & 4);
+    const int y_eo0 = (((y_col >> 3) ^ ((j16 >> 3) << 2)) << 3) + (y_col & 4);
+    const int y_eo1 = ((((y_col + 32) >> 3) ^ ((j16 >> 3) << 2)) << 3) + (y_col & 4);
+    auto tr = [&](const uint16_t* base) {
+        return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr_t)base);
     };
 
     f16v acc[2];
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int jn = 0; jn < 2; ++jn)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+        for (int v = 0; v < 16; ++v) acc[jn][v] = 0.f;
+    const bool active = kt0 + wave * 32 < p.K;           // wave-uniform
 
-    // Which 32 k-rows this wave multiplies.  Rotated by the split index so that the
-    // idle row blocks of a partly filled last k tile do not always land on the same SIMDs.
-    const int kblk = (wave + split) & 3;
-    const bool active = kt0 + kblk * 32 < Kout;          // wave-uniform
-    const int a_rd = ((kblk * 32) ^ (lh << 5)) + l32;    // physical float of this lane's k, rows m = 2t + lh
-    const int y_rd0 = l32 + (lh << 5);                   // logical n = l32
-    const int y_rd1 = l32 + ((lh ^ 1) << 5);             // logical n = 32 + l32
-    auto slab = [&](int mb, const float* la, const float* ly, float* na, float* ny, bool has_next) {
+    float dbsum = 0.f;
+    const int db_col = tid & 63, db_rg = tid >> 6;       // 4 row groups of 16 rows
+    auto add_columns = [&](const uint16_t* ly) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = db_rg * 16 + r;
+            const int e = (((db_col >> 3) ^ (((row >> 1) & 1) << 2)) << 3) + (db_col & 7);
+            dbsum += __uint_as_float((unsigned)ly[row * kWgBN + e] << 16);
+        }
+    };
+
+    auto slab = [&](int mb, const uint16_t* la, const uint16_t* ly, uint16_t* na, uint16_t* ny, bool has_next) {
         __builtin_amdgcn_s_waitcnt(0);                   // this wave's loads of the slab have landed
         __syncthreads();
-        if (has_next) issue(mb + kWgBR, na, ny);
+        if (has_next) issue(mb + BR, na, ny);
         if (do_db) add_columns(ly);
         if (active) {
-            float fa[2], fb0[2], fb1[2];
-            fa[0] = la[lh * kWgBK + a_rd];
-            fb0[0] = ly[lh * kWgBN + y_rd0];
-            fb1[0] = ly[lh * kWgBN + y_rd1];
 #pragma unroll
-            for (int t = 0; t < kWgBR / 2; ++t) {
-                if (t + 1 < kWgBR / 2) {
-                    fa[(t + 1) & 1] = la[(2 * t + 2 + lh) * kWgBK + a_rd];
-                    fb0[(t + 1) & 1] = ly[(2 * t + 2 + lh) * kWgBN + y_rd0];
-                    fb1[(t + 1) & 1] = ly[(2 * t + 2 + lh) * kWgBN + y_rd1];
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[t & 1], fb0[t & 1], acc[0], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[t & 1], fb1[t & 1], acc[1], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
+            for (int st = 0; st < BR / 16; ++st) {
+                const int r0 = st * 16 + t_row;
+                s4v a0 = tr(la + r0 * kWgBK + a_eo);
+                s4v a1 = tr(la + (r0 + 4) * kWgBK + a_eo);
+                s4v b00 = tr(ly + r0 * kWgBN + y_eo0);
+                s4v b01 = tr(ly + (r0 + 4) * kWgBN + y_eo0);
+                s4v b10 = tr(ly + r0 * kWgBN + y_eo1);
+                s4v b11 = tr(ly + (r0 + 4) * kWgBN + y_eo1);
+                typedef short s8v __attribute__((ext_vector_type(8)));
+                const s8v av = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+                const s8v bv0 = __builtin_shufflevector(b00, b01, 0, 1, 2, 3, 4, 5, 6, 7);
+                const s8v bv1 = __builtin_shufflevector(b10, b11, 0, 1, 2, 3, 4, 5, 6, 7);
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av),
+                                                                 __builtin_bit_cast(bf16x8, bv0), acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av),
+                                                                 __builtin_bit_cast(bf16x8, bv1), acc[1], 0, 0, 0);
             }
         }
     };
 
     if (m_begin < m_end) issue(m_begin, lds_a0, lds_y0);
-    for (int mb = m_begin; mb < m_end; mb += 2 * kWgBR) {
-        slab(mb, lds_a0, lds_y0, lds_a1, lds_y1, mb + kWgBR < m_end);
-        if (mb + kWgBR < m_end) slab(mb + kWgBR, lds_a1, lds_y1, lds_a0, lds_y0, mb + 2 * kWgBR < m_end);
+    for (int mb = m_begin; mb < m_end; mb += 2 * BR) {
+        slab(mb, lds_a0, lds_y0, lds_a1, lds_y1, mb + BR < m_end);
+        if (mb + BR < m_end) slab(mb + BR, lds_a1, lds_y1, lds_a0, lds_y0, mb + 2 * BR < m_end);
     }
 
     const size_t split_stride = (size_t)p.K * p.D + p.D;
     float* outp = p.out + (size_t)split * split_stride;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int n = n0 + 32 * j + l32;
+    for (int jn = 0; jn < 2; ++jn) {
+        const int n = n0 + 32 * jn + l32;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            const int k = kt0 + kblk * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-            if (k < Kout && n < p.D) outp[(size_t)k * p.D + n] = acc[j][v];
+            const int k = kt0 + wave * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            if (k < p.K && n < p.D) outp[(size_t)k * p.D + n] = acc[jn][v];
         }
     }
     if (do_db) {
-        __syncthreads();                                 // the slab buffers are free: reuse one for the 4 row groups
-        lds_y0[db_rg * 64 + db_col] = dbsum;
+        lds_db[db_rg * 64 + db_col] = dbsum;
         __syncthreads();
         if (tid < 64 && n0 + tid < p.D)
-            outp[(size_t)p.K * p.D + n0 + tid] = (lds_y0[tid] + lds_y0[64 + tid]) + (lds_y0[128 + tid] + lds_y0[192 + tid]);
+            outp[(size_t)p.K * p.D + n0 + tid] = (lds_db[tid] + lds_db[64 + tid]) + (lds_db[128 + tid] + lds_db[192 + tid]);
     }
 }
 
@@ -1164,18 +1372,33 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     constexpr int CE = Elem<T>::CE;
     const bool va = (C % CE == 0), vy = (D % CE == 0);
     const int64_t xb = (int64_t)S * H * W * C * (int64_t)sizeof(T), yb = (int64_t)p.M * D * (int64_t)sizeof(T);
-    const bool dma = sizeof(T) == 4 && va && vy && xb < ((int64_t)1 << 31) && yb < ((int64_t)1 << 31);
-    p.x_bytes = dma ? (unsigned)xb : 0u;
-    p.dy_bytes = dma ? (unsigned)yb : 0u;
-    const int kt = cdiv(p.K, kWgBK), nt = cdiv(D, kWgBN);
-    const int slabs = cdiv(p.M, kWgBR);
+    const bool fits = xb < ((int64_t)1 << 31) && yb < ((int64_t)1 << 31);
+    const bool dma = sizeof(T) == 4 && va && vy && fits;
+    const bool dma16 = sizeof(T) == 2 && va && vy && fits;      // bf16 MFMA kernel, 64-row slabs
+    p.x_bytes = (dma || dma16) ? (unsigned)xb : 0u;
+    p.dy_bytes = (dma || dma16) ? (unsigned)yb : 0u;
+    // 256-row k tiles (two row blocks per wave) move half the bytes per flop, but a
+    // partly filled last tile leaves whole workgroups nearly idle: use them only when
+    // K fills its 256-row tiles to 94 % or more (measured: K = 576 is 23 % slower).
+    int wkb_used = 1;
+    if (dma) {
+        const int t256 = cdiv(p.K, 2 * kWgBK);
+        if ((int64_t)p.K * 100 >= (int64_t)t256 * 2 * kWgBK * 94) wkb_used = 2;
+        if (const char* f = getenv("AETHER_WGRAD_WKB")) {     // tuning override: 1 or 2
+            const int v = atoi(f);
+            if (v == 1 || v == 2) wkb_used = v;
+        }
+    }
+    const int kt = cdiv(p.K, kWgBK * wkb_used), nt = cdiv(D, kWgBN);
+    const int slab_rows = dma16 ? 64 : kWgBR;
+    const int slabs = cdiv(p.M, slab_rows);           // fp32: counted in 32-row units for both tile shapes
     // about two rounds of resident workgroups (3 per CU for the LDS-direct kernel)
-    int splits = cdiv((dma ? 6 : 4) * c.prop.multiProcessorCount, kt * nt);
+    int splits = cdiv(((dma || dma16) ? 6 : 4) * c.prop.multiProcessorCount, kt * nt);
     if (splits > slabs) splits = slabs;
     if (splits < 1) splits = 1;
     int slabs_per = cdiv(slabs, splits);
     splits = cdiv(slabs, slabs_per);
-    p.m_per_split = slabs_per * kWgBR;
+    p.m_per_split = slabs_per * slab_rows;
     const int64_t kd = (int64_t)p.K * D;
     void* ws;
     rc = workspace((int64_t)splits * (kd + D) * sizeof(float), &ws);
@@ -1183,7 +1406,9 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     p.out = (float*)ws;
     p.kt = kt; p.nt = nt;
     dim3 grid(kt * nt * splits);
-    if (dma) hipLaunchKernelGGL(wgrad_gemm_dma, grid, dim3(kThreads), 0, c.stream, p);
+    if (dma16) hipLaunchKernelGGL(wgrad_gemm_dma_bf16, grid, dim3(kThreads), 0, c.stream, p);
+    else if (dma && wkb_used == 2) hipLaunchKernelGGL(wgrad_gemm_dma<2>, grid, dim3(kThreads), 0, c.stream, p);
+    else if (dma) hipLaunchKernelGGL(wgrad_gemm_dma<1>, grid, dim3(kThreads), 0, c.stream, p);
     else if (va && vy) hipLaunchKernelGGL((wgrad_gemm<T, CE, CE>), grid, dim3(kThreads), 0, c.stream, p);
     else if (va) hipLaunchKernelGGL((wgrad_gemm<T, CE, 1>), grid, dim3(kThreads), 0, c.stream, p);
     else if (vy) hipLaunchKernelGGL((wgrad_gemm<T, 1, CE>), grid, dim3(kThreads), 0, c.stream, p);
