@@ -156,15 +156,22 @@ def main():
         per[name] = {"ms": ms, "tflops": fl / (ms * 1e-3) / 1e12,
                      "frac_fp32_mfma_peak": fl / (ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS}
     slowest = max(per, key=lambda k: per[k]["ms"])
+    # HBM/fabric bytes per launch of the two big kernels, from the FETCH_SIZE / WRITE_SIZE
+    # counter runs summarised in profiles/conv_f32_resnet3x3_256x56x56x64.md (FETCH_SIZE scaled
+    # by 2.0 and WRITE_SIZE by 1.0 against the copy probe); algorithmic bytes are 411.2 MB.
+    measured_traffic = {"gather_gemm_dma": 208.4e6 + 205.5e6, "wgrad_gemm_dma": 479.8e6 + 45.2e6}
+    kernel = {"fprop": "gather_gemm_dma", "dgrad": "gather_gemm_dma", "wgrad": "wgrad_gemm_dma"}[slowest]
     roofline = {
         "bound": "mfma",
-        "kernel": {"fprop": "gather_gemm_f32", "dgrad": "gather_gemm_f32", "wgrad": "wgrad_gemm_f32"}[slowest],
+        "kernel": kernel,
         "direction": slowest,
         "achieved": per[slowest]["tflops"],
         "peak": FP32_MFMA_PEAK_TFLOPS,
         "unit": "TFLOP/s",
         "frac": per[slowest]["tflops"] / FP32_MFMA_PEAK_TFLOPS,
-        "traffic": None,
+        "traffic": measured_traffic[kernel],
+        "algorithmic_flops_per_launch": fl,
+        "algorithmic_bytes_per_launch": 4.0 * (2 * S * H * W * C + 9 * C * D + D),
     }
 
     extra = {"per_direction_fp32": per, "wall_ms_per_step": wall_ms,
