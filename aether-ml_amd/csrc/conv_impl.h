@@ -22,6 +22,7 @@
 //   bf16: a chunk is exactly the 8 k-values one lane supplies to
 //   v_mfma_f32_32x32x16_bf16.
 #pragma once
+#include <type_traits>
 
 #include "common.h"
 
@@ -85,6 +86,7 @@ struct GatherParams {
     int dense_out;       // 1: row m is stored at out + m*N
     unsigned src_bytes;  // extent of src / bt for the buffer descriptors (0: too large, not used)
     unsigned bt_bytes;
+    unsigned out_bytes;  // extent of out; 0: no 16-byte stores (too large, N not a multiple of 4, or unaligned)
     FastDiv div_hw, div_w, div_c, div_tw;
 };
 
@@ -102,38 +104,84 @@ __device__ __forceinline__ int xcd_contiguous_id(int wg, int total) {
     return xcd * per + (xcd < rem ? xcd : rem) + idx;
 }
 
-// Bias add and store of a wave's TM x TN accumulator tiles.  acc[i][j][v] holds row
-// 32*i + 8*(v/4) + 4*(lane/32) + v%4, column 32*j + lane%32 of the wave tile.
+// The MFMAs are issued with the operands swapped (filter rows as A, gathered pixels
+// as B), so the accumulators hold the TRANSPOSED output tile:
+//   acc[i][j][v] = out[m = mw0 + 32 i + lane%32][n = nw0 + 32 j + 8 (v/4) + 4 (lane/32) + v%4]
+// A lane owns one output row per tile and 4 consecutive channels per v/4: the tile
+// goes out in 16-byte stores whose addresses differ by compile-time constants, with
+// one row decode per lane.  fp32 MFMA and ordinary vector instructions compete for
+// the same issue cycles, so an epilogue of 32 scalar stores with per-element address
+// arithmetic costs measurable matrix time (9 % on the 56x56x64 layer).
+// The bias is added by starting the accumulators from it.
+template <int TM, int TN>
+__device__ __forceinline__ void init_acc(const GatherParams& p, f16v (&acc)[TM][TN], int nw0, int lh) {
+    const bool vec = p.out_bytes != 0 && (reinterpret_cast<uintptr_t>(p.bias) & 15) == 0;
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int n = nw0 + 32 * j + 8 * q + 4 * lh;
+            f4 bv = {0.f, 0.f, 0.f, 0.f};
+            if (p.bias != nullptr) {
+                if (vec) {
+                    if (n < p.N) bv = *reinterpret_cast<const f4*>(p.bias + n);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (n + e < p.N) bv[e] = p.bias[n + e];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = bv[e];
+        }
+}
+
 template <int TM, int TN>
 __device__ __forceinline__ void store_tile(const GatherParams& p, const f16v (&acc)[TM][TN], int mw0, int nw0,
                                            int l32, int lh) {
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    const bool full_n = nw0 + 32 * TN <= p.N;           // wave-uniform
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(p.out, 0, (int)p.out_bytes, 0x00020000);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int n = nw0 + 32 * j + l32;
-        const bool nok = n < p.N;
-        const float bv = (p.bias != nullptr && nok) ? p.bias[n] : 0.f;
+    for (int i = 0; i < TM; ++i) {
+        const int m = mw0 + 32 * i + l32;
+        const bool mok = m < p.M;
+        unsigned row = (unsigned)m;
+        if (!p.dense_out) {
+            unsigned s, rem, ii, jj;
+            p.div_hw.divmod(mok ? (unsigned)m : 0u, s, rem);
+            p.div_w.divmod(rem, ii, jj);
+            row = ((unsigned)s * p.Hof + p.oh0 + ii * p.ohs) * p.Wof + p.ow0 + jj * p.ows;
+        }
+        const unsigned elem = row * (unsigned)p.N + (unsigned)(nw0 + 4 * lh);   // < 2^31: checked by the host
+        if (p.out_bytes != 0) {
+            // rows past M (and, in edge tiles, channels past N) get a byte offset beyond
+            // the descriptor's extent: the hardware drops the store
+            const unsigned base = (elem * 4u) | ((unsigned)!mok << 31);
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int m = mw0 + 32 * i + 8 * (v >> 2) + 4 * lh + (v & 3);
-                if (nok && m < p.M) {
-                    size_t row;
-                    if (p.dense_out) {
-                        row = (size_t)m;
-                    } else {
-                        unsigned s, rem, ii, jj;
-                        p.div_hw.divmod((unsigned)m, s, rem);
-                        p.div_w.divmod(rem, ii, jj);
-                        row = ((size_t)s * p.Hof + p.oh0 + (size_t)ii * p.ohs) * p.Wof + p.ow0 + (size_t)jj * p.ows;
-                    }
-                    p.out[row * p.N + n] = acc[i][j][v] + bv;
+                for (int q = 0; q < 4; ++q) {
+                    const f4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                    unsigned off = base;
+                    if (!full_n) off |= (unsigned)!(nw0 + 32 * j + 8 * q + 4 * lh < p.N) << 31;
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, v), rsrc, (int)off,
+                                                           (32 * j + 8 * q) * 4, 0);
                 }
-            }
+        } else if (mok) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int n = nw0 + 32 * j + 8 * (v >> 2) + 4 * lh + (v & 3);
+                    if (n < p.N) p.out[(size_t)row * p.N + n] = acc[i][j][v];
+                }
         }
     }
 }
-
 
 template <typename T, int BM, int BN, int WM, int WN, int VEC>
 __global__ __launch_bounds__(kThreads, 3) void gather_gemm(const GatherParams p) {
@@ -242,12 +290,7 @@ __global__ __launch_bounds__(kThreads, 3) void gather_gemm(const GatherParams p)
     };
 
     f16v acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    init_acc<TM, TN>(p, acc, n0 + wn0, lh);
 
     if (p.Kpad > 0) {
         load_slab(0);
@@ -269,7 +312,7 @@ __global__ __launch_bounds__(kThreads, 3) void gather_gemm(const GatherParams p)
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) mma_chunk<T>(a[i], b[j], acc[i][j]);
+                for (int j = 0; j < TN; ++j) mma_chunk<T>(b[j], a[i], acc[i][j]);
         }
         __syncthreads();
         if (more) {
@@ -388,29 +431,23 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
     const __amdgpu_buffer_rsrc_t rsrc_b =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.bt), 0, (int)p.bt_bytes, 0x00020000);
 
-    auto issue = [&](int k0, f4* la, f4* lb) {
+    // The loads of a slab are issued in parts between the MFMA groups of the slab
+    // before it: a burst of AL + BL loads right after the barrier keeps the wave away
+    // from the matrix pipe for the time the memory pipeline takes to accept them.
+    // `prep` decodes the slab's tap(s) once, `issue_part(j)` issues load j of the
+    // wave (j < AL: 8 rows of A, else 8 rows of B).
+    unsigned ut_tap = 0, ut_tap_bytes = 0;              // UT: wave-uniform, scalar registers
+    int tap_off[2] = {0, 0}, tap_h[2] = {0, 0}, tap_w[2] = {0, 0};
+    bool kvalid[2] = {false, false};
+    auto prep = [&](int k0) {
         if (UT) {
-            // k0 is wave-uniform: this arithmetic runs on the scalar unit
-            unsigned tap, c0, th, tw;
-            p.div_c.divmod((unsigned)k0, tap, c0);
-            p.div_tw.divmod(tap, th, tw);
-            const unsigned tap_bytes = (unsigned)(((int)th * p.Ws + (int)tw) * p.Cs + (int)c0) * (unsigned)sizeof(T);
-#pragma unroll
-            for (int i = 0; i < AL; ++i) {
-                const unsigned bad = (a_inv[i] >> tap) & 1u;
-                const unsigned voff = (a_byte[i] + tap_bytes) | (bad << 31);
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(la + (wave * AL + i) * 64), 16,
-                                                         (int)voff, 0, 0, 0);
-            }
-#pragma unroll
-            for (int i = 0; i < BL; ++i)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(lb + (wave * BL + i) * 64), 16,
-                                                         (int)(b_off[i] + (unsigned)k0 * (unsigned)sizeof(T)), 0, 0, 0);
+            unsigned c0, th, tw;
+            p.div_c.divmod((unsigned)k0, ut_tap, c0);
+            p.div_tw.divmod(ut_tap, th, tw);
+            ut_tap_bytes = (unsigned)(((int)th * p.Ws + (int)tw) * p.Cs + (int)c0) * (unsigned)sizeof(T);
             return;
         }
         // tap decode for the two chunk columns a lane serves (even / odd 8-row blocks)
-        int tap_off[2], tap_h[2], tap_w[2];
-        bool kvalid[2];
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
             int kk = k0 + CE * (k4e ^ (q << 2));
@@ -422,31 +459,44 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
             tap_w[q] = (int)tw;
             tap_off[q] = ((int)th * p.Ws + (int)tw) * p.Cs + (int)c;
         }
-#pragma unroll
-        for (int i = 0; i < AL; ++i) {
-            const int q = i & 1;                    // AL is even: block parity = i & 1
+    };
+    auto issue_load = [&](int j, int k0, f4* la, f4* lb) {
+        if (j >= AL) {
+            const int i = j - AL;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(lb + (wave * BL + i) * 64), 16,
+                                                     (int)(b_off[i] + (unsigned)k0 * (unsigned)sizeof(T)), 0, 0, 0);
+            return;
+        }
+        const int i = j;
+        unsigned voff;
+        if (UT) {
+            const unsigned bad = (a_inv[i] >> ut_tap) & 1u;
+            voff = (a_byte[i] + ut_tap_bytes) | (bad << 31);
+        } else {
+            const int q = i & 1;                        // AL is even: block parity = i & 1
             int r = (base_rc[i] >> 16) + tap_h[q];
             int cc = ((int)((unsigned)base_rc[i] << 16) >> 16) + tap_w[q];
             // bitwise, not short-circuit: keeps the slab issue free of branches
             const unsigned bad =
                 (unsigned)!(kvalid[q] & ((unsigned)r < (unsigned)p.Hs) & ((unsigned)cc < (unsigned)p.Ws));
-            const unsigned voff = ((unsigned)(base_off[i] + tap_off[q]) * (unsigned)sizeof(T)) | (bad << 31);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(la + (wave * AL + i) * 64), 16, (int)voff, 0,
-                                                     0, 0);
+            voff = ((unsigned)(base_off[i] + tap_off[q]) * (unsigned)sizeof(T)) | (bad << 31);
         }
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(la + (wave * AL + i) * 64), 16, (int)voff, 0, 0, 0);
+    };
+    constexpr int NL = AL + BL;                          // loads per wave per slab
+    constexpr int LPG = (NL + 2) / 3;                    // spread over the first 3 of the 4 MFMA groups
+    auto issue_part = [&](int g, int k0, f4* la, f4* lb) {
 #pragma unroll
-        for (int i = 0; i < BL; ++i)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(lb + (wave * BL + i) * 64), 16,
-                                                     (int)(b_off[i] + (unsigned)k0 * (unsigned)sizeof(T)), 0, 0, 0);
+        for (int j = g * LPG; j < (g + 1) * LPG && j < NL; ++j) issue_load(j, k0, la, lb);
+    };
+    auto issue = [&](int k0, f4* la, f4* lb) {
+        prep(k0);
+#pragma unroll
+        for (int j = 0; j < NL; ++j) issue_load(j, k0, la, lb);
     };
 
     f16v acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    init_acc<TM, TN>(p, acc, n0 + wn0, lh);
 
     const int sw7 = (l32 >> 1) & 7;            // (row >> 1) & 7 of every operand row this lane reads
     f4 fa[2][TM], fb[2][TN];                   // operand fragments, double buffered across k groups
@@ -461,7 +511,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) mma_chunk<T>(fa[slot][i], fb[slot][j], acc[i][j]);
+            for (int j = 0; j < TN; ++j) mma_chunk<T>(fb[slot][j], fa[slot][i], acc[i][j]);
     };
     // One slab: the first operand reads go out right after the barrier, then the
     // loads of the next slab are issued (their address arithmetic overlaps the LDS
@@ -470,10 +520,11 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
         __builtin_amdgcn_s_waitcnt(0);         // this wave's loads of the slab have landed
         __syncthreads();                       // everyone's have; everyone is done reading the other buffer
         read_frags(la, lb, 0, 0);
-        if (has_next) issue(next_k0, na, nb);
+        if (has_next) prep(next_k0);
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             if (g < 3) read_frags(la, lb, g + 1, (g + 1) & 1);
+            if (has_next && g < 3) issue_part(g, next_k0, na, nb);
             // keep the prefetch ahead of the MFMAs (the scheduler would otherwise sink
             // the reads next to their first use and expose the LDS latency)
             __builtin_amdgcn_sched_barrier(0);
@@ -601,6 +652,9 @@ static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
         const int64_t lim = (int64_t)1 << 31;
         gs.gp.src_bytes = (sb < lim && bb < lim) ? (unsigned)sb : 0u;
         gs.gp.bt_bytes = (sb < lim && bb < lim) ? (unsigned)bb : 0u;
+        const int64_t ob = (g.dense_out ? (int64_t)g.M : (int64_t)g.S * g.Hof * g.Wof) * g.N * (int64_t)sizeof(float);
+        const bool ovec = ob < lim && g.N % 4 == 0 && (reinterpret_cast<uintptr_t>(g.out) & 15) == 0;
+        gs.gp.out_bytes = ovec ? (unsigned)ob : 0u;
     }
     if (total > 0) {
         hipLaunchKernelGGL(pack_filter<T>, dim3(cdiv(total, 256)), dim3(256), 0, c.stream, gs.pp);
@@ -746,6 +800,9 @@ struct WgradParams {
     int m_per_split;     // multiple of 32
     int kt, nt;          // output tiles along k and n
     unsigned x_bytes, dy_bytes;   // extents for the buffer descriptors (LDS-direct kernel)
+    // moving 32 rows of m ahead: 32 = qs*Ho*Wo + qh*Wo + qw.  step_c = qw*sW, step_r = qh*sH;
+    // byte offset += inc0 (+ inc1 when the column wraps) (+ inc2 when the row wraps)
+    int step_c, step_r, inc0, inc1, inc2;
     FastDiv div_howo, div_wo, div_c, div_fw;
 };
 
@@ -1144,6 +1201,244 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma(const WgradPar
 }
 
 // ------------------------------------------------------------------------------
+// wgrad, LDS-direct, wide-operand variant (fp32, C and D multiples of 4): the
+// default for fp32.  Tile 128 k x 64 n per workgroup, 32-row slabs of m as above,
+// but the A operand is read with ONE `ds_read_b128` per 4 MFMAs: lane i takes the
+// 4 consecutive k values 4i..4i+3 of slab row m and MFMA q (q = 0..3) multiplies
+// the column k = 4i + q, i.e. accumulator q holds the output rows k == q (mod 4).
+// Which rows an MFMA produces is free to choose, and this choice turns the
+// 3 x `ds_read_b32` per 2 MFMAs of wgrad_gemm_dma into 2 reads per 4 MFMAs
+// (a stand-alone loop: 118 -> 132 TFLOP/s).
+//   * the 4 waves are (n half) x (parity of the m pair): a wave owns all 128 k rows
+//     of one 32-wide n half and every other pair of slab rows; the two parities
+//     are added through LDS once, after the last slab;
+//   * a last k tile with at most 64 valid rows switches to `ds_read_b64` and two
+//     accumulators (k = 2i + q), so K = 576 multiplies no padding;
+//   * x rows are stored plainly (a 16-lane group reads 256 contiguous bytes);
+//     dy keeps the half-swap of odd rows for its `ds_read_b32`.
+// ------------------------------------------------------------------------------
+template <int CW>
+static __device__ __forceinline__ void wgrad_wide_body(const WgradParams& p, float* lds_a0, float* lds_a1, float* lds_y0,
+                                                       float* lds_y1) {
+    constexpr int BR = kWgBR;                            // 32 rows of m per slab
+    typedef float fcw __attribute__((ext_vector_type(CW)));
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int l32 = lane & 31;
+    const int lh = lane >> 5;
+    const int nt = wave & 1;                             // n half of this wave
+    const int mh = wave >> 1;                            // parity of the m pairs it multiplies
+
+    const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
+    const int tiles = p.kt * p.nt;
+    const int split = lid / tiles;
+    const int tile = lid - split * tiles;
+    const int ktile = tile % p.kt;
+    const int kt0 = ktile * kWgBK;
+    const int n0 = (tile / p.kt) * kWgBN;
+    const int m_begin = split * p.m_per_split;
+    int m_end = m_begin + p.m_per_split;
+    if (m_end > p.M) m_end = p.M;
+    const bool do_db = p.want_dbias && (ktile == 0);
+
+    // ---- x: one wave-level load = 2 slab rows x 32 chunks; 4 loads per wave per slab ----
+    // fp32 MFMA and ordinary vector (and scalar) instructions of a wave share its issue
+    // slots, so the address work per load is kept to a handful of instructions:
+    //  * lane l keeps the image position of slab row 8*wave + (l & 7) -- the 8 rows this
+    //    wave loads -- and moves it by 32 rows per slab with adds and two carries
+    //    (no division in the loop);
+    //  * load i takes the rows 2i and 2i+1 of those 8 from their lanes with `ds_bpermute`;
+    //  * the lane's own filter tap is tested against the row's position with the fields
+    //    (row, column) packed in one register and guard bits catching both bounds.
+    // Row state: rpos/cpos = position of tap (0,0) in the image + 64 (never negative),
+    // off = byte offset of that pixel (wraps for padding positions; only used when valid).
+    int st_r, st_c, st_off;
+    {
+        const int m = m_begin + 8 * wave + (lane & 7);
+        unsigned s_, rem, ho, wo;
+        p.div_howo.divmod((unsigned)m, s_, rem);
+        p.div_wo.divmod(rem, ho, wo);
+        st_r = (int)ho * p.sH - p.pH;
+        st_c = (int)wo * p.sW - p.pW;
+        st_off = ((((int)s_ * p.H + st_r) * p.W + st_c) * p.C) * 4;
+        st_r += 64;
+        st_c += 64;
+    }
+    const int thr_c = p.Wo * p.sW - p.pW + 64, thr_r = p.Ho * p.sH - p.pH + 64;
+    auto advance = [&]() {                               // m += 32
+        st_c += p.step_c;
+        const bool c1 = st_c >= thr_c;
+        st_c -= c1 ? p.Wo * p.sW : 0;
+        st_r += c1 ? p.step_r + p.sH : p.step_r;
+        const bool c2 = st_r >= thr_r;
+        st_r -= c2 ? p.Ho * p.sH : 0;
+        st_off += c1 ? p.inc0 + p.inc1 : p.inc0;
+        st_off += c2 ? p.inc2 : 0;
+    };
+    // per-lane tap constants
+    unsigned tap_lo, tap_hi;                             // guard-bit constants, see test below
+    int a_tap4;
+    {
+        const int kk = kt0 + 4 * (lane & 31);
+        unsigned tap, c, fx, fy;
+        p.div_c.divmod((unsigned)kk, tap, c);
+        p.div_fw.divmod(tap, fx, fy);
+        a_tap4 = (((int)fx * p.W + (int)fy) * p.C + (int)c) * 4;
+        const unsigned tapc = (fx << 16) | fy;
+        // t = rc + tapc has the fields (row + 64, column + 64) of the lane's tap.
+        // lo = 0x803f803f - t : bit 15 of a field is set iff that coordinate is < 0
+        // hi = t + (0x8000 - (H + 64), 0x8000 - (W + 64)) : set iff it is >= H (or W)
+        tap_lo = 0x803f803fu - tapc;
+        tap_hi = tapc + (((unsigned)(0x8000 - (p.H + 64)) << 16) | (unsigned)(0x8000 - (p.W + 64)));
+        if (kk >= p.K) tap_lo = 0xffffffffu;             // k past K: always out of range
+    }
+    const int perm0 = (lane >> 5) * 4;                   // byte index of source lane 0 / 1 (+ 8 i for load i)
+
+    // ---- dy: one wave-level load = 4 slab rows x 16 chunks; 2 loads per wave ------------
+    // Rows past M lie beyond the descriptors' extents (and m_per_split is a multiple of
+    // the slab height), so neither operand needs a test against m_end.
+    const int y_row = lane >> 4;
+    const int y_lc = (lane & 15) ^ ((y_row & 1) << 3);
+    const int y_n = n0 + 4 * y_lc;
+    const unsigned y_lane = ((unsigned)(y_row * p.D + y_n) * 4u) | ((unsigned)!(y_n < p.D) << 31);
+
+    const __amdgpu_buffer_rsrc_t rsrc_x =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.x), 0, (int)p.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_y =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.dy), 0, (int)p.dy_bytes, 0x00020000);
+
+    // loads of the slab whose first row is mb; the row state must stand at mb
+    auto issue = [&](int mb, float* la, float* ly) {
+        const int rc = (st_r << 16) | st_c;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const unsigned rc_i = (unsigned)__builtin_amdgcn_ds_bpermute(perm0 + 8 * i, rc);
+            const int off_i = __builtin_amdgcn_ds_bpermute(perm0 + 8 * i, st_off);
+            const unsigned z = (tap_lo - rc_i) | (rc_i + tap_hi);
+            const unsigned w = z | (z << 16);            // bit 31: row or column out of the image
+            const unsigned voff = (w & 0x80000000u) | (unsigned)(off_i + a_tap4);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + (wave * 4 + i) * 256), 16, (int)voff, 0,
+                                                     0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int m = mb + (wave_u * 2 + i) * 4;     // scalar
+            const unsigned voff = y_lane + (unsigned)(m * p.D) * 4u;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_y, (lds_ptr_t)(ly + (wave * 2 + i) * 256), 16, (int)voff, 0,
+                                                     0, 0);
+        }
+    };
+
+    float dbsum = 0.f;
+    const int db_col = tid & 63, db_rg = tid >> 6;
+    auto add_columns = [&](const float* ly) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dbsum += ly[(db_rg * 8 + j) * kWgBN + (db_col ^ ((j & 1) << 5))];
+    };
+
+    f16v acc[CW];
+#pragma unroll
+    for (int q = 0; q < CW; ++q)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[q][v] = 0.f;
+
+    // operand addresses of m pair t' (slab rows 2*(2t'+mh) + lh); odd rows of dy have halves swapped
+    const int row0 = 2 * mh + lh;                        // first slab row read; then +4 per step
+    const int y_rd = nt * 32 + l32;                      // logical n; physical = y_rd ^ (lh << 5)
+    // The MFMA takes dy as its A operand and x as B: accumulator q then holds
+    // dW[k = kt0 + CW * (lane % 32) + q][n = 32 nt + 8 (v/4) + 4 (lane/32) + v%4], four
+    // consecutive n per lane and v/4, which leave in 16-byte stores.
+    auto slab = [&](int mb, const float* la, const float* ly, float* na, float* ny, bool has_next) {
+        __builtin_amdgcn_s_waitcnt(0);                   // this wave's loads of the slab have landed
+        __syncthreads();
+        fcw fa[2];
+        float fb[2];
+        fa[0] = *reinterpret_cast<const fcw*>(la + row0 * kWgBK + CW * l32);
+        fb[0] = ly[row0 * kWgBN + (y_rd ^ (lh << 5))];
+        if (has_next) {
+            advance();
+            issue(mb + BR, na, ny);
+        }
+#pragma unroll
+        for (int t = 0; t < BR / 4; ++t) {
+            if (t + 1 < BR / 4) {
+                fa[(t + 1) & 1] = *reinterpret_cast<const fcw*>(la + (row0 + 4 * t + 4) * kWgBK + CW * l32);
+                fb[(t + 1) & 1] = ly[(row0 + 4 * t + 4) * kWgBN + (y_rd ^ (lh << 5))];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int q = 0; q < CW; ++q)
+                acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[t & 1], fa[t & 1][q], acc[q], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (do_db) add_columns(ly);
+    };
+
+    if (m_begin < m_end) issue(m_begin, lds_a0, lds_y0);
+    for (int mb = m_begin; mb < m_end; mb += 2 * BR) {
+        slab(mb, lds_a0, lds_y0, lds_a1, lds_y1, mb + BR < m_end);
+        if (mb + BR < m_end) slab(mb + BR, lds_a1, lds_y1, lds_a0, lds_y0, mb + 2 * BR < m_end);
+    }
+
+    // ---- add the two m parities: waves 2,3 hand their accumulators to waves 0,1 --------
+    __syncthreads();                                     // slab buffers are free now
+    f4* xch = reinterpret_cast<f4*>(nt == 0 ? lds_a0 : lds_a1);   // 16 x 16 B x 64 lanes = 16 KB per wave pair
+    if (mh == 1) {
+#pragma unroll
+        for (int q = 0; q < CW; ++q)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+                xch[(q * 4 + g) * 64 + lane] = f4{acc[q][4 * g], acc[q][4 * g + 1], acc[q][4 * g + 2], acc[q][4 * g + 3]};
+    }
+    __syncthreads();
+    const size_t split_stride = (size_t)p.K * p.D + p.D;
+    float* outp = p.out + (size_t)split * split_stride;
+    if (mh == 0) {
+        // one split's partial block is far below 2^31 bytes (K * D < 2^29 is checked by the host)
+        const __amdgpu_buffer_rsrc_t rsrc_o =
+            __builtin_amdgcn_make_buffer_rsrc(outp, 0, (int)((unsigned)p.K * (unsigned)p.D * 4u), 0x00020000);
+        const int nb = n0 + nt * 32 + 4 * lh;
+#pragma unroll
+        for (int q = 0; q < CW; ++q) {
+            const int k = kt0 + CW * l32 + q;            // rows past K fall outside the descriptor
+            const unsigned base = (unsigned)(k * p.D + nb) * 4u;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                f4 v = xch[(q * 4 + g) * 64 + lane];
+                v[0] += acc[q][4 * g];
+                v[1] += acc[q][4 * g + 1];
+                v[2] += acc[q][4 * g + 2];
+                v[3] += acc[q][4 * g + 3];
+                const unsigned off = base | ((unsigned)!(nb + 8 * g < p.D) << 31);
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, v), rsrc_o, (int)off, 8 * g * 4, 0);
+            }
+        }
+    }
+    if (do_db) {
+        __syncthreads();
+        lds_y0[db_rg * 64 + db_col] = dbsum;
+        __syncthreads();
+        if (tid < 64 && n0 + tid < p.D)
+            outp[(size_t)p.K * p.D + n0 + tid] = (lds_y0[tid] + lds_y0[64 + tid]) + (lds_y0[128 + tid] + lds_y0[192 + tid]);
+    }
+}
+
+static __global__ __launch_bounds__(kThreads, 3) void wgrad_gemm_dma_wide(const WgradParams p) {
+    __shared__ float lds_a0[kWgBR * kWgBK];
+    __shared__ float lds_a1[kWgBR * kWgBK];
+    __shared__ float lds_y0[kWgBR * kWgBN];
+    __shared__ float lds_y1[kWgBR * kWgBN];
+    static_assert(sizeof(lds_a0) >= 64 * 64 * sizeof(float), "accumulator exchange buffer");
+    const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
+    const int kt0 = ((lid % (p.kt * p.nt)) % p.kt) * kWgBK;
+    if (p.K - kt0 <= 64) wgrad_wide_body<2>(p, lds_a0, lds_a1, lds_y0, lds_y1);   // workgroup-uniform
+    else wgrad_wide_body<4>(p, lds_a0, lds_a1, lds_y0, lds_y1);
+}
+
+// ------------------------------------------------------------------------------
 // wgrad for bf16 inputs on v_mfma_f32_32x32x16_bf16 (C and D multiples of 8).
 // The MFMA reduces over m, so each lane needs 8 consecutive m of ONE k (or n)
 // column, while the slabs arrive m-major ([m][k], k contiguous) straight from
@@ -1369,6 +1664,14 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     p.fW = fW; p.sH = sH; p.sW = sW; p.pH = pH; p.pW = pW;
     p.want_dbias = dbias != nullptr;
     p.div_howo = FastDiv(Ho * Wo); p.div_wo = FastDiv(Wo); p.div_c = FastDiv(C); p.div_fw = FastDiv(fW);
+    {
+        const int qs = kWgBR / (Ho * Wo), rem = kWgBR % (Ho * Wo), qh = rem / Wo, qw = rem % Wo;
+        p.step_c = qw * sW;
+        p.step_r = qh * sH;
+        p.inc0 = 4 * C * (qw * sW + qh * sH * W + qs * H * W);
+        p.inc1 = 4 * C * (-Wo * sW + sH * W);
+        p.inc2 = 4 * C * (-Ho * sH * W + H * W);
+    }
     constexpr int CE = Elem<T>::CE;
     const bool va = (C % CE == 0), vy = (D % CE == 0);
     const int64_t xb = (int64_t)S * H * W * C * (int64_t)sizeof(T), yb = (int64_t)p.M * D * (int64_t)sizeof(T);
@@ -1377,16 +1680,14 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     const bool dma16 = sizeof(T) == 2 && va && vy && fits;      // bf16 MFMA kernel, 64-row slabs
     p.x_bytes = (dma || dma16) ? (unsigned)xb : 0u;
     p.dy_bytes = (dma || dma16) ? (unsigned)yb : 0u;
-    // 256-row k tiles (two row blocks per wave) move half the bytes per flop, but a
-    // partly filled last tile leaves whole workgroups nearly idle: use them only when
-    // K fills its 256-row tiles to 94 % or more (measured: K = 576 is 23 % slower).
+    // fp32 LDS-direct kernels: the wide-operand kernel unless AETHER_WGRAD_WKB names one
+    // of the `ds_read_b32` kernels (1: 128-row k tiles, 2: 256-row k tiles) for comparison.
     int wkb_used = 1;
+    bool wide = dma;
     if (dma) {
-        const int t256 = cdiv(p.K, 2 * kWgBK);
-        if ((int64_t)p.K * 100 >= (int64_t)t256 * 2 * kWgBK * 94) wkb_used = 2;
-        if (const char* f = getenv("AETHER_WGRAD_WKB")) {     // tuning override: 1 or 2
+        if (const char* f = getenv("AETHER_WGRAD_WKB")) {
             const int v = atoi(f);
-            if (v == 1 || v == 2) wkb_used = v;
+            if (v == 1 || v == 2) { wkb_used = v; wide = false; }
         }
     }
     const int kt = cdiv(p.K, kWgBK * wkb_used), nt = cdiv(D, kWgBN);
@@ -1407,6 +1708,7 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     p.kt = kt; p.nt = nt;
     dim3 grid(kt * nt * splits);
     if (dma16) hipLaunchKernelGGL(wgrad_gemm_dma_bf16, grid, dim3(kThreads), 0, c.stream, p);
+    else if (dma && wide) hipLaunchKernelGGL(wgrad_gemm_dma_wide, grid, dim3(kThreads), 0, c.stream, p);
     else if (dma && wkb_used == 2) hipLaunchKernelGGL(wgrad_gemm_dma<2>, grid, dim3(kThreads), 0, c.stream, p);
     else if (dma) hipLaunchKernelGGL(wgrad_gemm_dma<1>, grid, dim3(kThreads), 0, c.stream, p);
     else if (va && vy) hipLaunchKernelGGL((wgrad_gemm<T, CE, CE>), grid, dim3(kThreads), 0, c.stream, p);
