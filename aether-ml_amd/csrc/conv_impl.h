@@ -78,7 +78,7 @@ struct GatherParams {
     int S, Hs, Ws, Cs;
     int Hg, Wg;          // output pixel grid of this launch
     int M, N, K, Kpad;   // M = S*Hg*Wg, K = Th*Tw*Cs
-    int Tw;              // taps per filter row
+    int Tw, Th;          // taps per filter row, filter rows (Th is filled in by run_gather)
     int sh, sw;          // source step per output pixel
     int rh0, rw0;        // source offset of tap (0,0)
     // output element (s,i,j,n) lives at ((s*Hof + oh0 + i*ohs)*Wof + ow0 + j*ows)*N + n
@@ -402,19 +402,23 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
     // tap that says "outside the image" (all ones for rows past M)
     unsigned a_byte[AL], a_inv[AL];
     if (UT) {
-        const int ntaps = p.K / p.Cs;
 #pragma unroll
         for (int i = 0; i < AL; ++i) {
             const int br = base_rc[i] >> 16;
             const int bc = (int)((unsigned)base_rc[i] << 16) >> 16;
-            unsigned inv = 0;
-            int th = 0, tw = 0;
-            for (int t = 0; t < ntaps; ++t) {
-                const unsigned bad =
-                    (unsigned)!(((unsigned)(br + th) < (unsigned)p.Hs) & ((unsigned)(bc + tw) < (unsigned)p.Ws));
-                inv |= bad << t;
-                if (++tw == p.Tw) { tw = 0; ++th; }
-            }
+            // taps (th, tw) inside the image: th in [max(0,-br), min(Th, Hs-br)), same for tw;
+            // a row past M has br = kInvalidRow and an empty range
+            auto span = [](int lo, int hi) -> unsigned {     // bits [lo, hi) of a mask, 0 <= lo, hi <= 32
+                const unsigned upto_hi = hi > 0 ? ~0u >> (32 - hi) : 0u;
+                const unsigned upto_lo = lo > 0 ? ~0u >> (32 - lo) : 0u;
+                return hi > lo ? upto_hi & ~upto_lo : 0u;
+            };
+            const int lo_r = min(max(-br, 0), 32), hi_r = min(max(p.Hs - br, 0), p.Th);
+            const int lo_c = min(max(-bc, 0), 32), hi_c = min(max(p.Ws - bc, 0), p.Tw);
+            const unsigned rmask = span(lo_r, hi_r), cmask = span(lo_c, hi_c);
+            unsigned valid = 0;
+            for (int th = 0; th < p.Th; ++th) valid |= (((rmask >> th) & 1u) ? cmask : 0u) << (th * p.Tw);
+            const unsigned inv = ~valid;
             a_inv[i] = inv;
             a_byte[i] = (unsigned)(base_off[i] + CE * (k4e ^ ((i & 1) << 2))) * (unsigned)sizeof(T);
         }
@@ -650,6 +654,7 @@ static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
         int64_t sb = (int64_t)g.S * g.Hs * g.Ws * g.Cs * (int64_t)sizeof(T);
         int64_t bb = (int64_t)total * (int64_t)sizeof(T);
         const int64_t lim = (int64_t)1 << 31;
+        gs.gp.Th = (g.Tw > 0 && g.Cs > 0) ? (g.K / g.Cs) / g.Tw : 0;
         gs.gp.src_bytes = (sb < lim && bb < lim) ? (unsigned)sb : 0u;
         gs.gp.bt_bytes = (sb < lim && bb < lim) ? (unsigned)bb : 0u;
         const int64_t ob = (g.dense_out ? (int64_t)g.M : (int64_t)g.S * g.Hof * g.Wof) * g.N * (int64_t)sizeof(float);
@@ -1310,26 +1315,31 @@ static __device__ __forceinline__ void wgrad_wide_body(const WgradParams& p, flo
     const __amdgpu_buffer_rsrc_t rsrc_y =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.dy), 0, (int)p.dy_bytes, 0x00020000);
 
-    // loads of the slab whose first row is mb; the row state must stand at mb
-    auto issue = [&](int mb, float* la, float* ly) {
-        const int rc = (st_r << 16) | st_c;
+    // loads of the slab whose first row is mb; the row state must stand at mb.  The work
+    // is cut in three so that a slab can spread it between its MFMA groups: a burst of
+    // address arithmetic after the barrier keeps the wave off the matrix pipe, while the
+    // same instructions issued behind an MFMA run in its shadow.
+    unsigned perm_rc[4];
+    int perm_off[4];
+    // live == 0 (no next slab): rows read as (0, 0), which every tap sees as "above the image"
+    auto fetch_rows = [&](int live) {                    // 8 LDS-crossbar permutes, no LDS memory
+        const int rc = ((st_r << 16) | st_c) & live;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const unsigned rc_i = (unsigned)__builtin_amdgcn_ds_bpermute(perm0 + 8 * i, rc);
-            const int off_i = __builtin_amdgcn_ds_bpermute(perm0 + 8 * i, st_off);
-            const unsigned z = (tap_lo - rc_i) | (rc_i + tap_hi);
-            const unsigned w = z | (z << 16);            // bit 31: row or column out of the image
-            const unsigned voff = (w & 0x80000000u) | (unsigned)(off_i + a_tap4);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + (wave * 4 + i) * 256), 16, (int)voff, 0,
-                                                     0, 0);
+            perm_rc[i] = (unsigned)__builtin_amdgcn_ds_bpermute(perm0 + 8 * i, rc);
+            perm_off[i] = __builtin_amdgcn_ds_bpermute(perm0 + 8 * i, st_off);
         }
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int m = mb + (wave_u * 2 + i) * 4;     // scalar
-            const unsigned voff = y_lane + (unsigned)(m * p.D) * 4u;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_y, (lds_ptr_t)(ly + (wave * 2 + i) * 256), 16, (int)voff, 0,
-                                                     0, 0);
-        }
+    };
+    auto load_x = [&](int i, float* la) {
+        const unsigned z = (tap_lo - perm_rc[i]) | (perm_rc[i] + tap_hi);
+        const unsigned w = z | (z << 16);                // bit 31: row or column out of the image
+        const unsigned voff = (w & 0x80000000u) | (unsigned)(perm_off[i] + a_tap4);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + (wave * 4 + i) * 256), 16, (int)voff, 0, 0, 0);
+    };
+    auto load_y = [&](int i, int mb, float* ly, int live) {
+        const int m = mb + (wave_u * 2 + i) * 4;         // scalar
+        const unsigned voff = y_lane + (live ? (unsigned)(m * p.D) * 4u : 0x80000000u);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_y, (lds_ptr_t)(ly + (wave * 2 + i) * 256), 16, (int)voff, 0, 0, 0);
     };
 
     float dbsum = 0.f;
@@ -1358,16 +1368,19 @@ static __device__ __forceinline__ void wgrad_wide_body(const WgradParams& p, flo
         float fb[2];
         fa[0] = *reinterpret_cast<const fcw*>(la + row0 * kWgBK + CW * l32);
         fb[0] = ly[row0 * kWgBN + (y_rd ^ (lh << 5))];
-        if (has_next) {
-            advance();
-            issue(mb + BR, na, ny);
-        }
+        // no branch in here: without a next slab the loads are issued with offsets past
+        // the descriptors and fetch nothing
+        const int live = has_next ? -1 : 0;
+        advance();
+        fetch_rows(live);
 #pragma unroll
         for (int t = 0; t < BR / 4; ++t) {
             if (t + 1 < BR / 4) {
                 fa[(t + 1) & 1] = *reinterpret_cast<const fcw*>(la + (row0 + 4 * t + 4) * kWgBK + CW * l32);
                 fb[(t + 1) & 1] = ly[(row0 + 4 * t + 4) * kWgBN + (y_rd ^ (lh << 5))];
             }
+            if (t >= 1 && t <= 4) load_x(t - 1, na);
+            if (t == 5 || t == 6) load_y(t - 5, mb + BR, ny, live);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int q = 0; q < CW; ++q)
@@ -1377,7 +1390,13 @@ static __device__ __forceinline__ void wgrad_wide_body(const WgradParams& p, flo
         if (do_db) add_columns(ly);
     };
 
-    if (m_begin < m_end) issue(m_begin, lds_a0, lds_y0);
+    if (m_begin < m_end) {
+        fetch_rows(-1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) load_x(i, lds_a0);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) load_y(i, m_begin, lds_y0, -1);
+    }
     for (int mb = m_begin; mb < m_end; mb += 2 * BR) {
         slab(mb, lds_a0, lds_y0, lds_a1, lds_y1, mb + BR < m_end);
         if (mb + BR < m_end) slab(mb + BR, lds_a1, lds_y1, lds_a0, lds_y0, mb + 2 * BR < m_end);
