@@ -348,21 +348,32 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 //     the FP32 lanes with ordinary vector instructions, so every address instruction
 //     costs MFMA time; in this mode the tap decode runs on the scalar unit and each
 //     row's per-tap validity is a precomputed bit mask: 3 vector instructions per load.
-template <typename T, int BM, int BN, int WM, int WN, bool UT>
+//   * KC = 16-byte chunks per slab row: 8 (slab = 32 floats of k, 48 KB of LDS for a
+//     128 x 64 tile, 3 workgroups per CU) or 4 (16 floats, 24 KB, 5 per CU).  The
+//     shallow slab pays a barrier twice as often but keeps more workgroups resident, and
+//     those hide each other's set-up, first loads and epilogue.  With KC = 4 a wave-level
+//     load covers 16 rows, chunk c of row r lives at c ^ ((r >> 2) & 3), and a 16-lane
+//     read group (16 rows x 64 B) again covers the 64 banks exactly once.
+template <typename T, int BM, int BN, int WM, int WN, bool UT, int KC>
 __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p) {
     static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
-    static_assert((BM / 32) % 2 == 0, "8-row load blocks of a wave alternate even/odd");
+    static_assert(KC == 8 || KC == 4, "slab rows of 8 or 4 chunks");
     constexpr int CE = Elem<T>::CE;
-    constexpr int BK = Elem<T>::BK;
-    constexpr int AL = BM / 32;          // wave-level A loads per wave per slab (8 rows each)
-    constexpr int BL = BN / 32;
+    constexpr int BK = KC * CE;          // elements of k per slab
+    constexpr int RPL = 64 / KC;         // slab rows per wave-level load
+    constexpr int SH = KC == 8 ? 1 : 2;  // swizzle: chunk position = chunk ^ ((row >> SH) & (KC - 1))
+    constexpr int G = KC / 2;            // MFMA groups per slab (one 16-byte chunk per lane half each)
+    constexpr int AL = BM / (4 * RPL);   // wave-level A loads per wave per slab
+    constexpr int BL = BN / (4 * RPL);
+    static_assert(AL >= 1 && BL >= 1 && BM % (4 * RPL) == 0 && BN % (4 * RPL) == 0, "tile too small for KC");
+    static_assert(KC == 4 || AL % 2 == 0, "8-row load blocks of a wave alternate even/odd");
     constexpr int TM = WM / 32;
     constexpr int TN = WN / 32;
 
-    __shared__ f4 lds_a0[BM * 8];
-    __shared__ f4 lds_a1[BM * 8];
-    __shared__ f4 lds_b0[BN * 8];
-    __shared__ f4 lds_b1[BN * 8];
+    __shared__ f4 lds_a0[BM * KC];
+    __shared__ f4 lds_a1[BM * KC];
+    __shared__ f4 lds_b0[BN * KC];
+    __shared__ f4 lds_b1[BN * KC];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -376,15 +387,17 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
     const int m0 = (lid / ntile) * BM;
     const int n0 = (lid % ntile) * BN;
 
-    const int lr = lane >> 3;                  // row inside an 8-row load block
-    // logical chunk this lane fetches: (lane & 7) ^ ((row >> 1) & 7); the 8-row blocks
-    // alternate between row bits (0,lane>>4) and (4 | lane>>4)
-    const int k4e = (lane & 7) ^ (lane >> 4);  // even 8-row blocks; odd blocks use k4e ^ 4
+    const int lr = lane / KC;                  // row inside a load block
+    // logical chunk this lane fetches: (lane % KC) ^ swizzle(row).  KC == 8: the 8-row
+    // blocks alternate between row bits (0,lane>>4) and (4 | lane>>4), so odd blocks use
+    // k4e ^ 4; KC == 4: 16-row blocks, the same for every block
+    const int k4e = KC == 8 ? (lane & 7) ^ (lane >> 4) : (lane & 3) ^ (lane >> 4);
+    constexpr int ODD = KC == 8 ? 4 : 0;       // what an odd load block xors into the chunk
     int base_off[AL];
     int base_rc[AL];
 #pragma unroll
     for (int i = 0; i < AL; ++i) {
-        int m = m0 + (wave * AL + i) * 8 + lr;
+        int m = m0 + (wave * AL + i) * RPL + lr;
         if (m < p.M) {
             unsigned s, rem, ii, jj;
             p.div_hw.divmod((unsigned)m, s, rem);
@@ -420,14 +433,14 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
             for (int th = 0; th < p.Th; ++th) valid |= (((rmask >> th) & 1u) ? cmask : 0u) << (th * p.Tw);
             const unsigned inv = ~valid;
             a_inv[i] = inv;
-            a_byte[i] = (unsigned)(base_off[i] + CE * (k4e ^ ((i & 1) << 2))) * (unsigned)sizeof(T);
+            a_byte[i] = (unsigned)(base_off[i] + CE * (k4e ^ ((i & 1) ? ODD : 0))) * (unsigned)sizeof(T);
         }
     }
     unsigned b_off[BL];
 #pragma unroll
     for (int i = 0; i < BL; ++i) {
-        const int k4 = k4e ^ (((wave * BL + i) & 1) << 2);
-        b_off[i] = (unsigned)(((n0 + (wave * BL + i) * 8 + lr) * p.Kpad + CE * k4) * (int)sizeof(T));
+        const int k4 = k4e ^ (((wave * BL + i) & 1) ? ODD : 0);
+        b_off[i] = (unsigned)(((n0 + (wave * BL + i) * RPL + lr) * p.Kpad + CE * k4) * (int)sizeof(T));
     }
 
     const __amdgpu_buffer_rsrc_t rsrc_a =
@@ -454,7 +467,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
         // tap decode for the two chunk columns a lane serves (even / odd 8-row blocks)
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
-            int kk = k0 + CE * (k4e ^ (q << 2));
+            int kk = k0 + CE * (k4e ^ (q ? ODD : 0));
             unsigned tap, c, th, tw;
             p.div_c.divmod((unsigned)kk, tap, c);
             p.div_tw.divmod(tap, th, tw);
@@ -488,7 +501,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(la + (wave * AL + i) * 64), 16, (int)voff, 0, 0, 0);
     };
     constexpr int NL = AL + BL;                          // loads per wave per slab
-    constexpr int LPG = (NL + 2) / 3;                    // spread over the first 3 of the 4 MFMA groups
+    constexpr int LPG = (NL + G - 2) / (G - 1);          // spread over all MFMA groups but the last
     auto issue_part = [&](int g, int k0, f4* la, f4* lb) {
 #pragma unroll
         for (int j = g * LPG; j < (g + 1) * LPG && j < NL; ++j) issue_load(j, k0, la, lb);
@@ -502,14 +515,14 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
     f16v acc[TM][TN];
     init_acc<TM, TN>(p, acc, n0 + wn0, lh);
 
-    const int sw7 = (l32 >> 1) & 7;            // (row >> 1) & 7 of every operand row this lane reads
+    const int sw7 = (l32 >> SH) & (KC - 1);    // swizzle of every operand row this lane reads
     f4 fa[2][TM], fb[2][TN];                   // operand fragments, double buffered across k groups
     auto read_frags = [&](const f4* la, const f4* lb, int g, int slot) {
         const int pc = (2 * g + lh) ^ sw7;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fa[slot][i] = la[(wm0 + 32 * i + l32) * 8 + pc];
+        for (int i = 0; i < TM; ++i) fa[slot][i] = la[(wm0 + 32 * i + l32) * KC + pc];
 #pragma unroll
-        for (int j = 0; j < TN; ++j) fb[slot][j] = lb[(wn0 + 32 * j + l32) * 8 + pc];
+        for (int j = 0; j < TN; ++j) fb[slot][j] = lb[(wn0 + 32 * j + l32) * KC + pc];
     };
     auto mma_group = [&](int slot) {
 #pragma unroll
@@ -526,9 +539,9 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
         read_frags(la, lb, 0, 0);
         if (has_next) prep(next_k0);
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            if (g < 3) read_frags(la, lb, g + 1, (g + 1) & 1);
-            if (has_next && g < 3) issue_part(g, next_k0, na, nb);
+        for (int g = 0; g < G; ++g) {
+            if (g < G - 1) read_frags(la, lb, g + 1, (g + 1) & 1);
+            if (has_next && g < G - 1) issue_part(g, next_k0, na, nb);
             // keep the prefetch ahead of the MFMAs (the scheduler would otherwise sink
             // the reads next to their first use and expose the LDS latency)
             __builtin_amdgcn_sched_barrier(0);
@@ -583,13 +596,26 @@ __global__ void pack_filter(const PackParams p) {
     static_cast<T*>(p.bt)[idx] = v;
 }
 
+template <typename T, int BM, int BN, int WM, int WN, int KC>
+static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
+    dim3 grid(cdiv(gp.M, BM) * cdiv(gp.N, BN));
+    const bool ut = gp.Cs % (KC * Elem<T>::CE) == 0 && gp.K == gp.Kpad && gp.K / gp.Cs <= 32;
+    if (ut) hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC>), grid, dim3(kThreads), 0, st, gp);
+    else hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, false, KC>), grid, dim3(kThreads), 0, st, gp);
+}
+
+// kc4: shallow slabs (4 chunks of k per row) for the LDS-direct kernel where the tile allows it
 template <typename T, int BM, int BN, int WM, int WN>
-static void launch_gather_cfg(const GatherParams& gp, bool vec, hipStream_t st) {
+static void launch_gather_cfg(const GatherParams& gp, bool vec, bool kc4, hipStream_t st) {
     dim3 grid(cdiv(gp.M, BM) * cdiv(gp.N, BN));
     if (vec && gp.src_bytes != 0 && gp.bt_bytes != 0) {
-        const bool ut = gp.Cs % Elem<T>::BK == 0 && gp.K == gp.Kpad && gp.K / gp.Cs <= 32;
-        if (ut) hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true>), grid, dim3(kThreads), 0, st, gp);
-        else hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, false>), grid, dim3(kThreads), 0, st, gp);
+        if constexpr (BM >= 64 && BN >= 64) {
+            if (kc4) {
+                launch_gather_dma<T, BM, BN, WM, WN, 4>(gp, st);
+                return;
+            }
+        }
+        launch_gather_dma<T, BM, BN, WM, WN, 8>(gp, st);
     }
     else if (vec)
         hipLaunchKernelGGL((gather_gemm<T, BM, BN, WM, WN, Elem<T>::CE>), grid, dim3(kThreads), 0, st, gp);
@@ -625,13 +651,17 @@ static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t
     const int bn = gather_bn(gp.N);
     const bool dma = vec && gp.src_bytes != 0 && gp.bt_bytes != 0;
     const int bm = gather_bm(gp.M, gp.N, cus, dma);
+    // shallow slabs measure the same as deep ones on the 56x56 layers (within 2 % either
+    // way), so they stay a tuning switch: AETHER_GATHER_KC=4
+    bool kc4 = false;
+    if (const char* f = getenv("AETHER_GATHER_KC")) kc4 = atoi(f) == 4;
     if (bn == 32) {
-        if (bm == 256) launch_gather_cfg<T, 256, 32, 64, 32>(gp, vec, st);
-        else launch_gather_cfg<T, 128, 32, 32, 32>(gp, vec, st);
+        if (bm == 256) launch_gather_cfg<T, 256, 32, 64, 32>(gp, vec, false, st);
+        else launch_gather_cfg<T, 128, 32, 32, 32>(gp, vec, false, st);
     } else {
-        if (bm == 256) launch_gather_cfg<T, 256, 64, 64, 64>(gp, vec, st);
-        else if (bm == 128) launch_gather_cfg<T, 128, 64, 32, 64>(gp, vec, st);
-        else launch_gather_cfg<T, 64, 64, 32, 32>(gp, vec, st);
+        if (bm == 256) launch_gather_cfg<T, 256, 64, 64, 64>(gp, vec, kc4, st);
+        else if (bm == 128) launch_gather_cfg<T, 128, 64, 32, 64>(gp, vec, kc4, st);
+        else launch_gather_cfg<T, 64, 64, 32, 32>(gp, vec, kc4, st);
     }
 }
 
