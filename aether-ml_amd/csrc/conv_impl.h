@@ -629,16 +629,17 @@ static inline int gather_bn(int N) { return N <= 32 ? 32 : 64; }
 // 128-row tile (48 KB) lets three workgroups share a CU where a 256-row tile
 // (80 KB) allows one or two; measured on the 56x56x64 shape, 128 rows is 11 %
 // faster.  The register-staged kernel prefers 256 rows.
-static inline int gather_bm(int M, int N, int cus, bool dma) {
+static inline int gather_bm(int M, int N, int cus, bool dma, int elem_bytes = 4) {
     const int bn = gather_bn(N);
     if (const char* f = getenv("AETHER_GATHER_BM")) {       // tuning override: 256, 128 or 64
         int v = atoi(f);
         if (v == 256 || v == 128 || (v == 64 && bn == 64)) return v;
     }
     const int ntiles = cdiv(N, bn);
-    const int want = 2 * cus;
+    const int want = elem_bytes == 2 ? cus : 2 * cus;   // bf16: the taller tile pays off from one tile per CU on
     const int cands[3] = {256, 128, 64};
-    for (int i = dma ? 1 : 0; i < 3; ++i) {
+    // bf16 MFMAs are 8x shorter per slab: there the larger wave tile of the 256-row shape wins
+    for (int i = (dma && elem_bytes == 4) ? 1 : 0; i < 3; ++i) {
         int bm = cands[i];
         if (bn == 32 && bm == 64) break;
         if ((int64_t)cdiv(M, bm) * ntiles >= want) return bm;
@@ -650,7 +651,7 @@ template <typename T>
 static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t st) {
     const int bn = gather_bn(gp.N);
     const bool dma = vec && gp.src_bytes != 0 && gp.bt_bytes != 0;
-    const int bm = gather_bm(gp.M, gp.N, cus, dma);
+    const int bm = gather_bm(gp.M, gp.N, cus, dma, (int)sizeof(T));
     // shallow slabs measure the same as deep ones on the 56x56 layers (within 2 % either
     // way), so they stay a tuning switch: AETHER_GATHER_KC=4
     bool kc4 = false;
@@ -1045,215 +1046,29 @@ __global__ __launch_bounds__(kThreads) void wgrad_gemm(const WgradParams p) {
 }
 
 // ------------------------------------------------------------------------------
-// wgrad, LDS-direct variant (fp32, C and D multiples of 4).  Output tile
-// (128*WKB) k x 64 n per workgroup, each wave owns WKB blocks of 32 k-rows x 64 n;
-// the M range of a split is walked in slabs of 32/WKB rows:
-//   * x and dy slabs loaded straight into LDS (`buffer_load_dwordx4 ... lds`), two
-//     buffers, one barrier per slab, operand reads of step t+1 issued before the
-//     MFMAs of step t;
-//   * slab rows are unpadded; odd rows store the 32-float halves of every 64-float
-//     group swapped, so the two half-waves of an operand read (rows m and m+1) fall
-//     into different halves of the 64 banks;
-//   * WKB = 2 moves half the bytes per flop through L2 and LDS and issues one LDS
-//     read per MFMA instead of 1.5; it is used when K fills at least one 256-row tile;
-//   * dbias fused: the workgroups of k tile 0 also add up the columns of every dy
-//     slab they hold in LDS;
-//   * wave blocks whose 32 k-rows lie entirely past K issue no MFMAs; which wave
-//     gets which block rotates with the split index.
-// ------------------------------------------------------------------------------
-template <int WKB>
-static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma(const WgradParams p) {
-    constexpr int TK = kWgBK * WKB;          // k rows per workgroup tile
-    constexpr int BR = kWgBR / WKB;          // m rows per slab
-    constexpr int RPL = 256 / TK;            // A rows per wave-level load (1024 B): 2 or 1
-    constexpr int CPR = TK / 4;              // chunks per A row
-    constexpr int YL = BR / 16;              // dy loads per wave per slab (4 rows each)
-    __shared__ float lds_a0[BR * TK];
-    __shared__ float lds_a1[BR * TK];
-    __shared__ float lds_y0[kWgBR * kWgBN];  // BR rows used; sized for the dbias epilogue too
-    __shared__ float lds_y1[BR * kWgBN];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int l32 = lane & 31;
-    const int lh = lane >> 5;
-
-    const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
-    const int tiles = p.kt * p.nt;
-    const int split = lid / tiles;
-    const int tile = lid - split * tiles;
-    const int ktile = tile % p.kt;
-    const int kt0 = ktile * TK;
-    const int n0 = (tile / p.kt) * kWgBN;
-    const int m_begin = split * p.m_per_split;
-    int m_end = m_begin + p.m_per_split;
-    if (m_end > p.M) m_end = p.M;
-    const bool do_db = p.want_dbias && (ktile == 0);
-
-    // ---- A: a wave-level load covers RPL slab rows; 4 loads per wave per slab --------
-    const int a_row = lane / CPR;                        // row inside the load block (0 when RPL == 1)
-    const int a_pc = lane % CPR;                         // chunk position written by this lane
-    int a_tap_off[2], a_fx[2], a_fy[2];                  // tap of the chunk fetched for even / odd slab rows
-    bool a_kok[2];
-#pragma unroll
-    for (int q = 0; q < 2; ++q) {
-        int kk = kt0 + 4 * (a_pc ^ (q << 3));
-        unsigned tap, c, fx, fy;
-        p.div_c.divmod((unsigned)kk, tap, c);
-        p.div_fw.divmod(tap, fx, fy);
-        a_kok[q] = kk < p.K;
-        a_fx[q] = (int)fx - p.pH;
-        a_fy[q] = (int)fy - p.pW;
-        a_tap_off[q] = (a_fx[q] * p.W + a_fy[q]) * p.C + (int)c;
-    }
-    // ---- dy: one wave-level load = 4 slab rows x 16 chunks ---------------------------
-    const int y_row = lane >> 4;
-    const int y_lc = (lane & 15) ^ ((y_row & 1) << 3);
-    const int y_n = n0 + 4 * y_lc;
-    const bool y_nok = y_n < p.D;
-
-    const __amdgpu_buffer_rsrc_t rsrc_x =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.x), 0, (int)p.x_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrc_y =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.dy), 0, (int)p.dy_bytes, 0x00020000);
-
-    auto issue = [&](int mb, float* la, float* ly) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int ml = (wave * 4 + i) * RPL + a_row;
-            const int q = RPL == 2 ? a_row : (i & 1);    // row parity
-            const int m = mb + ml;
-            unsigned s, rem, ho, wo;
-            p.div_howo.divmod((unsigned)m, s, rem);
-            p.div_wo.divmod(rem, ho, wo);
-            const int r0 = (int)ho * p.sH, c0 = (int)wo * p.sW;
-            const int pix = (((int)s * p.H + r0) * p.W + c0) * p.C;
-            const unsigned bad = (unsigned)!((m < m_end) & a_kok[q] & ((unsigned)(r0 + a_fx[q]) < (unsigned)p.H) &
-                                             ((unsigned)(c0 + a_fy[q]) < (unsigned)p.W));
-            const unsigned voff = ((unsigned)(pix + a_tap_off[q]) * 4u) | (bad << 31);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + (wave * 4 + i) * 256), 16, (int)voff, 0,
-                                                     0, 0);
-        }
-#pragma unroll
-        for (int i = 0; i < YL; ++i) {
-            const int m = mb + (wave * YL + i) * 4 + y_row;
-            const unsigned bad = (unsigned)!((m < m_end) & y_nok);
-            const unsigned voff = ((unsigned)(m * p.D + y_n) * 4u) | (bad << 31);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_y, (lds_ptr_t)(ly + (wave * YL + i) * 256), 16, (int)voff,
-                                                     0, 0, 0);
-        }
-    };
-
-    // dbias: thread (column tid & 63, row group tid >> 6) adds BR/4 rows of each dy slab;
-    // odd rows keep their 32-float halves swapped
-    float dbsum = 0.f;
-    const int db_col = tid & 63, db_rg = tid >> 6;
-    auto add_columns = [&](const float* ly) {
-#pragma unroll
-        for (int j = 0; j < BR / 4; ++j) dbsum += ly[(db_rg * (BR / 4) + j) * kWgBN + (db_col ^ ((j & 1) << 5))];
-    };
-
-    f16v acc[WKB][2];
-#pragma unroll
-    for (int b = 0; b < WKB; ++b)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[b][j][v] = 0.f;
-
-    // Which k-row blocks this wave multiplies.  Rotated by the split index so that the
-    // idle blocks of a partly filled last k tile do not always land on the same SIMDs.
-    const int wv = (wave + split) & 3;
-    bool active[WKB];
-    int a_rd[WKB];                                       // physical float of this lane's k, rows m = 2t + lh
-#pragma unroll
-    for (int b = 0; b < WKB; ++b) {
-        const int kblk = wv * WKB + b;
-        active[b] = kt0 + kblk * 32 < p.K;               // wave-uniform
-        a_rd[b] = ((kblk * 32) ^ (lh << 5)) + l32;
-    }
-    const int y_rd0 = l32 + (lh << 5);                   // logical n = l32
-    const int y_rd1 = l32 + ((lh ^ 1) << 5);             // logical n = 32 + l32
-    auto slab = [&](int mb, const float* la, const float* ly, float* na, float* ny, bool has_next) {
-        __builtin_amdgcn_s_waitcnt(0);                   // this wave's loads of the slab have landed
-        __syncthreads();
-        if (has_next) issue(mb + BR, na, ny);
-        if (do_db) add_columns(ly);
-        if (active[0]) {
-            float fa[2][WKB], fb0[2], fb1[2];
-#pragma unroll
-            for (int b = 0; b < WKB; ++b) fa[0][b] = la[lh * TK + a_rd[b]];
-            fb0[0] = ly[lh * kWgBN + y_rd0];
-            fb1[0] = ly[lh * kWgBN + y_rd1];
-#pragma unroll
-            for (int t = 0; t < BR / 2; ++t) {
-                if (t + 1 < BR / 2) {
-#pragma unroll
-                    for (int b = 0; b < WKB; ++b) fa[(t + 1) & 1][b] = la[(2 * t + 2 + lh) * TK + a_rd[b]];
-                    fb0[(t + 1) & 1] = ly[(2 * t + 2 + lh) * kWgBN + y_rd0];
-                    fb1[(t + 1) & 1] = ly[(2 * t + 2 + lh) * kWgBN + y_rd1];
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int b = 0; b < WKB; ++b) {
-                    if (b == 0 || active[b]) {
-                        acc[b][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[t & 1][b], fb0[t & 1], acc[b][0], 0, 0, 0);
-                        acc[b][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[t & 1][b], fb1[t & 1], acc[b][1], 0, 0, 0);
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-    };
-
-    if (m_begin < m_end) issue(m_begin, lds_a0, lds_y0);
-    for (int mb = m_begin; mb < m_end; mb += 2 * BR) {
-        slab(mb, lds_a0, lds_y0, lds_a1, lds_y1, mb + BR < m_end);
-        if (mb + BR < m_end) slab(mb + BR, lds_a1, lds_y1, lds_a0, lds_y0, mb + 2 * BR < m_end);
-    }
-
-    const size_t split_stride = (size_t)p.K * p.D + p.D;
-    float* outp = p.out + (size_t)split * split_stride;
-#pragma unroll
-    for (int b = 0; b < WKB; ++b)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int n = n0 + 32 * j + l32;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int k = kt0 + (wv * WKB + b) * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-                if (k < p.K && n < p.D) outp[(size_t)k * p.D + n] = acc[b][j][v];
-            }
-        }
-    if (do_db) {
-        __syncthreads();                                 // the slab buffers are free: reuse one for the 4 row groups
-        lds_y0[db_rg * 64 + db_col] = dbsum;
-        __syncthreads();
-        if (tid < 64 && n0 + tid < p.D)
-            outp[(size_t)p.K * p.D + n0 + tid] = (lds_y0[tid] + lds_y0[64 + tid]) + (lds_y0[128 + tid] + lds_y0[192 + tid]);
-    }
-}
-
-// ------------------------------------------------------------------------------
-// wgrad, LDS-direct, wide-operand variant (fp32, C and D multiples of 4): the
-// default for fp32.  Tile 128 k x 64 n per workgroup, 32-row slabs of m as above,
-// but the A operand is read with ONE `ds_read_b128` per 4 MFMAs: lane i takes the
-// 4 consecutive k values 4i..4i+3 of slab row m and MFMA q (q = 0..3) multiplies
-// the column k = 4i + q, i.e. accumulator q holds the output rows k == q (mod 4).
-// Which rows an MFMA produces is free to choose, and this choice turns the
-// 3 x `ds_read_b32` per 2 MFMAs of wgrad_gemm_dma into 2 reads per 4 MFMAs
-// (a stand-alone loop: 118 -> 132 TFLOP/s).
+// wgrad, LDS-direct (fp32, C and D multiples of 4).  Output tile 128 k x 64 n per
+// workgroup; the M range of a split is walked in slabs of 32 rows:
+//   * x and dy slabs go straight into LDS (`buffer_load_dwordx4 ... lds`), two buffers,
+//     one barrier per slab, operand reads of step t+1 issued before the MFMAs of step t;
+//   * the x operand is read with ONE `ds_read_b128` per 4 MFMAs: lane i takes the 4
+//     consecutive k values 4i..4i+3 of slab row m and MFMA q (q = 0..3) multiplies the
+//     column k = 4i + q, i.e. accumulator q holds the output rows k == q (mod 4).  Which
+//     rows an MFMA produces is free to choose, and this choice needs 2 LDS reads per
+//     4 MFMAs where k-contiguous accumulator rows need 3 `ds_read_b32` per 2 (a
+//     stand-alone loop: 132 against 118 TFLOP/s);
 //   * the 4 waves are (n half) x (parity of the m pair): a wave owns all 128 k rows
 //     of one 32-wide n half and every other pair of slab rows; the two parities
 //     are added through LDS once, after the last slab;
-//   * a last k tile with at most 64 valid rows switches to `ds_read_b64` and two
-//     accumulators (k = 2i + q), so K = 576 multiplies no padding;
-//   * x rows are stored plainly (a 16-lane group reads 256 contiguous bytes);
-//     dy keeps the half-swap of odd rows for its `ds_read_b32`.
+//   * when all of K is at most 64 rows the kernel switches to `ds_read_b64` and two
+//     accumulators (k = 2i + q);
+//   * x rows are stored plainly (a 16-lane group reads 256 contiguous bytes); odd rows
+//     of dy store their 32-float halves swapped, so the two half-waves of a
+//     `ds_read_b32` (rows m and m+1) fall into different halves of the 64 banks;
+//   * dbias fused: the workgroups of k tile 0 also add up the columns of every dy
+//     slab they hold in LDS.
 // ------------------------------------------------------------------------------
 template <int CW>
-static __device__ __forceinline__ void wgrad_wide_body(const WgradParams& p, float* lds_a0, float* lds_a1, float* lds_y0,
+static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, float* lds_a0, float* lds_a1, float* lds_y0,
                                                        float* lds_y1) {
     constexpr int BR = kWgBR;                            // 32 rows of m per slab
     typedef float fcw __attribute__((ext_vector_type(CW)));
@@ -1475,16 +1290,19 @@ static __device__ __forceinline__ void wgrad_wide_body(const WgradParams& p, flo
     }
 }
 
-static __global__ __launch_bounds__(kThreads, 3) void wgrad_gemm_dma_wide(const WgradParams p) {
+static __global__ __launch_bounds__(kThreads, 3) void wgrad_gemm_dma(const WgradParams p) {
     __shared__ float lds_a0[kWgBR * kWgBK];
     __shared__ float lds_a1[kWgBR * kWgBK];
     __shared__ float lds_y0[kWgBR * kWgBN];
     __shared__ float lds_y1[kWgBR * kWgBN];
     static_assert(sizeof(lds_a0) >= 64 * 64 * sizeof(float), "accumulator exchange buffer");
-    const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
-    const int kt0 = ((lid % (p.kt * p.nt)) % p.kt) * kWgBK;
-    if (p.K - kt0 <= 64) wgrad_wide_body<2>(p, lds_a0, lds_a1, lds_y0, lds_y1);   // workgroup-uniform
-    else wgrad_wide_body<4>(p, lds_a0, lds_a1, lds_y0, lds_y1);
+    // The half-width form only when the whole of K fits in it.  As the LAST of several k
+    // tiles it would run at up to twice the pace of its neighbours; the k tiles of a split
+    // share their x and dy rows through L2 only while they move through m together
+    // (measured on K = 576: 722 MB fetched with a fast last tile, 445 MB with an even pace
+    // at 1.5 % more time for its padded MFMAs).
+    if (p.kt == 1 && p.K <= 64) wgrad_dma_body<2>(p, lds_a0, lds_a1, lds_y0, lds_y1);   // workgroup-uniform
+    else wgrad_dma_body<4>(p, lds_a0, lds_a1, lds_y0, lds_y1);
 }
 
 // ------------------------------------------------------------------------------
@@ -1729,17 +1547,7 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     const bool dma16 = sizeof(T) == 2 && va && vy && fits;      // bf16 MFMA kernel, 64-row slabs
     p.x_bytes = (dma || dma16) ? (unsigned)xb : 0u;
     p.dy_bytes = (dma || dma16) ? (unsigned)yb : 0u;
-    // fp32 LDS-direct kernels: the wide-operand kernel unless AETHER_WGRAD_WKB names one
-    // of the `ds_read_b32` kernels (1: 128-row k tiles, 2: 256-row k tiles) for comparison.
-    int wkb_used = 1;
-    bool wide = dma;
-    if (dma) {
-        if (const char* f = getenv("AETHER_WGRAD_WKB")) {
-            const int v = atoi(f);
-            if (v == 1 || v == 2) { wkb_used = v; wide = false; }
-        }
-    }
-    const int kt = cdiv(p.K, kWgBK * wkb_used), nt = cdiv(D, kWgBN);
+    const int kt = cdiv(p.K, kWgBK), nt = cdiv(D, kWgBN);
     const int slab_rows = dma16 ? 64 : kWgBR;
     const int slabs = cdiv(p.M, slab_rows);           // fp32: counted in 32-row units for both tile shapes
     // about two rounds of resident workgroups (3 per CU for the LDS-direct kernel)
@@ -1757,9 +1565,7 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     p.kt = kt; p.nt = nt;
     dim3 grid(kt * nt * splits);
     if (dma16) hipLaunchKernelGGL(wgrad_gemm_dma_bf16, grid, dim3(kThreads), 0, c.stream, p);
-    else if (dma && wide) hipLaunchKernelGGL(wgrad_gemm_dma_wide, grid, dim3(kThreads), 0, c.stream, p);
-    else if (dma && wkb_used == 2) hipLaunchKernelGGL(wgrad_gemm_dma<2>, grid, dim3(kThreads), 0, c.stream, p);
-    else if (dma) hipLaunchKernelGGL(wgrad_gemm_dma<1>, grid, dim3(kThreads), 0, c.stream, p);
+    else if (dma) hipLaunchKernelGGL(wgrad_gemm_dma, grid, dim3(kThreads), 0, c.stream, p);
     else if (va && vy) hipLaunchKernelGGL((wgrad_gemm<T, CE, CE>), grid, dim3(kThreads), 0, c.stream, p);
     else if (va) hipLaunchKernelGGL((wgrad_gemm<T, CE, 1>), grid, dim3(kThreads), 0, c.stream, p);
     else if (vy) hipLaunchKernelGGL((wgrad_gemm<T, 1, CE>), grid, dim3(kThreads), 0, c.stream, p);
