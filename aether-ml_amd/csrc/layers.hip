@@ -72,6 +72,54 @@ static void col_grid(int rows, int C, int* nblk, int* rows_per_block, dim3* grid
     *grid = dim3(nb, cdiv(C, 64));
 }
 
+// Same reduction for C % 4 == 0 and 16-byte aligned rows: a lane owns 4 consecutive
+// columns and reads them with one 16-byte load per row, four rows in flight.  The
+// partials land in the same part[v][block][c] layout.
+typedef float ew_f4 __attribute__((ext_vector_type(4)));
+
+template <int NV, typename F>
+__device__ __forceinline__ void column_partials4(int rows, int C, int rows_per_block, float* __restrict__ part, F f) {
+    __shared__ ew_f4 red4[NV][kEwThreads];
+    const int C4 = C >> 2;
+    const int lanes_c = (C4 < 64 && (64 % C4) == 0) ? C4 : 64;
+    const int sub_rows = 64 / lanes_c;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int c4 = blockIdx.y * 64 + (lane % lanes_c);
+    const int rl = wave * sub_rows + lane / lanes_c;
+    const int nrl = 4 * sub_rows;
+    const int rbeg = blockIdx.x * rows_per_block;
+    int rend = rbeg + rows_per_block;
+    if (rend > rows) rend = rows;
+    ew_f4 acc[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[v] = ew_f4{0.f, 0.f, 0.f, 0.f};
+    if (c4 < C4) {
+        int r = rbeg + rl;
+        for (; r + 3 * nrl < rend; r += 4 * nrl) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) f((size_t)(r + u * nrl) * C4 + c4, c4, acc);
+        }
+        for (; r < rend; r += nrl) f((size_t)r * C4 + c4, c4, acc);
+    }
+#pragma unroll
+    for (int v = 0; v < NV; ++v) red4[v][tid] = acc[v];
+    __syncthreads();
+    if (rl == 0 && c4 < C4) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            ew_f4 s = {0.f, 0.f, 0.f, 0.f};
+            for (int w = 0; w < 4; ++w)
+                for (int sr = 0; sr < sub_rows; ++sr) s += red4[v][w * 64 + sr * lanes_c + (lane % lanes_c)];
+            *reinterpret_cast<ew_f4*>(part + ((size_t)v * gridDim.x + blockIdx.x) * C + 4 * c4) = s;
+        }
+    }
+}
+
+static bool col_vec4(int C, const void* a, const void* b) {
+    return C % 4 == 0 && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) == 0;
+}
+
 // ---- batch norm ------------------------------------------------------------------
 // Sums part[v][b][c] over the blocks b for v = 0, 1.  Launched with 256 threads =
 // 64 channels x 4 block lanes; lane j adds blocks j, j+4, ... with four independent
@@ -110,6 +158,16 @@ __global__ __launch_bounds__(kEwThreads) void bn_stats_partial(const float* __re
                                                               int rpb, float* __restrict__ part) {
     column_partials<2>(rows, C, rpb, part, [&](size_t i, int c, float* acc) {
         float d = x[i] - x[c];
+        acc[0] += d;
+        acc[1] += d * d;
+    });
+}
+
+__global__ __launch_bounds__(kEwThreads) void bn_stats_partial4(const float* __restrict__ x, int rows, int C,
+                                                               int rpb, float* __restrict__ part) {
+    const ew_f4* __restrict__ x4 = reinterpret_cast<const ew_f4*>(x);
+    column_partials4<2>(rows, C, rpb, part, [&](size_t i, int c4, ew_f4* acc) {
+        const ew_f4 d = x4[i] - x4[c4];
         acc[0] += d;
         acc[1] += d * d;
     });
@@ -163,6 +221,19 @@ __global__ __launch_bounds__(kEwThreads) void bn_bwd_partial(const float* __rest
         float g = dy[i];
         acc[0] += g;
         acc[1] += g * (x[i] - mean[c]);
+    });
+}
+
+__global__ __launch_bounds__(kEwThreads) void bn_bwd_partial4(const float* __restrict__ x, const float* __restrict__ dy,
+                                                             const float* __restrict__ mean, int rows, int C, int rpb,
+                                                             float* __restrict__ part) {
+    const ew_f4* __restrict__ x4 = reinterpret_cast<const ew_f4*>(x);
+    const ew_f4* __restrict__ dy4 = reinterpret_cast<const ew_f4*>(dy);
+    const ew_f4* __restrict__ mean4 = reinterpret_cast<const ew_f4*>(mean);
+    column_partials4<2>(rows, C, rpb, part, [&](size_t i, int c4, ew_f4* acc) {
+        const ew_f4 g = dy4[i];
+        acc[0] += g;
+        acc[1] += g * (x4[i] - mean4[c4]);
     });
 }
 
@@ -310,6 +381,7 @@ __global__ __launch_bounds__(1024) void reduce_kernel(const float* __restrict__ 
 // ---- pooling ---------------------------------------------------------------------------
 struct PoolParams {
     int S, H, W, C, Ho, Wo, fH, fW, sH, sW;
+    FastDiv div_c, div_w, div_h, div_sh, div_sw;   // tensors are below 2^31 elements: 32-bit index arithmetic
 };
 
 __global__ void maxpool_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, uint8_t* __restrict__ idx,
@@ -343,28 +415,26 @@ __global__ void maxpool_fwd_kernel(const float* __restrict__ x, float* __restric
 // windows that contain it and whose argmax points at it
 __global__ void maxpool_bwd_kernel(const float* __restrict__ dy, const uint8_t* __restrict__ idx,
                                    float* __restrict__ dx, PoolParams p, int64_t n) {
-    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (; i < n; i += stride) {
-        int c = (int)(i % p.C);
-        int64_t t = i / p.C;
-        int col = (int)(t % p.W);
-        t /= p.W;
-        int row = (int)(t % p.H);
-        int s = (int)(t / p.H);
-        int h_lo = row - p.fH + 1;
-        h_lo = h_lo <= 0 ? 0 : (h_lo + p.sH - 1) / p.sH;
-        int h_hi = row / p.sH;
+    unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+    const unsigned stride = gridDim.x * blockDim.x;
+    for (; i < (unsigned)n; i += stride) {
+        unsigned t, u, c, col, row, s;
+        p.div_c.divmod(i, t, c);
+        p.div_w.divmod(t, u, col);
+        p.div_h.divmod(u, s, row);
+        int h_lo = (int)row - p.fH + 1;
+        h_lo = h_lo <= 0 ? 0 : (int)p.div_sh.div((unsigned)(h_lo + p.sH - 1));
+        int h_hi = (int)p.div_sh.div(row);
         if (h_hi > p.Ho - 1) h_hi = p.Ho - 1;
-        int w_lo = col - p.fW + 1;
-        w_lo = w_lo <= 0 ? 0 : (w_lo + p.sW - 1) / p.sW;
-        int w_hi = col / p.sW;
+        int w_lo = (int)col - p.fW + 1;
+        w_lo = w_lo <= 0 ? 0 : (int)p.div_sw.div((unsigned)(w_lo + p.sW - 1));
+        int w_hi = (int)p.div_sw.div(col);
         if (w_hi > p.Wo - 1) w_hi = p.Wo - 1;
         float acc = 0.f;
         for (int h = h_lo; h <= h_hi; ++h)
             for (int w = w_lo; w <= w_hi; ++w) {
-                size_t o = (((size_t)s * p.Ho + h) * p.Wo + w) * p.C + c;
-                int want = (row - h * p.sH) * p.fW + (col - w * p.sW);
+                const unsigned o = ((s * p.Ho + h) * p.Wo + w) * p.C + c;
+                const int want = ((int)row - h * p.sH) * p.fW + ((int)col - w * p.sW);
                 if ((int)idx[o] == want) acc += dy[o];
             }
         dx[i] = acc;
@@ -488,6 +558,7 @@ static int pool_dims(const char* fn, int S, int H, int W, int C, int fH, int fW,
     p->Ho = (H - fH) / sH + 1;
     p->Wo = (W - fW) / sW + 1;
     if ((int64_t)S * H * W * C >= ((int64_t)1 << 31)) return fail(AETH_E_INVALID, "%s: tensor too large", fn);
+    p->div_c = FastDiv(C); p->div_w = FastDiv(W); p->div_h = FastDiv(H); p->div_sh = FastDiv(sH); p->div_sw = FastDiv(sW);
     return AETH_OK;
 }
 
@@ -528,7 +599,11 @@ int aeth_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta,
     if (rc) return rc;
     float* part = (float*)ws;
     hipStream_t st = ctx().stream;
-    hipLaunchKernelGGL(bn_stats_partial, grid, dim3(kEwThreads), 0, st, x, rows, C, rpb, part);
+    if (col_vec4(C, x, part)) {
+        hipLaunchKernelGGL(bn_stats_partial4, dim3(grid.x, cdiv(C / 4, 64)), dim3(kEwThreads), 0, st, x, rows, C, rpb, part);
+    } else {
+        hipLaunchKernelGGL(bn_stats_partial, grid, dim3(kEwThreads), 0, st, x, rows, C, rpb, part);
+    }
     AETH_LAUNCH_CHECK();
     hipLaunchKernelGGL(bn_stats_final, dim3(cdiv(C, 64)), dim3(256), 0, st, x, part, nblk, rows, C, eps, momentum,
                        running_mean, running_var, save_mean, save_invstd);
@@ -562,7 +637,12 @@ int aeth_bn_bwd_f32(const float* x, const float* dy, const float* gamma, const f
     float* part = (float*)ws;
     float* coef = part + (int64_t)2 * nblk * C;
     hipStream_t st = ctx().stream;
-    hipLaunchKernelGGL(bn_bwd_partial, grid, dim3(kEwThreads), 0, st, x, dy, save_mean, rows, C, rpb, part);
+    if (col_vec4(C, x, dy) && col_vec4(C, save_mean, part)) {
+        hipLaunchKernelGGL(bn_bwd_partial4, dim3(grid.x, cdiv(C / 4, 64)), dim3(kEwThreads), 0, st, x, dy, save_mean, rows, C,
+                           rpb, part);
+    } else {
+        hipLaunchKernelGGL(bn_bwd_partial, grid, dim3(kEwThreads), 0, st, x, dy, save_mean, rows, C, rpb, part);
+    }
     AETH_LAUNCH_CHECK();
     hipLaunchKernelGGL(bn_bwd_final, dim3(cdiv(C, 64)), dim3(256), 0, st, part, nblk, rows, C, gamma, save_invstd,
                        dgamma, dbeta, coef);
