@@ -87,6 +87,7 @@ struct GatherParams {
     unsigned src_bytes;  // extent of src / bt for the buffer descriptors (0: too large, not used)
     unsigned bt_bytes;
     unsigned out_bytes;  // extent of out; 0: no 16-byte stores (too large, N not a multiple of 4, or unaligned)
+    int split_slabs;     // 0, or slabs of K per blockIdx.y: split y writes its partial product at out + y*M*N
     FastDiv div_hw, div_w, div_c, div_tw;
 };
 
@@ -114,21 +115,21 @@ __device__ __forceinline__ int xcd_contiguous_id(int wg, int total) {
 // arithmetic costs measurable matrix time (9 % on the 56x56x64 layer).
 // The bias is added by starting the accumulators from it.
 template <int TM, int TN>
-__device__ __forceinline__ void init_acc(const GatherParams& p, f16v (&acc)[TM][TN], int nw0, int lh) {
-    const bool vec = p.out_bytes != 0 && (reinterpret_cast<uintptr_t>(p.bias) & 15) == 0;
+__device__ __forceinline__ void init_acc(const GatherParams& p, const float* bias, f16v (&acc)[TM][TN], int nw0, int lh) {
+    const bool vec = p.out_bytes != 0 && (reinterpret_cast<uintptr_t>(bias) & 15) == 0;
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int n = nw0 + 32 * j + 8 * q + 4 * lh;
             f4 bv = {0.f, 0.f, 0.f, 0.f};
-            if (p.bias != nullptr) {
+            if (bias != nullptr) {
                 if (vec) {
-                    if (n < p.N) bv = *reinterpret_cast<const f4*>(p.bias + n);
+                    if (n < p.N) bv = *reinterpret_cast<const f4*>(bias + n);
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
-                        if (n + e < p.N) bv[e] = p.bias[n + e];
+                        if (n + e < p.N) bv[e] = bias[n + e];
                 }
             }
 #pragma unroll
@@ -139,12 +140,12 @@ __device__ __forceinline__ void init_acc(const GatherParams& p, f16v (&acc)[TM][
 }
 
 template <int TM, int TN>
-__device__ __forceinline__ void store_tile(const GatherParams& p, const f16v (&acc)[TM][TN], int mw0, int nw0,
-                                           int l32, int lh) {
+__device__ __forceinline__ void store_tile(const GatherParams& p, float* out, const f16v (&acc)[TM][TN], int mw0,
+                                           int nw0, int l32, int lh) {
     typedef unsigned u4 __attribute__((ext_vector_type(4)));
     const bool full_n = nw0 + 32 * TN <= p.N;           // wave-uniform
     const __amdgpu_buffer_rsrc_t rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(p.out, 0, (int)p.out_bytes, 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc(out, 0, (int)p.out_bytes, 0x00020000);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int m = mw0 + 32 * i + l32;
@@ -177,7 +178,7 @@ __device__ __forceinline__ void store_tile(const GatherParams& p, const f16v (&a
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int n = nw0 + 32 * j + 8 * (v >> 2) + 4 * lh + (v & 3);
-                    if (n < p.N) p.out[(size_t)row * p.N + n] = acc[i][j][v];
+                    if (n < p.N) out[(size_t)row * p.N + n] = acc[i][j][v];
                 }
         }
     }
@@ -290,7 +291,7 @@ __global__ __launch_bounds__(kThreads, 3) void gather_gemm(const GatherParams p)
     };
 
     f16v acc[TM][TN];
-    init_acc<TM, TN>(p, acc, n0 + wn0, lh);
+    init_acc<TM, TN>(p, p.bias, acc, n0 + wn0, lh);
 
     if (p.Kpad > 0) {
         load_slab(0);
@@ -321,7 +322,7 @@ __global__ __launch_bounds__(kThreads, 3) void gather_gemm(const GatherParams p)
         }
     }
 
-    store_tile<TM, TN>(p, acc, m0 + wm0, n0 + wn0, l32, lh);
+    store_tile<TM, TN>(p, p.out, acc, m0 + wm0, n0 + wn0, l32, lh);
 }
 
 // ------------------------------------------------------------------------------
@@ -512,8 +513,12 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
         for (int j = 0; j < NL; ++j) issue_load(j, k0, la, lb);
     };
 
+    // split K (launches with few tiles and a long K, e.g. a dense layer on a small batch):
+    // blockIdx.y walks its own range of slabs and writes a partial product; the bias goes
+    // into split 0 and `reduce_splits` adds the partials in order
+    const int split = (int)blockIdx.y;
     f16v acc[TM][TN];
-    init_acc<TM, TN>(p, acc, n0 + wn0, lh);
+    init_acc<TM, TN>(p, split == 0 ? p.bias : nullptr, acc, n0 + wn0, lh);
 
     const int sw7 = (l32 >> SH) & (KC - 1);    // swizzle of every operand row this lane reads
     f4 fa[2][TM], fb[2][TN];                   // operand fragments, double buffered across k groups
@@ -550,14 +555,18 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
         }
     };
 
-    const int nslabs = p.Kpad / BK;
-    if (nslabs > 0) issue(0, lds_a0, lds_b0);
-    for (int s = 0; s < nslabs; s += 2) {
+    int s_begin = 0, nslabs = p.Kpad / BK;
+    if (p.split_slabs > 0) {
+        s_begin = split * p.split_slabs;
+        if (s_begin + p.split_slabs < nslabs) nslabs = s_begin + p.split_slabs;
+    }
+    if (s_begin < nslabs) issue(s_begin * BK, lds_a0, lds_b0);
+    for (int s = s_begin; s < nslabs; s += 2) {
         slab(lds_a0, lds_b0, lds_a1, lds_b1, (s + 1) * BK, s + 1 < nslabs);
         if (s + 1 < nslabs) slab(lds_a1, lds_b1, lds_a0, lds_b0, (s + 2) * BK, s + 2 < nslabs);
     }
 
-    store_tile<TM, TN>(p, acc, m0 + wm0, n0 + wn0, l32, lh);
+    store_tile<TM, TN>(p, p.out + (size_t)split * p.M * p.N, acc, m0 + wm0, n0 + wn0, l32, lh);
 }
 
 // Packs the filter w[fH][fW][C][D] into bt[Npad][Kpad] (k contiguous) for one
@@ -599,6 +608,7 @@ __global__ void pack_filter(const PackParams p) {
 template <typename T, int BM, int BN, int WM, int WN, int KC>
 static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
     dim3 grid(cdiv(gp.M, BM) * cdiv(gp.N, BN));
+    if (gp.split_slabs > 0) grid.y = (unsigned)cdiv(gp.Kpad / (KC * Elem<T>::CE), gp.split_slabs);
     const bool ut = gp.Cs % (KC * Elem<T>::CE) == 0 && gp.K == gp.Kpad && gp.K / gp.Cs <= 32;
     if (ut) hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC>), grid, dim3(kThreads), 0, st, gp);
     else hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, false, KC>), grid, dim3(kThreads), 0, st, gp);
@@ -666,12 +676,110 @@ static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t
     }
 }
 
+// out[i] = sum_s part[s*stride + i] for i < n, in a fixed order: 4 split lanes per
+// output (splits s, s+4, ...), then the 4 lanes in order.  i < n_dw goes to dw,
+// the rest to dbias.
+static __global__ __launch_bounds__(kThreads) void reduce_splits(const float* __restrict__ part, float* __restrict__ dw,
+                                                         float* __restrict__ dbias, int n_dw, int n, int stride,
+                                                         int splits) {
+    __shared__ float red[4][64];
+    const int col = threadIdx.x & 63;
+    const int sl = threadIdx.x >> 6;
+    const int i = blockIdx.x * 64 + col;
+    float s = 0.f;
+    if (i < n) {
+        const float* q = part + i;
+        int k = sl;
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        for (; k + 12 < splits; k += 16) {
+            s0 += q[(size_t)k * stride];
+            s1 += q[(size_t)(k + 4) * stride];
+            s2 += q[(size_t)(k + 8) * stride];
+            s3 += q[(size_t)(k + 12) * stride];
+        }
+        for (; k < splits; k += 4) s0 += q[(size_t)k * stride];
+        s = (s0 + s1) + (s2 + s3);
+    }
+    red[sl][col] = s;
+    __syncthreads();
+    if (sl == 0 && i < n) {
+        float t = (red[0][col] + red[1][col]) + (red[2][col] + red[3][col]);
+        if (i < n_dw) dw[i] = t;
+        else if (dbias != nullptr) dbias[i - n_dw] = t;
+    }
+}
+
+// The same sum for 16-byte aligned partials (stride and n_dw multiples of 4): a thread
+// owns 4 consecutive outputs, 16 split lanes per output add splits j, j+16, ... with
+// four loads in flight, and the lanes are added in lane order.
+static __global__ __launch_bounds__(kThreads) void reduce_splits4(const float* __restrict__ part, float* __restrict__ dw,
+                                                          float* __restrict__ dbias, int n_dw, int n, int stride,
+                                                          int splits) {
+    __shared__ f4 red[16][16];
+    const int cg = threadIdx.x & 15;                     // group of 4 outputs
+    const int sl = threadIdx.x >> 4;                     // split lane
+    const int i = (blockIdx.x * 16 + cg) * 4;
+    f4 s = {0.f, 0.f, 0.f, 0.f};
+    if (i < n) {
+        const float* q = part + i;
+        int k = sl;
+        f4 s0 = s, s1 = s, s2 = s, s3 = s;
+        for (; k + 48 < splits; k += 64) {
+            s0 += *reinterpret_cast<const f4*>(q + (size_t)k * stride);
+            s1 += *reinterpret_cast<const f4*>(q + (size_t)(k + 16) * stride);
+            s2 += *reinterpret_cast<const f4*>(q + (size_t)(k + 32) * stride);
+            s3 += *reinterpret_cast<const f4*>(q + (size_t)(k + 48) * stride);
+        }
+        for (; k < splits; k += 16) s0 += *reinterpret_cast<const f4*>(q + (size_t)k * stride);
+        s = (s0 + s1) + (s2 + s3);
+    }
+    red[sl][cg] = s;
+    __syncthreads();
+    if (sl == 0 && i < n) {
+        f4 t = red[0][cg];
+#pragma unroll
+        for (int j = 1; j < 16; ++j) t += red[j][cg];
+        if (i < n_dw) *reinterpret_cast<f4*>(dw + i) = t;
+        else if (dbias != nullptr) *reinterpret_cast<f4*>(dbias + (i - n_dw)) = t;
+    }
+}
+
 // One gather-GEMM problem: pack the filter into the workspace at `ws_off`, launch.
 struct GatherSetup {
     GatherParams gp;
     PackParams pp;
     int64_t bt_bytes;
+    int nsplit = 1;          // > 1: split K, partial products behind the packed filter in the workspace
+    int64_t part_bytes = 0;
 };
+
+// Split K when the tiles alone would leave most of the chip idle: at most one tile per
+// two CUs and at least 8 slabs of K.  Only for the LDS-direct kernel with 16-byte stores
+// to a dense [M, N] output.  Aim: about two workgroups per CU, at least 4 slabs each.
+template <typename T>
+static void plan_split(GatherSetup& gs, bool vec, int cus) {
+    const GatherParams& g = gs.gp;
+    gs.nsplit = 1;
+    gs.part_bytes = 0;
+    const int64_t lim = (int64_t)1 << 31;
+    const int64_t sb = (int64_t)g.S * g.Hs * g.Ws * g.Cs * (int64_t)sizeof(T);
+    const int64_t ob = (int64_t)g.M * g.N * (int64_t)sizeof(float);
+    const bool dma = vec && sb < lim && gs.bt_bytes < lim;
+    if (!dma || !g.dense_out || g.N % 4 != 0 || ob >= lim || (reinterpret_cast<uintptr_t>(g.out) & 15) != 0) return;
+    if (getenv("AETHER_GATHER_KC") != nullptr) return;       // the tuning switch changes the slab depth
+    const int bn = gather_bn(g.N), bm = gather_bm(g.M, g.N, cus, true, (int)sizeof(T));
+    const int64_t tiles = (int64_t)cdiv(g.M, bm) * cdiv(g.N, bn);
+    const int nslabs = g.Kpad / Elem<T>::BK;
+    if (tiles * 2 > cus || nslabs < 8) return;
+    int n = (int)((2 * (int64_t)cus) / tiles);
+    if (n > nslabs / 4) n = nslabs / 4;
+    if (n > 64) n = 64;
+    if (n < 2) return;
+    const int per = cdiv(nslabs, n);
+    gs.gp.split_slabs = per;
+    gs.nsplit = cdiv(nslabs, per);
+    gs.part_bytes = round_up((int64_t)gs.nsplit * ob, 256);
+}
 
 template <typename T>
 static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
@@ -697,8 +805,16 @@ static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
         AETH_LAUNCH_CHECK();
     }
     if (gs.gp.M > 0 && gs.gp.N > 0) {
+        float* real_out = gs.gp.out;
+        if (gs.nsplit > 1) gs.gp.out = reinterpret_cast<float*>(ws + ws_off + round_up(gs.bt_bytes, 256));
         launch_gather<T>(gs.gp, vec, c.prop.multiProcessorCount, c.stream);
         AETH_LAUNCH_CHECK();
+        if (gs.nsplit > 1) {
+            const int n = gs.gp.M * gs.gp.N;
+            hipLaunchKernelGGL(reduce_splits4, dim3(cdiv(n, 64)), dim3(kThreads), 0, c.stream,
+                               (const float*)gs.gp.out, real_out, (float*)nullptr, n, n, n, gs.nsplit);
+            AETH_LAUNCH_CHECK();
+        }
     }
     return AETH_OK;
 }
@@ -748,8 +864,10 @@ int conv_fprop_impl(const char* fn, const T* x, const T* w, const float* bias, f
     pk.xa = 0; pk.xs = 1; pk.ya = 0; pk.ys = 1; pk.transposed = 0;
     pk.N = D; pk.K = g.K; pk.Npad = (int)round_up(D, 64); pk.Kpad = g.Kpad;
     gs.bt_bytes = (int64_t)pk.Npad * pk.Kpad * sizeof(T);
+    g.split_slabs = 0;
+    plan_split<T>(gs, C % Elem<T>::CE == 0, ctx().prop.multiProcessorCount);
     void* ws;
-    rc = workspace(gs.bt_bytes, &ws);
+    rc = workspace(round_up(gs.bt_bytes, 256) + gs.part_bytes, &ws);
     if (rc) return rc;
     return run_gather<T>(gs, (char*)ws, 0, C % Elem<T>::CE == 0);
 }
@@ -800,7 +918,9 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
             pk.xa = xmax; pk.xs = -sH; pk.ya = ymax; pk.ys = -sW; pk.transposed = 1;
             pk.N = C; pk.K = g.K; pk.Npad = (int)round_up(C, 64); pk.Kpad = g.Kpad;
             gs.bt_bytes = round_up((int64_t)pk.Npad * pk.Kpad * sizeof(T), 256);
-            total_bytes += gs.bt_bytes;
+            g.split_slabs = 0;
+            plan_split<T>(gs, D % Elem<T>::CE == 0, ctx().prop.multiProcessorCount);
+            total_bytes += gs.bt_bytes + gs.part_bytes;
             sets.push_back(gs);
         }
     }
@@ -811,7 +931,7 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
     for (auto& gs : sets) {
         rc = run_gather<T>(gs, (char*)ws, off, D % Elem<T>::CE == 0);
         if (rc) return rc;
-        off += gs.bt_bytes;
+        off += gs.bt_bytes + gs.part_bytes;
     }
     return AETH_OK;
 }
@@ -1481,74 +1601,6 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma_bf16(const Wgr
         __syncthreads();
         if (tid < 64 && n0 + tid < p.D)
             outp[(size_t)p.K * p.D + n0 + tid] = (lds_db[tid] + lds_db[64 + tid]) + (lds_db[128 + tid] + lds_db[192 + tid]);
-    }
-}
-
-// out[i] = sum_s part[s*stride + i] for i < n, in a fixed order: 4 split lanes per
-// output (splits s, s+4, ...), then the 4 lanes in order.  i < n_dw goes to dw,
-// the rest to dbias.
-static __global__ __launch_bounds__(kThreads) void reduce_splits(const float* __restrict__ part, float* __restrict__ dw,
-                                                         float* __restrict__ dbias, int n_dw, int n, int stride,
-                                                         int splits) {
-    __shared__ float red[4][64];
-    const int col = threadIdx.x & 63;
-    const int sl = threadIdx.x >> 6;
-    const int i = blockIdx.x * 64 + col;
-    float s = 0.f;
-    if (i < n) {
-        const float* q = part + i;
-        int k = sl;
-        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-        for (; k + 12 < splits; k += 16) {
-            s0 += q[(size_t)k * stride];
-            s1 += q[(size_t)(k + 4) * stride];
-            s2 += q[(size_t)(k + 8) * stride];
-            s3 += q[(size_t)(k + 12) * stride];
-        }
-        for (; k < splits; k += 4) s0 += q[(size_t)k * stride];
-        s = (s0 + s1) + (s2 + s3);
-    }
-    red[sl][col] = s;
-    __syncthreads();
-    if (sl == 0 && i < n) {
-        float t = (red[0][col] + red[1][col]) + (red[2][col] + red[3][col]);
-        if (i < n_dw) dw[i] = t;
-        else if (dbias != nullptr) dbias[i - n_dw] = t;
-    }
-}
-
-// The same sum for 16-byte aligned partials (stride and n_dw multiples of 4): a thread
-// owns 4 consecutive outputs, 16 split lanes per output add splits j, j+16, ... with
-// four loads in flight, and the lanes are added in lane order.
-static __global__ __launch_bounds__(kThreads) void reduce_splits4(const float* __restrict__ part, float* __restrict__ dw,
-                                                          float* __restrict__ dbias, int n_dw, int n, int stride,
-                                                          int splits) {
-    __shared__ f4 red[16][16];
-    const int cg = threadIdx.x & 15;                     // group of 4 outputs
-    const int sl = threadIdx.x >> 4;                     // split lane
-    const int i = (blockIdx.x * 16 + cg) * 4;
-    f4 s = {0.f, 0.f, 0.f, 0.f};
-    if (i < n) {
-        const float* q = part + i;
-        int k = sl;
-        f4 s0 = s, s1 = s, s2 = s, s3 = s;
-        for (; k + 48 < splits; k += 64) {
-            s0 += *reinterpret_cast<const f4*>(q + (size_t)k * stride);
-            s1 += *reinterpret_cast<const f4*>(q + (size_t)(k + 16) * stride);
-            s2 += *reinterpret_cast<const f4*>(q + (size_t)(k + 32) * stride);
-            s3 += *reinterpret_cast<const f4*>(q + (size_t)(k + 48) * stride);
-        }
-        for (; k < splits; k += 16) s0 += *reinterpret_cast<const f4*>(q + (size_t)k * stride);
-        s = (s0 + s1) + (s2 + s3);
-    }
-    red[sl][cg] = s;
-    __syncthreads();
-    if (sl == 0 && i < n) {
-        f4 t = red[0][cg];
-#pragma unroll
-        for (int j = 1; j < 16; ++j) t += red[j][cg];
-        if (i < n_dw) *reinterpret_cast<f4*>(dw + i) = t;
-        else if (dbias != nullptr) *reinterpret_cast<f4*>(dbias + (i - n_dw)) = t;
     }
 }
 

@@ -28,6 +28,9 @@ CASES = [
     (2, 9, 9, 6, 10, 3, 3, 1, 1, "same"),        # C,D not multiples of 4
     (2, 9, 9, 5, 7, 1, 1, 2, 2, "same"),         # 1x1 stride 2: dgrad classes without taps
     (40, 16, 16, 3, 32, 3, 3, 1, 1, "same"),     # config-1 channel counts
+    (2, 4, 4, 256, 64, 3, 3, 1, 1, "same"),      # one tile, K = 2304: fprop splits K
+    (1, 8, 16, 512, 256, 1, 1, 1, 1, "valid"),   # dense-like, batch 128, K = 512: fprop and dgrad split K
+    (3, 6, 6, 128, 96, 3, 3, 1, 1, "valid"),     # split K with a ragged last split (36 slabs)
 ]
 
 
