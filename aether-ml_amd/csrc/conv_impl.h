@@ -955,6 +955,7 @@ struct WgradParams {
     int fW, sH, sW, pH, pW;
     int m_per_split;     // multiple of 32
     int kt, nt;          // output tiles along k and n
+    int cw;              // fp32 LDS-direct kernel: floats of k per lane of an operand read (4, 2 or 1)
     unsigned x_bytes, dy_bytes;   // extents for the buffer descriptors (LDS-direct kernel)
     // moving 32 rows of m ahead: 32 = qs*Ho*Wo + qh*Wo + qw.  step_c = qw*sW, step_r = qh*sH;
     // byte offset += inc0 (+ inc1 when the column wraps) (+ inc2 when the row wraps)
@@ -1191,6 +1192,11 @@ template <int CW>
 static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, float* lds_a0, float* lds_a1, float* lds_y0,
                                                        float* lds_y1) {
     constexpr int BR = kWgBR;                            // 32 rows of m per slab
+    // CW = 1: any channel count.  A lane loads ONE float per slab row (`buffer_load_dword ... lds`),
+    // slab rows are 32 floats, the k tile is 32 wide and there is one accumulator.
+    constexpr int RS = CW == 1 ? 32 : kWgBK;             // floats per x slab row in LDS
+    constexpr int KSTEP = CW == 1 ? 1 : 4;               // k per lane of an x load
+    constexpr int TKW = 32 * KSTEP;                      // k tile width
     typedef float fcw __attribute__((ext_vector_type(CW)));
     typedef unsigned u4 __attribute__((ext_vector_type(4)));
     const int tid = threadIdx.x;
@@ -1207,7 +1213,7 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
     const int split = lid / tiles;
     const int tile = lid - split * tiles;
     const int ktile = tile % p.kt;
-    const int kt0 = ktile * kWgBK;
+    const int kt0 = ktile * TKW;
     const int n0 = (tile / p.kt) * kWgBN;
     const int m_begin = split * p.m_per_split;
     int m_end = m_begin + p.m_per_split;
@@ -1252,7 +1258,7 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
     unsigned tap_lo, tap_hi;                             // guard-bit constants, see test below
     int a_tap4;
     {
-        const int kk = kt0 + 4 * (lane & 31);
+        const int kk = kt0 + KSTEP * (lane & 31);
         unsigned tap, c, fx, fy;
         p.div_c.divmod((unsigned)kk, tap, c);
         p.div_fw.divmod(tap, fx, fy);
@@ -1299,7 +1305,10 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
         const unsigned z = (tap_lo - perm_rc[i]) | (perm_rc[i] + tap_hi);
         const unsigned w = z | (z << 16);                // bit 31: row or column out of the image
         const unsigned voff = (w & 0x80000000u) | (unsigned)(perm_off[i] + a_tap4);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + (wave * 4 + i) * 256), 16, (int)voff, 0, 0, 0);
+        if constexpr (CW == 1)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + (wave * 4 + i) * 2 * RS), 4, (int)voff, 0, 0, 0);
+        else
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + (wave * 4 + i) * 2 * RS), 16, (int)voff, 0, 0, 0);
     };
     auto load_y = [&](int i, int mb, float* ly, int live) {
         const int m = mb + (wave_u * 2 + i) * 4;         // scalar
@@ -1331,7 +1340,7 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
         __syncthreads();
         fcw fa[2];
         float fb[2];
-        fa[0] = *reinterpret_cast<const fcw*>(la + row0 * kWgBK + CW * l32);
+        fa[0] = *reinterpret_cast<const fcw*>(la + row0 * RS + CW * l32);
         fb[0] = ly[row0 * kWgBN + (y_rd ^ (lh << 5))];
         // no branch in here: without a next slab the loads are issued with offsets past
         // the descriptors and fetch nothing
@@ -1341,7 +1350,7 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
 #pragma unroll
         for (int t = 0; t < BR / 4; ++t) {
             if (t + 1 < BR / 4) {
-                fa[(t + 1) & 1] = *reinterpret_cast<const fcw*>(la + (row0 + 4 * t + 4) * kWgBK + CW * l32);
+                fa[(t + 1) & 1] = *reinterpret_cast<const fcw*>(la + (row0 + 4 * t + 4) * RS + CW * l32);
                 fb[(t + 1) & 1] = ly[(row0 + 4 * t + 4) * kWgBN + (y_rd ^ (lh << 5))];
             }
             if (t >= 1 && t <= 4) load_x(t - 1, na);
@@ -1421,7 +1430,9 @@ static __global__ __launch_bounds__(kThreads, 3) void wgrad_gemm_dma(const Wgrad
     // share their x and dy rows through L2 only while they move through m together
     // (measured on K = 576: 722 MB fetched with a fast last tile, 445 MB with an even pace
     // at 1.5 % more time for its padded MFMAs).
-    if (p.kt == 1 && p.K <= 64) wgrad_dma_body<2>(p, lds_a0, lds_a1, lds_y0, lds_y1);   // workgroup-uniform
+    // p.cw (workgroup-uniform): 1 for channel counts that are not multiples of 4
+    if (p.cw == 1) wgrad_dma_body<1>(p, lds_a0, lds_a1, lds_y0, lds_y1);
+    else if (p.cw == 2) wgrad_dma_body<2>(p, lds_a0, lds_a1, lds_y0, lds_y1);
     else wgrad_dma_body<4>(p, lds_a0, lds_a1, lds_y0, lds_y1);
 }
 
@@ -1630,11 +1641,13 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     const bool va = (C % CE == 0), vy = (D % CE == 0);
     const int64_t xb = (int64_t)S * H * W * C * (int64_t)sizeof(T), yb = (int64_t)p.M * D * (int64_t)sizeof(T);
     const bool fits = xb < ((int64_t)1 << 31) && yb < ((int64_t)1 << 31);
-    const bool dma = sizeof(T) == 4 && va && vy && fits;
+    // fp32: the LDS-direct kernel takes any C (one float per lane and load when C % 4 != 0)
+    const bool dma = sizeof(T) == 4 && vy && fits;
     const bool dma16 = sizeof(T) == 2 && va && vy && fits;      // bf16 MFMA kernel, 64-row slabs
     p.x_bytes = (dma || dma16) ? (unsigned)xb : 0u;
     p.dy_bytes = (dma || dma16) ? (unsigned)yb : 0u;
-    const int kt = cdiv(p.K, kWgBK), nt = cdiv(D, kWgBN);
+    p.cw = !va ? 1 : (p.K <= 64 ? 2 : 4);
+    const int kt = cdiv(p.K, (dma && !va) ? 32 : kWgBK), nt = cdiv(D, kWgBN);
     const int slab_rows = dma16 ? 64 : kWgBR;
     const int slabs = cdiv(p.M, slab_rows);           // fp32: counted in 32-row units for both tile shapes
     // about two rounds of resident workgroups (3 per CU for the LDS-direct kernel)
