@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("AETHER_HIP_LIB", os.path.join(_HERE, "lib", "libaether_hip.so"))
 
-_i, _f, _p, _i64 = C.c_int, C.c_float, C.c_void_p, C.c_int64
+_i, _f, _p, _i64, _d = C.c_int, C.c_float, C.c_void_p, C.c_int64, C.c_double
 _conv_dims = [_i] * 11
 
 # name -> argument types (all return int)
@@ -58,6 +58,12 @@ SIGNATURES = {
     "aeth_softmax_cce_bwd_f32": [_p, _p, _f, _p, _i, _i],
     "aeth_adam_f32": [_p, _p, _p, _p, _i64, _f, _f, _f, _f, _i],
     "aeth_adam_multi_f32": [_i, _p, _p, _p, _p, _p, _f, _f, _f, _f, _i],
+    "aeth_adam_state_step": [_p, _d, _d, _d, _d],
+    "aeth_adam_multi_dev_f32": [_i, _p, _p, _p, _p, _p, _f, _f, _f, _p],
+    "aeth_graph_begin": [],
+    "aeth_graph_end": [C.POINTER(_p)],
+    "aeth_graph_launch": [_p],
+    "aeth_graph_destroy": [_p],
 }
 
 AETH_E_INVALID = -1

@@ -453,10 +453,13 @@ def _sparse_labels(y_true):
 
 
 _label_cache = [None, None]     # (bytes of the last label batch, its device copy)
+_label_buffer = [None]          # while a step is being recorded: the buffer its kernels read labels from
 
 
 def _device_labels(y_true):
     """Labels on the device; the forward and backward pass of one step share the upload."""
+    if _label_buffer[0] is not None:
+        return _label_buffer[0]
     y = _sparse_labels(y_true)
     key = y.tobytes()
     if _label_cache[0] != key:
@@ -468,6 +471,29 @@ def _device_labels(y_true):
 class Loss:
     def remember_trainable_layers(self, trainable_layers):
         self.trainable_layers = trainable_layers
+
+    # ``calculate`` in two halves for Model.train_step: ``launch`` queues the loss kernel,
+    # ``finish`` reads its result.  With backward and the optimizer queued in between, the
+    # host never waits in the middle of a step.  Only for losses that offer
+    # ``forward_launch`` and when no regulariser is active (its sums must see the weights
+    # before the update).
+    def can_defer(self):
+        if not hasattr(self, "forward_launch"):
+            return False
+        return not any(l.weight_regularizer_l1 > 0 or l.weight_regularizer_l2 > 0 or l.bias_regularizer_l1 > 0
+                       or l.bias_regularizer_l2 > 0 for l in self.trainable_layers)
+
+    def launch(self, output, y, *, training=True):
+        return self.forward_launch(output, y, training)
+
+    def finish(self, pending, *, include_regularization=False):
+        sample_losses = self.forward_finish(pending)
+        data_loss = np.mean(sample_losses)
+        self.accumulated_sum += np.sum(sample_losses)
+        self.accumulated_count += len(sample_losses)
+        if not include_regularization:
+            return data_loss
+        return data_loss, self.regularization_loss()
 
     def calculate(self, output, y, *, include_regularization=False, training=True):
         sample_losses = self.forward(output, y, training)
@@ -512,6 +538,9 @@ class Loss_CategoricalCrossEntropy(Loss):
         self.label_smoothing = label_smoothing
 
     def forward(self, y_pred, y_true, training=True):
+        return self.forward_finish(self.forward_launch(y_pred, y_true, training))
+
+    def forward_launch(self, y_pred, y_true, training=True):
         y_pred = as_device(y_pred, _F32)
         rows, K = y_pred.shape
         labels = _device_labels(y_true)
@@ -519,6 +548,10 @@ class Loss_CategoricalCrossEntropy(Loss):
         # per-sample loss and row argmax side by side: one read-back for both
         buf = DeviceTensor(2 * rows, _F32)
         _ck(_L().aeth_cce_fwd_f32(y_pred.ptr, labels.ptr, ls, buf.ptr, buf.ptr + 4 * rows, rows, K))
+        return buf, rows, y_pred
+
+    def forward_finish(self, pending):
+        buf, rows, y_pred = pending
         host = buf.get()
         y_pred._cache = {"argmax": host[rows:].view(np.int32)}
         return host[:rows]
@@ -599,3 +632,43 @@ class Optimizer_Adam:
     def post_update_parameters(self):
         self._flush()
         self.iterations += 1
+
+    # -- recorded steps: the step number lives on the device -----------------------------
+    def device_state(self):
+        """{iterations, beta_1^iterations, beta_2^iterations, lr} as 4 doubles on the device,
+        brought in line with ``self.iterations`` whenever eager steps moved it."""
+        if getattr(self, "_state", None) is None:
+            self._state = DeviceTensor(4, np.float64)
+            self._state_iterations = None
+        if self._state_iterations != self.iterations:
+            b1, b2 = float(np.float32(self.beta_1)), float(np.float32(self.beta_2))   # what the kernels receive
+            self._state.set(np.array([self.iterations, b1 ** self.iterations, b2 ** self.iterations,
+                                      self.current_learning_rate], dtype=np.float64))
+            self._state_iterations = self.iterations
+        return self._state
+
+    def record_update(self, layers):
+        """Queue one whole optimizer step (pre_update, every layer, post_update) in a form
+        that can be replayed: learning rate and bias corrections come from device_state()."""
+        import ctypes as C
+        state = self._state
+        b1, b2 = float(np.float32(self.beta_1)), float(np.float32(self.beta_2))
+        _ck(_L().aeth_adam_state_step(state.ptr, float(self.learning_rate), float(self.decay), b1, b2))
+        batch = []
+        for layer in layers:
+            batch.append((layer.weights, layer.dweights, layer.weight_momentums, layer.weight_cache))
+            batch.append((layer.biases, layer.dbiases, layer.bias_momentums, layer.bias_cache))
+        while batch:
+            part, batch = batch[:32], batch[32:]
+            n = len(part)
+            arr = lambda k: (C.c_void_p * n)(*[t[k].ptr for t in part])
+            sizes = (C.c_int64 * n)(*[t[0].size for t in part])
+            _ck(_L().aeth_adam_multi_dev_f32(n, arr(0), arr(1), arr(2), arr(3), sizes, self.beta_1, self.beta_2,
+                                             self.epsilon, state.ptr))
+
+    def replayed(self):
+        """Host bookkeeping after a recorded step has run once more."""
+        if self.decay:
+            self.current_learning_rate = self.learning_rate * (1. / (1. + self.decay * self.iterations))
+        self.iterations += 1
+        self._state_iterations = self.iterations

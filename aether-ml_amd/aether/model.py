@@ -118,21 +118,119 @@ class Model:
         if validation_data is not None:
             self.evaluate(*validation_data, batch_size=batch_size)
 
+    # -- recorded steps ------------------------------------------------------------------
+    def record_steps(self, enabled=True):
+        """Replay training steps from a recording instead of launching every kernel from
+        Python (no counterpart in the reference).  The first step of a batch shape runs
+        normally, the second is recorded as a HIP graph, later ones replay it: one host
+        call per step.  Same kernels, same order, same results; the step number and the
+        learning rate live on the device.  Falls back to normal steps for models the
+        recording cannot express (dropout masks drawn on the host, active regularisers,
+        anything but Adam with the fused softmax / cross-entropy output)."""
+        self._record = bool(enabled)
+        if not enabled:
+            self._drop_recordings()
+
+    def _drop_recordings(self):
+        from . import _lib
+        for rec in getattr(self, "_recordings", {}).values():
+            if rec.get("graph"):
+                _lib.check(_lib.lib().aeth_graph_destroy(rec["graph"]))
+        self._recordings = {}
+
+    def _can_record(self):
+        from .layers import Layer_Dropout, Layer_Dropout_Spatial, Optimizer_Adam
+        if self.softmax_classifier_output is None or not isinstance(self.optimizer, Optimizer_Adam):
+            return False
+        if not self.loss.can_defer():
+            return False
+        if any(isinstance(layer, (Layer_Dropout, Layer_Dropout_Spatial)) for layer in self.layers):
+            return False                                 # their masks are drawn and uploaded by the host every step
+        return all(hasattr(l, "weight_cache") for l in self.trainable_layers)     # Adam state exists
+
+    def _recorded_step(self, batch_X, batch_y):
+        import ctypes as C
+        from . import _lib, layers as L
+        from .tensor import DeviceTensor
+        labels = L._sparse_labels(batch_y)
+        key = (tuple(batch_X.shape), labels.shape[0])
+        recs = self.__dict__.setdefault("_recordings", {})
+        rec = recs.get(key)
+        if rec is None:
+            # first step of this shape: a normal one (lazy initialisations, workspace sizes)
+            recs[key] = {"graph": None}
+            return None
+        lib = _lib.lib()
+        if rec["graph"] is None:
+            rec["x"] = DeviceTensor(batch_X.shape, np.float32)
+            rec["labels"] = DeviceTensor(labels.shape, np.int32)
+            self.optimizer.device_state()
+            _lib.check(lib.aeth_graph_begin())
+            L._label_buffer[0] = rec["labels"]
+            try:
+                output = self.forward(rec["x"], training=True)
+                rec["pending"] = self.loss.launch(output, batch_y, training=True)
+                rec["output"] = output
+                self.backward(output, batch_y)
+                self.optimizer.record_update(self.trainable_layers)
+            finally:
+                L._label_buffer[0] = None
+                handle = C.c_void_p()
+                rc = lib.aeth_graph_end(C.byref(handle))
+            _lib.check(rc)
+            rec["graph"] = handle
+            # what the layers point at after this step (output, dinputs, dweights, ...):
+            # replays fill the same buffers, so the attributes are put back after steps
+            # that ran in between (an evaluation, a step of another shape)
+            holders = list(self.layers) + [self.softmax_classifier_output, self.softmax_classifier_output.activation,
+                                           self.loss]
+            rec["bindings"] = [(obj, name, val) for obj in holders for name, val in vars(obj).items()
+                               if isinstance(val, DeviceTensor)]
+        # feed the recording and replay it
+        self.optimizer.device_state()
+        if isinstance(batch_X, DeviceTensor):
+            _lib.check(lib.aeth_memcpy_d2d(rec["x"].ptr, batch_X.ptr, rec["x"].nbytes))
+        else:
+            rec["x"].set(np.asarray(batch_X, dtype=np.float32))
+        rec["labels"].set(labels)
+        _lib.check(lib.aeth_graph_launch(rec["graph"]))
+        self.optimizer.replayed()
+        if self.layers[-1].__dict__.get("output") is not rec["output"]:
+            for obj, name, val in rec["bindings"]:
+                setattr(obj, name, val)
+        data_loss, regularization_loss = self.loss.finish(rec["pending"], include_regularization=True)
+        loss = data_loss + regularization_loss
+        predictions = self.output_layer_activation.predictions(rec["output"])
+        accuracy = self.accuracy.calculate(predictions, batch_y)
+        return loss, data_loss, regularization_loss, accuracy
+
     def train_step(self, batch_X, batch_y):
         """One iteration of the loop body of ``train`` (CNN_model_cupy.py:107-126):
         forward, loss, accuracy, backward, Adam.  Returns (loss, data_loss,
         regularization_loss, accuracy)."""
+        if getattr(self, "_record", False) and self._can_record():
+            result = self._recorded_step(batch_X, batch_y)
+            if result is not None:
+                return result
         output = self.forward(batch_X, training=True)
-        data_loss, regularization_loss = self.loss.calculate(output, batch_y, include_regularization=True,
-                                                             training=True)
-        loss = data_loss + regularization_loss
-        predictions = self.output_layer_activation.predictions(output)
-        accuracy = self.accuracy.calculate(predictions, batch_y)
+        # The loss kernel is queued here and read after backward and the update have been
+        # queued too, so the device never idles while the host prepares the backward pass.
+        defer = self.loss.can_defer()
+        if defer:
+            pending = self.loss.launch(output, batch_y, training=True)
+        else:
+            data_loss, regularization_loss = self.loss.calculate(output, batch_y, include_regularization=True,
+                                                                 training=True)
         self.backward(output, batch_y)
         self.optimizer.pre_update_parameters()
         for layer in self.trainable_layers:
             self.optimizer.update_parameters(layer)
         self.optimizer.post_update_parameters()
+        if defer:
+            data_loss, regularization_loss = self.loss.finish(pending, include_regularization=True)
+        loss = data_loss + regularization_loss
+        predictions = self.output_layer_activation.predictions(output)
+        accuracy = self.accuracy.calculate(predictions, batch_y)
         return loss, data_loss, regularization_loss, accuracy
 
     def forward(self, X, training):

@@ -360,6 +360,44 @@ __global__ void adam_multi_kernel(const AdamTable tb, float lr, float b1, float 
     }
 }
 
+// Adam with its step state on the device, for callers that replay a recorded step and
+// cannot pass a new step number from the host.  state = {t, beta1^t, beta2^t, lr_t} as
+// doubles.  adam_state_step advances it by one step; adam_multi_dev_kernel reads it.
+__global__ void adam_state_step_kernel(double* __restrict__ state, double lr, double decay, double b1, double b2) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        const double t = state[0];
+        state[3] = decay != 0.0 ? lr * (1.0 / (1.0 + decay * t)) : lr;   // learning rate of this step
+        state[0] = t + 1.0;
+        state[1] *= b1;
+        state[2] *= b2;
+    }
+}
+
+__global__ void adam_multi_dev_kernel(const AdamTable tb, float b1, float b2, float eps,
+                                      const double* __restrict__ state) {
+    const float lr = (float)state[3];
+    const float c1 = (float)(1.0 - state[1]);
+    const float c2 = (float)(1.0 - state[2]);
+    const int t = blockIdx.y;
+    float* __restrict__ theta = tb.theta[t];
+    const float* __restrict__ g = tb.grad[t];
+    float* __restrict__ m = tb.m[t];
+    float* __restrict__ v = tb.v[t];
+    const int64_t n = tb.n[t];
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        float gi = g[i];
+        float mi = b1 * m[i] + (1.0f - b1) * gi;
+        float vi = b2 * v[i] + (1.0f - b2) * (gi * gi);
+        m[i] = mi;
+        v[i] = vi;
+        float mh = mi / c1;
+        float vh = vi / c2;
+        theta[i] += -lr * mh / (sqrtf(vh) + eps);
+    }
+}
+
 // single block: out[0] = sum |x| or sum x^2, summed in a fixed tree
 __global__ __launch_bounds__(1024) void reduce_kernel(const float* __restrict__ x, int64_t n, int mode,
                                                       float* __restrict__ out) {
@@ -797,6 +835,39 @@ int aeth_adam_multi_f32(int count, float* const* host_theta, const float* const*
     if (bx > 256) bx = 256;
     hipLaunchKernelGGL(adam_multi_kernel, dim3(bx, count), dim3(kEwThreads), 0, ctx().stream, tb, lr, beta1, beta2,
                        eps, c1, c2);
+    AETH_LAUNCH_CHECK();
+    return AETH_OK;
+}
+
+int aeth_adam_state_step(double* state, double lr, double decay, double beta1, double beta2) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(state != nullptr);
+    hipLaunchKernelGGL(adam_state_step_kernel, dim3(1), dim3(64), 0, ctx().stream, state, lr, decay, beta1, beta2);
+    AETH_LAUNCH_CHECK();
+    return AETH_OK;
+}
+
+int aeth_adam_multi_dev_f32(int count, float* const* host_theta, const float* const* host_grad, float* const* host_m,
+                            float* const* host_v, const int64_t* host_n, float beta1, float beta2, float eps,
+                            const double* state) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(count >= 1 && count <= kAdamMax && state != nullptr);
+    AETH_CHECK_ARG(host_theta && host_grad && host_m && host_v && host_n);
+    AdamTable tb;
+    int64_t nmax = 0;
+    for (int i = 0; i < kAdamMax; ++i) {
+        const int j = i < count ? i : 0;
+        AETH_CHECK_ARG(host_n[j] >= 0);
+        AETH_CHECK_ARG(host_n[j] == 0 || (host_theta[j] && host_grad[j] && host_m[j] && host_v[j]));
+        tb.theta[i] = host_theta[j]; tb.grad[i] = host_grad[j]; tb.m[i] = host_m[j]; tb.v[i] = host_v[j];
+        tb.n[i] = i < count ? host_n[j] : 0;
+        if (tb.n[i] > nmax) nmax = tb.n[i];
+    }
+    if (nmax == 0) return AETH_OK;
+    int bx = (int)((nmax + 4 * kEwThreads - 1) / (4 * kEwThreads));
+    if (bx > 256) bx = 256;
+    hipLaunchKernelGGL(adam_multi_dev_kernel, dim3(bx, count), dim3(kEwThreads), 0, ctx().stream, tb, beta1, beta2, eps,
+                       state);
     AETH_LAUNCH_CHECK();
     return AETH_OK;
 }

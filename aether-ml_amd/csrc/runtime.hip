@@ -23,9 +23,14 @@ int fail(int code, const char* fmt, ...) {
     return code;
 }
 
+static bool g_recording = false;                       // a step is being recorded on the stream
+static bool recording_open() { return g_recording; }
+
 int workspace(int64_t bytes, void** out) {
     Context& c = ctx();
     if (bytes > c.ws_bytes) {
+        if (recording_open())
+            return fail(AETH_E_STATE, "the workspace would have to grow while a step is being recorded: run the step once first");
         int64_t want = round_up(bytes + bytes / 4, 1 << 20);
         if (c.ws) {
             AETH_HIP(hipStreamSynchronize(c.stream));
@@ -47,6 +52,11 @@ struct Pool {
     std::unordered_map<void*, size_t> live;            // pointer -> rounded size
     std::map<size_t, std::vector<void*>> free_blocks;  // rounded size -> idle blocks
     size_t cached_bytes = 0;
+    // Blocks handed out while a step is being recorded belong to the recording: its
+    // replays write to them, so a block the caller frees stays out of circulation until
+    // the recording is destroyed.  pointer -> "the caller has freed it".
+    std::unordered_map<void*, bool> reserved;
+    std::vector<void*>* recording = nullptr;           // blocks of the recording in progress
 
     static size_t rounded(int64_t bytes) {
         size_t b = bytes <= 0 ? 256 : (size_t)bytes;
@@ -141,6 +151,7 @@ int aeth_malloc(void** host_out_ptr, int64_t bytes) {
         it->second.pop_back();
         g_pool.cached_bytes -= sz;
         g_pool.live[p] = sz;
+        if (g_pool.recording) { g_pool.recording->push_back(p); g_pool.reserved[p] = false; }
         *host_out_ptr = p;
         return AETH_OK;
     }
@@ -157,6 +168,7 @@ int aeth_malloc(void** host_out_ptr, int64_t bytes) {
                     "aeth_malloc: hipMalloc(%lld bytes) -> %s", (long long)bytes, hipGetErrorString(e));
     }
     g_pool.live[p] = sz;
+    if (g_pool.recording) { g_pool.recording->push_back(p); g_pool.reserved[p] = false; }
     *host_out_ptr = p;
     return AETH_OK;
 }
@@ -166,6 +178,12 @@ int aeth_free(void* p) {
     if (!p) return AETH_OK;
     auto it = g_pool.live.find(p);
     if (it == g_pool.live.end()) return fail(AETH_E_INVALID, "aeth_free: %p was not returned by aeth_malloc", p);
+    auto rs = g_pool.reserved.find(p);
+    if (rs != g_pool.reserved.end()) {
+        if (rs->second) return fail(AETH_E_INVALID, "aeth_free: %p freed twice", p);
+        rs->second = true;                              // returned to the pool by aeth_graph_destroy
+        return AETH_OK;
+    }
     size_t sz = it->second;
     g_pool.live.erase(it);
     g_pool.free_blocks[sz].push_back(p);
@@ -175,6 +193,7 @@ int aeth_free(void* p) {
 
 int aeth_memcpy_h2d(void* dst, const void* host_src, int64_t bytes) {
     AETH_REQUIRE_INIT();
+    if (recording_open()) return fail(AETH_E_STATE, "aeth_memcpy_h2d: waits for the device, not possible while recording");
     AETH_CHECK_ARG(bytes >= 0);
     if (bytes == 0) return AETH_OK;
     AETH_CHECK_ARG(dst != nullptr && host_src != nullptr);
@@ -186,6 +205,7 @@ int aeth_memcpy_h2d(void* dst, const void* host_src, int64_t bytes) {
 
 int aeth_memcpy_d2h(void* host_dst, const void* src, int64_t bytes) {
     AETH_REQUIRE_INIT();
+    if (recording_open()) return fail(AETH_E_STATE, "aeth_memcpy_d2h: waits for the device, not possible while recording");
     AETH_CHECK_ARG(bytes >= 0);
     if (bytes == 0) return AETH_OK;
     AETH_CHECK_ARG(host_dst != nullptr && src != nullptr);
@@ -215,8 +235,101 @@ int aeth_fill_f32(float* dst, float value, int64_t n) {
     return AETH_OK;
 }
 
+// ---- recorded steps (HIP graphs) -----------------------------------------------------
+struct Recording {
+    hipGraphExec_t exec = nullptr;
+    std::vector<void*> blocks;
+};
+static Recording* g_open_recording = nullptr;
+#define AETH_NOT_RECORDING(fn)                                                                    \
+    do {                                                                                          \
+        if (g_open_recording) return fail(AETH_E_STATE, fn ": waits for the device, not possible while recording"); \
+    } while (0)
+
+int aeth_graph_begin(void) {
+    AETH_REQUIRE_INIT();
+    if (g_open_recording) return fail(AETH_E_STATE, "aeth_graph_begin: a recording is already open");
+    Context& c = ctx();
+    AETH_HIP(hipStreamSynchronize(c.stream));
+    Recording* r = new Recording();
+    hipError_t e = hipStreamBeginCapture(c.stream, hipStreamCaptureModeRelaxed);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        delete r;
+        return fail(AETH_E_HIP, "aeth_graph_begin: hipStreamBeginCapture -> %s", hipGetErrorString(e));
+    }
+    g_open_recording = r;
+    g_recording = true;
+    g_pool.recording = &r->blocks;
+    return AETH_OK;
+}
+
+static void release_recording_blocks(Recording* r) {
+    for (void* p : r->blocks) {
+        auto rs = g_pool.reserved.find(p);
+        if (rs == g_pool.reserved.end()) continue;
+        const bool freed = rs->second;
+        g_pool.reserved.erase(rs);
+        if (freed) {
+            auto it = g_pool.live.find(p);
+            if (it != g_pool.live.end()) {
+                const size_t sz = it->second;
+                g_pool.live.erase(it);
+                g_pool.free_blocks[sz].push_back(p);
+                g_pool.cached_bytes += sz;
+            }
+        }
+    }
+    r->blocks.clear();
+}
+
+int aeth_graph_end(void** host_out_graph) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(host_out_graph != nullptr);
+    *host_out_graph = nullptr;
+    if (!g_open_recording) return fail(AETH_E_STATE, "aeth_graph_end: no recording is open");
+    Recording* r = g_open_recording;
+    g_open_recording = nullptr;
+    g_recording = false;
+    g_pool.recording = nullptr;
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx().stream, &graph);
+    if (e == hipSuccess) {
+        e = hipGraphInstantiate(&r->exec, graph, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(graph);
+    }
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        release_recording_blocks(r);
+        delete r;
+        return fail(AETH_E_HIP, "aeth_graph_end: %s", hipGetErrorString(e));
+    }
+    *host_out_graph = r;
+    return AETH_OK;
+}
+
+int aeth_graph_launch(void* graph) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(graph != nullptr);
+    if (g_open_recording) return fail(AETH_E_STATE, "aeth_graph_launch: a recording is open");
+    AETH_HIP(hipGraphLaunch(static_cast<Recording*>(graph)->exec, ctx().stream));
+    return AETH_OK;
+}
+
+int aeth_graph_destroy(void* graph) {
+    AETH_REQUIRE_INIT();
+    if (!graph) return AETH_OK;
+    Recording* r = static_cast<Recording*>(graph);
+    AETH_HIP(hipStreamSynchronize(ctx().stream));
+    if (r->exec) (void)hipGraphExecDestroy(r->exec);
+    release_recording_blocks(r);
+    delete r;
+    return AETH_OK;
+}
+
 int aeth_sync(void) {
     AETH_REQUIRE_INIT();
+    AETH_NOT_RECORDING("aeth_sync");
     AETH_HIP(hipStreamSynchronize(ctx().stream));
     return AETH_OK;
 }

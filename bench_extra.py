@@ -127,22 +127,33 @@ def train_step(steps, warmup):
     np.random.seed(0)
     X = aether.DeviceTensor.from_numpy(np.random.rand(128, 32, 32, 3).astype(np.float32))
     y = np.random.randint(0, 10, 128)
-    model = build_cnn(aether)
-    model.loss.new_pass()
-    model.accuracy.new_pass()
-    for _ in range(warmup):
-        model.train_step(X, y)
-    _lib.sync()
-    times = []
-    for _ in range(steps):
-        t0 = time.perf_counter()
-        loss, data_loss, reg, acc = model.train_step(X, y)
+
+    def timed(model):
+        model.loss.new_pass()
+        model.accuracy.new_pass()
+        for _ in range(warmup):
+            model.train_step(X, y)
         _lib.sync()
-        times.append(time.perf_counter() - t0)
-    med = float(np.median(times))
-    return {"ms_per_step_median": med * 1e3, "images_per_sec": 128.0 / med, "batch": 128,
-            "last_loss": float(loss), "note": "forward + loss + accuracy + backward + Adam, batch resident in HBM, "
-                                              "includes the per-step scalar read-backs"}
+        times = []
+        for _ in range(steps):
+            t0 = time.perf_counter()
+            loss, data_loss, reg, acc = model.train_step(X, y)
+            _lib.sync()
+            times.append(time.perf_counter() - t0)
+        return float(np.median(times)), float(loss)
+
+    np.random.seed(0)
+    med, loss = timed(build_cnn(aether))
+    np.random.seed(0)
+    recorded = build_cnn(aether)
+    recorded.record_steps(True)
+    med_rec, loss_rec = timed(recorded)
+    return {"ms_per_step_median": med * 1e3, "images_per_sec": 128.0 / med, "batch": 128, "last_loss": loss,
+            "recorded_steps": {"ms_per_step_median": med_rec * 1e3, "images_per_sec": 128.0 / med_rec,
+                               "last_loss": loss_rec,
+                               "note": "Model.record_steps(True): the step replayed from a HIP graph, one host call"},
+            "note": "forward + loss + accuracy + backward + Adam, batch resident in HBM, "
+                    "includes the per-step scalar read-backs"}
 
 
 def run(steps, warmup):

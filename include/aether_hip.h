@@ -176,6 +176,34 @@ int aeth_adam_multi_f32(int count, float* const* host_theta, const float* const*
                         float* const* host_m, float* const* host_v, const int64_t* host_n,
                         float lr, float beta1, float beta2, float eps, int t);
 
+/* Adam with the step state on the device, for recorded steps (below) that cannot take a
+ * new step number from the host: state[4] doubles = {iterations, beta1^iterations,
+ * beta2^iterations, learning rate of the current step}.  aeth_adam_state_step does
+ * pre_update_parameters :693-697 and post_update_parameters :735-736 for one step
+ * (learning-rate decay from the old iteration count, then iterations += 1 and the two
+ * powers advance); aeth_adam_multi_dev_f32 is aeth_adam_multi_f32 reading lr and the bias
+ * corrections 1 - beta^iterations from `state`. */
+int aeth_adam_state_step(double* state, double lr, double decay, double beta1, double beta2);
+int aeth_adam_multi_dev_f32(int count, float* const* host_theta, const float* const* host_grad,
+                            float* const* host_m, float* const* host_v, const int64_t* host_n,
+                            float beta1, float beta2, float eps, const double* state);
+
+/* ---- recorded steps -------------------------------------------------------------------
+ * No counterpart in the reference (CuPy launches every kernel from Python each step).
+ * Between aeth_graph_begin and aeth_graph_end the library's stream records instead of
+ * executing: every launch and device-to-device copy of the calls made in between
+ * becomes a node of a HIP graph; nothing runs.  aeth_graph_launch replays the whole
+ * sequence with one host call.  Blocks returned by aeth_malloc while recording stay
+ * reserved for the graph until aeth_graph_destroy, also after aeth_free, because replays
+ * write to them.  While recording, calls that wait for the device (aeth_sync, host
+ * copies, a workspace that has to grow) fail with AETH_E_STATE: run the step once
+ * normally first.  Arguments are frozen at recording time: feed new data by copying
+ * into the buffers the recorded step reads. */
+int aeth_graph_begin(void);
+int aeth_graph_end(void** host_out_graph);
+int aeth_graph_launch(void* graph);
+int aeth_graph_destroy(void* graph);
+
 #ifdef __cplusplus
 }
 #endif

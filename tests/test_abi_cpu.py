@@ -56,6 +56,8 @@ def test_ctypes_table_matches_header(lib):
                 assert ct in (ctypes.c_void_p, ctypes.c_char_p) or hasattr(ct, "contents"), (name, decl)
             elif decl.startswith("float"):
                 assert ct is ctypes.c_float, (name, decl)
+            elif decl.startswith("double"):
+                assert ct is ctypes.c_double, (name, decl)
             elif decl.startswith("int64_t"):
                 assert ct is ctypes.c_int64, (name, decl)
             else:

@@ -234,3 +234,75 @@ def test_load_parameters_accepts_cupy_wrapped_float64_checkpoints(tmp_path):
     want = O.softmax(O.dense_forward(a.reshape(5, -1), params[2][0], params[2][1], dtype=np.float64))
     from tests import abi
     abi.close(got, want, rtol=1e-3)
+
+
+def test_recorded_steps_equal_eager_steps():
+    """Model.record_steps: a step replayed from a HIP graph must give what the same
+    step gives when every kernel is launched from Python.  Same kernels in the same
+    order, so the comparison is exact.  The replays are interleaved with eager work
+    of the same model (an evaluation, a step of another batch shape, a
+    synchronisation), every replay is checked, and learning-rate decay is on so that
+    the step state kept on the device matters."""
+    import aether
+    from aether import _lib
+
+    def make():
+        np.random.seed(3)
+        m = build_model(aether, hw=16)
+        m.optimizer.decay = 1e-2
+        m.loss.new_pass()
+        m.accuracy.new_pass()
+        return m
+
+    rng = np.random.RandomState(5)
+    Xs = [rng.rand(32, 16, 16, 3).astype(np.float32) for _ in range(3)]
+    ys = [rng.randint(0, 10, 32) for _ in range(3)]
+    Xodd, yodd = rng.rand(16, 16, 16, 3).astype(np.float32), rng.randint(0, 10, 16)
+    eager, rec = make(), make()
+    rec.record_steps(True)
+    for step in range(9):
+        X, y = Xs[step % 3], ys[step % 3]
+        a = eager.train_step(X, y)
+        b = rec.train_step(X, y)
+        assert a == b, "step %d: eager %r, recorded %r" % (step, a, b)
+        assert eager.optimizer.iterations == rec.optimizer.iterations
+        assert eager.optimizer.current_learning_rate == rec.optimizer.current_learning_rate
+        for la, lb in zip(eager.trainable_layers, rec.trainable_layers):
+            assert np.array_equal(np.asarray(la.weights), np.asarray(lb.weights)), "weights differ after step %d" % step
+            assert np.array_equal(np.asarray(la.dweights), np.asarray(lb.dweights)), "layer.dweights is stale"
+        if step == 4:
+            for m in (eager, rec):
+                m.evaluate(Xs[0], ys[0], batch_size=16)
+            _lib.sync()
+        if step == 6:
+            assert eager.train_step(Xodd, yodd) == rec.train_step(Xodd, yodd)      # another shape: runs eagerly
+    assert len([r for r in rec._recordings.values() if r.get("graph")]) == 1
+    rec.record_steps(False)
+    assert eager.train_step(Xs[0], ys[0]) == rec.train_step(Xs[0], ys[0])
+
+
+def test_recording_refuses_calls_that_wait_for_the_device():
+    import ctypes as C
+    import aether
+    from aether import _lib
+    lib = _lib.lib()
+    t = aether.DeviceTensor.zeros(8)
+    _lib.sync()
+    _lib.check(lib.aeth_graph_begin())
+    try:
+        assert lib.aeth_sync() == _lib.AETH_E_STATE
+        host = np.zeros(8, np.float32)
+        assert lib.aeth_memcpy_d2h(host.ctypes.data, t.ptr, 32) == _lib.AETH_E_STATE
+        assert lib.aeth_graph_begin() == _lib.AETH_E_STATE
+        _lib.check(lib.aeth_fill_f32(t.ptr, 2.0, 8))
+    finally:
+        g = C.c_void_p()
+        rc = lib.aeth_graph_end(C.byref(g))
+    _lib.check(rc)
+    assert np.all(t.get() == 0)                     # recorded, not run
+    for _ in range(3):
+        _lib.check(lib.aeth_fill_f32(t.ptr, 1.0, 8))
+        _lib.check(lib.aeth_graph_launch(g))
+        assert np.all(t.get() == 2)
+    _lib.check(lib.aeth_graph_destroy(g))
+    assert lib.aeth_graph_end(C.byref(g)) == _lib.AETH_E_STATE
