@@ -83,3 +83,57 @@ def test_full_size_conv(cfg):
     dyd.set(dy1)
     _lib.check(L.aeth_conv_wgrad_f32(xd.ptr, dyd.ptr, dw.ptr, None, *dims))
     abi.close(dw_h, first + dw.get().astype(np.float64), rms_scaled=True)
+
+
+@pytest.mark.parametrize("cfg", FULL, ids=lambda c: c[0] + "_bf16")
+def test_full_size_conv_bf16(cfg):
+    """The bf16-input kernels at the same full-size shapes.  Inputs are rounded to bf16
+    on the device; the oracle gets the same rounded values, so the fp32 tolerance
+    applies (bf16 products are exact in fp32, accumulation is fp32).  The adjoint
+    identities hold for the rounded operands: <y - b, r(dy)> = <r(x), dx> when dx is
+    computed from r(dy) and r(w), and likewise for dW."""
+    from aether import _lib
+    from aether.tensor import DeviceTensor
+    from tests import abi
+    name, S, H, W, C, D, fH, fW, st, pad = cfg
+    stride = (st, st)
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((S, H, W, C), dtype=np.float32)
+    w = (rng.standard_normal((fH, fW, C, D), dtype=np.float32) * np.float32(np.sqrt(2.0 / (fH * fW * C))))
+    b = rng.standard_normal(D, dtype=np.float32)
+    dims, yshape = abi.conv_dims(x.shape, w.shape, stride, pad)
+    dy = rng.standard_normal(yshape, dtype=np.float32)
+    xr, wr, dyr = (O.round_to_bf16(a) for a in (x, w, dy))
+    L = _lib.lib()
+    xd, wd, dyd = (abi.to_bf16_device(a) for a in (x, w, dy))
+    bd = DeviceTensor.from_numpy(b)
+    y = DeviceTensor.full(yshape, np.nan)
+    dx = DeviceTensor.full(x.shape, np.nan)
+    dw = DeviceTensor.full(w.shape, np.nan)
+    db = DeviceTensor.full(D, np.nan)
+    _lib.check(L.aeth_conv_fprop_bf16(xd.ptr, wd.ptr, bd.ptr, y.ptr, *dims))
+    _lib.check(L.aeth_conv_dgrad_bf16(dyd.ptr, wd.ptr, dx.ptr, *dims))
+    _lib.check(L.aeth_conv_wgrad_bf16(xd.ptr, dyd.ptr, dw.ptr, db.ptr, *dims))
+    y_h, dx_h, dw_h, db_h = y.get(), dx.get(), dw.get(), db.get()
+    assert np.all(np.isfinite(y_h)) and np.all(np.isfinite(dx_h)) and np.all(np.isfinite(dw_h))
+
+    for s in (0, S // 2 + 1, S - 1):
+        abi.close(y_h[s:s + 1], O.conv_fprop(xr[s:s + 1], wr, b, stride, pad, dtype=np.float64))
+        abi.close(dx_h[s:s + 1], O.conv_dgrad(dyr[s:s + 1], wr, (H, W), stride, pad, dtype=np.float64))
+
+    lhs = float(np.sum((y_h.astype(np.float64) - b.astype(np.float64)) * dyr))
+    rhs_x = float(np.sum(xr.astype(np.float64) * dx_h))
+    rhs_w = float(np.sum(wr.astype(np.float64) * dw_h))
+    scale = float(np.sqrt(np.sum(y_h.astype(np.float64) ** 2)) * np.sqrt(np.sum(dyr.astype(np.float64) ** 2)))
+    assert abs(lhs - rhs_x) <= 1e-6 * scale, (lhs, rhs_x)
+    assert abs(lhs - rhs_w) <= 1e-6 * scale, (lhs, rhs_w)
+    abi.close(db_h, np.sum(dyr.astype(np.float64), axis=(0, 1, 2)), rms_scaled=True)
+
+    # one-sample-supported gradient: wgrad of that sample alone
+    s = S - 1
+    dy1 = np.zeros_like(dy)
+    dy1[s] = dy[s]
+    dyd1 = abi.to_bf16_device(dy1)
+    _lib.check(L.aeth_conv_wgrad_bf16(xd.ptr, dyd1.ptr, dw.ptr, db.ptr, *dims))
+    want = O.conv_wgrad(xr[s:s + 1], dyr[s:s + 1], (fH, fW), stride, pad, dtype=np.float64)
+    abi.close(dw.get(), want, rms_scaled=True)
