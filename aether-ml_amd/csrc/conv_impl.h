@@ -355,7 +355,11 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 //     those hide each other's set-up, first loads and epilogue.  With KC = 4 a wave-level
 //     load covers 16 rows, chunk c of row r lives at c ^ ((r >> 2) & 3), and a 16-lane
 //     read group (16 rows x 64 B) again covers the 64 banks exactly once.
-template <typename T, int BM, int BN, int WM, int WN, bool UT, int KC>
+//   * NLOOP: for a K of at most two slabs and several n tiles (1x1 convolutions onto many
+//     channels: the HBM-bound case, where a one-tile workgroup is mostly set-up).  The
+//     workgroup keeps its A tile, both slabs, in the two A buffers and walks over all n
+//     tiles: one set-up and one fetch of A per m tile instead of one per output tile.
+template <typename T, int BM, int BN, int WM, int WN, bool UT, int KC, bool NLOOP>
 __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p) {
     static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
     static_assert(KC == 8 || KC == 4, "slab rows of 8 or 4 chunks");
@@ -385,8 +389,8 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
     const int wn0 = (wave / (BM / WM)) * WN;
     const int ntile = (p.N + BN - 1) / BN;
     const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
-    const int m0 = (lid / ntile) * BM;
-    const int n0 = (lid % ntile) * BN;
+    const int m0 = NLOOP ? lid * BM : (lid / ntile) * BM;
+    int n0 = NLOOP ? 0 : (lid % ntile) * BN;
 
     const int lr = lane / KC;                  // row inside a load block
     // logical chunk this lane fetches: (lane % KC) ^ swizzle(row).  KC == 8: the 8-row
@@ -438,11 +442,14 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
         }
     }
     unsigned b_off[BL];
+    auto set_b_off = [&]() {
 #pragma unroll
-    for (int i = 0; i < BL; ++i) {
-        const int k4 = k4e ^ (((wave * BL + i) & 1) ? ODD : 0);
-        b_off[i] = (unsigned)(((n0 + (wave * BL + i) * RPL + lr) * p.Kpad + CE * k4) * (int)sizeof(T));
-    }
+        for (int i = 0; i < BL; ++i) {
+            const int k4 = k4e ^ (((wave * BL + i) & 1) ? ODD : 0);
+            b_off[i] = (unsigned)(((n0 + (wave * BL + i) * RPL + lr) * p.Kpad + CE * k4) * (int)sizeof(T));
+        }
+    };
+    set_b_off();
 
     const __amdgpu_buffer_rsrc_t rsrc_a =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.src), 0, (int)p.src_bytes, 0x00020000);
@@ -555,6 +562,63 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
         }
     };
 
+    if constexpr (NLOOP) {
+        // A (at most two slabs) stays in the two A buffers; the B slabs of all n tiles pass
+        // through the two B buffers as one double-buffered sequence f = (n tile, slab):
+        // the loads of step f+1 fly while step f is multiplied.
+        const int nslabs = p.Kpad / BK;                // 1 or 2
+        const int total = ntile * nslabs;
+        prep(0);
+#pragma unroll
+        for (int j = 0; j < AL; ++j) issue_load(j, 0, lds_a0, lds_b0);
+        if (nslabs > 1) {
+            prep(BK);
+#pragma unroll
+            for (int j = 0; j < AL; ++j) issue_load(j, BK, lds_a1, lds_b1);
+        }
+#pragma unroll
+        for (int j = AL; j < NL; ++j) issue_load(j, 0, lds_a0, lds_b0);         // B of step 0
+        // one step; `last_slab`: this slab completes an n tile
+        auto step = [&](int f, const f4* la, const f4* lb, f4* nb, bool last_slab) __attribute__((always_inline)) {
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+            read_frags(la, lb, 0, 0);
+            const int tile_now = n0;
+            if (f + 1 < total) {
+                const int fn = f + 1;
+                const int nt_next = nslabs == 2 ? fn >> 1 : fn;
+                const int k0_next = nslabs == 2 ? (fn & 1) * BK : 0;
+                n0 = nt_next * BN;
+                set_b_off();
+#pragma unroll
+                for (int j = AL; j < NL; ++j) issue_load(j, k0_next, lds_a0, nb);
+            }
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                if (g < G - 1) read_frags(la, lb, g + 1, (g + 1) & 1);
+                __builtin_amdgcn_sched_barrier(0);
+                mma_group(g & 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (last_slab) {
+                store_tile<TM, TN>(p, p.out, acc, m0 + wm0, tile_now + wn0, l32, lh);
+                if (f + 1 < total) init_acc<TM, TN>(p, p.bias, acc, n0 + wn0, lh);
+            }
+        };
+        if (nslabs == 2) {
+            for (int f = 0; f < total; f += 2) {
+                step(f, lds_a0, lds_b0, lds_b1, false);
+                step(f + 1, lds_a1, lds_b1, lds_b0, true);
+            }
+        } else {
+            for (int f = 0; f < total; f += 2) {
+                step(f, lds_a0, lds_b0, lds_b1, true);
+                if (f + 1 < total) step(f + 1, lds_a0, lds_b1, lds_b0, true);
+            }
+        }
+        return;
+    }
+
     int s_begin = 0, nslabs = p.Kpad / BK;
     if (p.split_slabs > 0) {
         s_begin = split * p.split_slabs;
@@ -610,8 +674,17 @@ static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
     dim3 grid(cdiv(gp.M, BM) * cdiv(gp.N, BN));
     if (gp.split_slabs > 0) grid.y = (unsigned)cdiv(gp.Kpad / (KC * Elem<T>::CE), gp.split_slabs);
     const bool ut = gp.Cs % (KC * Elem<T>::CE) == 0 && gp.K == gp.Kpad && gp.K / gp.Cs <= 32;
-    if (ut) hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC>), grid, dim3(kThreads), 0, st, gp);
-    else hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, false, KC>), grid, dim3(kThreads), 0, st, gp);
+    // short K, several n tiles: one workgroup per m tile walks the n tiles (128 x 64 tiles only)
+    if constexpr (BM == 128 && BN == 64 && KC == 8) {
+        if (gp.split_slabs == 0 && gp.Kpad / (KC * Elem<T>::CE) <= 2 && gp.N > BN && getenv("AETHER_GATHER_NLOOP_OFF") == nullptr) {
+            grid.x = (unsigned)cdiv(gp.M, BM);
+            if (ut) hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, true>), grid, dim3(kThreads), 0, st, gp);
+            else hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, false, KC, true>), grid, dim3(kThreads), 0, st, gp);
+            return;
+        }
+    }
+    if (ut) hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false>), grid, dim3(kThreads), 0, st, gp);
+    else hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, false, KC, false>), grid, dim3(kThreads), 0, st, gp);
 }
 
 // kc4: shallow slabs (4 chunks of k per row) for the LDS-direct kernel where the tile allows it

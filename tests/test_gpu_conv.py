@@ -31,6 +31,9 @@ CASES = [
     (2, 4, 4, 256, 64, 3, 3, 1, 1, "same"),      # one tile, K = 2304: fprop splits K
     (1, 8, 16, 512, 256, 1, 1, 1, 1, "valid"),   # dense-like, batch 128, K = 512: fprop and dgrad split K
     (3, 6, 6, 128, 96, 3, 3, 1, 1, "valid"),     # split K with a ragged last split (36 slabs)
+    (8, 48, 48, 64, 256, 1, 1, 1, 1, "valid"),   # K of two slabs, 4 n tiles: one workgroup walks the n tiles
+    (8, 48, 48, 32, 192, 1, 1, 1, 1, "valid"),   # same with one slab, 3 n tiles
+    (8, 48, 48, 48, 136, 1, 1, 1, 1, "valid"),   # same, padded second slab, ragged last n tile
 ]
 
 
@@ -127,3 +130,36 @@ def test_bad_arguments_are_errors_not_crashes():
         _lib.check(L.aeth_conv_wgrad_f32(t.ptr, t.ptr, t.ptr, None, 1, 2, 2, 1, 1, 1, 1, 0, 1, 0, 0))
     with pytest.raises(ValueError):
         _lib.check(L.aeth_free(12345))
+
+
+def _random_cases(n, seed):
+    """Seeded random geometries: channel counts around the vector widths and tile edges,
+    strides 1-3, filters 1-5, both paddings, batch sizes that leave ragged row tiles."""
+    r = np.random.RandomState(seed)
+    out = []
+    chans = [1, 2, 3, 4, 5, 8, 12, 16, 20, 31, 32, 33, 48, 64, 72, 96, 128, 136]
+    while len(out) < n:
+        fH, fW = int(r.choice([1, 2, 3, 3, 3, 5])), int(r.choice([1, 2, 3, 3, 3, 4]))
+        sH, sW = int(r.choice([1, 1, 1, 2, 3])), int(r.choice([1, 1, 1, 2, 3]))
+        H, W = int(r.randint(fH, 20)), int(r.randint(fW, 20))
+        C, D = int(r.choice(chans)), int(r.choice(chans))
+        S = int(r.choice([1, 2, 3, 5, 9, 17]))
+        pad = "same" if r.rand() < 0.5 else "valid"
+        if S * H * W * C * D * fH * fW > 3e8:
+            continue
+        out.append((S, H, W, C, D, fH, fW, sH, sW, pad))
+    return out
+
+
+@pytest.mark.parametrize("case", _random_cases(48, 20240607), ids=lambda c: "x".join(str(v) for v in c))
+def test_random_geometries(case):
+    """All three directions on random geometries (the fixed list above names the paths;
+    this one looks for the combinations nobody thought of)."""
+    from tests import abi
+    S, H, W, C, D, fH, fW, sH, sW, pad = case
+    x, w, b, dy = _case(case, 11)
+    abi.close(abi.fprop(x, w, b, (sH, sW), pad), O.conv_fprop(x, w, b, (sH, sW), pad, dtype=np.float64))
+    abi.close(abi.dgrad(dy, w, x.shape, (sH, sW), pad), O.conv_dgrad(dy, w, (H, W), (sH, sW), pad, dtype=np.float64))
+    dw, db = abi.wgrad(x, dy, w.shape, (sH, sW), pad)
+    abi.close(dw, O.conv_wgrad(x, dy, (fH, fW), (sH, sW), pad, dtype=np.float64), rms_scaled=True)
+    abi.close(db, O.conv_dbias(dy, dtype=np.float64), rms_scaled=True)
