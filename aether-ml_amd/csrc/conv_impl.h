@@ -1267,9 +1267,17 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
     constexpr int BR = kWgBR;                            // 32 rows of m per slab
     // CW = 1: any channel count.  A lane loads ONE float per slab row (`buffer_load_dword ... lds`),
     // slab rows are 32 floats, the k tile is 32 wide and there is one accumulator.
-    constexpr int RS = CW == 1 ? 32 : kWgBK;             // floats per x slab row in LDS
+    // CW = 6: a 192-wide k tile (K = 576 is 3 of them: no padded rows where 128-wide tiles
+    // pad 10 %).  Accumulators 0..3 hold k = 4i + q of the first 128 columns, 4 and 5 hold
+    // k = 128 + 2i + (q - 4) of the last 64 (one `ds_read_b128` and one `ds_read_b64`, both
+    // aligned).  64 KB of LDS and 96 accumulator registers: 2 workgroups per CU, which a
+    // stand-alone loop measured at 135 TFLOP/s against 132 for the 128-wide form at 3.
+    constexpr int RS = CW == 1 ? 32 : (CW == 6 ? 192 : kWgBK);   // floats per x slab row in LDS
     constexpr int KSTEP = CW == 1 ? 1 : 4;               // k per lane of an x load
-    constexpr int TKW = 32 * KSTEP;                      // k tile width
+    constexpr int CPR = RS / KSTEP;                      // load lanes per slab row (32 or 48)
+    constexpr int TKW = RS;                              // k tile width
+    constexpr int XL = CPR / 8;                          // x loads per wave per slab: 8 rows x CPR lanes / 64
+    constexpr int NA = CW == 6 ? 4 : CW;                 // accumulators fed by the first (wide) operand read
     typedef float fcw __attribute__((ext_vector_type(CW)));
     typedef unsigned u4 __attribute__((ext_vector_type(4)));
     const int tid = threadIdx.x;
@@ -1293,7 +1301,8 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
     if (m_end > p.M) m_end = p.M;
     const bool do_db = p.want_dbias && (ktile == 0);
 
-    // ---- x: one wave-level load = 2 slab rows x 32 chunks; 4 loads per wave per slab ----
+    // ---- x: a wave loads 8 slab rows with XL loads; lane l of load j is load lane 64 j + l ----
+    //      of those rows: row (64 j + l) / CPR, chunk (64 j + l) % CPR
     // fp32 MFMA and ordinary vector (and scalar) instructions of a wave share its issue
     // slots, so the address work per load is kept to a handful of instructions:
     //  * lane l keeps the image position of slab row 8*wave + (l & 7) -- the 8 rows this
@@ -1327,24 +1336,28 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
         st_off += c1 ? p.inc0 + p.inc1 : p.inc0;
         st_off += c2 ? p.inc2 : 0;
     };
-    // per-lane tap constants
-    unsigned tap_lo, tap_hi;                             // guard-bit constants, see test below
-    int a_tap4;
-    {
-        const int kk = kt0 + KSTEP * (lane & 31);
+    // per-lane tap constants, one set per load (with 32 lanes per row they coincide)
+    unsigned tap_lo[XL], tap_hi[XL];                     // guard-bit constants, see test below
+    int a_tap4[XL];
+    int perm_idx[XL];                                    // byte index of the lane that tracks this load's row
+#pragma unroll
+    for (int j = 0; j < XL; ++j) {
+        const int flat = 64 * j + lane;
+        const int row = flat / CPR, chunk = flat % CPR;
+        perm_idx[j] = row * 4;
+        const int kk = kt0 + KSTEP * chunk;
         unsigned tap, c, fx, fy;
         p.div_c.divmod((unsigned)kk, tap, c);
         p.div_fw.divmod(tap, fx, fy);
-        a_tap4 = (((int)fx * p.W + (int)fy) * p.C + (int)c) * 4;
+        a_tap4[j] = (((int)fx * p.W + (int)fy) * p.C + (int)c) * 4;
         const unsigned tapc = (fx << 16) | fy;
         // t = rc + tapc has the fields (row + 64, column + 64) of the lane's tap.
         // lo = 0x803f803f - t : bit 15 of a field is set iff that coordinate is < 0
         // hi = t + (0x8000 - (H + 64), 0x8000 - (W + 64)) : set iff it is >= H (or W)
-        tap_lo = 0x803f803fu - tapc;
-        tap_hi = tapc + (((unsigned)(0x8000 - (p.H + 64)) << 16) | (unsigned)(0x8000 - (p.W + 64)));
-        if (kk >= p.K) tap_lo = 0xffffffffu;             // k past K: always out of range
+        tap_lo[j] = 0x803f803fu - tapc;
+        tap_hi[j] = tapc + (((unsigned)(0x8000 - (p.H + 64)) << 16) | (unsigned)(0x8000 - (p.W + 64)));
+        if (kk >= p.K) tap_lo[j] = 0xffffffffu;          // k past K: always out of range
     }
-    const int perm0 = (lane >> 5) * 4;                   // byte index of source lane 0 / 1 (+ 8 i for load i)
 
     // ---- dy: one wave-level load = 4 slab rows x 16 chunks; 2 loads per wave ------------
     // Rows past M lie beyond the descriptors' extents (and m_per_split is a multiple of
@@ -1363,25 +1376,26 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
     // is cut in three so that a slab can spread it between its MFMA groups: a burst of
     // address arithmetic after the barrier keeps the wave off the matrix pipe, while the
     // same instructions issued behind an MFMA run in its shadow.
-    unsigned perm_rc[4];
-    int perm_off[4];
+    unsigned perm_rc[XL];
+    int perm_off[XL];
     // live == 0 (no next slab): rows read as (0, 0), which every tap sees as "above the image"
     auto fetch_rows = [&](int live) {                    // 8 LDS-crossbar permutes, no LDS memory
         const int rc = ((st_r << 16) | st_c) & live;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            perm_rc[i] = (unsigned)__builtin_amdgcn_ds_bpermute(perm0 + 8 * i, rc);
-            perm_off[i] = __builtin_amdgcn_ds_bpermute(perm0 + 8 * i, st_off);
+        for (int i = 0; i < XL; ++i) {
+            perm_rc[i] = (unsigned)__builtin_amdgcn_ds_bpermute(perm_idx[i], rc);
+            perm_off[i] = __builtin_amdgcn_ds_bpermute(perm_idx[i], st_off);
         }
     };
     auto load_x = [&](int i, float* la) {
-        const unsigned z = (tap_lo - perm_rc[i]) | (perm_rc[i] + tap_hi);
+        const unsigned z = (tap_lo[i] - perm_rc[i]) | (perm_rc[i] + tap_hi[i]);
         const unsigned w = z | (z << 16);                // bit 31: row or column out of the image
-        const unsigned voff = (w & 0x80000000u) | (unsigned)(perm_off[i] + a_tap4);
+        const unsigned voff = (w & 0x80000000u) | (unsigned)(perm_off[i] + a_tap4[i]);
+        // the wave's 8 rows are contiguous in LDS; load i fills the next 64 lanes' worth of them
         if constexpr (CW == 1)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + (wave * 4 + i) * 2 * RS), 4, (int)voff, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + wave * 8 * RS + i * 64), 4, (int)voff, 0, 0, 0);
         else
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + (wave * 4 + i) * 2 * RS), 16, (int)voff, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + wave * 8 * RS + i * 256), 16, (int)voff, 0, 0, 0);
     };
     auto load_y = [&](int i, int mb, float* ly, int live) {
         const int m = mb + (wave_u * 2 + i) * 4;         // scalar
@@ -1408,13 +1422,20 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
     // The MFMA takes dy as its A operand and x as B: accumulator q then holds
     // dW[k = kt0 + CW * (lane % 32) + q][n = 32 nt + 8 (v/4) + 4 (lane/32) + v%4], four
     // consecutive n per lane and v/4, which leave in 16-byte stores.
+    typedef float fna __attribute__((ext_vector_type(NA)));
+    typedef float f2v __attribute__((ext_vector_type(2)));
     auto slab = [&](int mb, const float* la, const float* ly, float* na, float* ny, bool has_next) {
         __builtin_amdgcn_s_waitcnt(0);                   // this wave's loads of the slab have landed
         __syncthreads();
-        fcw fa[2];
+        fna fa[2];
+        f2v fa2[2];                                      // CW == 6: columns 128 + 2i, 128 + 2i + 1
         float fb[2];
-        fa[0] = *reinterpret_cast<const fcw*>(la + row0 * RS + CW * l32);
-        fb[0] = ly[row0 * kWgBN + (y_rd ^ (lh << 5))];
+        auto read_operands = [&](int row, int slot) {
+            fa[slot] = *reinterpret_cast<const fna*>(la + row * RS + NA * l32);
+            if constexpr (CW == 6) fa2[slot] = *reinterpret_cast<const f2v*>(la + row * RS + 128 + 2 * l32);
+            fb[slot] = ly[row * kWgBN + (y_rd ^ (lh << 5))];
+        };
+        read_operands(row0, 0);
         // no branch in here: without a next slab the loads are issued with offsets past
         // the descriptors and fetch nothing
         const int live = has_next ? -1 : 0;
@@ -1422,16 +1443,19 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
         fetch_rows(live);
 #pragma unroll
         for (int t = 0; t < BR / 4; ++t) {
-            if (t + 1 < BR / 4) {
-                fa[(t + 1) & 1] = *reinterpret_cast<const fcw*>(la + (row0 + 4 * t + 4) * RS + CW * l32);
-                fb[(t + 1) & 1] = ly[(row0 + 4 * t + 4) * kWgBN + (y_rd ^ (lh << 5))];
-            }
-            if (t >= 1 && t <= 4) load_x(t - 1, na);
-            if (t == 5 || t == 6) load_y(t - 5, mb + BR, ny, live);
+            if (t + 1 < BR / 4) read_operands(row0 + 4 * t + 4, (t + 1) & 1);
+            // one load per MFMA step: dy in steps 0 and 1 (XL == 6) or 5 and 6, x from step 1 on
+            constexpr int Y0 = XL == 6 ? 0 : 5;
+            if (t >= 1 && t <= XL) load_x(t - 1, na);
+            if (t == Y0 || t == Y0 + 1) load_y(t - Y0, mb + BR, ny, live);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int q = 0; q < CW; ++q)
+            for (int q = 0; q < NA; ++q)
                 acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[t & 1], fa[t & 1][q], acc[q], 0, 0, 0);
+            if constexpr (CW == 6) {
+                acc[4] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[t & 1], fa2[t & 1][0], acc[4], 0, 0, 0);
+                acc[5] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[t & 1], fa2[t & 1][1], acc[5], 0, 0, 0);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
         if (do_db) add_columns(ly);
@@ -1440,7 +1464,7 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
     if (m_begin < m_end) {
         fetch_rows(-1);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) load_x(i, lds_a0);
+        for (int i = 0; i < XL; ++i) load_x(i, lds_a0);
 #pragma unroll
         for (int i = 0; i < 2; ++i) load_y(i, m_begin, lds_y0, -1);
     }
@@ -1451,7 +1475,7 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
 
     // ---- add the two m parities: waves 2,3 hand their accumulators to waves 0,1 --------
     __syncthreads();                                     // slab buffers are free now
-    f4* xch = reinterpret_cast<f4*>(nt == 0 ? lds_a0 : lds_a1);   // 16 x 16 B x 64 lanes = 16 KB per wave pair
+    f4* xch = reinterpret_cast<f4*>(nt == 0 ? lds_a0 : lds_a1);   // CW x 4 x 16 B x 64 lanes per wave pair: one x buffer
     if (mh == 1) {
 #pragma unroll
         for (int q = 0; q < CW; ++q)
@@ -1469,7 +1493,7 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
         const int nb = n0 + nt * 32 + 4 * lh;
 #pragma unroll
         for (int q = 0; q < CW; ++q) {
-            const int k = kt0 + CW * l32 + q;            // rows past K fall outside the descriptor
+            const int k = q < NA ? kt0 + NA * l32 + q : kt0 + 128 + 2 * l32 + (q - NA);   // rows past K fall outside the descriptor
             const unsigned base = (unsigned)(k * p.D + nb) * 4u;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
@@ -1507,6 +1531,16 @@ static __global__ __launch_bounds__(kThreads, 3) void wgrad_gemm_dma(const Wgrad
     if (p.cw == 1) wgrad_dma_body<1>(p, lds_a0, lds_a1, lds_y0, lds_y1);
     else if (p.cw == 2) wgrad_dma_body<2>(p, lds_a0, lds_a1, lds_y0, lds_y1);
     else wgrad_dma_body<4>(p, lds_a0, lds_a1, lds_y0, lds_y1);
+}
+
+// The 192-wide k tile: 64 KB of LDS, two workgroups per CU.
+static __global__ __launch_bounds__(kThreads, 2) void wgrad_gemm_dma192(const WgradParams p) {
+    __shared__ float lds_a0[kWgBR * 192];
+    __shared__ float lds_a1[kWgBR * 192];
+    __shared__ float lds_y0[kWgBR * kWgBN];
+    __shared__ float lds_y1[kWgBR * kWgBN];
+    static_assert(sizeof(lds_a0) >= 6 * 16 * 64 * sizeof(float), "accumulator exchange buffer");
+    wgrad_dma_body<6>(p, lds_a0, lds_a1, lds_y0, lds_y1);
 }
 
 // ------------------------------------------------------------------------------
@@ -1719,12 +1753,20 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     const bool dma16 = sizeof(T) == 2 && va && vy && fits;      // bf16 MFMA kernel, 64-row slabs
     p.x_bytes = (dma || dma16) ? (unsigned)xb : 0u;
     p.dy_bytes = (dma || dma16) ? (unsigned)yb : 0u;
+    // operand width of the fp32 LDS-direct kernel: 192-wide k tiles where they pad fewer rows than 128-wide ones
     p.cw = !va ? 1 : (p.K <= 64 ? 2 : 4);
-    const int kt = cdiv(p.K, (dma && !va) ? 32 : kWgBK), nt = cdiv(D, kWgBN);
+    if (dma && p.cw == 4 && cdiv(p.K, 192) * 192 < cdiv(p.K, kWgBK) * kWgBK) p.cw = 6;
+    if (const char* f = getenv("AETHER_WGRAD_CW")) {
+        if (dma && va && p.K > 64 && (atoi(f) == 4 || atoi(f) == 6)) p.cw = atoi(f);
+    }
+    const int tkw = !dma ? kWgBK : (p.cw == 1 ? 32 : (p.cw == 6 ? 192 : kWgBK));
+    const int kt = cdiv(p.K, tkw), nt = cdiv(D, kWgBN);
     const int slab_rows = dma16 ? 64 : kWgBR;
     const int slabs = cdiv(p.M, slab_rows);           // fp32: counted in 32-row units for both tile shapes
-    // about two rounds of resident workgroups (3 per CU for the LDS-direct kernel)
-    int splits = cdiv(((dma || dma16) ? 6 : 4) * c.prop.multiProcessorCount, kt * nt);
+    // two rounds of resident workgroups (3 per CU for the LDS-direct kernels, 2 for the 192-wide
+    // one and the register-staged one), rounded down so that the last round is not a nearly empty one
+    const int per_cu2 = ((dma && p.cw != 6) || dma16) ? 6 : 4;
+    int splits = (per_cu2 * c.prop.multiProcessorCount) / (kt * nt);
     // a workgroup's set-up, epilogue and its share of the reduction are worth several slabs
     // (training step of the 3-block CNN: 0.672 ms with 1, 0.642 with 4, 0.611 with 8, 0.658 with 16)
     const int min_slabs = 8;
@@ -1741,6 +1783,7 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     p.kt = kt; p.nt = nt;
     dim3 grid(kt * nt * splits);
     if (dma16) hipLaunchKernelGGL(wgrad_gemm_dma_bf16, grid, dim3(kThreads), 0, c.stream, p);
+    else if (dma && p.cw == 6) hipLaunchKernelGGL(wgrad_gemm_dma192, grid, dim3(kThreads), 0, c.stream, p);
     else if (dma) hipLaunchKernelGGL(wgrad_gemm_dma, grid, dim3(kThreads), 0, c.stream, p);
     else if (va && vy) hipLaunchKernelGGL((wgrad_gemm<T, CE, CE>), grid, dim3(kThreads), 0, c.stream, p);
     else if (va) hipLaunchKernelGGL((wgrad_gemm<T, CE, 1>), grid, dim3(kThreads), 0, c.stream, p);
