@@ -711,7 +711,10 @@ static inline int gather_bn(int N) { return N <= 32 ? 32 : 64; }
 // Tile height.  The LDS-direct kernel keeps two slabs per operand in LDS, so a
 // 128-row tile (48 KB) lets three workgroups share a CU where a 256-row tile
 // (80 KB) allows one or two; measured on the 56x56x64 shape, 128 rows is 11 %
-// faster.  The register-staged kernel prefers 256 rows.
+// faster.  64-row tiles (32 KB, five per CU) run at the same rate and leave a
+// smaller last round, so fp32 takes 128 rows only from about 8 rounds of tiles on
+// (6272 tiles, 56x56x64: 0.483 ms either way; 1568 tiles, 56x56x256 batch 64: 0.503 ms
+// with 128 rows, 0.488 with 64).  The register-staged kernel prefers 256 rows.
 static inline int gather_bm(int M, int N, int cus, bool dma, int elem_bytes = 4) {
     const int bn = gather_bn(N);
     if (const char* f = getenv("AETHER_GATHER_BM")) {       // tuning override: 256, 128 or 64
@@ -725,7 +728,9 @@ static inline int gather_bm(int M, int N, int cus, bool dma, int elem_bytes = 4)
     for (int i = (dma && elem_bytes == 4) ? 1 : 0; i < 3; ++i) {
         int bm = cands[i];
         if (bn == 32 && bm == 64) break;
-        if ((int64_t)cdiv(M, bm) * ntiles >= want) return bm;
+        const int64_t tiles = (int64_t)cdiv(M, bm) * ntiles;
+        if (dma && elem_bytes == 4 && bm == 128 && bn == 64 && tiles < 24 * (int64_t)cus) continue;
+        if (tiles >= want) return bm;
     }
     return bn == 32 ? 128 : 64;
 }
