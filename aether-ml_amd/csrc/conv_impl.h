@@ -114,29 +114,53 @@ __device__ __forceinline__ int xcd_contiguous_id(int wg, int total) {
 // the same issue cycles, so an epilogue of 32 scalar stores with per-element address
 // arithmetic costs measurable matrix time (9 % on the 56x56x64 layer).
 // The bias is added by starting the accumulators from it.
+// Bias values for the accumulator layout above, through a buffer descriptor that ends
+// after channel N (after nothing when there is no bias): channels past N read as zero
+// without a branch.  Per-lane branches around ordinary loads made the compiler wait
+// for each load in turn, several microseconds at the start of every workgroup.
+template <int TN>
+__device__ __forceinline__ void load_bias(const GatherParams& p, const float* bias, f4 (&bv)[TN][4], int nw0, int lh) {
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(bias), 0, bias != nullptr ? p.N * 4 : 0, 0x00020000);
+    if (p.N % 4 == 0) {                                 // whole groups of 4 channels: inside or outside as one
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n = nw0 + 32 * j + 8 * q + 4 * lh;
+                bv[j][q] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, n * 4, 0, 0));
+            }
+    } else {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int n = nw0 + 32 * j + 8 * q + 4 * lh + e;
+                    bv[j][q][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, n * 4, 0, 0));
+                }
+    }
+}
+
 template <int TM, int TN>
-__device__ __forceinline__ void init_acc(const GatherParams& p, const float* bias, f16v (&acc)[TM][TN], int nw0, int lh) {
-    const bool vec = p.out_bytes != 0 && (reinterpret_cast<uintptr_t>(bias) & 15) == 0;
+__device__ __forceinline__ void fill_acc(const f4 (&bv)[TN][4], f16v (&acc)[TM][TN]) {
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int n = nw0 + 32 * j + 8 * q + 4 * lh;
-            f4 bv = {0.f, 0.f, 0.f, 0.f};
-            if (bias != nullptr) {
-                if (vec) {
-                    if (n < p.N) bv = *reinterpret_cast<const f4*>(bias + n);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (n + e < p.N) bv[e] = bias[n + e];
-                }
-            }
+        for (int q = 0; q < 4; ++q)
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = bv[e];
-        }
+                for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = bv[j][q][e];
+}
+
+template <int TM, int TN>
+__device__ __forceinline__ void init_acc(const GatherParams& p, const float* bias, f16v (&acc)[TM][TN], int nw0, int lh) {
+    f4 bv[TN][4];
+    load_bias<TN>(p, bias, bv, nw0, lh);
+    fill_acc<TM, TN>(bv, acc);
 }
 
 template <int TM, int TN>
@@ -392,38 +416,39 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
     const int m0 = NLOOP ? lid * BM : (lid / ntile) * BM;
     int n0 = NLOOP ? 0 : (lid % ntile) * BN;
 
+    // The bias is fetched first: its latency passes behind the row decode.
+    const int split = (int)blockIdx.y;
+    f4 bv[TN][4];
+    load_bias<TN>(p, split == 0 ? p.bias : nullptr, bv, n0 + wn0, lh);
+
     const int lr = lane / KC;                  // row inside a load block
     // logical chunk this lane fetches: (lane % KC) ^ swizzle(row).  KC == 8: the 8-row
     // blocks alternate between row bits (0,lane>>4) and (4 | lane>>4), so odd blocks use
     // k4e ^ 4; KC == 4: 16-row blocks, the same for every block
     const int k4e = KC == 8 ? (lane & 7) ^ (lane >> 4) : (lane & 3) ^ (lane >> 4);
     constexpr int ODD = KC == 8 ? 4 : 0;       // what an odd load block xors into the chunk
-    int base_off[AL];
-    int base_rc[AL];
-#pragma unroll
-    for (int i = 0; i < AL; ++i) {
-        int m = m0 + (wave * AL + i) * RPL + lr;
+    // Row decode: thread t works out the image position of row m0 + t once, and the
+    // KC lanes that fetch a row take it from a table in LDS (decoding AL rows in every
+    // lane made the set-up a quarter of the life of a 9-slab workgroup).  An entry is
+    // (element offset of tap (0,0), aux); aux is, in uniform-tap mode, one bit per tap
+    // that says "outside the image" (all ones for rows past M), else (row << 16 | column).
+    // The table sits in the second B buffer, which is first written after the first
+    // barrier of the K loop.
+    static_assert(BM <= kThreads && BM * sizeof(int2) <= BN * KC * sizeof(f4), "row table fits the B buffer");
+    int2* rowtab = reinterpret_cast<int2*>(lds_b1);
+    if (tid < BM) {
+        const int m = m0 + tid;
+        int off = 0, br = kInvalidRow, bc = 0;
         if (m < p.M) {
             unsigned s, rem, ii, jj;
             p.div_hw.divmod((unsigned)m, s, rem);
             p.div_w.divmod(rem, ii, jj);
-            int br = (int)ii * p.sh + p.rh0;
-            int bc = (int)jj * p.sw + p.rw0;
-            base_off[i] = (((int)s * p.Hs + br) * p.Ws + bc) * p.Cs;
-            base_rc[i] = (int)(((unsigned)br << 16) | ((unsigned)bc & 0xffffu));
-        } else {
-            base_off[i] = 0;
-            base_rc[i] = (int)((unsigned)kInvalidRow << 16);
+            br = (int)ii * p.sh + p.rh0;
+            bc = (int)jj * p.sw + p.rw0;
+            off = (((int)s * p.Hs + br) * p.Ws + bc) * p.Cs;
         }
-    }
-    // uniform-tap mode: byte offset of this lane's chunk at tap (0,0), and one bit per
-    // tap that says "outside the image" (all ones for rows past M)
-    unsigned a_byte[AL], a_inv[AL];
-    if (UT) {
-#pragma unroll
-        for (int i = 0; i < AL; ++i) {
-            const int br = base_rc[i] >> 16;
-            const int bc = (int)((unsigned)base_rc[i] << 16) >> 16;
+        int aux = (int)(((unsigned)br << 16) | ((unsigned)bc & 0xffffu));
+        if (UT) {
             // taps (th, tw) inside the image: th in [max(0,-br), min(Th, Hs-br)), same for tw;
             // a row past M has br = kInvalidRow and an empty range
             auto span = [](int lo, int hi) -> unsigned {     // bits [lo, hi) of a mask, 0 <= lo, hi <= 32
@@ -436,10 +461,21 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
             const unsigned rmask = span(lo_r, hi_r), cmask = span(lo_c, hi_c);
             unsigned valid = 0;
             for (int th = 0; th < p.Th; ++th) valid |= (((rmask >> th) & 1u) ? cmask : 0u) << (th * p.Tw);
-            const unsigned inv = ~valid;
-            a_inv[i] = inv;
-            a_byte[i] = (unsigned)(base_off[i] + CE * (k4e ^ ((i & 1) ? ODD : 0))) * (unsigned)sizeof(T);
+            aux = (int)~valid;
         }
+        rowtab[tid] = int2{off, aux};
+    }
+    __syncthreads();
+    int base_off[AL];
+    int base_rc[AL];
+    unsigned a_byte[AL], a_inv[AL];
+#pragma unroll
+    for (int i = 0; i < AL; ++i) {
+        const int2 e = rowtab[(wave * AL + i) * RPL + lr];
+        base_off[i] = e.x;
+        base_rc[i] = e.y;
+        a_inv[i] = (unsigned)e.y;
+        a_byte[i] = (unsigned)(e.x + CE * (k4e ^ ((i & 1) ? ODD : 0))) * (unsigned)sizeof(T);
     }
     unsigned b_off[BL];
     auto set_b_off = [&]() {
@@ -523,9 +559,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
     // split K (launches with few tiles and a long K, e.g. a dense layer on a small batch):
     // blockIdx.y walks its own range of slabs and writes a partial product; the bias goes
     // into split 0 and `reduce_splits` adds the partials in order
-    const int split = (int)blockIdx.y;
     f16v acc[TM][TN];
-    init_acc<TM, TN>(p, split == 0 ? p.bias : nullptr, acc, n0 + wn0, lh);
 
     const int sw7 = (l32 >> SH) & (KC - 1);    // swizzle of every operand row this lane reads
     f4 fa[2][TM], fb[2][TN];                   // operand fragments, double buffered across k groups
@@ -578,6 +612,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
         }
 #pragma unroll
         for (int j = AL; j < NL; ++j) issue_load(j, 0, lds_a0, lds_b0);         // B of step 0
+        fill_acc<TM, TN>(bv, acc);
         // one step; `last_slab`: this slab completes an n tile
         auto step = [&](int f, const f4* la, const f4* lb, f4* nb, bool last_slab) __attribute__((always_inline)) {
             __builtin_amdgcn_s_waitcnt(0);
@@ -625,6 +660,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
         if (s_begin + p.split_slabs < nslabs) nslabs = s_begin + p.split_slabs;
     }
     if (s_begin < nslabs) issue(s_begin * BK, lds_a0, lds_b0);
+    fill_acc<TM, TN>(bv, acc);
     for (int s = s_begin; s < nslabs; s += 2) {
         slab(lds_a0, lds_b0, lds_a1, lds_b1, (s + 1) * BK, s + 1 < nslabs);
         if (s + 1 < nslabs) slab(lds_a1, lds_b1, lds_a0, lds_b0, (s + 2) * BK, s + 2 < nslabs);
