@@ -92,6 +92,7 @@ struct GatherParams {
 };
 
 constexpr int kInvalidRow = -16384;
+constexpr int kNloopMaxN = 1024;   // widest output the n-loop mode of the gather kernel takes (its bias sits in LDS)
 constexpr int kXcds = 8;
 
 // Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has its
@@ -163,7 +164,8 @@ __device__ __forceinline__ void init_acc(const GatherParams& p, const float* bia
     fill_acc<TM, TN>(bv, acc);
 }
 
-template <int TM, int TN>
+// VEC_ONLY: the caller guarantees p.out_bytes != 0 (16-byte stores through the descriptor)
+template <int TM, int TN, bool VEC_ONLY = false>
 __device__ __forceinline__ void store_tile(const GatherParams& p, float* out, const f16v (&acc)[TM][TN], int mw0,
                                            int nw0, int l32, int lh) {
     typedef unsigned u4 __attribute__((ext_vector_type(4)));
@@ -182,7 +184,7 @@ __device__ __forceinline__ void store_tile(const GatherParams& p, float* out, co
             row = ((unsigned)s * p.Hof + p.oh0 + ii * p.ohs) * p.Wof + p.ow0 + jj * p.ows;
         }
         const unsigned elem = row * (unsigned)p.N + (unsigned)(nw0 + 4 * lh);   // < 2^31: checked by the host
-        if (p.out_bytes != 0) {
+        if (VEC_ONLY || p.out_bytes != 0) {
             // rows past M (and, in edge tiles, channels past N) get a byte offset beyond
             // the descriptor's extent: the hardware drops the store
             const unsigned base = (elem * 4u) | ((unsigned)!mok << 31);
@@ -602,6 +604,15 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
         // the loads of step f+1 fly while step f is multiplied.
         const int nslabs = p.Kpad / BK;                // 1 or 2
         const int total = ntile * nslabs;
+        // the bias of every n tile, kept in LDS: a tile's accumulators start from it without a
+        // global load between the steps (tile 0 takes the registers fetched above)
+        __shared__ __attribute__((aligned(16))) float lds_bias[kNloopMaxN];
+        float bias_mine[kNloopMaxN / kThreads];
+#pragma unroll
+        for (int i = 0; i < kNloopMaxN / kThreads; ++i) {
+            const int n = i * kThreads + tid;
+            bias_mine[i] = (p.bias != nullptr && n < p.N) ? p.bias[n] : 0.f;
+        }
         prep(0);
 #pragma unroll
         for (int j = 0; j < AL; ++j) issue_load(j, 0, lds_a0, lds_b0);
@@ -613,13 +624,37 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
 #pragma unroll
         for (int j = AL; j < NL; ++j) issue_load(j, 0, lds_a0, lds_b0);         // B of step 0
         fill_acc<TM, TN>(bv, acc);
-        // one step; `last_slab`: this slab completes an n tile
-        auto step = [&](int f, const f4* la, const f4* lb, f4* nb, bool last_slab) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < kNloopMaxN / kThreads; ++i) lds_bias[i * kThreads + tid] = bias_mine[i];
+        // One step.  `first_slab` / `last_slab`: this slab begins / completes an n tile.
+        // A finished tile is copied to `done` and stored at the beginning of the next step,
+        // after that step's loads are issued: the stores then have a whole step to drain
+        // before the next wait.  (Waiting for "all but the stores" is not possible: loads
+        // and stores of a wave may complete out of order with respect to each other, and
+        // stores issued at the end of a step are waited for in full by the next one.)
+        f16v done[TM][TN];
+        auto step = [&](int f, const f4* la, const f4* lb, f4* nb, bool first_slab, bool last_slab) __attribute__((always_inline)) {
             __builtin_amdgcn_s_waitcnt(0);
             __syncthreads();
             read_frags(la, lb, 0, 0);
             const int tile_now = n0;
-            if (f + 1 < total) {
+            const bool more = f + 1 < total;
+            const bool pending = first_slab && f > 0;     // the tile before this one waits in `done`
+            if (pending) {
+                // before this step's loads are issued: with an LDS-direct load in flight the
+                // compiler makes every other LDS read wait for it
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const f4 v = *reinterpret_cast<const f4*>(lds_bias + tile_now + wn0 + 32 * j + 8 * q + 4 * lh);
+#pragma unroll
+                        for (int i = 0; i < TM; ++i)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = v[e];
+                    }
+            }
+            if (more) {
                 const int fn = f + 1;
                 const int nt_next = nslabs == 2 ? fn >> 1 : fn;
                 const int k0_next = nslabs == 2 ? (fn & 1) * BK : 0;
@@ -628,6 +663,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
 #pragma unroll
                 for (int j = AL; j < NL; ++j) issue_load(j, k0_next, lds_a0, nb);
             }
+            if (pending) store_tile<TM, TN, true>(p, p.out, done, m0 + wm0, tile_now - BN + wn0, l32, lh);
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 if (g < G - 1) read_frags(la, lb, g + 1, (g + 1) & 1);
@@ -636,19 +672,25 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (last_slab) {
-                store_tile<TM, TN>(p, p.out, acc, m0 + wm0, tile_now + wn0, l32, lh);
-                if (f + 1 < total) init_acc<TM, TN>(p, p.bias, acc, n0 + wn0, lh);
+                if (more) {
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) done[i][j] = acc[i][j];
+                } else {
+                    store_tile<TM, TN, true>(p, p.out, acc, m0 + wm0, tile_now + wn0, l32, lh);
+                }
             }
         };
         if (nslabs == 2) {
             for (int f = 0; f < total; f += 2) {
-                step(f, lds_a0, lds_b0, lds_b1, false);
-                step(f + 1, lds_a1, lds_b1, lds_b0, true);
+                step(f, lds_a0, lds_b0, lds_b1, true, false);
+                step(f + 1, lds_a1, lds_b1, lds_b0, false, true);
             }
         } else {
             for (int f = 0; f < total; f += 2) {
-                step(f, lds_a0, lds_b0, lds_b1, true);
-                if (f + 1 < total) step(f + 1, lds_a0, lds_b1, lds_b0, true);
+                step(f, lds_a0, lds_b0, lds_b1, true, true);
+                if (f + 1 < total) step(f + 1, lds_a0, lds_b1, lds_b0, true, true);
             }
         }
         return;
@@ -712,7 +754,8 @@ static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
     const bool ut = gp.Cs % (KC * Elem<T>::CE) == 0 && gp.K == gp.Kpad && gp.K / gp.Cs <= 32;
     // short K, several n tiles: one workgroup per m tile walks the n tiles (128 x 64 tiles only)
     if constexpr (BM == 128 && BN == 64 && KC == 8) {
-        if (gp.split_slabs == 0 && gp.Kpad / (KC * Elem<T>::CE) <= 2 && gp.N > BN && getenv("AETHER_GATHER_NLOOP_OFF") == nullptr) {
+        if (gp.split_slabs == 0 && gp.Kpad / (KC * Elem<T>::CE) <= 2 && gp.N > BN && gp.N <= kNloopMaxN && gp.out_bytes != 0 &&
+            getenv("AETHER_GATHER_NLOOP_OFF") == nullptr) {
             grid.x = (unsigned)cdiv(gp.M, BM);
             if (ut) hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, true>), grid, dim3(kThreads), 0, st, gp);
             else hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, false, KC, true>), grid, dim3(kThreads), 0, st, gp);
@@ -1804,9 +1847,15 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     const int kt = cdiv(p.K, tkw), nt = cdiv(D, kWgBN);
     const int slab_rows = dma16 ? 64 : kWgBR;
     const int slabs = cdiv(p.M, slab_rows);           // fp32: counted in 32-row units for both tile shapes
-    // two rounds of resident workgroups (3 per CU for the LDS-direct kernels, 2 for the 192-wide
-    // one and the register-staged one), rounded down so that the last round is not a nearly empty one
-    const int per_cu2 = ((dma && p.cw != 6) || dma16) ? 6 : 4;
+    // one round of resident workgroups (3 per CU for the LDS-direct kernels, 2 for the 192-wide
+    // one and the register-staged one), rounded down so that no second, nearly empty round follows.
+    // Every further round costs a set-up, an epilogue and a share of the reduction per workgroup
+    // (56x56x64: 0.485 ms with one round, 0.493 with two, 0.509 with four).
+    int rounds = 1;
+    if (const char* f = getenv("AETHER_WGRAD_ROUNDS")) {      // tuning override: 1 to 4
+        if (atoi(f) >= 1 && atoi(f) <= 4) rounds = atoi(f);
+    }
+    const int per_cu2 = (((dma && p.cw != 6) || dma16) ? 3 : 2) * rounds;
     int splits = (per_cu2 * c.prop.multiProcessorCount) / (kt * nt);
     // a workgroup's set-up, epilogue and its share of the reduction are worth several slabs
     // (training step of the 3-block CNN: 0.672 ms with 1, 0.642 with 4, 0.611 with 8, 0.658 with 16)
