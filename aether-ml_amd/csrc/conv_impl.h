@@ -88,7 +88,8 @@ struct GatherParams {
     unsigned bt_bytes;
     unsigned out_bytes;  // extent of out; 0: no 16-byte stores (too large, N not a multiple of 4, or unaligned)
     int split_slabs;     // 0, or slabs of K per blockIdx.y: split y writes its partial product at out + y*M*N
-    FastDiv div_hw, div_w, div_c, div_tw;
+    int halo_wp, halo_tiles;   // gather_halo_bf16: columns of the padded source row, 256-row tiles per image
+    FastDiv div_hw, div_w, div_c, div_tw, div_halo_wp, div_halo_tiles;
 };
 
 constexpr int kInvalidRow = -16384;
@@ -165,9 +166,11 @@ __device__ __forceinline__ void init_acc(const GatherParams& p, const float* bia
 }
 
 // VEC_ONLY: the caller guarantees p.out_bytes != 0 (16-byte stores through the descriptor)
+// m_end: rows from here on are not stored (default: p.M)
 template <int TM, int TN, bool VEC_ONLY = false>
 __device__ __forceinline__ void store_tile(const GatherParams& p, float* out, const f16v (&acc)[TM][TN], int mw0,
-                                           int nw0, int l32, int lh) {
+                                           int nw0, int l32, int lh, int m_end = -1) {
+    if (m_end < 0) m_end = p.M;
     typedef unsigned u4 __attribute__((ext_vector_type(4)));
     const bool full_n = nw0 + 32 * TN <= p.N;           // wave-uniform
     const __amdgpu_buffer_rsrc_t rsrc =
@@ -175,7 +178,7 @@ __device__ __forceinline__ void store_tile(const GatherParams& p, float* out, co
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int m = mw0 + 32 * i + l32;
-        const bool mok = m < p.M;
+        const bool mok = m < m_end;
         unsigned row = (unsigned)m;
         if (!p.dense_out) {
             unsigned s, rem, ii, jj;
@@ -711,6 +714,204 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
     store_tile<TM, TN>(p, p.out + (size_t)split * p.M * p.N, acc, m0 + wm0, n0 + wn0, l32, lh);
 }
 
+// ------------------------------------------------------------------------------
+// gather_halo_bf16: unit-stride gathers with several filter taps on bf16 inputs
+// (3x3 stride-1 fprop, every dgrad class with 4 taps or more).
+// The bf16 MFMAs of a slab take a fifth of the time its LDS-direct loads need to
+// arrive, and with the taps of a filter walked one slab at a time every source
+// pixel is fetched once per tap (9 times for 3x3): gather_gemm_dma on these shapes
+// waits for its loads (without the A loads of slabs 1..8 it runs 1.5x faster).
+// Here a workgroup fetches the source pixels of its 256 output pixels ONCE, as a
+// span of the zero-padded image in row-major order ("halo", 64 channels = 128 B per
+// pixel slot, at most kHaloSlots slots), and every tap reads it at a shifted slot:
+//     slot(pixel (i, j), tap (th, tw)) = (i + th) * Wp + (j + tw) - first,  Wp = Wg + Tw - 1
+// Padding pixels are slots the loads fill with zeros (offsets outside the buffer
+// descriptor), so no tap needs a validity test.  Only the filter slabs stream, 8 KB
+// per tap through a ring of four buffers, three taps ahead.  Tiles do not cross
+// images (the span would grow by (Th - 1) rows), so the last tile of an image is
+// partly empty: used when that costs at most 10 % of the rows.
+//   * slot s keeps logical 16-byte chunk c at position c ^ ((s >> 1) & 7), like the
+//     slab rows of gather_gemm_dma: 16 consecutive pixels cover the 64 banks once;
+//   * channel blocks beyond the first reload the halo (Cs = 64 j: j passes over the taps).
+// ------------------------------------------------------------------------------
+// A 16-byte-per-lane LDS-direct load the compiler does not see as one.  It orders every LDS
+// read behind the LDS-direct loads it knows to be in flight unless it can prove where they
+// land, and with a ring of buffers in a loop it cannot: the reads of a step then wait for the
+// slabs fetched for later steps.  The caller waits (vmcnt + barrier) before reading what a
+// load brings.  lds_base: wave-uniform LDS byte address; the lanes land at lds_base + 16 * lane.
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void lds_direct_load16(const u32x4& rsrc, unsigned lds_base, unsigned voff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :: "s"(lds_base), "v"(voff), "s"(rsrc) : "memory", "m0");
+}
+__device__ __forceinline__ u32x4 raw_rsrc(const void* base, unsigned bytes) {
+    const unsigned long long a = reinterpret_cast<unsigned long long>(base);
+    return u32x4{(unsigned)a, (unsigned)(a >> 32) & 0xffffu, bytes, 0x00020000u};
+}
+__device__ __forceinline__ unsigned lds_address(const void* q) {
+    return (unsigned)reinterpret_cast<uintptr_t>((lds_ptr_t)const_cast<void*>(q));
+}
+
+constexpr int kHaloSlots = 384;      // 48 KB; with the 4 x 8 KB ring 80 KB: two workgroups per CU
+constexpr int kHaloBM = 256;
+
+static __global__ __launch_bounds__(kThreads, 2) void gather_halo_bf16(const GatherParams p) {
+    constexpr int BM = kHaloBM, BN = 64, TM = 2, TN = 2, KC = 8, BK = 64;
+    constexpr int HL = kHaloSlots / 8 / 4;               // halo loads per wave (8 slots each)
+    __shared__ f4 halo[kHaloSlots * KC];
+    __shared__ f4 ring0[BN * KC];
+    __shared__ f4 ring1[BN * KC];
+    __shared__ f4 ring2[BN * KC];
+    __shared__ f4 ring3[BN * KC];
+    static_assert(kHaloSlots * sizeof(int) <= sizeof(ring3), "slot table fits a ring buffer");
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int l32 = lane & 31;
+    const int lh = lane >> 5;
+    const int wm0 = wave * 64;
+    const int ntile = (p.N + BN - 1) / BN;
+    const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
+    const int mt = lid / ntile;
+    const int n0 = (lid - mt * ntile) * BN;
+    unsigned s_img, t_img;
+    p.div_halo_tiles.divmod((unsigned)mt, s_img, t_img);
+    const int hw = p.Hg * p.Wg;
+    const int pm0 = (int)t_img * BM;
+    const int Wp = p.halo_wp;
+    const int T = p.Th * p.Tw;
+    const int nsteps = (p.Cs / BK) * T;
+
+    f4 bv[TN][4];
+    load_bias<TN>(p, p.bias, bv, n0, lh);
+
+    // the span: from the slot of tap (0,0) of the tile's first pixel to that of the last tap of its last pixel
+    unsigned i0, j0, i1, j1;
+    p.div_w.divmod((unsigned)pm0, i0, j0);
+    p.div_w.divmod((unsigned)min(pm0 + BM, hw) - 1u, i1, j1);
+    const int lfirst = (int)i0 * Wp + (int)j0;
+    const int span = ((int)i1 + p.Th - 1) * Wp + (int)j1 + p.Tw - lfirst;     // <= kHaloSlots, checked by the host
+    // slot -> byte offset of the pixel's channel 0 (bit 31: padding or past the span), one slot per
+    // thread, through LDS to the lanes that fetch it.  The table sits in the last ring buffer, which
+    // the filter loads reach after the first barrier of the loop.
+    int* tab = reinterpret_cast<int*>(ring3);
+    for (int sl = tid; sl < kHaloSlots; sl += kThreads) {
+        unsigned rr, cc;
+        p.div_halo_wp.divmod((unsigned)(lfirst + sl), rr, cc);
+        const int srow = (int)rr + p.rh0, scol = (int)cc + p.rw0;
+        const bool ok = sl < span && (unsigned)srow < (unsigned)p.Hs && (unsigned)scol < (unsigned)p.Ws;
+        const unsigned off = (unsigned)((((int)s_img * p.Hs + srow) * p.Ws + scol) * p.Cs) * 2u;
+        tab[sl] = (int)(ok ? off : 0x80000000u);
+    }
+    __syncthreads();
+    unsigned hoff[HL];
+#pragma unroll
+    for (int k = 0; k < HL; ++k) {
+        const int sl = (wave * HL + k) * 8 + (lane >> 3);
+        hoff[k] = (unsigned)tab[sl] + (unsigned)((((lane & 7) ^ (sl >> 1)) & 7) * 16);
+    }
+    // slot of tap (0,0) for the pixels this lane multiplies (rows past the image: slot 0, never stored)
+    int pslot[TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int pm = pm0 + wm0 + 32 * i + l32;
+        unsigned ii, jj;
+        p.div_w.divmod((unsigned)min(pm, hw - 1), ii, jj);
+        pslot[i] = pm < hw ? (int)ii * Wp + (int)jj - lfirst : 0;
+    }
+    // filter slab loads: as in gather_gemm_dma (rows of 8 chunks, chunk c of row r at c ^ ((r >> 1) & 7))
+    const int k4e = (lane & 7) ^ (lane >> 4);
+    unsigned b_off[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int k4 = k4e ^ (((wave * 2 + i) & 1) ? 4 : 0);
+        b_off[i] = (unsigned)(((n0 + (wave * 2 + i) * 8 + (lane >> 3)) * p.Kpad + 8 * k4) * 2);
+    }
+    const u32x4 rsrc_a = raw_rsrc(p.src, p.src_bytes);
+    const u32x4 rsrc_b = raw_rsrc(p.bt, p.bt_bytes);
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    auto load_halo = [&](int cb) __attribute__((always_inline)) {
+        const unsigned base = lds_address(halo) + (unsigned)(wave_u * HL) * 1024u;
+#pragma unroll
+        for (int k = 0; k < HL; ++k) lds_direct_load16(rsrc_a, base + k * 1024u, hoff[k] + (unsigned)(cb * BK * 2));
+    };
+    // filter slab of step u = (channel block, tap): k0 = tap * Cs + 64 * block, as a byte offset
+    auto load_filter = [&](unsigned k0_bytes, f4* lb) __attribute__((always_inline)) {
+        const unsigned base = lds_address(lb) + (unsigned)(wave_u * 2) * 1024u;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) lds_direct_load16(rsrc_b, base + i * 1024u, b_off[i] + k0_bytes);
+    };
+    // prefetch position: three steps ahead of the one being multiplied.  Every step issues
+    // exactly one slab, past the last step with an offset outside the descriptor (no memory
+    // access): the wait of a step is then the same count in every step, without a branch
+    // (with conditional loads the compiler cannot tell which loads a count leaves in
+    // flight and waits for all of them before the first LDS read).
+    int pf_tap = 0, pf_cb = 0;
+    auto pf_next = [&]() __attribute__((always_inline)) {
+        const unsigned k0_bytes = pf_cb < p.Cs / BK ? (unsigned)(pf_tap * p.Cs + pf_cb * BK) * 2u : 0x80000000u;
+        if (++pf_tap == T) { pf_tap = 0; ++pf_cb; }
+        return k0_bytes;
+    };
+    load_halo(0);
+    load_filter(pf_next(), ring0);
+    load_filter(pf_next(), ring1);
+    load_filter(pf_next(), ring2);
+
+    f16v acc[TM][TN];
+    fill_acc<TM, TN>(bv, acc);
+
+    const int sw7 = (l32 >> 1) & 7;
+    int th = 0, tw = 0, cb = 0;                          // the step being multiplied
+    auto step = [&](int u, const f4* lb, f4* nb) __attribute__((always_inline)) {
+        // loads complete in the order of issue (no stores are pending here): all but the
+        // two younger filter slabs
+        __builtin_amdgcn_s_waitcnt(4 | (7 << 4) | (15 << 8));
+        // a bare barrier: the fence of __syncthreads() would wait for every load in flight
+        asm volatile("s_barrier" ::: "memory");
+        if (th == 0 && tw == 0 && cb > 0) {              // next channel block: everyone is done with the halo
+            load_halo(cb);
+            __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
+            asm volatile("s_barrier" ::: "memory");
+        }
+        load_filter(pf_next(), nb);
+        const int shift = th * Wp + tw;
+        int x0[TM];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int sl = pslot[i] + shift;
+            x0[i] = sl * 8 + ((lh ^ (sl >> 1)) & 7);
+        }
+        // all operand reads of the step go out at once (64 registers): with a read-ahead of one
+        // k group the MFMAs of every group waited for LDS, whose queue under 8 waves of 16-byte
+        // reads is longer than the four MFMAs that were meant to cover it
+        f4 fa[4][TM], fb[4][TN];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) fa[g][i] = halo[x0[i] ^ (g << 1)];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fb[g][j] = lb[(32 * j + l32) * KC + ((2 * g + lh) ^ sw7)];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) mma_chunk<uint16_t>(fb[g][j], fa[g][i], acc[i][j]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (++tw == p.Tw) { tw = 0; if (++th == p.Th) { th = 0; ++cb; } }
+    };
+    for (int u = 0; u < nsteps; u += 4) {
+        step(u, ring0, ring3);
+        if (u + 1 < nsteps) step(u + 1, ring1, ring0);
+        if (u + 2 < nsteps) step(u + 2, ring2, ring1);
+        if (u + 3 < nsteps) step(u + 3, ring3, ring2);
+    }
+    store_tile<TM, TN>(p, p.out, acc, (int)s_img * hw + pm0 + wm0, n0, l32, lh, ((int)s_img + 1) * hw);
+}
+
 // Packs the filter w[fH][fW][C][D] into bt[Npad][Kpad] (k contiguous) for one
 // gather-GEMM launch.  k = (th*Tw + tw)*Ck + kc ; filter tap x = xa + xs*th,
 // y = ya + ys*tw.  transposed == 0: n is the output channel d and kc the input
@@ -814,10 +1015,43 @@ static inline int gather_bm(int M, int N, int cus, bool dma, int elem_bytes = 4)
     return bn == 32 ? 128 : 64;
 }
 
+// gather_halo_bf16 applies to unit-stride gathers of 4 to 32 taps over whole 64-channel blocks
+// whose images are large enough for 256-row tiles that do not cross them.  Fills the halo
+// fields of gp when it does.
+static bool plan_halo(GatherParams& gp, bool dma) {
+    if (!dma || gp.sh != 1 || gp.sw != 1 || gp.Cs % 64 != 0 || gp.K != gp.Kpad || gp.split_slabs != 0) return false;
+    const int taps = gp.Th * gp.Tw;
+    if (taps < 4 || taps > 32 || gp.N <= 32 || gp.Cs <= 0 || gp.K != taps * gp.Cs) return false;
+    if (getenv("AETHER_GATHER_HALO_OFF") != nullptr) return false;
+    const int hw = gp.Hg * gp.Wg;
+    const int tiles = cdiv(hw, kHaloBM);
+    if ((int64_t)tiles * kHaloBM * 10 > (int64_t)hw * 11) return false;       // more than 10 % empty rows
+    const int wp = gp.Wg + gp.Tw - 1;
+    for (int t = 0; t < tiles; ++t) {
+        const int first = t * kHaloBM, last = std::min(first + kHaloBM, hw) - 1;
+        const int l0 = (first / gp.Wg) * wp + first % gp.Wg;
+        const int l1 = (last / gp.Wg + gp.Th - 1) * wp + last % gp.Wg + gp.Tw - 1;
+        if (l1 - l0 + 1 > kHaloSlots) return false;
+    }
+    gp.halo_wp = wp;
+    gp.halo_tiles = tiles;
+    gp.div_halo_wp = FastDiv(wp);
+    gp.div_halo_tiles = FastDiv(tiles);
+    return true;
+}
+
 template <typename T>
 static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t st) {
     const int bn = gather_bn(gp.N);
     const bool dma = vec && gp.src_bytes != 0 && gp.bt_bytes != 0;
+    if constexpr (sizeof(T) == 2) {
+        GatherParams hp = gp;
+        if (plan_halo(hp, dma)) {
+            dim3 grid((unsigned)(gp.S * hp.halo_tiles * cdiv(gp.N, 64)));
+            hipLaunchKernelGGL(gather_halo_bf16, grid, dim3(kThreads), 0, st, hp);
+            return;
+        }
+    }
     const int bm = gather_bm(gp.M, gp.N, cus, dma, (int)sizeof(T));
     // shallow slabs measure the same as deep ones on the 56x56 layers (within 2 % either
     // way), so they stay a tuning switch: AETHER_GATHER_KC=4
@@ -924,6 +1158,7 @@ static void plan_split(GatherSetup& gs, bool vec, int cus) {
     const bool dma = vec && sb < lim && gs.bt_bytes < lim;
     if (!dma || !g.dense_out || g.N % 4 != 0 || ob >= lim || (reinterpret_cast<uintptr_t>(g.out) & 15) != 0) return;
     if (getenv("AETHER_GATHER_KC") != nullptr) return;       // the tuning switch changes the slab depth
+    if (getenv("AETHER_GATHER_SPLIT_OFF") != nullptr) return; // lets small inputs reach the kernels of large ones
     const int bn = gather_bn(g.N), bm = gather_bm(g.M, g.N, cus, true, (int)sizeof(T));
     const int64_t tiles = (int64_t)cdiv(g.M, bm) * cdiv(g.N, bn);
     const int nslabs = g.Kpad / Elem<T>::BK;

@@ -93,3 +93,31 @@ def test_conv_layer_bf16_precision_switch():
     _loose(layer.dinputs.get(), O.conv_dgrad(dy, w, (10, 10), (1, 1), "same", dtype=np.float64))
     _loose(layer.dweights.get(), O.conv_wgrad(x, dy, (3, 3), (1, 1), "same", dtype=np.float64))
     _loose(layer.dbiases.get(), O.conv_dbias(dy, dtype=np.float64))
+
+
+# Unit-stride gathers over whole 64-channel blocks on images of about a multiple of 256 pixels
+# take the kernel that keeps the source pixels of a tile in LDS for all taps.  Small inputs
+# would split K instead; the tuning switch turns that off so that they reach the same code.
+HALO_CASES = [
+    (3, 16, 16, 64, 64, 3, 3, 1, 1, "same"),      # one tile per image
+    (2, 16, 32, 128, 96, 3, 3, 1, 1, "same"),     # two channel blocks, two n tiles (the second ragged)
+    (1, 50, 50, 64, 64, 3, 3, 1, 1, "same"),      # ten tiles, the last one partly empty
+    (2, 17, 17, 64, 64, 2, 2, 1, 1, "valid"),     # even filter
+    (2, 31, 31, 64, 64, 3, 3, 2, 2, "valid"),     # stride 2: the dgrad class of 2x2 taps on a 16x16 grid
+    (2, 16, 16, 64, 64, 3, 5, 1, 1, "same"),      # 3x5 filter, pad 1 on both axes: columns lose their border
+    (1, 16, 16, 64, 64, 5, 5, 1, 1, "same"),      # 25 taps: span too long for the buffer, the slab kernel runs
+]
+
+
+@pytest.mark.parametrize("case", HALO_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_bf16_fprop_dgrad_without_split_k(case, monkeypatch):
+    from tests import abi
+    monkeypatch.setenv("AETHER_GATHER_SPLIT_OFF", "1")
+    x, w, b, dy = _case(case, 5)
+    stride, pad = (case[7], case[8]), case[9]
+    xr, wr, dyr = O.round_to_bf16(x), O.round_to_bf16(w), O.round_to_bf16(dy)
+    abi.close(abi.fprop_bf16(x, w, b, stride, pad), O.conv_fprop(xr, wr, b, stride, pad, dtype=np.float64))
+    abi.close(abi.fprop_bf16(x, w, None, stride, pad), O.conv_fprop(xr, wr, None, stride, pad, dtype=np.float64))
+    abi.close(abi.dgrad_bf16(dy, w, x.shape, stride, pad),
+              O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
+

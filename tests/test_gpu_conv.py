@@ -163,3 +163,28 @@ def test_random_geometries(case):
     dw, db = abi.wgrad(x, dy, w.shape, (sH, sW), pad)
     abi.close(dw, O.conv_wgrad(x, dy, (fH, fW), (sH, sW), pad, dtype=np.float64), rms_scaled=True)
     abi.close(db, O.conv_dbias(dy, dtype=np.float64), rms_scaled=True)
+
+
+# The mode in which one workgroup keeps its rows of x in LDS and walks all n tiles is chosen
+# for 128-row tiles only, which the library takes from about 800 000 output pixels on; the
+# tuning switch forces that tile height so that small inputs reach the same code.
+NLOOP_CASES = [
+    (8, 48, 48, 64, 256, 1, 1, 1, 1, "valid"),    # K of two slabs, 4 n tiles
+    (8, 48, 48, 32, 192, 1, 1, 1, 1, "valid"),    # one slab, 3 n tiles
+    (8, 48, 48, 48, 136, 1, 1, 1, 1, "valid"),    # padded second slab, ragged last n tile
+    (3, 37, 41, 64, 1024, 1, 1, 1, 1, "valid"),   # the widest output it takes, rows past M in the last tile
+    (3, 37, 41, 16, 1088, 1, 1, 1, 1, "valid"),   # wider: back to one workgroup per tile
+    (2, 40, 40, 4, 128, 3, 3, 1, 1, "same"),      # K = 36: two slabs of a 3x3 filter, taps decoded per lane
+]
+
+
+@pytest.mark.parametrize("case", NLOOP_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_fprop_parity_with_128_row_tiles(case, monkeypatch):
+    from tests import abi
+    monkeypatch.setenv("AETHER_GATHER_BM", "128")
+    x, w, b, dy = _case(case, 11)
+    stride, pad = (case[7], case[8]), case[9]
+    want = O.conv_fprop(x, w, b, stride, pad, dtype=np.float64)
+    abi.close(abi.fprop(x, w, b, stride, pad), want)
+    abi.close(abi.fprop(x, w, None, stride, pad), O.conv_fprop(x, w, None, stride, pad, dtype=np.float64))
+
