@@ -1235,12 +1235,183 @@ static inline void set_out_divs(GatherParams& g) {
     g.div_tw = FastDiv(g.Tw > 0 ? g.Tw : 1);
 }
 
+// ------------------------------------------------------------------------------
+// Direct kernels for convolutions on 1 to 3 input channels (the first layer of an
+// image network: K = fH*fW*C is 9 to 27).  An implicit GEMM pads such a K to a slab
+// and, for dgrad, N = C to a 32-wide tile: up to 10 times the useful MFMA work, and
+// the gather moves single floats.  Here the filter sits in LDS as fp32 and a lane
+// owns 4 output channels d of one pixel, so that the lanes of a pixel read (dgrad)
+// or write (fprop) one contiguous row:
+//   fprop: y[m][4q..4q+3] = b + sum_{tap,c} x[pixel(m,tap)][c] * w[tap][c][4q..4q+3]
+//   dgrad: dx[p][c] = sum over the lanes q of the pixel of
+//                     sum_{tap: p = stride*o + tap - pad} dy[o][4q..4q+3] . w[tap][c][4q..4q+3]
+// D is a multiple of 4 and at most 256 (D/4 a power of two up to 64 for dgrad, whose
+// lanes add up with xor-shuffles), fH*fW*C*D floats fit 32 KB of LDS.
+// ------------------------------------------------------------------------------
+struct DirectParams {
+    const void* a;       // fprop: x [S,H,W,C];  dgrad: dy [S,Ho,Wo,D]
+    const void* w;       // [fH,fW,C,D]
+    const float* bias;   // fprop only, may be null
+    float* out;          // fprop: y [S,Ho,Wo,D];  dgrad: dx [S,H,W,C]
+    int S, H, W, C, Ho, Wo, D;
+    int fH, fW, sH, sW, pH, pW;
+    int M;               // pixels: S*Ho*Wo (fprop) or S*H*W (dgrad)
+    int q_shift;         // log2(D / 4): lanes per pixel
+    FastDiv div_hw, div_w;
+};
+
+constexpr int kDirectMaxW = 8192;    // floats of filter a direct kernel keeps in LDS
+
+template <typename T>
+__device__ __forceinline__ void direct_load_filter(const DirectParams& p, float* wl) {
+    const T* __restrict__ w = static_cast<const T*>(p.w);
+    const int n = p.fH * p.fW * p.C * p.D;
+    for (int i = (int)threadIdx.x; i < n; i += kThreads) wl[i] = Elem<T>::to_f32(w[i]);
+    __syncthreads();
+}
+
+// FH, FW, C are compile-time so that the taps unroll and their loads go out together; the
+// filter takes as much LDS as it has floats (dynamic), so that a CU holds 8 workgroups.
+template <typename T, int FH, int FW, int C>
+static __global__ __launch_bounds__(kThreads) void direct_fprop_smallc(const DirectParams p) {
+    extern __shared__ __attribute__((aligned(16))) float wl[];
+    direct_load_filter<T>(p, wl);
+    const T* __restrict__ x = static_cast<const T*>(p.a);
+    const int g = (int)(blockIdx.x * kThreads + threadIdx.x);
+    const int m = g >> p.q_shift;
+    const int q = g & ((1 << p.q_shift) - 1);
+    if (m >= p.M) return;
+    unsigned s_, rem, ho, wo;
+    p.div_hw.divmod((unsigned)m, s_, rem);
+    p.div_w.divmod(rem, ho, wo);
+    f4 acc = p.bias != nullptr ? *reinterpret_cast<const f4*>(p.bias + 4 * q) : f4{0.f, 0.f, 0.f, 0.f};
+    const float* wq = wl + 4 * q;
+    float xv[FH * FW * C];
+#pragma unroll
+    for (int fx = 0; fx < FH; ++fx)
+#pragma unroll
+        for (int fy = 0; fy < FW; ++fy) {
+            const int r = (int)ho * p.sH + fx - p.pH;
+            const int cc = (int)wo * p.sW + fy - p.pW;
+            const bool ok = (unsigned)r < (unsigned)p.H && (unsigned)cc < (unsigned)p.W;
+            const T* px = x + (size_t)((((int)s_ * p.H + (ok ? r : 0)) * p.W + (ok ? cc : 0)) * C);
+#pragma unroll
+            for (int c = 0; c < C; ++c) xv[(fx * FW + fy) * C + c] = ok ? Elem<T>::to_f32(px[c]) : 0.f;
+        }
+#pragma unroll
+    for (int k = 0; k < FH * FW * C; ++k) {
+        const f4 wv = *reinterpret_cast<const f4*>(wq + k * p.D);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] = fmaf(xv[k], wv[e], acc[e]);
+    }
+    *reinterpret_cast<f4*>(p.out + (size_t)m * p.D + 4 * q) = acc;
+}
+
+template <typename T, int FH, int FW, int C>
+static __global__ __launch_bounds__(kThreads) void direct_dgrad_smallc(const DirectParams p) {
+    extern __shared__ __attribute__((aligned(16))) float wl[];
+    direct_load_filter<T>(p, wl);
+    const T* __restrict__ dy = static_cast<const T*>(p.a);
+    const int g = (int)(blockIdx.x * kThreads + threadIdx.x);
+    const int m = g >> p.q_shift;                            // a pixel's lanes sit in one wave: q_shift <= 6
+    const int q = g & ((1 << p.q_shift) - 1);
+    unsigned s_, rem, i, j;
+    p.div_hw.divmod((unsigned)min(m, p.M - 1), s_, rem);
+    p.div_w.divmod(rem, i, j);
+    float acc[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) acc[c] = 0.f;
+    const float* wq = wl + 4 * q;
+    f4 gv[FH * FW];
+    bool oks[FH * FW];
+#pragma unroll
+    for (int fx = 0; fx < FH; ++fx)
+#pragma unroll
+        for (int fy = 0; fy < FW; ++fy) {
+            const int t = (int)i + p.pH - fx, u = (int)j + p.pW - fy;        // = ho * sH, wo * sW
+            const int ho = t / p.sH, wo = u / p.sW;
+            const bool ok = t >= 0 && u >= 0 && ho * p.sH == t && wo * p.sW == u && ho < p.Ho && wo < p.Wo;
+            const T* pd = dy + (size_t)(((int)s_ * p.Ho + (ok ? ho : 0)) * p.Wo + (ok ? wo : 0)) * p.D + 4 * q;
+            oks[fx * FW + fy] = ok;
+            if constexpr (sizeof(T) == 4) {
+                gv[fx * FW + fy] = *reinterpret_cast<const f4*>(pd);
+            } else {
+                const uint2 v = *reinterpret_cast<const uint2*>(pd);
+                gv[fx * FW + fy] = f4{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u),
+                                      __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u)};
+            }
+        }
+#pragma unroll
+    for (int tap = 0; tap < FH * FW; ++tap) {
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const f4 wv = *reinterpret_cast<const f4*>(wq + (tap * C + c) * p.D);
+            float d = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) d = fmaf(gv[tap][e], wv[e], d);
+            acc[c] += oks[tap] ? d : 0.f;
+        }
+    }
+    // add up the lanes of the pixel; every lane ends with the full sums and lane q < C stores channel q
+    for (int sh = 1; sh < (1 << p.q_shift); sh <<= 1) {
+#pragma unroll
+        for (int c = 0; c < C; ++c) acc[c] += __shfl_xor(acc[c], sh);
+    }
+    if (m < p.M) {
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+            if (q == c) p.out[(size_t)m * C + c] = acc[c];
+    }
+}
+
+// The shapes the direct kernels take; everything else goes to the gather kernels.
+template <typename T>
+static bool launch_direct(DirectParams& dp, bool dgrad, hipStream_t st) {
+    if (getenv("AETHER_DIRECT_OFF") != nullptr) return false;
+    const int chunks = dp.D / 4;
+    if (dp.C > 3 || dp.D % 4 != 0 || chunks < 4 || chunks > 64 || (chunks & (chunks - 1)) != 0) return false;
+    if ((int64_t)dp.fH * dp.fW * dp.C * dp.D > kDirectMaxW || (int64_t)dp.M * chunks >= ((int64_t)1 << 31)) return false;
+    if ((reinterpret_cast<uintptr_t>(dp.a) & 15) != 0 || (reinterpret_cast<uintptr_t>(dp.out) & 15) != 0 ||
+        (dp.bias != nullptr && (reinterpret_cast<uintptr_t>(dp.bias) & 15) != 0))
+        return false;
+    dp.q_shift = 0;
+    while ((1 << dp.q_shift) < chunks) ++dp.q_shift;
+    const dim3 grid((unsigned)cdiv((int64_t)dp.M * chunks, kThreads));
+    const size_t lds = (size_t)dp.fH * dp.fW * dp.C * dp.D * sizeof(float);
+#define AETH_DIRECT_CASE(FH_, FW_, C_)                                                                              \
+    if (dp.fH == FH_ && dp.fW == FW_ && dp.C == C_) {                                                               \
+        if (dgrad) hipLaunchKernelGGL((direct_dgrad_smallc<T, FH_, FW_, C_>), grid, dim3(kThreads), lds, st, dp);   \
+        else hipLaunchKernelGGL((direct_fprop_smallc<T, FH_, FW_, C_>), grid, dim3(kThreads), lds, st, dp);         \
+        return true;                                                                                                \
+    }
+    AETH_DIRECT_CASE(3, 3, 1)
+    AETH_DIRECT_CASE(3, 3, 2)
+    AETH_DIRECT_CASE(3, 3, 3)
+    AETH_DIRECT_CASE(5, 5, 1)
+    AETH_DIRECT_CASE(5, 5, 3)
+#undef AETH_DIRECT_CASE
+    return false;
+}
+
 template <typename T>
 int conv_fprop_impl(const char* fn, const T* x, const T* w, const float* bias, float* y,
                     int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW) {
     int Ho, Wo;
     int rc = check_conv_dims(fn, S, H, W, C, D, fH, fW, sH, sW, pH, pW, &Ho, &Wo);
     if (rc) return rc;
+    if (C <= 3) {
+        DirectParams dp;
+        dp.a = x; dp.w = w; dp.bias = bias; dp.out = y;
+        dp.S = S; dp.H = H; dp.W = W; dp.C = C; dp.Ho = Ho; dp.Wo = Wo; dp.D = D;
+        dp.fH = fH; dp.fW = fW; dp.sH = sH; dp.sW = sW; dp.pH = pH; dp.pW = pW;
+        dp.M = S * Ho * Wo;
+        dp.div_hw = FastDiv(Ho * Wo);
+        dp.div_w = FastDiv(Wo);
+        if (launch_direct<T>(dp, false, ctx().stream)) {
+            AETH_LAUNCH_CHECK();
+            return AETH_OK;
+        }
+    }
     constexpr int BK = Elem<T>::BK;
     GatherSetup gs;
     GatherParams& g = gs.gp;
@@ -1278,6 +1449,19 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
     constexpr int BK = Elem<T>::BK;
     const int nclass = sH * sW;
     if (nclass > 64) return fail(AETH_E_INVALID, "%s: stride too large", fn);
+    if (C <= 3) {
+        DirectParams dp;
+        dp.a = dy; dp.w = w; dp.bias = nullptr; dp.out = dx;
+        dp.S = S; dp.H = H; dp.W = W; dp.C = C; dp.Ho = Ho; dp.Wo = Wo; dp.D = D;
+        dp.fH = fH; dp.fW = fW; dp.sH = sH; dp.sW = sW; dp.pH = pH; dp.pW = pW;
+        dp.M = S * H * W;
+        dp.div_hw = FastDiv(H * W);
+        dp.div_w = FastDiv(W);
+        if (launch_direct<T>(dp, true, ctx().stream)) {
+            AETH_LAUNCH_CHECK();
+            return AETH_OK;
+        }
+    }
     std::vector<GatherSetup> sets;
     int64_t total_bytes = 0;
     for (int a = 0; a < sH; ++a) {

@@ -25,6 +25,9 @@ CASES = [
     (3, 13, 13, 128, 256, 3, 3, 2, 2, "valid"),
     (5, 9, 9, 24, 40, 3, 3, 1, 1, "same"),
     (40, 16, 16, 3, 32, 3, 3, 1, 1, "same"),
+    (5, 28, 28, 1, 32, 3, 3, 1, 1, "same"),       # direct kernels on bf16 inputs
+    (3, 12, 12, 2, 16, 5, 5, 2, 2, "same"),       # 5x5 on 2 channels: not built, gather kernels
+    (2, 11, 13, 3, 64, 5, 5, 1, 1, "same"),
 ]
 
 

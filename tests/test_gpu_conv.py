@@ -34,6 +34,13 @@ CASES = [
     (8, 48, 48, 64, 256, 1, 1, 1, 1, "valid"),   # K of two slabs, 4 n tiles: one workgroup walks the n tiles
     (8, 48, 48, 32, 192, 1, 1, 1, 1, "valid"),   # same with one slab, 3 n tiles
     (8, 48, 48, 48, 136, 1, 1, 1, 1, "valid"),   # same, padded second slab, ragged last n tile
+    # 1 to 3 input channels, 3x3 or 5x5, D/4 a power of two: the direct kernels (filter in LDS, a lane per 4 channels)
+    (5, 28, 28, 1, 32, 3, 3, 1, 1, "same"),      # first layer of the 28x28x1 topology
+    (3, 12, 12, 2, 16, 3, 3, 2, 2, "same"),      # stride 2: dgrad taps that do not divide
+    (2, 11, 13, 3, 64, 5, 5, 1, 1, "same"),
+    (2, 9, 9, 3, 256, 3, 3, 1, 1, "valid"),      # 64 lanes per pixel
+    (2, 9, 9, 3, 48, 3, 3, 1, 1, "same"),        # D/4 = 12: not a power of two, gather kernels
+    (3, 10, 10, 1, 32, 5, 5, 3, 2, "valid"),     # 5x5 on one channel, strides 3 and 2
 ]
 
 
