@@ -48,6 +48,8 @@ SIGNATURES = {
     "aeth_relu_fwd_f32": [_p, _p, _f, _i64],
     "aeth_relu_bwd_f32": [_p, _p, _p, _f, _i64],
     "aeth_maxpool_fwd_f32": [_p, _p, _p] + [_i] * 8,
+    "aeth_bn_relu_maxpool2_fwd_f32": [_p] * 11 + [_i] * 4 + [_f, _f, _f],
+    "aeth_maxpool2_relu_bwd_f32": [_p] * 5 + [_i] * 4 + [_f],
     "aeth_maxpool_bwd_f32": [_p, _p, _p] + [_i] * 8,
     "aeth_avgpool_fwd_f32": [_p, _p] + [_i] * 8,
     "aeth_avgpool_bwd_f32": [_p, _p] + [_i] * 8,

@@ -134,6 +134,9 @@ class Pooling:
         self.pooling_type = pooling_type
 
     def forward(self, inputs, training):
+        if _take_prefilled(self, inputs):       # a Batch_Norm two layers up has done this pass
+            return self.output
+        self._fused_relu = None
         inputs = as_device(inputs, _F32)
         if inputs.ndim != 4:
             raise ValueError(f"Expected a 4D tensor, got {inputs.ndim} instead.")
@@ -165,6 +168,15 @@ class Pooling:
         fH, fW = self.filter_size
         sH, sW = self.strides
         self.dinputs = DeviceTensor(self.inputs.shape, _F32)
+        relu = getattr(self, "_fused_relu", None)
+        if relu is not None:
+            # the forward pass of this block was fused: one kernel for this layer's and the
+            # activation's backward pass (the activation then finds its dinputs in place)
+            relu.dinputs = DeviceTensor(self.inputs.shape, _F32)
+            _ck(_L().aeth_maxpool2_relu_bwd_f32(dvalues.ptr, self.max_indicies.ptr, relu.inputs.ptr, self.dinputs.ptr,
+                                                relu.dinputs.ptr, S, H_in, W_in, C, _relu_alpha(relu)))
+            relu._bwd_prefilled_for = self.dinputs
+            return self.dinputs
         if self.pooling_type == "max":
             _ck(_L().aeth_maxpool_bwd_f32(dvalues.ptr, self.max_indicies.ptr, self.dinputs.ptr,
                                           S, H_in, W_in, C, fH, fW, sH, sW))
@@ -294,8 +306,32 @@ class Layer_Dropout_Spatial:
 # ----------------------------------------------------------------------------------
 # ReLU / Leaky_ReLU  (CNN_classes_cupy.py:406-428)
 # ----------------------------------------------------------------------------------
+def _take_prefilled(layer, inputs):
+    """True when a fused kernel further up has already produced this layer's output
+    for exactly this input tensor (see Batch_Norm._forward_block)."""
+    if getattr(layer, "_prefilled_for", None) is inputs and inputs is not None:
+        layer._prefilled_for = None
+        return True
+    layer._prefilled_for = None
+    return False
+
+
+def _take_bwd_prefilled(layer, dvalues):
+    if getattr(layer, "_bwd_prefilled_for", None) is dvalues and dvalues is not None:
+        layer._bwd_prefilled_for = None
+        return True
+    layer._bwd_prefilled_for = None
+    return False
+
+
+def _relu_alpha(layer):
+    return float(layer.alpha) if isinstance(layer, Leaky_ReLU) else 0.0
+
+
 class ReLU:
     def forward(self, inputs, training):
+        if _take_prefilled(self, inputs):
+            return self.output
         inputs = as_device(inputs, _F32)
         self.inputs = inputs
         self.output = DeviceTensor(inputs.shape, _F32)
@@ -303,6 +339,8 @@ class ReLU:
         return self.output
 
     def backward(self, dvalues):
+        if _take_bwd_prefilled(self, dvalues):
+            return
         dvalues = as_device(dvalues, _F32)
         self.dinputs = DeviceTensor(dvalues.shape, _F32)
         _ck(_L().aeth_relu_bwd_f32(self.inputs.ptr, dvalues.ptr, self.dinputs.ptr, 0.0, dvalues.size))
@@ -313,6 +351,8 @@ class Leaky_ReLU:
         self.alpha = alpha
 
     def forward(self, inputs, training):
+        if _take_prefilled(self, inputs):
+            return self.output
         inputs = as_device(inputs, _F32)
         self.inputs = inputs
         self.output = DeviceTensor(inputs.shape, _F32)
@@ -320,6 +360,8 @@ class Leaky_ReLU:
         return self.output
 
     def backward(self, dvalues):
+        if _take_bwd_prefilled(self, dvalues):
+            return
         dvalues = as_device(dvalues, _F32)
         self.dinputs = DeviceTensor(dvalues.shape, _F32)
         _ck(_L().aeth_relu_bwd_f32(self.inputs.ptr, dvalues.ptr, self.dinputs.ptr, self.alpha, dvalues.size))
@@ -367,9 +409,13 @@ class Batch_Norm:
         if training:
             self.batch_mean = DeviceTensor(C, _F32)
             self.batch_invstd = DeviceTensor(C, _F32)
-            _ck(_L().aeth_bn_fwd_train_f32(inputs.ptr, self.gamma.ptr, self.beta.ptr, self.running_mean.ptr,
-                                           self.running_var.ptr, self.batch_mean.ptr, self.batch_invstd.ptr,
-                                           self.output.ptr, rows, C, self.epsilon, self.momentum))
+            block = self._block_tail(inputs)
+            if block is not None:
+                self._forward_block(inputs, *block)
+            else:
+                _ck(_L().aeth_bn_fwd_train_f32(inputs.ptr, self.gamma.ptr, self.beta.ptr, self.running_mean.ptr,
+                                               self.running_var.ptr, self.batch_mean.ptr, self.batch_invstd.ptr,
+                                               self.output.ptr, rows, C, self.epsilon, self.momentum))
             # the reference's running statistics take the keepdims shape after a
             # training step (:475-476); keep that shape for get_parameters()
             keep = (1,) * (inputs.ndim - 1) + (C,)
@@ -380,6 +426,40 @@ class Batch_Norm:
             _ck(_L().aeth_bn_fwd_infer_f32(inputs.ptr, self.gamma.ptr, self.beta.ptr, self.running_mean.ptr,
                                            self.running_var.ptr, self.output.ptr, rows, C, self.epsilon))
         return self.output
+
+    # The usual convolution block is Batch_Norm -> ReLU / Leaky_ReLU -> Pooling(max, 2x2, stride 2).
+    # In training the three layers run as one pass over the tensor that writes all three
+    # outputs; the two layers behind find theirs in place when the model calls them with
+    # this layer's output.  AETHER_FUSE_BLOCK=0 keeps the layers apart.
+    def _block_tail(self, inputs):
+        if os.environ.get("AETHER_FUSE_BLOCK", "1") == "0" or inputs.ndim != 4:
+            return None
+        act = getattr(self, "next", None)
+        pool = getattr(act, "next", None)
+        if not isinstance(act, (ReLU, Leaky_ReLU)) or not isinstance(pool, Pooling):
+            return None
+        if (pool.pooling_type != "max" or pool.padding != "valid" or tuple(pool.filter_size) != (2, 2)
+                or tuple(pool.strides) != (2, 2)):
+            return None
+        S, H, W, C = inputs.shape
+        if H % 2 or W % 2 or C % 4:
+            return None
+        return act, pool
+
+    def _forward_block(self, inputs, act, pool):
+        S, H, W, C = inputs.shape
+        act.inputs = self.output
+        act.output = DeviceTensor(inputs.shape, _F32)
+        pool.inputs = act.output
+        pool.output = DeviceTensor((S, H // 2, W // 2, C), _F32)
+        pool.max_indicies = DeviceTensor((S, H // 2, W // 2, C), np.uint8)
+        _ck(_L().aeth_bn_relu_maxpool2_fwd_f32(
+            inputs.ptr, self.gamma.ptr, self.beta.ptr, self.running_mean.ptr, self.running_var.ptr,
+            self.batch_mean.ptr, self.batch_invstd.ptr, self.output.ptr, act.output.ptr, pool.output.ptr,
+            pool.max_indicies.ptr, S, H, W, C, self.epsilon, self.momentum, _relu_alpha(act)))
+        act._prefilled_for = self.output
+        pool._prefilled_for = act.output
+        pool._fused_relu = act
 
     def backward(self, dvalues):
         dvalues = as_device(dvalues, _F32)

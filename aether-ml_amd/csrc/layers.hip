@@ -615,6 +615,86 @@ static void adam_corrections(float beta1, float beta2, int t, float* c1, float* 
 
 using namespace aeth;
 
+// ---- batch norm + (leaky) ReLU + 2x2 stride-2 max pooling in one pass ----------------
+// The three layers of a convolution block read and write the same tensor three times
+// over.  One thread takes a pooling window and 4 channels: it reads the 4 pixels once
+// and writes what each layer would have written (the layers keep their outputs for
+// the backward pass and for callers that look at them).  H and W even, C % 4 == 0.
+struct Pool2Params {
+    int S, H, W, C4, Ho, Wo;
+    FastDiv div_c4, div_wo, div_ho;
+};
+
+__global__ __launch_bounds__(kEwThreads) void bn_relu_maxpool2_fwd_kernel(
+    const ew_f4* __restrict__ x, const ew_f4* __restrict__ gamma, const ew_f4* __restrict__ beta,
+    const ew_f4* __restrict__ mean, const ew_f4* __restrict__ invstd, ew_f4* __restrict__ bn_out,
+    ew_f4* __restrict__ relu_out, ew_f4* __restrict__ pool_out, uint32_t* __restrict__ idx, float alpha,
+    Pool2Params p, unsigned n) {
+    const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    unsigned t, c4, u, wo, s, ho;
+    p.div_c4.divmod(i, t, c4);
+    p.div_wo.divmod(t, u, wo);
+    p.div_ho.divmod(u, s, ho);
+    const unsigned base = ((s * p.H + 2u * ho) * p.W + 2u * wo) * p.C4 + c4;
+    const ew_f4 g = gamma[c4], b = beta[c4], m = mean[c4], is = invstd[c4];
+    ew_f4 best;
+    unsigned bi = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const unsigned off = base + ((unsigned)(k >> 1) * p.W + (unsigned)(k & 1)) * p.C4;
+        const ew_f4 v = x[off];
+        ew_f4 y, r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            y[e] = g[e] * ((v[e] - m[e]) * is[e]) + b[e];
+            r[e] = y[e] > 0.f ? y[e] : alpha * y[e];
+        }
+        bn_out[off] = y;
+        relu_out[off] = r;
+        if (k == 0) {
+            best = r;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (r[e] > best[e]) {        // strict: the first maximum keeps its place
+                    best[e] = r[e];
+                    bi = (bi & ~(0xffu << (8 * e))) | ((unsigned)k << (8 * e));
+                }
+        }
+    }
+    pool_out[i] = best;
+    idx[i] = bi;
+}
+
+// backward of the pooling and the ReLU of such a block: every pixel belongs to one window
+__global__ __launch_bounds__(kEwThreads) void maxpool2_relu_bwd_kernel(
+    const ew_f4* __restrict__ dy, const uint32_t* __restrict__ idx, const ew_f4* __restrict__ relu_in,
+    ew_f4* __restrict__ pool_dx, ew_f4* __restrict__ relu_dx, float alpha, Pool2Params p, unsigned n) {
+    const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    unsigned t, c4, u, wo, s, ho;
+    p.div_c4.divmod(i, t, c4);
+    p.div_wo.divmod(t, u, wo);
+    p.div_ho.divmod(u, s, ho);
+    const unsigned base = ((s * p.H + 2u * ho) * p.W + 2u * wo) * p.C4 + c4;
+    const ew_f4 g = dy[i];
+    const unsigned bi = idx[i];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const unsigned off = base + ((unsigned)(k >> 1) * p.W + (unsigned)(k & 1)) * p.C4;
+        const ew_f4 xin = relu_in[off];
+        ew_f4 d, r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            d[e] = ((bi >> (8 * e)) & 0xffu) == (unsigned)k ? g[e] : 0.f;
+            r[e] = xin[e] < 0.f ? alpha * d[e] : d[e];
+        }
+        pool_dx[off] = d;
+        relu_dx[off] = r;
+    }
+}
+
 #define EW_LAUNCH(kernel, n, ...)                                                          \
     do {                                                                                   \
         hipLaunchKernelGGL(kernel, dim3(ew_blocks(n)), dim3(kEwThreads), 0, ctx().stream, __VA_ARGS__); \
@@ -648,6 +728,75 @@ int aeth_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta,
     AETH_LAUNCH_CHECK();
     int64_t n = (int64_t)rows * C;
     EW_LAUNCH(bn_apply, n, x, gamma, beta, save_mean, save_invstd, y, n, C);
+    return AETH_OK;
+}
+
+static int pool2_params(int S, int H, int W, int C, Pool2Params* p, unsigned* n) {
+    if (S <= 0 || H <= 0 || W <= 0 || C <= 0 || H % 2 != 0 || W % 2 != 0 || C % 4 != 0) return AETH_E_INVALID;
+    if ((int64_t)S * H * W * C >= ((int64_t)1 << 31)) return AETH_E_INVALID;
+    p->S = S; p->H = H; p->W = W; p->C4 = C / 4; p->Ho = H / 2; p->Wo = W / 2;
+    p->div_c4 = FastDiv(p->C4);
+    p->div_wo = FastDiv(p->Wo);
+    p->div_ho = FastDiv(p->Ho);
+    *n = (unsigned)((int64_t)S * p->Ho * p->Wo * p->C4);
+    return AETH_OK;
+}
+
+static inline bool aligned16(const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; }
+
+int aeth_bn_relu_maxpool2_fwd_f32(const float* x, const float* gamma, const float* beta, float* running_mean,
+                                  float* running_var, float* save_mean, float* save_invstd, float* bn_out,
+                                  float* relu_out, float* pool_out, uint8_t* idx, int S, int H, int W, int C,
+                                  float eps, float momentum, float alpha) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(x && gamma && beta && running_mean && running_var && save_mean && save_invstd);
+    AETH_CHECK_ARG(bn_out && relu_out && pool_out && idx);
+    Pool2Params p;
+    unsigned n;
+    if (pool2_params(S, H, W, C, &p, &n) != AETH_OK)
+        return fail(AETH_E_INVALID, "%s: needs even H and W, C %% 4 == 0 and fewer than 2^31 elements", __func__);
+    AETH_CHECK_ARG(aligned16(x) && aligned16(gamma) && aligned16(beta) && aligned16(save_mean) &&
+                   aligned16(save_invstd) && aligned16(bn_out) && aligned16(relu_out) && aligned16(pool_out) &&
+                   aligned16(idx));
+    const int rows = S * H * W;
+    int nblk, rpb;
+    dim3 grid;
+    col_grid(rows, C, &nblk, &rpb, &grid);
+    void* ws;
+    int rc = workspace((int64_t)2 * nblk * C * sizeof(float), &ws);
+    if (rc) return rc;
+    float* part = (float*)ws;
+    hipStream_t st = ctx().stream;
+    if (col_vec4(C, x, part)) {
+        hipLaunchKernelGGL(bn_stats_partial4, dim3(grid.x, cdiv(C / 4, 64)), dim3(kEwThreads), 0, st, x, rows, C, rpb, part);
+    } else {
+        hipLaunchKernelGGL(bn_stats_partial, grid, dim3(kEwThreads), 0, st, x, rows, C, rpb, part);
+    }
+    AETH_LAUNCH_CHECK();
+    hipLaunchKernelGGL(bn_stats_final, dim3(cdiv(C, 64)), dim3(256), 0, st, x, part, nblk, rows, C, eps, momentum,
+                       running_mean, running_var, save_mean, save_invstd);
+    AETH_LAUNCH_CHECK();
+    hipLaunchKernelGGL(bn_relu_maxpool2_fwd_kernel, dim3(cdiv(n, kEwThreads)), dim3(kEwThreads), 0, st,
+                       (const ew_f4*)x, (const ew_f4*)gamma, (const ew_f4*)beta, (const ew_f4*)save_mean,
+                       (const ew_f4*)save_invstd, (ew_f4*)bn_out, (ew_f4*)relu_out, (ew_f4*)pool_out, (uint32_t*)idx,
+                       alpha, p, n);
+    AETH_LAUNCH_CHECK();
+    return AETH_OK;
+}
+
+int aeth_maxpool2_relu_bwd_f32(const float* dy, const uint8_t* idx, const float* relu_in, float* pool_dx,
+                               float* relu_dx, int S, int H, int W, int C, float alpha) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(dy && idx && relu_in && pool_dx && relu_dx);
+    Pool2Params p;
+    unsigned n;
+    if (pool2_params(S, H, W, C, &p, &n) != AETH_OK)
+        return fail(AETH_E_INVALID, "%s: needs even H and W, C %% 4 == 0 and fewer than 2^31 elements", __func__);
+    AETH_CHECK_ARG(aligned16(dy) && aligned16(idx) && aligned16(relu_in) && aligned16(pool_dx) && aligned16(relu_dx));
+    hipLaunchKernelGGL(maxpool2_relu_bwd_kernel, dim3(cdiv(n, kEwThreads)), dim3(kEwThreads), 0, ctx().stream,
+                       (const ew_f4*)dy, (const uint32_t*)idx, (const ew_f4*)relu_in, (ew_f4*)pool_dx, (ew_f4*)relu_dx,
+                       alpha, p, n);
+    AETH_LAUNCH_CHECK();
     return AETH_OK;
 }
 

@@ -203,7 +203,7 @@ def main():
         "extra": extra,
     }
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(32, H, W, C, D)
+        out["cpu_baseline"] = cpu_baseline(96, H, W, C, D)
     print(json.dumps(out))
 
 

@@ -144,6 +144,22 @@ int aeth_maxpool_fwd_f32(const float* x, float* y, uint8_t* idx,
                          int S, int H, int W, int C, int fH, int fW, int sH, int sW);
 int aeth_maxpool_bwd_f32(const float* dy, const uint8_t* idx, float* dx,
                          int S, int H, int W, int C, int fH, int fW, int sH, int sW);
+/* One pass over a convolution block's Batch_Norm (training branch, as bn_fwd_train),
+ * ReLU / Leaky_ReLU and 2x2 stride-2 "valid" max pooling: writes the three outputs
+ * the layers would have written one after the other (:467-476, :406-428, :212-273)
+ * and the pooling indices.  x is [S,H,W,C] with even H and W and C % 4 == 0, all
+ * pointers 16-byte aligned; AETH_E_INVALID otherwise (callers then use the three
+ * separate entry points).  maxpool2_relu_bwd is the backward pass of the pooling
+ * and the activation of such a block (:275-300, :412-415): pool_dx = Pooling.dinputs,
+ * relu_dx = ReLU.dinputs, relu_in = the activation's input (Batch_Norm's output). */
+int aeth_bn_relu_maxpool2_fwd_f32(const float* x, const float* gamma, const float* beta,
+                                  float* running_mean, float* running_var,
+                                  float* save_mean, float* save_invstd,
+                                  float* bn_out, float* relu_out, float* pool_out, uint8_t* idx,
+                                  int S, int H, int W, int C, float eps, float momentum, float alpha);
+int aeth_maxpool2_relu_bwd_f32(const float* dy, const uint8_t* idx, const float* relu_in,
+                               float* pool_dx, float* relu_dx,
+                               int S, int H, int W, int C, float alpha);
 /* Pooling "average" :267-268 and the scatter kernel :163-202. */
 int aeth_avgpool_fwd_f32(const float* x, float* y,
                          int S, int H, int W, int C, int fH, int fW, int sH, int sW);

@@ -302,3 +302,60 @@ def test_regularization_loss_and_adam():
     assert opt.iterations == 4
     _close(dense.weight_momentums, m[0])
     _close(dense.weight_cache, v[0], atol=1e-7)
+
+
+def _block(aether, alpha):
+    """Batch_Norm -> activation -> Pooling wired the way Model.finalize wires them."""
+    bn = aether.Batch_Norm()
+    act = aether.ReLU() if alpha is None else aether.Leaky_ReLU(alpha=alpha)
+    pool = aether.Pooling()
+    bn.next, act.next = act, pool
+    return bn, act, pool
+
+
+@pytest.mark.parametrize("shape,alpha", [((8, 16, 16, 32), None), ((3, 6, 10, 8), 0.01), ((5, 4, 2, 64), None),
+                                         ((2, 7, 6, 8), None), ((2, 6, 6, 6), None)])
+def test_fused_block_equals_the_three_layers(shape, alpha, monkeypatch):
+    import aether
+    r = np.random.RandomState(5)
+    x = (r.randn(*shape) * 2.0 + 0.5).astype(np.float32)
+    x[0, :2, :2, 0] = 1.25                      # a window of equal values: the first one wins the pooling
+    dy = r.randn(shape[0], shape[1] // 2, shape[2] // 2, shape[3]).astype(np.float32)
+    got = {}
+    for fuse in ("1", "0"):
+        monkeypatch.setenv("AETHER_FUSE_BLOCK", fuse)
+        bn, act, pool = _block(aether, alpha)
+        bn.forward(x, True)
+        act.forward(bn.output, True)
+        pool.forward(act.output, True)
+        pool.backward(dy)
+        act.backward(pool.dinputs)
+        bn.backward(act.dinputs)
+        got[fuse] = [t.get() for t in (bn.output, act.output, pool.output, pool.max_indicies, pool.dinputs,
+                                       act.dinputs, bn.dinputs, bn.dweights, bn.dbiases, bn.running_mean,
+                                       bn.running_var)]
+        fused_ran = getattr(pool, "_fused_relu", None) is not None
+        even = shape[1] % 2 == 0 and shape[2] % 2 == 0 and shape[3] % 4 == 0
+        assert fused_ran == (fuse == "1" and even)
+    for a, b in zip(got["1"], got["0"]):
+        assert a.shape == b.shape
+        assert np.allclose(a, b, rtol=1e-6, atol=1e-6)
+    # the indices agree exactly wherever the activations do
+    same = np.all(got["1"][1] == got["0"][1])
+    assert not same or np.array_equal(got["1"][3], got["0"][3])
+
+
+def test_fused_block_entry_points_reject_what_they_do_not_cover():
+    from aether import _lib
+    from aether.tensor import DeviceTensor
+    L = _lib.lib()
+    t = DeviceTensor.zeros(4 * 4 * 4 * 8)
+    c = DeviceTensor.zeros(8)
+    i8 = DeviceTensor((4 * 2 * 2 * 8,), np.uint8)
+    args = (t.ptr, c.ptr, c.ptr, c.ptr, c.ptr, c.ptr, c.ptr, t.ptr, t.ptr, t.ptr, i8.ptr)
+    assert L.aeth_bn_relu_maxpool2_fwd_f32(*args, 4, 3, 4, 8, 1e-5, 0.9, 0.0) == _lib.AETH_E_INVALID     # odd H
+    assert L.aeth_bn_relu_maxpool2_fwd_f32(*args, 4, 4, 4, 6, 1e-5, 0.9, 0.0) == _lib.AETH_E_INVALID     # C % 4
+    assert L.aeth_maxpool2_relu_bwd_f32(t.ptr, i8.ptr, t.ptr, t.ptr, t.ptr, 4, 4, 5, 8, 0.0) == _lib.AETH_E_INVALID
+    assert L.aeth_maxpool2_relu_bwd_f32(None, i8.ptr, t.ptr, t.ptr, t.ptr, 4, 4, 4, 8, 0.0) == _lib.AETH_E_INVALID
+    assert L.aeth_bn_relu_maxpool2_fwd_f32(*args, 4, 4, 4, 8, 1e-5, 0.9, 0.0) == 0
+
