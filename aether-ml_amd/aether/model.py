@@ -161,6 +161,12 @@ class Model:
             recs[key] = {"graph": None}
             return None
         lib = _lib.lib()
+        # a recording reads and writes the parameter buffers it was made with: parameters set
+        # anew since then (set_parameters, load_parameters) make it stale
+        params = [(id(l), l.weights.ptr, l.biases.ptr) for l in self.trainable_layers]
+        if rec["graph"] is not None and rec.get("params") != params:
+            _lib.check(lib.aeth_graph_destroy(rec["graph"]))
+            recs[key] = rec = {"graph": None}
         if rec["graph"] is None:
             rec["x"] = DeviceTensor(batch_X.shape, np.float32)
             rec["labels"] = DeviceTensor(labels.shape, np.int32)
@@ -179,6 +185,7 @@ class Model:
                 rc = lib.aeth_graph_end(C.byref(handle))
             _lib.check(rc)
             rec["graph"] = handle
+            rec["params"] = params
             # what the layers point at after this step (output, dinputs, dweights, ...):
             # replays fill the same buffers, so the attributes are put back after steps
             # that ran in between (an evaluation, a step of another shape)

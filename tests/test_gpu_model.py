@@ -276,6 +276,11 @@ def test_recorded_steps_equal_eager_steps():
             _lib.sync()
         if step == 6:
             assert eager.train_step(Xodd, yodd) == rec.train_step(Xodd, yodd)      # another shape: runs eagerly
+        if step == 7:
+            # parameters set anew live in new buffers: the recording made with the old ones must not be replayed
+            for m in (eager, rec):
+                host = [tuple(np.array(np.asarray(t)) for t in ps) for ps in m.get_parameters()]
+                m.set_parameters(host)
     assert len([r for r in rec._recordings.values() if r.get("graph")]) == 1
     rec.record_steps(False)
     assert eager.train_step(Xs[0], ys[0]) == rec.train_step(Xs[0], ys[0])
