@@ -50,6 +50,7 @@ SIGNATURES = {
     "aeth_maxpool_fwd_f32": [_p, _p, _p] + [_i] * 8,
     "aeth_bn_relu_maxpool2_fwd_f32": [_p] * 11 + [_i] * 4 + [_f, _f, _f],
     "aeth_maxpool2_relu_bwd_f32": [_p] * 5 + [_i] * 4 + [_f],
+    "aeth_maxpool2_relu_bn_bwd_f32": [_p] * 12 + [_i] * 4 + [_f],
     "aeth_maxpool_bwd_f32": [_p, _p, _p] + [_i] * 8,
     "aeth_avgpool_fwd_f32": [_p, _p] + [_i] * 8,
     "aeth_avgpool_bwd_f32": [_p, _p] + [_i] * 8,

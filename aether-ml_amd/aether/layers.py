@@ -136,7 +136,7 @@ class Pooling:
     def forward(self, inputs, training):
         if _take_prefilled(self, inputs):       # a Batch_Norm two layers up has done this pass
             return self.output
-        self._fused_relu = None
+        self._fused_relu = self._fused_bn = None
         inputs = as_device(inputs, _F32)
         if inputs.ndim != 4:
             raise ValueError(f"Expected a 4D tensor, got {inputs.ndim} instead.")
@@ -171,10 +171,24 @@ class Pooling:
         relu = getattr(self, "_fused_relu", None)
         if relu is not None:
             # the forward pass of this block was fused: one kernel for this layer's and the
-            # activation's backward pass (the activation then finds its dinputs in place)
+            # activation's backward pass (the activation then finds its dinputs in place),
+            # which also takes the batch norm's column sums when the channel count allows it
             relu.dinputs = DeviceTensor(self.inputs.shape, _F32)
-            _ck(_L().aeth_maxpool2_relu_bwd_f32(dvalues.ptr, self.max_indicies.ptr, relu.inputs.ptr, self.dinputs.ptr,
-                                                relu.dinputs.ptr, S, H_in, W_in, C, _relu_alpha(relu)))
+            bn = getattr(self, "_fused_bn", None)
+            c4 = C // 4
+            if bn is not None and 256 % c4 == 0:
+                bn.dinputs = DeviceTensor(self.inputs.shape, _F32)
+                bn.dweights = DeviceTensor(C, _F32)
+                bn.dbiases = DeviceTensor(C, _F32)
+                _ck(_L().aeth_maxpool2_relu_bn_bwd_f32(
+                    dvalues.ptr, self.max_indicies.ptr, relu.inputs.ptr, bn.inputs.ptr, bn.gamma.ptr,
+                    bn.batch_mean.ptr, bn.batch_invstd.ptr, self.dinputs.ptr, relu.dinputs.ptr, bn.dinputs.ptr,
+                    bn.dweights.ptr, bn.dbiases.ptr, S, H_in, W_in, C, _relu_alpha(relu)))
+                bn._bwd_prefilled_for = relu.dinputs
+            else:
+                _ck(_L().aeth_maxpool2_relu_bwd_f32(dvalues.ptr, self.max_indicies.ptr, relu.inputs.ptr,
+                                                    self.dinputs.ptr, relu.dinputs.ptr, S, H_in, W_in, C,
+                                                    _relu_alpha(relu)))
             relu._bwd_prefilled_for = self.dinputs
             return self.dinputs
         if self.pooling_type == "max":
@@ -460,8 +474,11 @@ class Batch_Norm:
         act._prefilled_for = self.output
         pool._prefilled_for = act.output
         pool._fused_relu = act
+        pool._fused_bn = self
 
     def backward(self, dvalues):
+        if _take_bwd_prefilled(self, dvalues):
+            return self.dinputs
         dvalues = as_device(dvalues, _F32)
         C = self.inputs.shape[-1]
         rows = self.inputs.size // C

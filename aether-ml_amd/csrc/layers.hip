@@ -695,6 +695,73 @@ __global__ __launch_bounds__(kEwThreads) void maxpool2_relu_bwd_kernel(
     }
 }
 
+// The same backward pass with the batch norm's column sums taken on the way: s1 = sum dz,
+// s2 = sum dz * (x - mean) over the rows, dz = the activation's input gradient.  A thread
+// keeps its channel group over the windows it walks (the stride is a multiple of C4) and
+// the threads of a block that share a group are added through LDS in a fixed order: the
+// partials land in the part[v][block][c] layout of bn_bwd_final.  256 % C4 == 0.
+__global__ __launch_bounds__(kEwThreads) void maxpool2_relu_bnpart_bwd_kernel(
+    const ew_f4* __restrict__ dy, const uint32_t* __restrict__ idx, const ew_f4* __restrict__ relu_in,
+    const ew_f4* __restrict__ x, const ew_f4* __restrict__ mean, ew_f4* __restrict__ pool_dx,
+    ew_f4* __restrict__ relu_dx, float* __restrict__ part, float alpha, Pool2Params p, unsigned n) {
+    __shared__ ew_f4 red[2][kEwThreads];
+    const unsigned tid = threadIdx.x;
+    const unsigned stride = gridDim.x * blockDim.x;
+    const unsigned c4 = tid % (unsigned)p.C4;            // the same for every window of this thread
+    const ew_f4 mu = mean[c4];
+    ew_f4 s1 = {0.f, 0.f, 0.f, 0.f}, s2 = {0.f, 0.f, 0.f, 0.f};
+    for (unsigned i = blockIdx.x * blockDim.x + tid; i < n; i += stride) {
+        unsigned t, u, wo, s, ho;
+        t = p.div_c4.div(i);
+        p.div_wo.divmod(t, u, wo);
+        p.div_ho.divmod(u, s, ho);
+        const unsigned base = ((s * p.H + 2u * ho) * p.W + 2u * wo) * p.C4 + c4;
+        const ew_f4 g = dy[i];
+        const unsigned bi = idx[i];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const unsigned off = base + ((unsigned)(k >> 1) * p.W + (unsigned)(k & 1)) * p.C4;
+            const ew_f4 xin = relu_in[off];
+            const ew_f4 xv = x[off];
+            ew_f4 d, r;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                d[e] = ((bi >> (8 * e)) & 0xffu) == (unsigned)k ? g[e] : 0.f;
+                r[e] = xin[e] < 0.f ? alpha * d[e] : d[e];
+            }
+            pool_dx[off] = d;
+            relu_dx[off] = r;
+            s1 += r;
+            s2 += r * (xv - mu);
+        }
+    }
+    red[0][tid] = s1;
+    red[1][tid] = s2;
+    __syncthreads();
+    if (tid < (unsigned)p.C4) {
+        ew_f4 a = {0.f, 0.f, 0.f, 0.f}, b = {0.f, 0.f, 0.f, 0.f};
+        for (unsigned r = tid; r < kEwThreads; r += (unsigned)p.C4) {
+            a += red[0][r];
+            b += red[1][r];
+        }
+        const int C = 4 * p.C4;
+        *reinterpret_cast<ew_f4*>(part + (size_t)blockIdx.x * C + 4 * tid) = a;
+        *reinterpret_cast<ew_f4*>(part + ((size_t)gridDim.x + blockIdx.x) * C + 4 * tid) = b;
+    }
+}
+
+// dx = coef0 * dy + A * (x - mean) + B on groups of 4 channels
+__global__ __launch_bounds__(kEwThreads) void bn_bwd_apply4(const ew_f4* __restrict__ x, const ew_f4* __restrict__ dy,
+                                                           const ew_f4* __restrict__ mean, const float* __restrict__ coef,
+                                                           ew_f4* __restrict__ dx, unsigned n4, int C4) {
+    const unsigned stride = gridDim.x * blockDim.x;
+    const ew_f4* c0 = reinterpret_cast<const ew_f4*>(coef);
+    for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+        const unsigned c4 = i % (unsigned)C4;
+        dx[i] = c0[c4] * dy[i] + c0[C4 + c4] * (x[i] - mean[c4]) + c0[2 * C4 + c4];
+    }
+}
+
 #define EW_LAUNCH(kernel, n, ...)                                                          \
     do {                                                                                   \
         hipLaunchKernelGGL(kernel, dim3(ew_blocks(n)), dim3(kEwThreads), 0, ctx().stream, __VA_ARGS__); \
@@ -796,6 +863,43 @@ int aeth_maxpool2_relu_bwd_f32(const float* dy, const uint8_t* idx, const float*
     hipLaunchKernelGGL(maxpool2_relu_bwd_kernel, dim3(cdiv(n, kEwThreads)), dim3(kEwThreads), 0, ctx().stream,
                        (const ew_f4*)dy, (const uint32_t*)idx, (const ew_f4*)relu_in, (ew_f4*)pool_dx, (ew_f4*)relu_dx,
                        alpha, p, n);
+    AETH_LAUNCH_CHECK();
+    return AETH_OK;
+}
+
+int aeth_maxpool2_relu_bn_bwd_f32(const float* dy, const uint8_t* idx, const float* relu_in, const float* x,
+                                  const float* gamma, const float* save_mean, const float* save_invstd,
+                                  float* pool_dx, float* relu_dx, float* bn_dx, float* dgamma, float* dbeta,
+                                  int S, int H, int W, int C, float alpha) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(dy && idx && relu_in && x && gamma && save_mean && save_invstd);
+    AETH_CHECK_ARG(pool_dx && relu_dx && bn_dx && dgamma && dbeta);
+    Pool2Params p;
+    unsigned n;
+    if (pool2_params(S, H, W, C, &p, &n) != AETH_OK || kEwThreads % p.C4 != 0)
+        return fail(AETH_E_INVALID, "%s: needs even H and W, C / 4 a divisor of %d and fewer than 2^31 elements",
+                    __func__, kEwThreads);
+    AETH_CHECK_ARG(aligned16(dy) && aligned16(idx) && aligned16(relu_in) && aligned16(x) && aligned16(save_mean) &&
+                   aligned16(pool_dx) && aligned16(relu_dx) && aligned16(bn_dx));
+    const int rows = S * H * W;
+    int nblk = cdiv(n, kEwThreads);
+    if (nblk > 256) nblk = 256;
+    void* ws;
+    int rc = workspace(((int64_t)2 * nblk * C + 3 * C) * sizeof(float), &ws);
+    if (rc) return rc;
+    float* part = (float*)ws;
+    float* coef = part + (int64_t)2 * nblk * C;
+    hipStream_t st = ctx().stream;
+    hipLaunchKernelGGL(maxpool2_relu_bnpart_bwd_kernel, dim3(nblk), dim3(kEwThreads), 0, st, (const ew_f4*)dy,
+                       (const uint32_t*)idx, (const ew_f4*)relu_in, (const ew_f4*)x, (const ew_f4*)save_mean,
+                       (ew_f4*)pool_dx, (ew_f4*)relu_dx, part, alpha, p, n);
+    AETH_LAUNCH_CHECK();
+    hipLaunchKernelGGL(bn_bwd_final, dim3(cdiv(C, 64)), dim3(256), 0, st, part, nblk, rows, C, gamma, save_invstd,
+                       dgamma, dbeta, coef);
+    AETH_LAUNCH_CHECK();
+    const unsigned n4 = (unsigned)((int64_t)rows * C / 4);
+    hipLaunchKernelGGL(bn_bwd_apply4, dim3(ew_blocks(n4)), dim3(kEwThreads), 0, st, (const ew_f4*)x,
+                       (const ew_f4*)relu_dx, (const ew_f4*)save_mean, coef, (ew_f4*)bn_dx, n4, C / 4);
     AETH_LAUNCH_CHECK();
     return AETH_OK;
 }

@@ -160,6 +160,15 @@ int aeth_bn_relu_maxpool2_fwd_f32(const float* x, const float* gamma, const floa
 int aeth_maxpool2_relu_bwd_f32(const float* dy, const uint8_t* idx, const float* relu_in,
                                float* pool_dx, float* relu_dx,
                                int S, int H, int W, int C, float alpha);
+/* The same with Batch_Norm.backward (:484-508) behind it: the column sums of the
+ * batch norm are taken while the activation's gradient is written.  x is the batch
+ * norm's input, bn_dx its dinputs.  Additionally needs C / 4 to divide 256. */
+int aeth_maxpool2_relu_bn_bwd_f32(const float* dy, const uint8_t* idx, const float* relu_in,
+                                  const float* x, const float* gamma,
+                                  const float* save_mean, const float* save_invstd,
+                                  float* pool_dx, float* relu_dx, float* bn_dx,
+                                  float* dgamma, float* dbeta,
+                                  int S, int H, int W, int C, float alpha);
 /* Pooling "average" :267-268 and the scatter kernel :163-202. */
 int aeth_avgpool_fwd_f32(const float* x, float* y,
                          int S, int H, int W, int C, int fH, int fW, int sH, int sW);

@@ -314,7 +314,7 @@ def _block(aether, alpha):
 
 
 @pytest.mark.parametrize("shape,alpha", [((8, 16, 16, 32), None), ((3, 6, 10, 8), 0.01), ((5, 4, 2, 64), None),
-                                         ((2, 7, 6, 8), None), ((2, 6, 6, 6), None)])
+                                         ((2, 7, 6, 8), None), ((2, 6, 6, 6), None), ((2, 4, 4, 24), 0.2)])
 def test_fused_block_equals_the_three_layers(shape, alpha, monkeypatch):
     import aether
     r = np.random.RandomState(5)
@@ -339,7 +339,8 @@ def test_fused_block_equals_the_three_layers(shape, alpha, monkeypatch):
         assert fused_ran == (fuse == "1" and even)
     for a, b in zip(got["1"], got["0"]):
         assert a.shape == b.shape
-        assert np.allclose(a, b, rtol=1e-6, atol=1e-6)
+        # the column sums of the batch norm's backward pass are added in another order
+        assert np.allclose(a, b, rtol=2e-5, atol=2e-5 * max(1.0, float(np.abs(b).max())))
     # the indices agree exactly wherever the activations do
     same = np.all(got["1"][1] == got["0"][1])
     assert not same or np.array_equal(got["1"][3], got["0"][3])
