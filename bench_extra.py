@@ -47,13 +47,15 @@ def _time(fn, steps, warmup):
     return e0.elapsed_ms(e1) / steps
 
 
-def conv_table(steps, warmup):
+def conv_table(steps, warmup, only=None):
     from aether import _lib
     from aether.tensor import DeviceTensor
     L = _lib.lib()
     rng = np.random.default_rng(0)
     out = {}
     for name, S, H, W, C, D, f, st, P, with_bf16 in SHAPES:
+        if only is not None and name != only:
+            continue
         Ho = (H + 2 * P - f) // st + 1
         Wo = (W + 2 * P - f) // st + 1
         dims = (S, H, W, C, D, f, f, st, st, P, P)
@@ -164,5 +166,8 @@ if __name__ == "__main__":
     import json
     if "--train-only" in sys.argv:
         print(json.dumps(train_step(50, 10), indent=1))
+    elif "--shape" in sys.argv:
+        # one shape of the list only, e.g. --shape cfg4_1x1_64_to256 (for profiler runs)
+        print(json.dumps(conv_table(10, 2, only=sys.argv[sys.argv.index("--shape") + 1]), indent=1))
     else:
         print(json.dumps(run(20, 5), indent=1))
