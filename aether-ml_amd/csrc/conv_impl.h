@@ -1764,10 +1764,12 @@ __global__ __launch_bounds__(kThreads) void wgrad_gemm(const WgradParams p) {
 //   * dbias fused: the workgroups of k tile 0 also add up the columns of every dy
 //     slab they hold in LDS.
 // ------------------------------------------------------------------------------
-template <int CW>
+template <int CW, int BR = kWgBR>                        // BR rows of m per slab: 32, or 16 (CW == 6 only)
 static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, float* lds_a0, float* lds_a1, float* lds_y0,
                                                        float* lds_y1) {
-    constexpr int BR = kWgBR;                            // 32 rows of m per slab
+    static_assert(BR == 32 || (BR == 16 && CW == 6), "slab heights");
+    constexpr int RW = BR / 4;                           // slab rows a wave loads
+    constexpr int YL = BR / 16;                          // dy loads per wave per slab (4 rows x 16 chunks each)
     // CW = 1: any channel count.  A lane loads ONE float per slab row (`buffer_load_dword ... lds`),
     // slab rows are 32 floats, the k tile is 32 wide and there is one accumulator.
     // CW = 6: a 192-wide k tile (K = 576 is 3 of them: no padded rows where 128-wide tiles
@@ -1779,7 +1781,7 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
     constexpr int KSTEP = CW == 1 ? 1 : 4;               // k per lane of an x load
     constexpr int CPR = RS / KSTEP;                      // load lanes per slab row (32 or 48)
     constexpr int TKW = RS;                              // k tile width
-    constexpr int XL = CPR / 8;                          // x loads per wave per slab: 8 rows x CPR lanes / 64
+    constexpr int XL = CPR * RW / 64;                    // x loads per wave per slab: RW rows x CPR lanes / 64
     constexpr int NA = CW == 6 ? 4 : CW;                 // accumulators fed by the first (wide) operand read
     typedef float fcw __attribute__((ext_vector_type(CW)));
     typedef unsigned u4 __attribute__((ext_vector_type(4)));
@@ -1818,7 +1820,7 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
     // off = byte offset of that pixel (wraps for padding positions; only used when valid).
     int st_r, st_c, st_off;
     {
-        const int m = m_begin + 8 * wave + (lane & 7);
+        const int m = m_begin + RW * wave + (lane & (RW - 1));
         unsigned s_, rem, ho, wo;
         p.div_howo.divmod((unsigned)m, s_, rem);
         p.div_wo.divmod(rem, ho, wo);
@@ -1829,7 +1831,7 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
         st_c += 64;
     }
     const int thr_c = p.Wo * p.sW - p.pW + 64, thr_r = p.Ho * p.sH - p.pH + 64;
-    auto advance = [&]() {                               // m += 32
+    auto advance = [&]() {                               // m += BR
         st_c += p.step_c;
         const bool c1 = st_c >= thr_c;
         st_c -= c1 ? p.Wo * p.sW : 0;
@@ -1894,23 +1896,23 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
         const unsigned z = (tap_lo[i] - perm_rc[i]) | (perm_rc[i] + tap_hi[i]);
         const unsigned w = z | (z << 16);                // bit 31: row or column out of the image
         const unsigned voff = (w & 0x80000000u) | (unsigned)(perm_off[i] + a_tap4[i]);
-        // the wave's 8 rows are contiguous in LDS; load i fills the next 64 lanes' worth of them
+        // the wave's RW rows are contiguous in LDS; load i fills the next 64 lanes' worth of them
         if constexpr (CW == 1)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + wave * 8 * RS + i * 64), 4, (int)voff, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + wave * RW * RS + i * 64), 4, (int)voff, 0, 0, 0);
         else
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + wave * 8 * RS + i * 256), 16, (int)voff, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(la + wave * RW * RS + i * 256), 16, (int)voff, 0, 0, 0);
     };
     auto load_y = [&](int i, int mb, float* ly, int live) {
-        const int m = mb + (wave_u * 2 + i) * 4;         // scalar
+        const int m = mb + (wave_u * YL + i) * 4;        // scalar
         const unsigned voff = y_lane + (live ? (unsigned)(m * p.D) * 4u : 0x80000000u);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_y, (lds_ptr_t)(ly + (wave * 2 + i) * 256), 16, (int)voff, 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_y, (lds_ptr_t)(ly + (wave * YL + i) * 256), 16, (int)voff, 0, 0, 0);
     };
 
     float dbsum = 0.f;
     const int db_col = tid & 63, db_rg = tid >> 6;
     auto add_columns = [&](const float* ly) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) dbsum += ly[(db_rg * 8 + j) * kWgBN + (db_col ^ ((j & 1) << 5))];
+        for (int j = 0; j < RW; ++j) dbsum += ly[(db_rg * RW + j) * kWgBN + (db_col ^ ((j & 1) << 5))];
     };
 
     f16v acc[CW];
@@ -1947,10 +1949,11 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
 #pragma unroll
         for (int t = 0; t < BR / 4; ++t) {
             if (t + 1 < BR / 4) read_operands(row0 + 4 * t + 4, (t + 1) & 1);
-            // one load per MFMA step: dy in steps 0 and 1 (XL == 6) or 5 and 6, x from step 1 on
-            constexpr int Y0 = XL == 6 ? 0 : 5;
+            // one load per MFMA step: dy from step 0 (wide tiles) or 5 on, x from step 1 on
+            constexpr int Y0 = (XL == 6 || BR == 16) ? 0 : 5;
+            static_assert(XL <= BR / 4 - 1 && Y0 + YL <= BR / 4, "a slab's loads fit its steps");
             if (t >= 1 && t <= XL) load_x(t - 1, na);
-            if (t == Y0 || t == Y0 + 1) load_y(t - Y0, mb + BR, ny, live);
+            if (t >= Y0 && t < Y0 + YL) load_y(t - Y0, mb + BR, ny, live);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int q = 0; q < NA; ++q)
@@ -1969,7 +1972,7 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
 #pragma unroll
         for (int i = 0; i < XL; ++i) load_x(i, lds_a0);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) load_y(i, m_begin, lds_y0, -1);
+        for (int i = 0; i < YL; ++i) load_y(i, m_begin, lds_y0, -1);
     }
     for (int mb = m_begin; mb < m_end; mb += 2 * BR) {
         slab(mb, lds_a0, lds_y0, lds_a1, lds_y1, mb + BR < m_end);
@@ -1977,36 +1980,43 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
     }
 
     // ---- add the two m parities: waves 2,3 hand their accumulators to waves 0,1 --------
-    __syncthreads();                                     // slab buffers are free now
-    f4* xch = reinterpret_cast<f4*>(nt == 0 ? lds_a0 : lds_a1);   // CW x 4 x 16 B x 64 lanes per wave pair: one x buffer
-    if (mh == 1) {
-#pragma unroll
-        for (int q = 0; q < CW; ++q)
-#pragma unroll
-            for (int g = 0; g < 4; ++g)
-                xch[(q * 4 + g) * 64 + lane] = f4{acc[q][4 * g], acc[q][4 * g + 1], acc[q][4 * g + 2], acc[q][4 * g + 3]};
-    }
-    __syncthreads();
+    // through one x buffer per wave pair, QP accumulators (4 x 16 B x 64 lanes each) at a time
+    constexpr int QP = (BR * RS * 4 >= CW * 4096) ? CW : CW / 2;
+    static_assert(BR * RS * 4 >= QP * 4096 && CW % QP == 0, "accumulator exchange buffer");
+    f4* xch = reinterpret_cast<f4*>(nt == 0 ? lds_a0 : lds_a1);
     const size_t split_stride = (size_t)p.K * p.D + p.D;
     float* outp = p.out + (size_t)split * split_stride;
-    if (mh == 0) {
-        // one split's partial block is far below 2^31 bytes (K * D < 2^29 is checked by the host)
-        const __amdgpu_buffer_rsrc_t rsrc_o =
-            __builtin_amdgcn_make_buffer_rsrc(outp, 0, (int)((unsigned)p.K * (unsigned)p.D * 4u), 0x00020000);
-        const int nb = n0 + nt * 32 + 4 * lh;
+    // one split's partial block is far below 2^31 bytes (K * D < 2^29 is checked by the host)
+    const __amdgpu_buffer_rsrc_t rsrc_o =
+        __builtin_amdgcn_make_buffer_rsrc(outp, 0, (int)((unsigned)p.K * (unsigned)p.D * 4u), 0x00020000);
+    const int nb = n0 + nt * 32 + 4 * lh;
 #pragma unroll
-        for (int q = 0; q < CW; ++q) {
-            const int k = q < NA ? kt0 + NA * l32 + q : kt0 + 128 + 2 * l32 + (q - NA);   // rows past K fall outside the descriptor
-            const unsigned base = (unsigned)(k * p.D + nb) * 4u;
+    for (int q0 = 0; q0 < CW; q0 += QP) {
+        __syncthreads();                                 // slab buffers (or the pass before) are free now
+        if (mh == 1) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                f4 v = xch[(q * 4 + g) * 64 + lane];
-                v[0] += acc[q][4 * g];
-                v[1] += acc[q][4 * g + 1];
-                v[2] += acc[q][4 * g + 2];
-                v[3] += acc[q][4 * g + 3];
-                const unsigned off = base | ((unsigned)!(nb + 8 * g < p.D) << 31);
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, v), rsrc_o, (int)off, 8 * g * 4, 0);
+            for (int q = q0; q < q0 + QP; ++q)
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                    xch[((q - q0) * 4 + g) * 64 + lane] =
+                        f4{acc[q][4 * g], acc[q][4 * g + 1], acc[q][4 * g + 2], acc[q][4 * g + 3]};
+        }
+        __syncthreads();
+        if (mh == 0) {
+#pragma unroll
+            for (int q = q0; q < q0 + QP; ++q) {
+                const int k = q < NA ? kt0 + NA * l32 + q : kt0 + 128 + 2 * l32 + (q - NA);   // rows past K fall outside the descriptor
+                const unsigned base = (unsigned)(k * p.D + nb) * 4u;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    f4 v = xch[((q - q0) * 4 + g) * 64 + lane];
+                    v[0] += acc[q][4 * g];
+                    v[1] += acc[q][4 * g + 1];
+                    v[2] += acc[q][4 * g + 2];
+                    v[3] += acc[q][4 * g + 3];
+                    const unsigned off = base | ((unsigned)!(nb + 8 * g < p.D) << 31);
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, v), rsrc_o, (int)off, 8 * g * 4, 0);
+                }
             }
         }
     }
@@ -2042,8 +2052,17 @@ static __global__ __launch_bounds__(kThreads, 2) void wgrad_gemm_dma192(const Wg
     __shared__ float lds_a1[kWgBR * 192];
     __shared__ float lds_y0[kWgBR * kWgBN];
     __shared__ float lds_y1[kWgBR * kWgBN];
-    static_assert(sizeof(lds_a0) >= 6 * 16 * 64 * sizeof(float), "accumulator exchange buffer");
     wgrad_dma_body<6>(p, lds_a0, lds_a1, lds_y0, lds_y1);
+}
+
+// The same with 16-row slabs: 32 KB of LDS and half the per-load state, so that three
+// workgroups fit a CU (a stand-alone loop: 140 TFLOP/s against 134 with 32-row slabs).
+static __global__ __launch_bounds__(kThreads, 3) void wgrad_gemm_dma192h(const WgradParams p) {
+    __shared__ float lds_a0[16 * 192];
+    __shared__ float lds_a1[16 * 192];
+    __shared__ float lds_y0[16 * kWgBN];
+    __shared__ float lds_y1[16 * kWgBN];
+    wgrad_dma_body<6, 16>(p, lds_a0, lds_a1, lds_y0, lds_y1);
 }
 
 // ------------------------------------------------------------------------------
@@ -2239,14 +2258,6 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     p.fW = fW; p.sH = sH; p.sW = sW; p.pH = pH; p.pW = pW;
     p.want_dbias = dbias != nullptr;
     p.div_howo = FastDiv(Ho * Wo); p.div_wo = FastDiv(Wo); p.div_c = FastDiv(C); p.div_fw = FastDiv(fW);
-    {
-        const int qs = kWgBR / (Ho * Wo), rem = kWgBR % (Ho * Wo), qh = rem / Wo, qw = rem % Wo;
-        p.step_c = qw * sW;
-        p.step_r = qh * sH;
-        p.inc0 = 4 * C * (qw * sW + qh * sH * W + qs * H * W);
-        p.inc1 = 4 * C * (-Wo * sW + sH * W);
-        p.inc2 = 4 * C * (-Ho * sH * W + H * W);
-    }
     constexpr int CE = Elem<T>::CE;
     const bool va = (C % CE == 0), vy = (D % CE == 0);
     const int64_t xb = (int64_t)S * H * W * C * (int64_t)sizeof(T), yb = (int64_t)p.M * D * (int64_t)sizeof(T);
@@ -2262,6 +2273,24 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     if (const char* f = getenv("AETHER_WGRAD_CW")) {
         if (dma && va && p.K > 64 && (atoi(f) == 4 || atoi(f) == 6)) p.cw = atoi(f);
     }
+    // slab height of the 192-wide kernel: 16 rows (three workgroups per CU) where a workgroup walks at
+    // least 64 of them (56x56x64: 0.481 ms against 0.487 with 32 rows; 8x8x64 -> 128, batch 128, 8 slabs of
+    // 32 per workgroup: 27.2 us with 32 rows, 28.3 with 16); AETHER_WGRAD_BR overrides
+    int br = kWgBR;
+    if (dma && p.cw == 6) {
+        const int kt6 = cdiv(p.K, 192), nt6 = cdiv(D, kWgBN);
+        const int64_t wgs = (int64_t)3 * c.prop.multiProcessorCount;
+        if ((int64_t)cdiv(p.M, 32) * kt6 * nt6 >= 32 * wgs) br = 16;
+        if (const char* f = getenv("AETHER_WGRAD_BR")) br = atoi(f) == 32 ? 32 : (atoi(f) == 16 ? 16 : br);
+    }
+    {
+        const int qs = br / (Ho * Wo), rem = br % (Ho * Wo), qh = rem / Wo, qw = rem % Wo;
+        p.step_c = qw * sW;
+        p.step_r = qh * sH;
+        p.inc0 = 4 * C * (qw * sW + qh * sH * W + qs * H * W);
+        p.inc1 = 4 * C * (-Wo * sW + sH * W);
+        p.inc2 = 4 * C * (-Ho * sH * W + H * W);
+    }
     const int tkw = !dma ? kWgBK : (p.cw == 1 ? 32 : (p.cw == 6 ? 192 : kWgBK));
     const int kt = cdiv(p.K, tkw), nt = cdiv(D, kWgBN);
     const int slab_rows = dma16 ? 64 : kWgBR;
@@ -2274,7 +2303,7 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     if (const char* f = getenv("AETHER_WGRAD_ROUNDS")) {      // tuning override: 1 to 4
         if (atoi(f) >= 1 && atoi(f) <= 4) rounds = atoi(f);
     }
-    const int per_cu2 = (((dma && p.cw != 6) || dma16) ? 3 : 2) * rounds;
+    const int per_cu2 = (((dma && (p.cw != 6 || br == 16)) || dma16) ? 3 : 2) * rounds;
     int splits = (per_cu2 * c.prop.multiProcessorCount) / (kt * nt);
     // a workgroup's set-up, epilogue and its share of the reduction are worth several slabs
     // (training step of the 3-block CNN: 0.672 ms with 1, 0.642 with 4, 0.611 with 8, 0.658 with 16)
@@ -2292,6 +2321,7 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     p.kt = kt; p.nt = nt;
     dim3 grid(kt * nt * splits);
     if (dma16) hipLaunchKernelGGL(wgrad_gemm_dma_bf16, grid, dim3(kThreads), 0, c.stream, p);
+    else if (dma && p.cw == 6 && br == 16) hipLaunchKernelGGL(wgrad_gemm_dma192h, grid, dim3(kThreads), 0, c.stream, p);
     else if (dma && p.cw == 6) hipLaunchKernelGGL(wgrad_gemm_dma192, grid, dim3(kThreads), 0, c.stream, p);
     else if (dma) hipLaunchKernelGGL(wgrad_gemm_dma, grid, dim3(kThreads), 0, c.stream, p);
     else if (va && vy) hipLaunchKernelGGL((wgrad_gemm<T, CE, CE>), grid, dim3(kThreads), 0, c.stream, p);
