@@ -124,3 +124,49 @@ def test_bf16_fprop_dgrad_without_split_k(case, monkeypatch):
     abi.close(abi.dgrad_bf16(dy, w, x.shape, stride, pad),
               O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
 
+
+def _random_halo_cases(n, seed):
+    """Seeded random geometries around the conditions of the kernel that keeps a tile's source
+    pixels in LDS (whole 64-channel blocks on the gathered side, output images of about a multiple
+    of 256 pixels, 4 taps or more, unit stride): two thirds are drawn inside them, the rest around."""
+    r = np.random.RandomState(seed)
+    grids = [(16, 16), (16, 32), (32, 16), (8, 32), (32, 24), (16, 48), (20, 38), (25, 31), (51, 5)]
+    out = []
+    while len(out) < n:
+        S = int(r.choice([1, 2, 3]))
+        if r.rand() < 0.67:
+            Ho, Wo = grids[r.randint(len(grids))]
+            kind = r.randint(4)
+            if kind == 0:
+                fH, fW, pad, H, W = 3, 3, "same", Ho, Wo
+            elif kind == 1:
+                fH, fW, pad, H, W = 2, 2, "valid", Ho + 1, Wo + 1
+            elif kind == 2:
+                fH, fW, pad, H, W = 3, 3, "valid", Ho + 2, Wo + 2
+            else:
+                fH, fW, pad, H, W = 3, 2, "same", Ho, Wo - 1          # pad 1 on both axes: Wo = W + 2 - 2 + 1
+            st = 1
+            C, D = int(r.choice([64, 128])), int(r.choice([64, 128, 40]))
+        else:
+            fH, fW = int(r.choice([2, 3, 3, 4, 5])), int(r.choice([1, 2, 3, 3, 5]))
+            st = int(r.choice([1, 2]))
+            H, W = int(r.randint(10, 34)), int(r.randint(10, 34))
+            C, D = int(r.choice([64, 128, 8])), int(r.choice([64, 128, 40, 8]))
+            pad = "same" if r.rand() < 0.6 else "valid"
+        if H < fH or W < fW or S * H * W * C * D * fH * fW > 6e8:
+            continue
+        out.append((S, H, W, C, D, fH, fW, st, st, pad))
+    return out
+
+
+@pytest.mark.parametrize("case", _random_halo_cases(28, 777), ids=lambda c: "x".join(str(v) for v in c))
+def test_bf16_random_geometries_without_split_k(case, monkeypatch):
+    from tests import abi
+    monkeypatch.setenv("AETHER_GATHER_SPLIT_OFF", "1")
+    x, w, b, dy = _case(case, 9)
+    stride, pad = (case[7], case[8]), case[9]
+    xr, wr, dyr = O.round_to_bf16(x), O.round_to_bf16(w), O.round_to_bf16(dy)
+    abi.close(abi.fprop_bf16(x, w, b, stride, pad), O.conv_fprop(xr, wr, b, stride, pad, dtype=np.float64))
+    abi.close(abi.dgrad_bf16(dy, w, x.shape, stride, pad),
+              O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
+
