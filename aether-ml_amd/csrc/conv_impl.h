@@ -88,8 +88,10 @@ struct GatherParams {
     unsigned bt_bytes;
     unsigned out_bytes;  // extent of out; 0: no 16-byte stores (too large, N not a multiple of 4, or unaligned)
     int split_slabs;     // 0, or slabs of K per blockIdx.y: split y writes its partial product at out + y*M*N
-    int halo_wp, halo_tiles;   // gather_halo_bf16: columns of the padded source row, 256-row tiles per image
-    FastDiv div_hw, div_w, div_c, div_tw, div_halo_wp, div_halo_tiles;
+    // gather_halo_bf16: columns and rows of the padded source image, 256-row tiles per image (0: tiles
+    // run over image boundaries)
+    int halo_wp, halo_hp, halo_tiles;
+    FastDiv div_hw, div_w, div_c, div_tw, div_halo_wp, div_halo_hp, div_halo_tiles;
 };
 
 constexpr int kInvalidRow = -16384;
@@ -716,20 +718,24 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
 
 // ------------------------------------------------------------------------------
 // gather_halo_bf16: unit-stride gathers with several filter taps on bf16 inputs
-// (3x3 stride-1 fprop, every dgrad class with 4 taps or more).
+// (3x3 stride-1 fprop, every dgrad class with 2 taps or more).
 // The bf16 MFMAs of a slab take a fifth of the time its LDS-direct loads need to
 // arrive, and with the taps of a filter walked one slab at a time every source
 // pixel is fetched once per tap (9 times for 3x3): gather_gemm_dma on these shapes
 // waits for its loads (without the A loads of slabs 1..8 it runs 1.5x faster).
 // Here a workgroup fetches the source pixels of its 256 output pixels ONCE, as a
-// span of the zero-padded image in row-major order ("halo", 64 channels = 128 B per
-// pixel slot, at most kHaloSlots slots), and every tap reads it at a shifted slot:
-//     slot(pixel (i, j), tap (th, tw)) = (i + th) * Wp + (j + tw) - first,  Wp = Wg + Tw - 1
+// span of the zero-padded source tensor [S][Hp][Wp] in row-major order ("halo", 64
+// channels = 128 B per pixel slot, at most kHaloSlots slots), and every tap reads it
+// at a shifted slot:
+//     slot(pixel (s, i, j), tap (th, tw)) = (s * Hp + i + th) * Wp + (j + tw) - first,
+//     Hp = Hg + Th - 1, Wp = Wg + Tw - 1
 // Padding pixels are slots the loads fill with zeros (offsets outside the buffer
 // descriptor), so no tap needs a validity test.  Only the filter slabs stream, 8 KB
-// per tap through a ring of four buffers, three taps ahead.  Tiles do not cross
-// images (the span would grow by (Th - 1) rows), so the last tile of an image is
-// partly empty: used when that costs at most 10 % of the rows.
+// per tap through a ring of three buffers, two taps ahead.
+//   * A tile that runs over the end of an image needs (Th - 1) * Wp more slots.  Where
+//     that does not fit (56x56: 500), tiles are cut per image and an image's last tile
+//     is partly empty: taken when that costs at most 10 % of the rows; else tiles run
+//     over all of M if every span fits; else gather_gemm_dma runs.
 //   * slot s keeps logical 16-byte chunk c at position c ^ ((s >> 1) & 7), like the
 //     slab rows of gather_gemm_dma: 16 consecutive pixels cover the 64 banks once;
 //   * channel blocks beyond the first reload the halo (Cs = 64 j: j passes over the taps).
@@ -752,18 +758,36 @@ __device__ __forceinline__ unsigned lds_address(const void* q) {
     return (unsigned)reinterpret_cast<uintptr_t>((lds_ptr_t)const_cast<void*>(q));
 }
 
-constexpr int kHaloSlots = 384;      // 48 KB; with the 4 x 8 KB ring 80 KB: two workgroups per CU
+// STAGES ring buffers of 8 KB and the rest of 80 KB (two workgroups per CU) for the halo:
+// 4 stages (three taps ahead) and 384 slots where every span fits that, else 3 and 448
+// (56x56x64: 0.098 ms with 4 stages, 0.102 with 3).
+constexpr int halo_slots(int stages) { return stages == 4 ? 384 : 448; }
+// an LDS array of N 16-byte elements that takes no space for N == 0
+template <int N> struct LdsBlock {
+    static __device__ __forceinline__ f4* get() {
+        __shared__ f4 block[N];
+        return block;
+    }
+};
+template <> struct LdsBlock<0> {
+    static __device__ __forceinline__ f4* get() { return nullptr; }
+};
+constexpr int kHaloSlotsMax = 448;
 constexpr int kHaloBM = 256;
 
+template <int STAGES>
 static __global__ __launch_bounds__(kThreads, 2) void gather_halo_bf16(const GatherParams p) {
     constexpr int BM = kHaloBM, BN = 64, TM = 2, TN = 2, KC = 8, BK = 64;
+    constexpr int kHaloSlots = halo_slots(STAGES);
     constexpr int HL = kHaloSlots / 8 / 4;               // halo loads per wave (8 slots each)
+    static_assert(STAGES == 3 || STAGES == 4, "ring of 3 or 4 filter slabs");
     __shared__ f4 halo[kHaloSlots * KC];
     __shared__ f4 ring0[BN * KC];
     __shared__ f4 ring1[BN * KC];
     __shared__ f4 ring2[BN * KC];
-    __shared__ f4 ring3[BN * KC];
-    static_assert(kHaloSlots * sizeof(int) <= sizeof(ring3), "slot table fits a ring buffer");
+    f4* const ring3 = LdsBlock<STAGES == 4 ? BN * KC : 0>::get();    // no bytes when unused: 80 KB exactly either way
+    f4* const ring_last = STAGES == 4 ? ring3 : ring2;
+    static_assert(kHaloSlots * sizeof(int) <= sizeof(ring2), "slot table fits a ring buffer");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -775,11 +799,25 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_bf16(const Gat
     const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
     const int mt = lid / ntile;
     const int n0 = (lid - mt * ntile) * BN;
-    unsigned s_img, t_img;
-    p.div_halo_tiles.divmod((unsigned)mt, s_img, t_img);
     const int hw = p.Hg * p.Wg;
-    const int pm0 = (int)t_img * BM;
-    const int Wp = p.halo_wp;
+    int m0, m_end;                                       // the tile's rows and where its image (or M) ends
+    if (p.halo_tiles > 0) {
+        unsigned s_img, t_img;
+        p.div_halo_tiles.divmod((unsigned)mt, s_img, t_img);
+        m0 = (int)s_img * hw + (int)t_img * BM;
+        m_end = ((int)s_img + 1) * hw;
+    } else {
+        m0 = mt * BM;
+        m_end = p.M;
+    }
+    const int Wp = p.halo_wp, Hp = p.halo_hp;
+    // slot of tap (0,0) of output pixel m in the padded source tensor
+    auto slot0 = [&](int m) __attribute__((always_inline)) {
+        unsigned s_, rem, ii, jj;
+        p.div_hw.divmod((unsigned)m, s_, rem);
+        p.div_w.divmod(rem, ii, jj);
+        return ((int)s_ * Hp + (int)ii) * Wp + (int)jj;
+    };
     const int T = p.Th * p.Tw;
     const int nsteps = (p.Cs / BK) * T;
 
@@ -787,21 +825,19 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_bf16(const Gat
     load_bias<TN>(p, p.bias, bv, n0, lh);
 
     // the span: from the slot of tap (0,0) of the tile's first pixel to that of the last tap of its last pixel
-    unsigned i0, j0, i1, j1;
-    p.div_w.divmod((unsigned)pm0, i0, j0);
-    p.div_w.divmod((unsigned)min(pm0 + BM, hw) - 1u, i1, j1);
-    const int lfirst = (int)i0 * Wp + (int)j0;
-    const int span = ((int)i1 + p.Th - 1) * Wp + (int)j1 + p.Tw - lfirst;     // <= kHaloSlots, checked by the host
+    const int lfirst = slot0(m0);
+    const int span = slot0(min(m0 + BM, m_end) - 1) + (p.Th - 1) * Wp + p.Tw - lfirst;   // <= kHaloSlots, checked by the host
     // slot -> byte offset of the pixel's channel 0 (bit 31: padding or past the span), one slot per
     // thread, through LDS to the lanes that fetch it.  The table sits in the last ring buffer, which
     // the filter loads reach after the first barrier of the loop.
-    int* tab = reinterpret_cast<int*>(ring3);
+    int* tab = reinterpret_cast<int*>(ring_last);
     for (int sl = tid; sl < kHaloSlots; sl += kThreads) {
-        unsigned rr, cc;
-        p.div_halo_wp.divmod((unsigned)(lfirst + sl), rr, cc);
+        unsigned rg, cc, s_, rr;
+        p.div_halo_wp.divmod((unsigned)(lfirst + sl), rg, cc);
+        p.div_halo_hp.divmod(rg, s_, rr);
         const int srow = (int)rr + p.rh0, scol = (int)cc + p.rw0;
-        const bool ok = sl < span && (unsigned)srow < (unsigned)p.Hs && (unsigned)scol < (unsigned)p.Ws;
-        const unsigned off = (unsigned)((((int)s_img * p.Hs + srow) * p.Ws + scol) * p.Cs) * 2u;
+        const bool ok = sl < span && (unsigned)srow < (unsigned)p.Hs && (unsigned)scol < (unsigned)p.Ws && (int)s_ < p.S;
+        const unsigned off = (unsigned)((((int)s_ * p.Hs + srow) * p.Ws + scol) * p.Cs) * 2u;
         tab[sl] = (int)(ok ? off : 0x80000000u);
     }
     __syncthreads();
@@ -811,14 +847,12 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_bf16(const Gat
         const int sl = (wave * HL + k) * 8 + (lane >> 3);
         hoff[k] = (unsigned)tab[sl] + (unsigned)((((lane & 7) ^ (sl >> 1)) & 7) * 16);
     }
-    // slot of tap (0,0) for the pixels this lane multiplies (rows past the image: slot 0, never stored)
+    // slot of tap (0,0) for the pixels this lane multiplies (rows past the end: slot 0, never stored)
     int pslot[TM];
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-        const int pm = pm0 + wm0 + 32 * i + l32;
-        unsigned ii, jj;
-        p.div_w.divmod((unsigned)min(pm, hw - 1), ii, jj);
-        pslot[i] = pm < hw ? (int)ii * Wp + (int)jj - lfirst : 0;
+        const int m = m0 + wm0 + 32 * i + l32;
+        pslot[i] = m < m_end ? slot0(m) - lfirst : 0;
     }
     // filter slab loads: as in gather_gemm_dma (rows of 8 chunks, chunk c of row r at c ^ ((r >> 1) & 7))
     const int k4e = (lane & 7) ^ (lane >> 4);
@@ -842,7 +876,7 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_bf16(const Gat
 #pragma unroll
         for (int i = 0; i < 2; ++i) lds_direct_load16(rsrc_b, base + i * 1024u, b_off[i] + k0_bytes);
     };
-    // prefetch position: three steps ahead of the one being multiplied.  Every step issues
+    // prefetch position: STAGES - 1 steps ahead of the one being multiplied.  Every step issues
     // exactly one slab, past the last step with an offset outside the descriptor (no memory
     // access): the wait of a step is then the same count in every step, without a branch
     // (with conditional loads the compiler cannot tell which loads a count leaves in
@@ -856,7 +890,7 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_bf16(const Gat
     load_halo(0);
     load_filter(pf_next(), ring0);
     load_filter(pf_next(), ring1);
-    load_filter(pf_next(), ring2);
+    if constexpr (STAGES == 4) load_filter(pf_next(), ring2);
 
     f16v acc[TM][TN];
     fill_acc<TM, TN>(bv, acc);
@@ -865,8 +899,8 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_bf16(const Gat
     int th = 0, tw = 0, cb = 0;                          // the step being multiplied
     auto step = [&](int u, const f4* lb, f4* nb) __attribute__((always_inline)) {
         // loads complete in the order of issue (no stores are pending here): all but the
-        // two younger filter slabs
-        __builtin_amdgcn_s_waitcnt(4 | (7 << 4) | (15 << 8));
+        // younger filter slabs (two loads each)
+        __builtin_amdgcn_s_waitcnt((2 * (STAGES - 2)) | (7 << 4) | (15 << 8));
         // a bare barrier: the fence of __syncthreads() would wait for every load in flight
         asm volatile("s_barrier" ::: "memory");
         if (th == 0 && tw == 0 && cb > 0) {              // next channel block: everyone is done with the halo
@@ -903,13 +937,21 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_bf16(const Gat
         __builtin_amdgcn_sched_barrier(0);
         if (++tw == p.Tw) { tw = 0; if (++th == p.Th) { th = 0; ++cb; } }
     };
-    for (int u = 0; u < nsteps; u += 4) {
-        step(u, ring0, ring3);
-        if (u + 1 < nsteps) step(u + 1, ring1, ring0);
-        if (u + 2 < nsteps) step(u + 2, ring2, ring1);
-        if (u + 3 < nsteps) step(u + 3, ring3, ring2);
+    if constexpr (STAGES == 4) {
+        for (int u = 0; u < nsteps; u += 4) {
+            step(u, ring0, ring3);
+            if (u + 1 < nsteps) step(u + 1, ring1, ring0);
+            if (u + 2 < nsteps) step(u + 2, ring2, ring1);
+            if (u + 3 < nsteps) step(u + 3, ring3, ring2);
+        }
+    } else {
+        for (int u = 0; u < nsteps; u += 3) {
+            step(u, ring0, ring2);
+            if (u + 1 < nsteps) step(u + 1, ring1, ring0);
+            if (u + 2 < nsteps) step(u + 2, ring2, ring1);
+        }
     }
-    store_tile<TM, TN>(p, p.out, acc, (int)s_img * hw + pm0 + wm0, n0, l32, lh, ((int)s_img + 1) * hw);
+    store_tile<TM, TN>(p, p.out, acc, m0 + wm0, n0, l32, lh, m_end);
 }
 
 // Packs the filter w[fH][fW][C][D] into bt[Npad][Kpad] (k contiguous) for one
@@ -1015,28 +1057,52 @@ static inline int gather_bm(int M, int N, int cus, bool dma, int elem_bytes = 4)
     return bn == 32 ? 128 : 64;
 }
 
-// gather_halo_bf16 applies to unit-stride gathers of 4 to 32 taps over whole 64-channel blocks
-// whose images are large enough for 256-row tiles that do not cross them.  Fills the halo
-// fields of gp when it does.
-static bool plan_halo(GatherParams& gp, bool dma) {
+// gather_halo_bf16 applies to unit-stride gathers of 2 to 32 taps over whole 64-channel blocks
+// when the span of every tile fits its buffer: with tiles cut per image (at most 10 % of empty
+// rows) or, failing that, running over image boundaries.  Fills the halo fields of gp and the
+// number of 256-row tiles when it does.
+static bool plan_halo(GatherParams& gp, bool dma, int* mtiles, int* stages) {
     if (!dma || gp.sh != 1 || gp.sw != 1 || gp.Cs % 64 != 0 || gp.K != gp.Kpad || gp.split_slabs != 0) return false;
     const int taps = gp.Th * gp.Tw;
-    if (taps < 4 || taps > 32 || gp.N <= 32 || gp.Cs <= 0 || gp.K != taps * gp.Cs) return false;
+    if (taps < 2 || taps > 32 || gp.N <= 32 || gp.Cs <= 0 || gp.K != taps * gp.Cs) return false;
     if (getenv("AETHER_GATHER_HALO_OFF") != nullptr) return false;
     const int hw = gp.Hg * gp.Wg;
-    const int tiles = cdiv(hw, kHaloBM);
-    if ((int64_t)tiles * kHaloBM * 10 > (int64_t)hw * 11) return false;       // more than 10 % empty rows
-    const int wp = gp.Wg + gp.Tw - 1;
-    for (int t = 0; t < tiles; ++t) {
-        const int first = t * kHaloBM, last = std::min(first + kHaloBM, hw) - 1;
-        const int l0 = (first / gp.Wg) * wp + first % gp.Wg;
-        const int l1 = (last / gp.Wg + gp.Th - 1) * wp + last % gp.Wg + gp.Tw - 1;
-        if (l1 - l0 + 1 > kHaloSlots) return false;
+    const int wp = gp.Wg + gp.Tw - 1, hp = gp.Hg + gp.Th - 1;
+    if ((int64_t)gp.S * hp * wp >= ((int64_t)1 << 30)) return false;
+    auto slot0 = [&](int64_t m) {
+        const int64_t s = m / hw, rem = m % hw;
+        return (s * hp + rem / gp.Wg) * wp + rem % gp.Wg;
+    };
+    int64_t longest = 0;
+    auto fits = [&](int64_t first, int64_t last) {
+        const int64_t span = slot0(last) + (int64_t)(gp.Th - 1) * wp + gp.Tw - slot0(first);
+        longest = std::max(longest, span);
+        return span <= kHaloSlotsMax;
+    };
+    // tiles cut per image: every image has the same tiles
+    const int per_img = cdiv(hw, kHaloBM);
+    bool ok = (int64_t)per_img * kHaloBM * 10 <= (int64_t)hw * 11;
+    for (int t = 0; ok && t < per_img; ++t) ok = fits((int64_t)t * kHaloBM, std::min((t + 1) * kHaloBM, hw) - 1);
+    if (!ok) longest = 0;
+    if (ok) {
+        gp.halo_tiles = per_img;
+        *mtiles = gp.S * per_img;
+    } else {
+        const int n = cdiv(gp.M, kHaloBM);
+        if (n > (1 << 20)) return false;
+        ok = true;
+        for (int t = 0; ok && t < n; ++t)
+            ok = fits((int64_t)t * kHaloBM, std::min<int64_t>((int64_t)(t + 1) * kHaloBM, gp.M) - 1);
+        if (!ok) return false;
+        gp.halo_tiles = 0;
+        *mtiles = n;
     }
+    *stages = longest <= halo_slots(4) ? 4 : 3;
     gp.halo_wp = wp;
-    gp.halo_tiles = tiles;
+    gp.halo_hp = hp;
     gp.div_halo_wp = FastDiv(wp);
-    gp.div_halo_tiles = FastDiv(tiles);
+    gp.div_halo_hp = FastDiv(hp);
+    gp.div_halo_tiles = FastDiv(gp.halo_tiles > 0 ? gp.halo_tiles : 1);
     return true;
 }
 
@@ -1046,9 +1112,11 @@ static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t
     const bool dma = vec && gp.src_bytes != 0 && gp.bt_bytes != 0;
     if constexpr (sizeof(T) == 2) {
         GatherParams hp = gp;
-        if (plan_halo(hp, dma)) {
-            dim3 grid((unsigned)(gp.S * hp.halo_tiles * cdiv(gp.N, 64)));
-            hipLaunchKernelGGL(gather_halo_bf16, grid, dim3(kThreads), 0, st, hp);
+        int mtiles = 0, stages = 0;
+        if (plan_halo(hp, dma, &mtiles, &stages)) {
+            dim3 grid((unsigned)(mtiles * cdiv(gp.N, 64)));
+            if (stages == 4) hipLaunchKernelGGL(gather_halo_bf16<4>, grid, dim3(kThreads), 0, st, hp);
+            else hipLaunchKernelGGL(gather_halo_bf16<3>, grid, dim3(kThreads), 0, st, hp);
             return;
         }
     }
