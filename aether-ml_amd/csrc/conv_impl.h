@@ -954,6 +954,177 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_bf16(const Gat
     store_tile<TM, TN>(p, p.out, acc, m0 + wm0, n0, l32, lh, m_end);
 }
 
+// ------------------------------------------------------------------------------
+// gather_halo_res_bf16: the halo gather for filters that fit LDS whole (at most 9 taps of 64 x 64
+// bf16 = 72 KB: 3x3 on 64 channels), as one persistent workgroup of 8 waves per CU.
+// gather_halo_bf16 pays per tile for a set-up, the latency of its halo and a store phase, each with
+// the matrix pipe idle in that workgroup, and its filter slabs queue behind the other workgroup's
+// stores in the CU's memory pipeline.  Here the filter is fetched once per workgroup, wave 7 does
+// nothing but fetch the halo of the NEXT tile (two halo buffers) and waves 0..6 multiply the current
+// one, 32 rows x 64 columns each, straight out of LDS: no wait on memory inside a tile, one barrier
+// per tile, and since the multiplying waves issue no loads, nothing they wait for sits behind their
+// stores.
+// Tiles are 224 rows = whole image rows (Wg divides 224: 4 rows of 56) of one image (its last tile
+// may be short), so every tile starts in column 0: where a slot lies relative to the tile's first
+// pixel, and whether it is a padding column, is the same for all tiles and worked out once per
+// lane; per tile only the rows above and below the image change.
+// ------------------------------------------------------------------------------
+constexpr int kResBM = 224;
+constexpr int kResThreads = 512;
+constexpr int kResSlots = 352;        // 2 x 352 x 128 B of halo + 72 KB of filter = 160 KB
+constexpr int kResMaxTaps = 9;
+
+static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(const GatherParams p, const int mtiles) {
+    constexpr int BM = kResBM, BN = 64, TN = 2, KC = 8, NL = kResSlots / 8;
+    __shared__ f4 filt[kResMaxTaps * BN * KC];
+    __shared__ f4 halo[2][kResSlots * KC];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31;
+    const int lh = lane >> 5;
+    const int G = (int)gridDim.x;
+    const int lid = xcd_contiguous_id((int)blockIdx.x, G);
+    // tiles of this workgroup: a contiguous run of them, so that a tile's upper halo rows are the
+    // lower rows of the tile the same CU has just had in its L2
+    const int per = (mtiles + G - 1) / G;
+    const int tile0 = lid * per;
+    const int ntl = max(0, min(per, mtiles - tile0));
+    const int hw = p.Hg * p.Wg;
+    const int Wp = p.halo_wp;
+    const int T = p.Th * p.Tw;
+    const int tile_rows = BM / p.Wg;                       // image rows per tile (the host checks BM % Wg == 0)
+
+    // the filter: T slabs of 64 rows x 128 B, laid out like the slabs of gather_gemm_dma
+    // (chunk c of row r at c ^ ((r >> 1) & 7)); wave w fetches the 1 KB pieces w, w + 8, ...
+    {
+        const u32x4 rsrc_b = raw_rsrc(p.bt, p.bt_bytes);
+        const int k4e = (lane & 7) ^ (lane >> 4);
+        for (int q = wave; q < T * 8; q += 8) {
+            const int tap = q >> 3, part = q & 7;
+            const int k4 = k4e ^ ((part & 1) ? 4 : 0);
+            const unsigned off = (unsigned)(((part * 8 + (lane >> 3)) * p.Kpad + 8 * k4 + tap * p.Cs) * 2);
+            lds_direct_load16(rsrc_b, lds_address(filt) + (unsigned)q * 1024u, off);
+        }
+    }
+
+    if (wave == 7) {
+        // ---- the loading wave ----
+        // Load i of a tile brings the 8 slots 8 i .. 8 i + 7 (lane / 8 picks the slot, lane % 8 the
+        // chunk).  rel[i]: byte offset of the lane's chunk from the pixel of slot 0 (row -pad, column
+        // -pad of the tile); colbad: bit i set where the slot is a padding column.  Per tile a slot is
+        // valid if its padded row lies inside the image: slot in [lo, hi).  Offsets of invalid slots
+        // get bit 31, outside the buffer descriptor: the load writes zeros.  The offsets of a tile are
+        // worked out while the loads of the tile before it are in flight.
+        const u32x4 rsrc_a = raw_rsrc(p.src, p.src_bytes);
+        const int lslot = lane >> 3;
+        int rel[NL];
+        unsigned colbad_lo = 0, colbad_hi = 0;
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            const int sl = i * 8 + lslot;
+            unsigned r, c;
+            p.div_halo_wp.divmod((unsigned)sl, r, c);
+            rel[i] = ((int)r * p.Ws + (int)c) * 128 + (((lane & 7) ^ (sl >> 1)) & 7) * 16;
+            const unsigned bad = (unsigned)((int)c + p.rw0) >= (unsigned)p.Ws ? 1u : 0u;
+            if (i < 32) colbad_lo |= bad << i;
+            else colbad_hi |= bad << (i - 32);
+        }
+        unsigned offs[NL];
+        auto addresses = [&](int tile) __attribute__((always_inline)) {
+            unsigned s_img, t_img;
+            p.div_halo_tiles.divmod((unsigned)tile, s_img, t_img);
+            const int R0 = (int)t_img * tile_rows + p.rh0;                 // image row of padded row 0 of the tile
+            const int base = (((int)s_img * p.Hs + R0) * p.Ws + p.rw0) * 128;
+            const int a0 = lslot + R0 * Wp;                                // slot - lo, lo = -R0 * Wp
+            const int b0 = (p.Hs - R0) * Wp - 1 - lslot;                   // hi - 1 - slot, hi = (Hs - R0) * Wp
+#pragma unroll
+            for (int i = 0; i < NL; ++i) {
+                const unsigned rowbad = (unsigned)((a0 + 8 * i) | (b0 - 8 * i)) & 0x80000000u;
+                const unsigned colbad = i < 32 ? (colbad_lo << (31 - i)) : (colbad_hi << (63 - i));
+                offs[i] = (unsigned)(base + rel[i]) | rowbad | (colbad & 0x80000000u);
+            }
+        };
+        auto issue = [&](int buf) __attribute__((always_inline)) {
+            const unsigned lbase = lds_address(&halo[buf][0]);
+#pragma unroll
+            for (int i = 0; i < NL; ++i) lds_direct_load16(rsrc_a, lbase + (unsigned)i * 1024u, offs[i]);
+        };
+        if (ntl > 0) {
+            addresses(tile0);
+            issue(0);
+        }
+        if (ntl > 1) addresses(tile0 + 1);
+        __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
+        asm volatile("s_barrier" ::: "memory");
+        for (int t = 0; t < ntl; ++t) {
+            // the multiplying waves are done with tile t - 1, whose buffer takes tile t + 1
+            if (t + 1 < ntl) issue((t + 1) & 1);
+            if (t + 2 < ntl) addresses(tile0 + t + 2);
+            __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
+            asm volatile("s_barrier" ::: "memory");
+        }
+        return;
+    }
+
+    // ---- the multiplying waves ----
+    f4 bv[TN][4];
+    load_bias<TN>(p, p.bias, bv, 0, lh);
+    const int sw7 = (l32 >> 1) & 7;
+    int pslot;                                                             // slot of tap (0,0) of this lane's row
+    {
+        unsigned r, c;
+        p.div_w.divmod((unsigned)(wave * 32 + l32), r, c);
+        pslot = (int)r * Wp + (int)c;
+    }
+    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));                  // this wave's pieces of the filter
+    asm volatile("s_barrier" ::: "memory");
+    for (int t = 0; t < ntl; ++t) {
+        unsigned s_img, t_img;
+        p.div_halo_tiles.divmod((unsigned)(tile0 + t), s_img, t_img);
+        const int m0 = (int)s_img * hw + (int)t_img * BM;
+        const int m_end = ((int)s_img + 1) * hw;                           // rows past the image: multiplied, never stored
+        const f4* h = halo[t & 1];
+        f16v acc[1][TN];
+        fill_acc<1, TN>(bv, acc);
+        // the operands of tap u + 1 are read while the MFMAs of tap u run (two sets of 48 registers)
+        int th = 0, tw = 0;
+        f4 fa[2][4], fb[2][4][TN];
+        auto read_tap = [&](int tap, f4 (&ra)[4], f4 (&rb)[4][TN]) __attribute__((always_inline)) {
+            const int sl = pslot + th * Wp + tw;
+            const int x0 = sl * 8 + ((lh ^ (sl >> 1)) & 7);
+            const f4* lb = filt + tap * (BN * KC);
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                ra[g] = h[x0 ^ (g << 1)];
+#pragma unroll
+                for (int j = 0; j < TN; ++j) rb[g][j] = lb[(32 * j + l32) * KC + ((2 * g + lh) ^ sw7)];
+            }
+            if (++tw == p.Tw) { tw = 0; ++th; }
+        };
+        auto multiply = [&](const f4 (&ra)[4], const f4 (&rb)[4][TN]) __attribute__((always_inline)) {
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) mma_chunk<uint16_t>(rb[g][j], ra[g], acc[0][j]);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        read_tap(0, fa[0], fb[0]);
+        for (int tap = 0; tap < T; tap += 2) {
+            if (tap + 1 < T) read_tap(tap + 1, fa[1], fb[1]);
+            multiply(fa[0], fb[0]);
+            if (tap + 1 < T) {
+                if (tap + 2 < T) read_tap(tap + 2, fa[0], fb[0]);
+                multiply(fa[1], fb[1]);
+            }
+        }
+        store_tile<1, TN>(p, p.out, acc, m0 + wave * 32, 0, l32, lh, m_end);
+        asm volatile("s_barrier" ::: "memory");
+    }
+}
+
 // Packs the filter w[fH][fW][C][D] into bt[Npad][Kpad] (k contiguous) for one
 // gather-GEMM launch.  k = (th*Tw + tw)*Ck + kc ; filter tap x = xa + xs*th,
 // y = ya + ys*tw.  transposed == 0: n is the output channel d and kc the input
@@ -1106,6 +1277,42 @@ static bool plan_halo(GatherParams& gp, bool dma, int* mtiles, int* stages) {
     return true;
 }
 
+// gather_halo_res_bf16 applies to unit-stride gathers of 2 to 9 taps over one 64-channel block
+// with N in one tile, when 224-row tiles are whole rows of one image (Wg divides 224, at most
+// 15 % of empty rows in an image's last tile), a tile's rows and its halo fit a halo buffer and
+// there are at least 4 tiles per CU to walk (AETHER_GATHER_RES=1 drops the last condition,
+// =0 turns the kernel off).
+static bool plan_halo_res(GatherParams& gp, bool dma, int cus, int* mtiles) {
+    if (!dma || gp.sh != 1 || gp.sw != 1 || gp.Cs != 64 || gp.K != gp.Kpad || gp.split_slabs != 0) return false;
+    const int taps = gp.Th * gp.Tw;
+    if (taps < 2 || taps > kResMaxTaps || gp.N <= 32 || gp.N > 64 || gp.K != taps * gp.Cs) return false;
+    bool force = false;
+    if (const char* f = getenv("AETHER_GATHER_RES")) {
+        if (atoi(f) == 0) return false;
+        force = true;
+    }
+    if (getenv("AETHER_GATHER_HALO_OFF") != nullptr) return false;
+    if (gp.Wg <= 0 || kResBM % gp.Wg != 0) return false;
+    const int hw = gp.Hg * gp.Wg;
+    const int wp = gp.Wg + gp.Tw - 1, hp = gp.Hg + gp.Th - 1;
+    const int rows = kResBM / gp.Wg;                                     // image rows per tile
+    if ((int64_t)(rows + gp.Th - 1) * wp > kResSlots) return false;      // the tile's rows and the halo below them
+    const int per_img = cdiv(hw, kResBM);
+    if ((int64_t)per_img * kResBM * 100 > (int64_t)hw * 115) return false;
+    const int64_t n = (int64_t)gp.S * per_img;
+    if (n > (1 << 24) || (!force && n < 4 * (int64_t)cus)) return false;
+    // byte offsets are formed in 32 bits from the pixel above and left of the image
+    if (((int64_t)gp.S * gp.Hs + hp) * gp.Ws * 128 >= ((int64_t)1 << 31)) return false;
+    *mtiles = (int)n;
+    gp.halo_tiles = per_img;
+    gp.halo_wp = wp;
+    gp.halo_hp = hp;
+    gp.div_halo_wp = FastDiv(wp);
+    gp.div_halo_hp = FastDiv(hp);
+    gp.div_halo_tiles = FastDiv(per_img);
+    return true;
+}
+
 template <typename T>
 static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t st) {
     const int bn = gather_bn(gp.N);
@@ -1113,6 +1320,12 @@ static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t
     if constexpr (sizeof(T) == 2) {
         GatherParams hp = gp;
         int mtiles = 0, stages = 0;
+        if (plan_halo_res(hp, dma, cus, &mtiles)) {
+            hipLaunchKernelGGL(gather_halo_res_bf16, dim3((unsigned)std::min(mtiles, cus)), dim3(kResThreads), 0, st, hp,
+                               mtiles);
+            return;
+        }
+        hp = gp;
         if (plan_halo(hp, dma, &mtiles, &stages)) {
             dim3 grid((unsigned)(mtiles * cdiv(gp.N, 64)));
             if (stages == 4) hipLaunchKernelGGL(gather_halo_bf16<4>, grid, dim3(kThreads), 0, st, hp);

@@ -170,3 +170,39 @@ def test_bf16_random_geometries_without_split_k(case, monkeypatch):
     abi.close(abi.dgrad_bf16(dy, w, x.shape, stride, pad),
               O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
 
+
+
+# A filter of at most 9 taps on 64 channels and at most 64 output channels stays in LDS whole: one
+# persistent workgroup per CU, one wave fetching the source pixels of the next 224-row tile while
+# seven multiply the current one.  Tiles are whole image rows (the width divides 224).  The library
+# takes that kernel from 4 tiles per CU on; AETHER_GATHER_RES=1 lets small inputs reach it.
+RES_CASES = [
+    (2, 56, 56, 64, 64, 3, 3, 1, 1, "same"),      # the 56x56x64 layer: 14 tiles of 4 image rows per image
+    (3, 28, 28, 64, 64, 3, 3, 1, 1, "same"),      # 784 pixels per image: the fourth tile is half empty
+    (9, 14, 14, 64, 64, 3, 3, 1, 1, "same"),      # 196 pixels per image: one short tile each
+    (2, 30, 30, 64, 48, 3, 3, 1, 1, "valid"),     # ragged N (no bias beyond channel 48), no padding
+    (2, 29, 17, 64, 64, 2, 2, 1, 1, "valid"),     # even filter, 16 columns
+    (2, 28, 28, 64, 64, 3, 3, 2, 2, "valid"),     # stride 2: dgrad classes of 4, 2 and 2 taps on a 14x14 grid
+    (2, 8, 56, 64, 36, 1, 3, 1, 1, "same"),       # one filter row
+    (100, 28, 28, 64, 64, 3, 3, 1, 1, "same"),    # 400 tiles on 256 workgroups: two tiles, or none
+    (1, 16, 112, 64, 64, 3, 3, 1, 1, "same"),     # two rows per tile, but four rows of 114 slots do not fit: other kernels
+    (2, 20, 20, 64, 64, 3, 3, 1, 1, "same"),      # width does not divide 224: other kernels
+]
+
+
+@pytest.mark.parametrize("case", RES_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_bf16_fprop_dgrad_with_the_filter_resident_in_lds(case, monkeypatch):
+    from tests import abi
+    monkeypatch.setenv("AETHER_GATHER_SPLIT_OFF", "1")
+    monkeypatch.setenv("AETHER_GATHER_RES", "1")
+    x, w, b, dy = _case(case, 11)
+    stride, pad = (case[7], case[8]), case[9]
+    xr, wr, dyr = O.round_to_bf16(x), O.round_to_bf16(w), O.round_to_bf16(dy)
+    got = abi.fprop_bf16(x, w, b, stride, pad)
+    abi.close(got, O.conv_fprop(xr, wr, b, stride, pad, dtype=np.float64))
+    abi.close(abi.fprop_bf16(x, w, None, stride, pad), O.conv_fprop(xr, wr, None, stride, pad, dtype=np.float64))
+    dx = abi.dgrad_bf16(dy, w, x.shape, stride, pad)
+    abi.close(dx, O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
+    # the same sums of the same products in another order of taps and tiles
+    monkeypatch.setenv("AETHER_GATHER_RES", "0")
+    abi.close(abi.fprop_bf16(x, w, b, stride, pad), got, rtol=1e-5, atol=1e-5)
