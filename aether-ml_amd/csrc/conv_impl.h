@@ -954,6 +954,17 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_bf16(const Gat
     store_tile<TM, TN>(p, p.out, acc, m0 + wm0, n0, l32, lh, m_end);
 }
 
+struct PackParams {
+    const void* w;
+    void* bt;
+    int fW, C, D;
+    int Tw, Ck;
+    int xa, xs, ya, ys;
+    int transposed;
+    int N, K, Npad, Kpad;
+    int64_t w_elems;     // fH * fW * C * D
+};
+
 // ------------------------------------------------------------------------------
 // gather_halo_res_bf16: the halo gather for filters that fit LDS whole (at most 9 taps of 64 x 64
 // bf16 = 72 KB: 3x3 on 64 channels), as one persistent workgroup of 8 waves per CU.
@@ -974,7 +985,8 @@ constexpr int kResThreads = 512;
 constexpr int kResSlots = 352;        // 2 x 352 x 128 B of halo + 72 KB of filter = 160 KB
 constexpr int kResMaxTaps = 9;
 
-static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(const GatherParams p, const int mtiles) {
+static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(const GatherParams p, const PackParams pk,
+                                                                               const int mtiles) {
     constexpr int BM = kResBM, BN = 64, TN = 2, KC = 8, NL = kResSlots / 8;
     __shared__ f4 filt[kResMaxTaps * BN * KC];
     __shared__ f4 halo[2][kResSlots * KC];
@@ -996,16 +1008,52 @@ static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(co
     const int T = p.Th * p.Tw;
     const int tile_rows = BM / p.Wg;                       // image rows per tile (the host checks BM % Wg == 0)
 
-    // the filter: T slabs of 64 rows x 128 B, laid out like the slabs of gather_gemm_dma
-    // (chunk c of row r at c ^ ((r >> 1) & 7)); wave w fetches the 1 KB pieces w, w + 8, ...
+    // The filter, straight from w[fH][fW][C][D] (no packing launch): T slabs of 64 rows (n) x 128 B
+    // (the 64 k of one tap), laid out like the slabs of gather_gemm_dma (chunk c of row r at
+    // c ^ ((r >> 1) & 7)).  Slab t holds tap x = xa + xs * (t / Tw), y = ya + ys * (t % Tw).
     {
-        const u32x4 rsrc_b = raw_rsrc(p.bt, p.bt_bytes);
-        const int k4e = (lane & 7) ^ (lane >> 4);
-        for (int q = wave; q < T * 8; q += 8) {
-            const int tap = q >> 3, part = q & 7;
-            const int k4 = k4e ^ ((part & 1) ? 4 : 0);
-            const unsigned off = (unsigned)(((part * 8 + (lane >> 3)) * p.Kpad + 8 * k4 + tap * p.Cs) * 2);
-            lds_direct_load16(rsrc_b, lds_address(filt) + (unsigned)q * 1024u, off);
+        const unsigned w_bytes = (unsigned)(pk.w_elems * 2);
+        if (pk.transposed) {
+            // dgrad: n is the input channel c and k the output channel d, which is contiguous in w:
+            // rows are copied as they are; wave w fetches the 1 KB pieces w, w + 8, ...
+            const u32x4 rsrc_w = raw_rsrc(pk.w, w_bytes);
+            const int k4e = (lane & 7) ^ (lane >> 4);
+            for (int q = wave; q < T * 8; q += 8) {
+                const int tap = q >> 3, part = q & 7;
+                unsigned t_h, t_w;
+                p.div_tw.divmod((unsigned)tap, t_h, t_w);
+                const int x = pk.xa + pk.xs * (int)t_h, y = pk.ya + pk.ys * (int)t_w;
+                const int n = part * 8 + (lane >> 3);
+                const int k4 = k4e ^ ((part & 1) ? 4 : 0);
+                const unsigned off = (unsigned)((((x * pk.fW + y) * pk.C + n) * pk.D + 8 * k4) * 2) |
+                                     ((unsigned)(n >= p.N) << 31);
+                lds_direct_load16(rsrc_w, lds_address(filt) + (unsigned)q * 1024u, off);
+            }
+        } else {
+            // fprop: n is the output channel d, contiguous in w, and k the input channel c: a
+            // transposition.  Half a wave reads two adjacent n of two adjacent c (4 bytes each) and
+            // writes the two (n, c pair) words; row pairs 2 (8 i + wave) + half of the T * 32 pairs.
+            const __amdgpu_buffer_rsrc_t rsrc_w =
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(pk.w), 0, (int)w_bytes, 0x00020000);
+            const int n2 = 2 * (lane & 31);
+            const unsigned nbad = (unsigned)(n2 >= p.N) << 31;             // N is even here (checked by the host)
+            char* const fbytes = reinterpret_cast<char*>(filt);
+#pragma unroll
+            for (int i = 0; i < 2 * kResMaxTaps; ++i) {
+                if (i < 2 * T) {
+                    const int r = 2 * ((i * 8 + wave) * 2 + lh);                // row = tap * 64 + c, c even
+                    const int tap = r >> 6, c = r & 63;
+                    unsigned t_h, t_w;
+                    p.div_tw.divmod((unsigned)tap, t_h, t_w);
+                    const int x = pk.xa + pk.xs * (int)t_h, y = pk.ya + pk.ys * (int)t_w;
+                    const unsigned off = (unsigned)((((x * pk.fW + y) * pk.C + c) * pk.D + n2) * 2) | nbad;
+                    const unsigned a = __builtin_amdgcn_raw_buffer_load_b32(rsrc_w, (int)off, 0, 0);
+                    const unsigned b = __builtin_amdgcn_raw_buffer_load_b32(rsrc_w, (int)off, pk.D * 2, 0);
+                    const int pos = ((c >> 3) ^ ((n2 >> 1) & 7)) * 16 + (c & 7) * 2;   // n2 and n2 + 1 share the key
+                    *reinterpret_cast<unsigned*>(fbytes + tap * 8192 + n2 * 128 + pos) = (a & 0xffffu) | (b << 16);
+                    *reinterpret_cast<unsigned*>(fbytes + tap * 8192 + (n2 + 1) * 128 + pos) = (a >> 16) | (b & 0xffff0000u);
+                }
+            }
         }
     }
 
@@ -1056,7 +1104,7 @@ static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(co
             issue(0);
         }
         if (ntl > 1) addresses(tile0 + 1);
-        __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
+        __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (0 << 8));                // its loads and its part of the filter
         asm volatile("s_barrier" ::: "memory");
         for (int t = 0; t < ntl; ++t) {
             // the multiplying waves are done with tile t - 1, whose buffer takes tile t + 1
@@ -1078,7 +1126,11 @@ static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(co
         p.div_w.divmod((unsigned)(wave * 32 + l32), r, c);
         pslot = (int)r * Wp + (int)c;
     }
-    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));                  // this wave's pieces of the filter
+    f16v done[1][TN];                                                      // the tile before the current one
+    int done_m0 = 0, done_end = 0;
+    bool have_done = false;
+    const int store_after = min(wave + 1, T - 1);
+    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (0 << 8));                   // this wave's part of the filter
     asm volatile("s_barrier" ::: "memory");
     for (int t = 0; t < ntl; ++t) {
         unsigned s_img, t_img;
@@ -1111,34 +1163,35 @@ static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(co
                 for (int j = 0; j < TN; ++j) mma_chunk<uint16_t>(rb[g][j], ra[g], acc[0][j]);
             __builtin_amdgcn_sched_barrier(0);
         };
+        // All seven waves finish a tile together; if they also stored together, each would wait
+        // for room in the CU's memory pipeline with nobody left to use the matrix pipe.  A wave
+        // keeps its finished tile in registers and stores it during the next tile, wave w after
+        // tap w + 1, so that the stores of a CU are spread over the tile.
         read_tap(0, fa[0], fb[0]);
         for (int tap = 0; tap < T; tap += 2) {
             if (tap + 1 < T) read_tap(tap + 1, fa[1], fb[1]);
             multiply(fa[0], fb[0]);
+            if (tap == store_after && have_done) store_tile<1, TN>(p, p.out, done, done_m0, 0, l32, lh, done_end);
             if (tap + 1 < T) {
                 if (tap + 2 < T) read_tap(tap + 2, fa[0], fb[0]);
                 multiply(fa[1], fb[1]);
+                if (tap + 1 == store_after && have_done) store_tile<1, TN>(p, p.out, done, done_m0, 0, l32, lh, done_end);
             }
         }
-        store_tile<1, TN>(p, p.out, acc, m0 + wave * 32, 0, l32, lh, m_end);
+        have_done = true;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) done[0][j] = acc[0][j];
+        done_m0 = m0 + wave * 32;
+        done_end = m_end;
         asm volatile("s_barrier" ::: "memory");
     }
+    if (have_done) store_tile<1, TN>(p, p.out, done, done_m0, 0, l32, lh, done_end);
 }
 
 // Packs the filter w[fH][fW][C][D] into bt[Npad][Kpad] (k contiguous) for one
 // gather-GEMM launch.  k = (th*Tw + tw)*Ck + kc ; filter tap x = xa + xs*th,
 // y = ya + ys*tw.  transposed == 0: n is the output channel d and kc the input
 // channel c (fprop).  transposed == 1: n is c and kc is d (dgrad).
-struct PackParams {
-    const void* w;
-    void* bt;
-    int fW, C, D;
-    int Tw, Ck;
-    int xa, xs, ya, ys;
-    int transposed;
-    int N, K, Npad, Kpad;
-};
-
 template <typename T>
 __global__ void pack_filter(const PackParams p) {
     int idx = blockIdx.x * blockDim.x + threadIdx.x;
@@ -1320,12 +1373,6 @@ static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t
     if constexpr (sizeof(T) == 2) {
         GatherParams hp = gp;
         int mtiles = 0, stages = 0;
-        if (plan_halo_res(hp, dma, cus, &mtiles)) {
-            hipLaunchKernelGGL(gather_halo_res_bf16, dim3((unsigned)std::min(mtiles, cus)), dim3(kResThreads), 0, st, hp,
-                               mtiles);
-            return;
-        }
-        hp = gp;
         if (plan_halo(hp, dma, &mtiles, &stages)) {
             dim3 grid((unsigned)(mtiles * cdiv(gp.N, 64)));
             if (stages == 4) hipLaunchKernelGGL(gather_halo_bf16<4>, grid, dim3(kThreads), 0, st, hp);
@@ -1472,6 +1519,18 @@ static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
         const int64_t ob = (g.dense_out ? (int64_t)g.M : (int64_t)g.S * g.Hof * g.Wof) * g.N * (int64_t)sizeof(float);
         const bool ovec = ob < lim && g.N % 4 == 0 && (reinterpret_cast<uintptr_t>(g.out) & 15) == 0;
         gs.gp.out_bytes = ovec ? (unsigned)ob : 0u;
+    }
+    if constexpr (sizeof(T) == 2) {
+        // the kernel that keeps the whole filter in LDS reads it from w itself
+        GatherParams hp = gs.gp;
+        int mtiles = 0;
+        const bool dma = vec && hp.src_bytes != 0 && gs.pp.w_elems * 2 < ((int64_t)1 << 31) && gs.pp.N % 2 == 0;
+        if (gs.nsplit == 1 && hp.M > 0 && plan_halo_res(hp, dma, c.prop.multiProcessorCount, &mtiles)) {
+            hipLaunchKernelGGL(gather_halo_res_bf16, dim3((unsigned)std::min(mtiles, c.prop.multiProcessorCount)),
+                               dim3(kResThreads), 0, c.stream, hp, gs.pp, mtiles);
+            AETH_LAUNCH_CHECK();
+            return AETH_OK;
+        }
     }
     if (total > 0) {
         hipLaunchKernelGGL(pack_filter<T>, dim3(cdiv(total, 256)), dim3(256), 0, c.stream, gs.pp);
@@ -1704,7 +1763,7 @@ int conv_fprop_impl(const char* fn, const T* x, const T* w, const float* bias, f
     g.Hof = Ho; g.Wof = Wo; g.oh0 = 0; g.ow0 = 0; g.ohs = 1; g.ows = 1; g.dense_out = 1;
     set_out_divs(g);
     PackParams& pk = gs.pp;
-    pk.w = w; pk.fW = fW; pk.C = C; pk.D = D; pk.Tw = fW; pk.Ck = C;
+    pk.w = w; pk.fW = fW; pk.C = C; pk.D = D; pk.Tw = fW; pk.Ck = C; pk.w_elems = (int64_t)fH * fW * C * D;
     pk.xa = 0; pk.xs = 1; pk.ya = 0; pk.ys = 1; pk.transposed = 0;
     pk.N = D; pk.K = g.K; pk.Npad = (int)round_up(D, 64); pk.Kpad = g.Kpad;
     gs.bt_bytes = (int64_t)pk.Npad * pk.Kpad * sizeof(T);
@@ -1771,7 +1830,7 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
             g.dense_out = (nclass == 1);
             set_out_divs(g);
             PackParams& pk = gs.pp;
-            pk.w = w; pk.fW = fW; pk.C = C; pk.D = D; pk.Tw = Tw > 0 ? Tw : 1; pk.Ck = D;
+            pk.w = w; pk.fW = fW; pk.C = C; pk.D = D; pk.Tw = Tw > 0 ? Tw : 1; pk.Ck = D; pk.w_elems = (int64_t)fH * fW * C * D;
             pk.xa = xmax; pk.xs = -sH; pk.ya = ymax; pk.ys = -sW; pk.transposed = 1;
             pk.N = C; pk.K = g.K; pk.Npad = (int)round_up(C, 64); pk.Kpad = g.Kpad;
             gs.bt_bytes = round_up((int64_t)pk.Npad * pk.Kpad * sizeof(T), 256);
