@@ -2584,6 +2584,275 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma_bf16(const Wgr
     }
 }
 
+// ------------------------------------------------------------------------------
+// wgrad_halo_bf16: bf16 wgrad of a unit-stride filter of at most 9 taps on 64 input channels and
+// at most 64 output channels, as one persistent workgroup per CU that holds the WHOLE K x N
+// result in registers: wave t owns filter tap t (64 k rows x 64 n columns, four 32 x 32
+// accumulators), one more wave does nothing but load.
+// wgrad_gemm_dma_bf16 gives a workgroup 128 k rows: 4.5 workgroups read every dy row again, each
+// x pixel is fetched once per tap, and a 64-row slab is 24 KB of loads for 1 MFLOP, which
+// bounds the kernel by what L2 delivers (1.55 times the operands fetched from memory at 1.9 TB/s,
+// matrix pipe 22 % busy).  Here a slab is some whole output rows (R rows, R * Wo a multiple of
+// 16 and at most 128: two rows of 56) and the loading wave fetches, once, the padded image rows
+// under them ("halo", (R + fH - 1) x (Wo + fW - 1) pixel slots of 128 B, padding as zeros from
+// offsets outside the buffer descriptor) and the slab's dy rows, two buffers each, a slab ahead;
+// tap (fx, fy) reads the halo at slots shifted by fx * Wp + fy.  The MFMA reduces over m, 8
+// consecutive m of one k (or n) column per lane, while both tiles lie m-major in LDS:
+// `ds_read_b64_tr_b16` transposes on the way (see wgrad_gemm_dma_bf16); chunk q of a 128-byte row
+// is stored at q ^ (((row >> 1) & 1) << 2), row = slot number or dy row.
+// The loading wave also adds up the dy columns for dbias.  Partial results go to
+// out + z * (K * D + D) like those of the other wgrad kernels.
+// ------------------------------------------------------------------------------
+struct WgradHaloParams {
+    const void* x;       // [S,H,W,64] bf16
+    const void* dy;      // [S,Ho,Wo,D] bf16
+    float* out;          // [splits][K*D + D]
+    unsigned x_bytes, dy_bytes;
+    int S, H, W, Ho, Wo, D, fH, fW, pH, pW;
+    int R;               // output rows per slab
+    int slab_m;          // R * Wo: multiple of 16, at most kWhRows
+    int Wp;              // Wo + fW - 1
+    int hslots;          // (R + fH - 1) * Wp, at most kWhSlots
+    int nslabs;          // S * Ho / R
+    int per;             // slabs per workgroup
+    int want_dbias;
+    FastDiv div_wp, div_wo, div_fw, div_spi;   // spi: slabs per image = Ho / R
+};
+constexpr int kWhSlots = 256;       // halo buffer: 256 pixel slots of 128 B
+constexpr int kWhRows = 128;        // dy buffer: 128 rows of 128 B
+constexpr int kWhMaxTaps = 9;
+
+static __global__ __launch_bounds__(64 * (kWhMaxTaps + 1), 1) void wgrad_halo_bf16(const WgradHaloParams p) {
+    constexpr int NLH = kWhSlots / 8, NLD = kWhRows / 8, STEPS = kWhRows / 16;
+    __shared__ uint16_t halo[2][kWhSlots * 64];
+    __shared__ uint16_t dyb[2][kWhRows * 64];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31;
+    const int lh = lane >> 5;
+    const int T = p.fH * p.fW;
+    const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
+    const int sl0 = lid * p.per;
+    const int nsl = max(0, min(p.per, p.nslabs - sl0));
+    const int K = T * 64;
+    float* const outp = p.out + (size_t)lid * ((size_t)K * p.D + p.D);
+    const int steps = p.slab_m >> 4;
+
+    if (wave == T) {
+        // ---- the loading wave ----
+        // Halo load i brings the slots 8 i .. 8 i + 7, dy load j the rows 8 j .. 8 j + 7 (lane / 8 picks
+        // the slot or row, lane % 8 the chunk position).  relx / rely: byte offset of the lane's chunk
+        // from the slab's first padded pixel / first dy element; a slot is a padding column for all
+        // slabs or not (colbad), and lies in a padded row inside the image or not per slab: slot in
+        // [lo, hi).  Invalid pieces get bit 31, outside the buffer descriptor: zeros.
+        const u32x4 rsrc_x = raw_rsrc(p.x, p.x_bytes);
+        const u32x4 rsrc_y = raw_rsrc(p.dy, p.dy_bytes);
+        const int lrow = lane >> 3;
+        int relx[NLH], rely[NLD];
+        unsigned colbad = 0;
+#pragma unroll
+        for (int i = 0; i < NLH; ++i) {
+            const int slot = 8 * i + lrow;
+            unsigned r, c;
+            p.div_wp.divmod((unsigned)slot, r, c);
+            relx[i] = ((int)r * p.W + (int)c) * 128 + (((lane & 7) ^ (((slot >> 1) & 1) << 2)) * 16);
+            colbad |= ((unsigned)((int)c - p.pW) >= (unsigned)p.W ? 1u : 0u) << i;
+        }
+#pragma unroll
+        for (int j = 0; j < NLD; ++j) {
+            const int row = 8 * j + lrow;
+            const int n8 = 8 * ((lane & 7) ^ (((row >> 1) & 1) << 2));
+            rely[j] = (row * p.D + n8) * 2;
+            if (n8 >= p.D || row >= p.slab_m) rely[j] = (int)0x80000000;
+        }
+        unsigned offx[NLH], offy[NLD];
+        auto addresses = [&](int slab) __attribute__((always_inline)) {
+            unsigned s_img, r_img;
+            p.div_spi.divmod((unsigned)slab, s_img, r_img);
+            const int R0 = (int)r_img * p.R - p.pH;                         // image row of padded row 0 of the slab
+            const int base = (((int)s_img * p.H + R0) * p.W - p.pW) * 128;
+            const int a0 = lrow + R0 * p.Wp;                                // slot - lo
+            const int b0 = (p.H - R0) * p.Wp - 1 - lrow;                    // hi - 1 - slot
+#pragma unroll
+            for (int i = 0; i < NLH; ++i) {
+                const unsigned rowbad = (unsigned)((a0 + 8 * i) | (b0 - 8 * i)) & 0x80000000u;
+                offx[i] = (unsigned)(base + relx[i]) | rowbad | ((colbad << (31 - i)) & 0x80000000u);
+            }
+            const int ybase = (((int)s_img * p.Ho + (int)r_img * p.R) * p.Wo) * p.D * 2;
+#pragma unroll
+            for (int j = 0; j < NLD; ++j) offy[j] = (unsigned)(ybase + rely[j]) | ((unsigned)rely[j] & 0x80000000u);
+        };
+        auto issue = [&](int buf) __attribute__((always_inline)) {
+            const unsigned hb = lds_address(&halo[buf][0]), yb = lds_address(&dyb[buf][0]);
+#pragma unroll
+            for (int i = 0; i < NLH; ++i)
+                if (8 * i < p.hslots) lds_direct_load16(rsrc_x, hb + (unsigned)i * 1024u, offx[i]);
+#pragma unroll
+            for (int j = 0; j < NLD; ++j)
+                if (8 * j < p.slab_m) lds_direct_load16(rsrc_y, yb + (unsigned)j * 1024u, offy[j]);
+        };
+        // dbias: the lane adds up 8 columns (one chunk position) of the rows lrow, lrow + 8, ...
+        float db[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        auto add_columns = [&](int buf) __attribute__((always_inline)) {
+            const f4* yb = reinterpret_cast<const f4*>(&dyb[buf][0]);
+#pragma unroll
+            for (int j = 0; j < NLD; ++j) {
+                if (8 * j < p.slab_m) {
+                    const f4 v = yb[(8 * j + lrow) * 8 + (lane & 7)];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const unsigned u = __float_as_uint(v[e]);
+                        db[2 * e] += __uint_as_float(u << 16);
+                        db[2 * e + 1] += __uint_as_float(u & 0xffff0000u);
+                    }
+                }
+            }
+        };
+        if (nsl > 0) {
+            addresses(sl0);
+            issue(0);
+        }
+        if (nsl > 1) addresses(sl0 + 1);
+        __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
+        if (p.want_dbias && nsl > 0) add_columns(0);
+        asm volatile("s_barrier" ::: "memory");
+        for (int t = 0; t < nsl; ++t) {
+            // the multiplying waves are done with slab t - 1, whose buffers take slab t + 1
+            if (t + 1 < nsl) issue((t + 1) & 1);
+            if (t + 2 < nsl) addresses(sl0 + t + 2);
+            __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
+            if (p.want_dbias && t + 1 < nsl) add_columns((t + 1) & 1);
+            asm volatile("s_barrier" ::: "memory");
+        }
+        if (p.want_dbias) {
+            // lanes with the same chunk position hold different rows; the logical chunk is the position
+            // with bit 2 flipped for rows whose bit 1 is set (lrow & 2)
+            float* red = reinterpret_cast<float*>(&halo[0][0]);             // everyone is past the last barrier
+            const int lc = (lane & 7) ^ (((lrow >> 1) & 1) << 2);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) red[lrow * 64 + 8 * lc + e] = db[e];
+            __builtin_amdgcn_s_waitcnt(0);
+            float sum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) sum += red[r * 64 + lane];
+            if (lane < p.D) outp[(size_t)K * p.D + lane] = sum;
+        }
+        return;
+    }
+    if (wave > T) return;                                                  // waves beyond the taps and the loader
+
+    // ---- the multiplying waves: wave t owns tap t ----
+    unsigned fx, fy;
+    p.div_fw.divmod((unsigned)wave, fx, fy);
+    const int shift = (int)fx * p.Wp + (int)fy;
+    // transposing reads: 16-lane group G covers columns 16 (G & 1).. and rows 8 (G >> 1)..; lane j of the
+    // group points at row j >> 2 (second read: + 4), elements 4 (j & 3)..+3
+    const int tr_row = 8 * (lane >> 5) + ((lane & 15) >> 2);
+    const int col0 = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    int offa[STEPS][2];                                                    // element offsets into a halo buffer (k block 0; ^ 32: block 1)
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int row = min(16 * st + tr_row + 4 * h, p.slab_m - 1);
+            unsigned r, wo;
+            p.div_wo.divmod((unsigned)row, r, wo);
+            const int slot = (int)r * p.Wp + (int)wo + shift;
+            offa[st][h] = slot * 64 + ((((col0 >> 3) ^ (((slot >> 1) & 1) << 2)) << 3) + (col0 & 4));
+        }
+    int offb[2];                                                           // into a dy buffer, step 0 (n block 0; ^ 32: block 1)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int row = tr_row + 4 * h;
+        offb[h] = row * 64 + ((((col0 >> 3) ^ (((row >> 1) & 1) << 2)) << 3) + (col0 & 4));
+    }
+    f16v acc[2][2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[kb][nb][v] = 0.f;
+    typedef short s8v __attribute__((ext_vector_type(8)));
+    auto tr = [&](const uint16_t* q) __attribute__((always_inline)) {
+        return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr_t)q);
+    };
+    asm volatile("s_barrier" ::: "memory");
+    for (int t = 0; t < nsl; ++t) {
+        const uint16_t* hb = halo[t & 1];
+        const uint16_t* yb = dyb[t & 1];
+#pragma unroll
+        for (int st = 0; st < STEPS; ++st) {
+            if (st < steps) {
+                s8v a[2], b[2];
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    a[q] = __builtin_shufflevector(tr(hb + (offa[st][0] ^ (32 * q))), tr(hb + (offa[st][1] ^ (32 * q))), 0, 1,
+                                                   2, 3, 4, 5, 6, 7);
+                    b[q] = __builtin_shufflevector(tr(yb + st * 1024 + (offb[0] ^ (32 * q))),
+                                                   tr(yb + st * 1024 + (offb[1] ^ (32 * q))), 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int nb = 0; nb < 2; ++nb)
+                        acc[kb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[kb]),
+                                                                              __builtin_bit_cast(bf16x8, b[nb]), acc[kb][nb],
+                                                                              0, 0, 0);
+            }
+        }
+        asm volatile("s_barrier" ::: "memory");
+    }
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            const int n = 32 * nb + l32;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int k = wave * 64 + 32 * kb + 8 * (v >> 2) + 4 * lh + (v & 3);
+                if (n < p.D) outp[(size_t)k * p.D + n] = acc[kb][nb][v];
+            }
+        }
+}
+
+// Fills the plan of wgrad_halo_bf16 and returns the number of workgroups (= splits), or 0 when the
+// kernel does not apply: unit stride, 64 input channels, D a multiple of 8 up to 64, at most 9 taps,
+// slabs of whole output rows (R rows with R * Wo a multiple of 16 up to 128, R dividing Ho) whose
+// padded source rows fit the halo buffer, and at least 4 slabs per CU (AETHER_WGRAD_HALO=1 drops
+// the last condition, =0 turns the kernel off).
+static int plan_wgrad_halo(WgradHaloParams& p, int C, int sH, int sW, int cus) {
+    if (sH != 1 || sW != 1 || C != 64 || p.D % 8 != 0 || p.D > 64 || p.fH * p.fW > kWhMaxTaps) return 0;
+    bool force = false;
+    if (const char* f = getenv("AETHER_WGRAD_HALO")) {
+        if (atoi(f) == 0) return 0;
+        force = true;
+    }
+    int R = 0;
+    for (int r = 1; r * p.Wo <= kWhRows; ++r)
+        if ((r * p.Wo) % 16 == 0 && p.Ho % r == 0) R = r;                  // the tallest slab that fits
+    if (R == 0) return 0;
+    p.R = R;
+    p.slab_m = R * p.Wo;
+    p.Wp = p.Wo + p.fW - 1;
+    p.hslots = (R + p.fH - 1) * p.Wp;
+    if (p.hslots > kWhSlots) return 0;
+    const int64_t nslabs = (int64_t)p.S * (p.Ho / R);
+    if (nslabs > (1 << 24) || (!force && nslabs < 4 * (int64_t)cus)) return 0;
+    // byte offsets are formed in 32 bits from the pixel above and left of the image
+    if (((int64_t)p.S * p.H + p.fH) * p.W * 128 >= ((int64_t)1 << 31)) return 0;
+    p.nslabs = (int)nslabs;
+    const int wgs = (int)std::min<int64_t>(nslabs, cus);
+    p.per = cdiv(p.nslabs, wgs);
+    p.div_wp = FastDiv(p.Wp);
+    p.div_wo = FastDiv(p.Wo);
+    p.div_fw = FastDiv(p.fW);
+    p.div_spi = FastDiv(p.Ho / R);
+    return cdiv(p.nslabs, p.per);
+}
+
 template <typename T>
 int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* dbias,
                     int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW) {
@@ -2607,6 +2876,34 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     const bool dma16 = sizeof(T) == 2 && va && vy && fits;      // bf16 MFMA kernel, 64-row slabs
     p.x_bytes = (dma || dma16) ? (unsigned)xb : 0u;
     p.dy_bytes = (dma || dma16) ? (unsigned)yb : 0u;
+    if constexpr (sizeof(T) == 2) {
+        WgradHaloParams hp;
+        hp.x = x; hp.dy = dy;
+        hp.x_bytes = p.x_bytes; hp.dy_bytes = p.dy_bytes;
+        hp.S = S; hp.H = H; hp.W = W; hp.Ho = Ho; hp.Wo = Wo; hp.D = D; hp.fH = fH; hp.fW = fW; hp.pH = pH; hp.pW = pW;
+        hp.want_dbias = dbias != nullptr;
+        const int splits = dma16 ? plan_wgrad_halo(hp, C, sH, sW, c.prop.multiProcessorCount) : 0;
+        if (splits > 0) {
+            const int64_t kd = (int64_t)p.K * D;
+            void* ws;
+            rc = workspace((int64_t)splits * (kd + D) * sizeof(float), &ws);
+            if (rc) return rc;
+            hp.out = (float*)ws;
+            hipLaunchKernelGGL(wgrad_halo_bf16, dim3(splits), dim3(64 * (fH * fW + 1)), 0, c.stream, hp);
+            AETH_LAUNCH_CHECK();
+            const int n = (int)(kd + (dbias ? D : 0));
+            const bool r4 = (reinterpret_cast<uintptr_t>(dw) & 15) == 0 &&
+                            (dbias == nullptr || (reinterpret_cast<uintptr_t>(dbias) & 15) == 0);
+            if (r4)
+                hipLaunchKernelGGL(reduce_splits4, dim3(cdiv(n, 64)), dim3(kThreads), 0, c.stream, (const float*)ws, dw,
+                                   dbias, (int)kd, n, (int)(kd + D), splits);
+            else
+                hipLaunchKernelGGL(reduce_splits, dim3(cdiv(n, 64)), dim3(kThreads), 0, c.stream, (const float*)ws, dw,
+                                   dbias, (int)kd, n, (int)(kd + D), splits);
+            AETH_LAUNCH_CHECK();
+            return AETH_OK;
+        }
+    }
     // operand width of the fp32 LDS-direct kernel: 192-wide k tiles where they pad fewer rows than 128-wide ones
     p.cw = !va ? 1 : (p.K <= 64 ? 2 : 4);
     if (dma && p.cw == 4 && cdiv(p.K, 192) * 192 < cdiv(p.K, kWgBK) * kWgBK) p.cw = 6;

@@ -206,3 +206,39 @@ def test_bf16_fprop_dgrad_with_the_filter_resident_in_lds(case, monkeypatch):
     # the same sums of the same products in another order of taps and tiles
     monkeypatch.setenv("AETHER_GATHER_RES", "0")
     abi.close(abi.fprop_bf16(x, w, b, stride, pad), got, rtol=1e-5, atol=1e-5)
+
+
+# wgrad of a unit-stride filter of at most 9 taps on 64 input channels and at most 64 output channels:
+# one persistent workgroup per CU keeps the whole K x N result in registers (a wave per tap) and a
+# loading wave brings slabs of whole output rows with the padded source rows under them.  The library
+# takes that kernel from 4 slabs per CU on; AETHER_WGRAD_HALO=1 lets small inputs reach it.
+WGRAD_HALO_CASES = [
+    (2, 56, 56, 64, 64, 3, 3, 1, 1, "same"),      # slabs of 2 rows of 56
+    (3, 28, 28, 64, 64, 3, 3, 1, 1, "same"),      # 4 rows of 28
+    (2, 30, 30, 64, 48, 3, 3, 1, 1, "valid"),     # no padding, 48 output channels
+    (2, 18, 34, 64, 64, 3, 3, 1, 1, "valid"),     # 4 rows of 32: full 128-row slabs
+    (2, 17, 17, 64, 64, 2, 2, 1, 1, "valid"),     # even filter, 8 rows of 16
+    (2, 8, 58, 64, 40, 1, 3, 1, 1, "valid"),      # one filter row
+    (24, 56, 56, 64, 64, 3, 3, 1, 1, "same"),     # 672 slabs on 224 workgroups of 3
+    (2, 14, 14, 64, 64, 3, 3, 1, 1, "same"),      # 8 rows of 14 would make a slab, but 8 does not divide 14: other kernel
+    (2, 16, 16, 128, 64, 3, 3, 1, 1, "same"),     # 128 input channels: other kernel
+]
+
+
+@pytest.mark.parametrize("case", WGRAD_HALO_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_bf16_wgrad_with_the_whole_result_in_registers(case, monkeypatch):
+    from tests import abi
+    monkeypatch.setenv("AETHER_WGRAD_HALO", "1")
+    x, w, b, dy = _case(case, 13)
+    stride, pad = (case[7], case[8]), case[9]
+    xr, dyr = O.round_to_bf16(x), O.round_to_bf16(dy)
+    dw, db = abi.wgrad_bf16(x, dy, w.shape, stride, pad)
+    abi.close(dw, O.conv_wgrad(xr, dyr, w.shape[:2], stride, pad, dtype=np.float64), rms_scaled=True)
+    abi.close(db, O.conv_dbias(dyr, dtype=np.float64), rms_scaled=True)
+    dw2, db2 = abi.wgrad_bf16(x, dy, w.shape, stride, pad)
+    assert np.array_equal(dw, dw2) and np.array_equal(db, db2)            # deterministic
+    # the same sums of the same products in another order
+    monkeypatch.setenv("AETHER_WGRAD_HALO", "0")
+    dw3, db3 = abi.wgrad_bf16(x, dy, w.shape, stride, pad)
+    abi.close(dw3, dw, rtol=1e-4, atol=1e-5, rms_scaled=True)
+    abi.close(db3, db, rtol=1e-4, atol=1e-5, rms_scaled=True)
