@@ -2658,7 +2658,7 @@ static __global__ __launch_bounds__(64 * (kWhMaxTaps + 1), 1) void wgrad_halo_bf
             unsigned r, c;
             p.div_wp.divmod((unsigned)slot, r, c);
             relx[i] = ((int)r * p.W + (int)c) * 128 + (((lane & 7) ^ (((slot >> 1) & 1) << 2)) * 16);
-            colbad |= ((unsigned)((int)c - p.pW) >= (unsigned)p.W ? 1u : 0u) << i;
+            colbad |= ((unsigned)((int)c - p.pW) >= (unsigned)p.W || 8 * i >= p.hslots ? 1u : 0u) << i;
         }
 #pragma unroll
         for (int j = 0; j < NLD; ++j) {
@@ -2686,29 +2686,12 @@ static __global__ __launch_bounds__(64 * (kWhMaxTaps + 1), 1) void wgrad_halo_bf
         };
         auto issue = [&](int buf) __attribute__((always_inline)) {
             const unsigned hb = lds_address(&halo[buf][0]), yb = lds_address(&dyb[buf][0]);
+            // every load is issued, without a branch; those past the slab have offsets outside the
+            // descriptors (no memory access, zeros into buffer space nobody reads)
 #pragma unroll
-            for (int i = 0; i < NLH; ++i)
-                if (8 * i < p.hslots) lds_direct_load16(rsrc_x, hb + (unsigned)i * 1024u, offx[i]);
+            for (int i = 0; i < NLH; ++i) lds_direct_load16(rsrc_x, hb + (unsigned)i * 1024u, offx[i]);
 #pragma unroll
-            for (int j = 0; j < NLD; ++j)
-                if (8 * j < p.slab_m) lds_direct_load16(rsrc_y, yb + (unsigned)j * 1024u, offy[j]);
-        };
-        // dbias: the lane adds up 8 columns (one chunk position) of the rows lrow, lrow + 8, ...
-        float db[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        auto add_columns = [&](int buf) __attribute__((always_inline)) {
-            const f4* yb = reinterpret_cast<const f4*>(&dyb[buf][0]);
-#pragma unroll
-            for (int j = 0; j < NLD; ++j) {
-                if (8 * j < p.slab_m) {
-                    const f4 v = yb[(8 * j + lrow) * 8 + (lane & 7)];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const unsigned u = __float_as_uint(v[e]);
-                        db[2 * e] += __uint_as_float(u << 16);
-                        db[2 * e + 1] += __uint_as_float(u & 0xffff0000u);
-                    }
-                }
-            }
+            for (int j = 0; j < NLD; ++j) lds_direct_load16(rsrc_y, yb + (unsigned)j * 1024u, offy[j]);
         };
         if (nsl > 0) {
             addresses(sl0);
@@ -2716,28 +2699,13 @@ static __global__ __launch_bounds__(64 * (kWhMaxTaps + 1), 1) void wgrad_halo_bf
         }
         if (nsl > 1) addresses(sl0 + 1);
         __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
-        if (p.want_dbias && nsl > 0) add_columns(0);
         asm volatile("s_barrier" ::: "memory");
         for (int t = 0; t < nsl; ++t) {
             // the multiplying waves are done with slab t - 1, whose buffers take slab t + 1
             if (t + 1 < nsl) issue((t + 1) & 1);
             if (t + 2 < nsl) addresses(sl0 + t + 2);
             __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
-            if (p.want_dbias && t + 1 < nsl) add_columns((t + 1) & 1);
             asm volatile("s_barrier" ::: "memory");
-        }
-        if (p.want_dbias) {
-            // lanes with the same chunk position hold different rows; the logical chunk is the position
-            // with bit 2 flipped for rows whose bit 1 is set (lrow & 2)
-            float* red = reinterpret_cast<float*>(&halo[0][0]);             // everyone is past the last barrier
-            const int lc = (lane & 7) ^ (((lrow >> 1) & 1) << 2);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) red[lrow * 64 + 8 * lc + e] = db[e];
-            __builtin_amdgcn_s_waitcnt(0);
-            float sum = 0.f;
-#pragma unroll
-            for (int r = 0; r < 8; ++r) sum += red[r * 64 + lane];
-            if (lane < p.D) outp[(size_t)K * p.D + lane] = sum;
         }
         return;
     }
@@ -2779,31 +2747,67 @@ static __global__ __launch_bounds__(64 * (kWhMaxTaps + 1), 1) void wgrad_halo_bf
     auto tr = [&](const uint16_t* q) __attribute__((always_inline)) {
         return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr_t)q);
     };
+    // dbias: wave t adds up the dy rows of the 8-row groups t, t + T, ... of every slab; a lane takes one
+    // chunk position (8 columns) of row lrow of those groups
+    const int lrow = lane >> 3;
+    float db[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     asm volatile("s_barrier" ::: "memory");
     for (int t = 0; t < nsl; ++t) {
         const uint16_t* hb = halo[t & 1];
         const uint16_t* yb = dyb[t & 1];
+        if (p.want_dbias) {
+            for (int j = wave; 8 * j < p.slab_m; j += T) {
+                const f4 v = reinterpret_cast<const f4*>(yb)[(8 * j + lrow) * 8 + (lane & 7)];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const unsigned u = __float_as_uint(v[e]);
+                    db[2 * e] += __uint_as_float(u << 16);
+                    db[2 * e + 1] += __uint_as_float(u & 0xffff0000u);
+                }
+            }
+        }
+        // the operands of step st + 1 are read while the four MFMAs of step st run
+        s8v a[2][2], b[2][2];
+        auto read_step = [&](int st, s8v (&ra)[2], s8v (&rb)[2]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                ra[q] = __builtin_shufflevector(tr(hb + (offa[st][0] ^ (32 * q))), tr(hb + (offa[st][1] ^ (32 * q))), 0, 1, 2,
+                                                3, 4, 5, 6, 7);
+                rb[q] = __builtin_shufflevector(tr(yb + st * 1024 + (offb[0] ^ (32 * q))),
+                                                tr(yb + st * 1024 + (offb[1] ^ (32 * q))), 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+        };
+        read_step(0, a[0], b[0]);
 #pragma unroll
         for (int st = 0; st < STEPS; ++st) {
             if (st < steps) {
-                s8v a[2], b[2];
-#pragma unroll
-                for (int q = 0; q < 2; ++q) {
-                    a[q] = __builtin_shufflevector(tr(hb + (offa[st][0] ^ (32 * q))), tr(hb + (offa[st][1] ^ (32 * q))), 0, 1,
-                                                   2, 3, 4, 5, 6, 7);
-                    b[q] = __builtin_shufflevector(tr(yb + st * 1024 + (offb[0] ^ (32 * q))),
-                                                   tr(yb + st * 1024 + (offb[1] ^ (32 * q))), 0, 1, 2, 3, 4, 5, 6, 7);
-                }
+                if (st + 1 < STEPS && st + 1 < steps) read_step(st + 1, a[(st + 1) & 1], b[(st + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                     for (int nb = 0; nb < 2; ++nb)
-                        acc[kb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[kb]),
-                                                                              __builtin_bit_cast(bf16x8, b[nb]), acc[kb][nb],
-                                                                              0, 0, 0);
+                        acc[kb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[st & 1][kb]),
+                                                                              __builtin_bit_cast(bf16x8, b[st & 1][nb]),
+                                                                              acc[kb][nb], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         asm volatile("s_barrier" ::: "memory");
+    }
+    if (p.want_dbias) {
+        // everyone is past the last barrier of the loop: the first halo buffer is free.  Row lrow of wave
+        // t holds its sums by logical chunk: the position with bit 2 flipped for rows whose bit 1 is set.
+        float* red = reinterpret_cast<float*>(&halo[0][0]);
+        const int lc = (lane & 7) ^ (((lrow >> 1) & 1) << 2);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) red[(wave * 8 + lrow) * 64 + 8 * lc + e] = db[e];
+        __syncthreads();
+        if (wave == 0 && lane < p.D) {
+            float sum = 0.f;
+            for (int r = 0; r < 8 * T; ++r) sum += red[r * 64 + lane];
+            outp[(size_t)K * p.D + lane] = sum;
+        }
     }
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
