@@ -213,6 +213,14 @@ __device__ __forceinline__ void store_tile(const GatherParams& p, float* out, co
                 }
         }
     }
+    // The stored registers stay untouched for a few cycles after the last store has been issued.
+    // Where the instruction after a 16-byte store was free to reuse its data registers (a
+    // persistent workgroup whose scheduler had moved the next tile's address arithmetic up), the
+    // last lanes of each row of 16 now and then stored the new value instead.
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) asm volatile("s_nop 3" :: "v"(acc[i][j]));
 }
 
 template <typename T, int BM, int BN, int WM, int WN, int VEC>
@@ -1192,6 +1200,165 @@ static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(co
 // gather-GEMM launch.  k = (th*Tw + tw)*Ck + kc ; filter tap x = xa + xs*th,
 // y = ya + ys*tw.  transposed == 0: n is the output channel d and kc the input
 // channel c (fprop).  transposed == 1: n is c and kc is d (dgrad).
+// ------------------------------------------------------------------------------
+// dense_res_f32: y[M, N] = x[M, K] . w + bias in fp32 for a short K (one or two slabs: K = 32 or 64)
+// and N up to 256 -- a 1x1 convolution that widens the channels (64 -> 256 on 56x56 images: 205 MB in,
+// 822 MB out, 26 GFLOP: the fp32 matrix pipe and the memory system need about the same time).  The
+// n-loop mode of gather_gemm_dma reaches 63 % of what a plain copy moves there: its waves wait for
+// the loads of the next filter slab together with the stores of the tile before.  Here one
+// persistent workgroup of 8 waves per CU keeps the whole packed filter in LDS (64 KB), walks tiles
+// of 128 rows x N (wave = 64 x 64, two A buffers of 32 KB) and never waits for a store: wave 0
+// fetches the A rows of the next tile at the start of a tile; a wave keeps its finished tile in
+// registers and stores it during the next one, wave w after k group w of the 8, so that the stores
+// of a CU are spread over the tile and those of wave 0 have long left when it waits for its loads.
+// ------------------------------------------------------------------------------
+constexpr int kD1BM = 128;
+constexpr int kD1Threads = 512;
+constexpr int kD1MaxN = 256;
+
+template <int NSLAB>                                   // K = 32 * NSLAB
+static __global__ __launch_bounds__(kD1Threads, 1) void dense_res_f32(const GatherParams p, const int mtiles) {
+    constexpr int BM = kD1BM, KC = 8, TM = 2, TN = 2, nslab = NSLAB;
+    __shared__ f4 filt[2][kD1MaxN * KC];                 // slab s: rows n of 128 B, chunk c at c ^ ((n >> 1) & 7)
+    __shared__ f4 abuf[2][2][BM * KC];                   // [buffer][slab]
+    __shared__ f4 bias_lds[kD1MaxN / 4];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31;
+    const int lh = lane >> 5;
+    const int G = (int)gridDim.x;
+    const int lid = xcd_contiguous_id((int)blockIdx.x, G);
+    const int per = (mtiles + G - 1) / G;
+    const int tile0 = lid * per;
+    const int ntl = max(0, min(per, mtiles - tile0));
+    const int wm0 = 64 * (wave & 1), wn0 = 64 * (wave >> 1);
+    const bool active = wn0 < p.N;                       // wave-uniform
+
+    // 1 KB pieces: 8 rows x 8 chunks, lane / 8 picks the row, lane % 8 the chunk position
+    const int prow = lane >> 3;
+    const int k4e = (lane & 7) ^ (lane >> 4);            // logical chunk at this position for even pieces (odd: ^ 4)
+    {
+        const u32x4 rsrc_b = raw_rsrc(p.bt, p.bt_bytes);
+        const int pieces = kD1MaxN / 8;                  // per slab; rows past the packed filter read as zeros
+        for (int q = wave; q < nslab * pieces; q += 8) {
+            const int sl = q / pieces, part = q - sl * pieces;
+            const int k4 = k4e ^ ((part & 1) ? 4 : 0);
+            const unsigned off = (unsigned)(((part * 8 + prow) * p.Kpad + 32 * sl + 4 * k4) * 4);
+            lds_direct_load16(rsrc_b, lds_address(&filt[sl][0]) + (unsigned)part * 1024u, off);
+        }
+        if (tid < kD1MaxN / 4) {
+            f4 b = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (p.bias != nullptr && 4 * tid + e < p.N) b[e] = p.bias[4 * tid + e];
+            bias_lds[tid] = b;
+        }
+    }
+    // A rows of a tile: 16 pieces per slab; rows past M lie outside the descriptor and read as zeros
+    const u32x4 rsrc_a = raw_rsrc(p.src, p.src_bytes);
+    unsigned rela[2 * (BM / 8)];
+#pragma unroll
+    for (int i = 0; i < 2 * (BM / 8); ++i) {
+        const int sl = i / (BM / 8), part = i % (BM / 8);
+        const int k4 = k4e ^ ((part & 1) ? 4 : 0);
+        rela[i] = (unsigned)(((part * 8 + prow) * p.Cs + 32 * sl + 4 * k4) * 4);
+    }
+    auto fetch = [&](int tile, int buf) __attribute__((always_inline)) {
+        const unsigned base = (unsigned)tile * (unsigned)(BM * p.Cs * 4);
+#pragma unroll
+        for (int i = 0; i < 2 * (BM / 8); ++i) {
+            if (i < nslab * (BM / 8)) {
+                const int sl = i / (BM / 8), part = i % (BM / 8);
+                lds_direct_load16(rsrc_a, lds_address(&abuf[buf][sl][0]) + (unsigned)part * 1024u, base + rela[i]);
+            }
+        }
+    };
+    if (wave == 0 && ntl > 0) fetch(tile0, 0);
+    __builtin_amdgcn_s_waitcnt(0);
+    asm volatile("s_barrier" ::: "memory");
+
+    const int sw7 = (l32 >> 1) & 7;
+    f16v acc[TM][TN], done[TM][TN];
+    int done_m0 = 0;
+    bool have_done = false;
+    auto store_done = [&]() __attribute__((always_inline)) {
+        store_tile<TM, TN, true>(p, p.out, done, done_m0 + wm0, wn0, l32, lh);
+    };
+    for (int t = 0; t < ntl; ++t) {
+        if (wave == 0 && t + 1 < ntl) fetch(tile0 + t + 1, (t + 1) & 1);
+        if (active) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const f4 b = bias_lds[(wn0 + 32 * j + 8 * q + 4 * lh) >> 2];
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = b[e];
+                }
+            // k groups u = 4 slab + g of 8 k each; the operands of group u + 1 are read during the MFMAs of group u
+            f4 fa[2][TM], fb[2][TN];
+            auto read_frags = [&](int u, int slot) __attribute__((always_inline)) {
+                const int sl = u >> 2, g = u & 3;
+                const f4* la = abuf[t & 1][sl];
+                const f4* lb = filt[sl];
+                const int pc = (2 * g + lh) ^ sw7;
+#pragma unroll
+                for (int i = 0; i < TM; ++i) fa[slot][i] = la[(wm0 + 32 * i + l32) * KC + pc];
+#pragma unroll
+                for (int j = 0; j < TN; ++j) fb[slot][j] = lb[(wn0 + 32 * j + l32) * KC + pc];
+            };
+            read_frags(0, 0);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (u < 4 * nslab) {
+                    if (u + 1 < 4 * nslab) read_frags(u + 1, (u + 1) & 1);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) mma_chunk<float>(fb[u & 1][j], fa[u & 1][i], acc[i][j]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                // the finished tile leaves after k group `wave` (a few 16-byte pieces after every group
+                // were slower: 0.298 ms against 0.266 on 56x56, 64 -> 256)
+                if (have_done && u == min(wave, 4 * nslab - 1)) store_done();
+            }
+            have_done = true;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) done[i][j] = acc[i][j];
+            done_m0 = (tile0 + t) * BM;
+        }
+        if (wave == 0) __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));   // the next tile's rows (and its own old stores)
+        asm volatile("s_barrier" ::: "memory");
+    }
+    if (active && have_done) store_done();
+}
+
+// dense_res_f32 applies to fp32 gathers that are plain matrix products (one tap, unit stride, no
+// padding), K = 32 or 64 whole, N a multiple of 4 up to 256 with more than one 64-wide tile, a dense
+// output with 16-byte stores, and at least 4 tiles of 128 rows per CU (AETHER_DENSE_RES=1 drops the
+// last condition, =0 turns the kernel off).
+static bool plan_dense_res(const GatherParams& gp, bool dma, int cus, int* mtiles) {
+    if (!dma || gp.sh != 1 || gp.sw != 1 || gp.rh0 != 0 || gp.rw0 != 0 || gp.Hs != gp.Hg || gp.Ws != gp.Wg) return false;
+    if (gp.K != gp.Cs || gp.K != gp.Kpad || (gp.K != 32 && gp.K != 64) || gp.split_slabs != 0) return false;
+    if (gp.N <= 64 || gp.N > kD1MaxN || !gp.dense_out || gp.out_bytes == 0) return false;
+    bool force = false;
+    if (const char* f = getenv("AETHER_DENSE_RES")) {
+        if (atoi(f) == 0) return false;
+        force = true;
+    }
+    const int n = cdiv(gp.M, kD1BM);
+    if (!force && n < 4 * cus) return false;
+    *mtiles = n;
+    return true;
+}
+
 template <typename T>
 __global__ void pack_filter(const PackParams p) {
     int idx = blockIdx.x * blockDim.x + threadIdx.x;
@@ -1377,6 +1544,15 @@ static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t
             dim3 grid((unsigned)(mtiles * cdiv(gp.N, 64)));
             if (stages == 4) hipLaunchKernelGGL(gather_halo_bf16<4>, grid, dim3(kThreads), 0, st, hp);
             else hipLaunchKernelGGL(gather_halo_bf16<3>, grid, dim3(kThreads), 0, st, hp);
+            return;
+        }
+    }
+    if constexpr (sizeof(T) == 4) {
+        int mtiles = 0;
+        if (plan_dense_res(gp, dma, cus, &mtiles)) {
+            const dim3 grid((unsigned)std::min(mtiles, cus));
+            if (gp.Kpad == 64) hipLaunchKernelGGL(dense_res_f32<2>, grid, dim3(kD1Threads), 0, st, gp, mtiles);
+            else hipLaunchKernelGGL(dense_res_f32<1>, grid, dim3(kD1Threads), 0, st, gp, mtiles);
             return;
         }
     }

@@ -195,3 +195,32 @@ def test_fprop_parity_with_128_row_tiles(case, monkeypatch):
     abi.close(abi.fprop(x, w, b, stride, pad), want)
     abi.close(abi.fprop(x, w, None, stride, pad), O.conv_fprop(x, w, None, stride, pad, dtype=np.float64))
 
+
+
+# Plain matrix products with a short K (32 or 64) and a wide output (up to 256 columns, e.g. the 1x1
+# convolution 64 -> 256): one persistent workgroup per CU with the whole filter in LDS.  The library
+# takes that kernel from 4 tiles of 128 rows per CU on; AETHER_DENSE_RES=1 lets small inputs reach it.
+DENSE_RES_CASES = [
+    (8, 48, 48, 64, 256, 1, 1, 1, 1, "valid"),    # 144 tiles: one each
+    (8, 48, 48, 32, 192, 1, 1, 1, 1, "valid"),    # one slab, 3 n tiles: two waves have nothing to multiply
+    (3, 50, 50, 64, 136, 1, 1, 1, 1, "valid"),    # ragged last n tile, rows past M in the last tile
+    (40, 56, 56, 64, 256, 1, 1, 1, 1, "valid"),   # 980 tiles on 256 workgroups: 4 each, the last ones fewer
+    (1000, 1, 1, 64, 100, 1, 1, 1, 1, "valid"),   # a dense layer
+    (8, 48, 48, 64, 256, 1, 1, 1, 1, "same"),     # "same" with a 1x1 filter pads nothing either
+    (8, 24, 24, 48, 256, 1, 1, 1, 1, "valid"),    # K = 48 is not a whole slab: the other kernels
+    (8, 24, 24, 64, 256, 1, 1, 2, 2, "valid"),    # stride 2: the other kernels
+]
+
+
+@pytest.mark.parametrize("case", DENSE_RES_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_fprop_with_the_filter_resident_in_lds(case, monkeypatch):
+    from tests import abi
+    monkeypatch.setenv("AETHER_DENSE_RES", "1")
+    x, w, b, dy = _case(case, 12)
+    stride, pad = (case[7], case[8]), case[9]
+    got = abi.fprop(x, w, b, stride, pad)
+    abi.close(got, O.conv_fprop(x, w, b, stride, pad, dtype=np.float64))
+    abi.close(abi.fprop(x, w, None, stride, pad), O.conv_fprop(x, w, None, stride, pad, dtype=np.float64))
+    # the other kernels add the same products in the same order of k
+    monkeypatch.setenv("AETHER_DENSE_RES", "0")
+    assert np.array_equal(got, abi.fprop(x, w, b, stride, pad))
