@@ -217,10 +217,12 @@ __device__ __forceinline__ void store_tile(const GatherParams& p, float* out, co
     // Where the instruction after a 16-byte store was free to reuse its data registers (a
     // persistent workgroup whose scheduler had moved the next tile's address arithmetic up), the
     // last lanes of each row of 16 now and then stored the new value instead.
+#if defined(__HIP_DEVICE_COMPILE__)                      // the host pass does not know the register class
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) asm volatile("s_nop 3" :: "v"(acc[i][j]));
+#endif
 }
 
 template <typename T, int BM, int BN, int WM, int WN, int VEC>
@@ -3033,6 +3035,202 @@ static int plan_wgrad_halo(WgradHaloParams& p, int C, int sH, int sW, int cus) {
     return cdiv(p.nslabs, p.per);
 }
 
+// ------------------------------------------------------------------------------
+// wgrad_halo_f32: the fp32 twin of wgrad_halo_bf16 for 64 input channels, at most 64 output
+// channels and at most 9 unit-stride taps.  One persistent workgroup per CU holds the whole
+// K x N result in registers, 12 multiplying waves of three 32 x 32 accumulators each (wave w: n block
+// w & 1, k blocks 3 (w >> 1) .. + 2, a k block being half a tap: 32 channels), three per SIMD, and a
+// thirteenth wave that only loads.  A slab is ONE output row (Wo pixels = NPAIRS pairs: an MFMA
+// 32x32x2 reduces over two pixels) and the three padded source rows under it (fH x Wp pixel slots
+// of 256 B), two buffers each, loaded a slab ahead.  A lane's operand of pixel pair p is one float
+// at a constant offset plus 512 p bytes from a per-lane base (ds_read_b32 with an immediate offset):
+// the loop is four LDS reads and three MFMAs per pair, no address arithmetic, no wait on memory.
+// A pixel's 64 floats are stored with their 128-byte halves swapped in odd slots (dy: odd rows), so
+// that the two pixels of a pair, read by the two halves of a wave, fall into different banks.
+// dbias: the waves of k blocks 0..2 add up the dy values they multiply.
+// ------------------------------------------------------------------------------
+constexpr int kFhSlots = 176;       // halo buffer: 176 pixel slots of 256 B (3 padded rows of 58)
+constexpr int kFhRows = 64;         // dy buffer: 64 rows of 256 B
+constexpr int kFhWaves = 13;
+
+template <int NPAIRS>
+static __global__ __launch_bounds__(64 * kFhWaves, 1) void wgrad_halo_f32(const WgradHaloParams p) {
+    constexpr int NLH = kFhSlots / 4, NLD = kFhRows / 4;
+    __shared__ float halo[2][kFhSlots * 64];
+    __shared__ float dyb[2][kFhRows * 64];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31;
+    const int lh = lane >> 5;
+    const int T = p.fH * p.fW;
+    const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
+    const int sl0 = lid * p.per;
+    const int nsl = max(0, min(p.per, p.nslabs - sl0));
+    const int K = T * 64;
+    float* const outp = p.out + (size_t)lid * ((size_t)K * p.D + p.D);
+
+    if (wave == kFhWaves - 1) {
+        // ---- the loading wave ----
+        // Halo load i brings the slots 4 i .. 4 i + 3, dy load j the rows 4 j .. 4 j + 3 (lane / 16 picks
+        // the slot or row, lane % 16 the 16-byte chunk position; odd slots and rows hold chunk c at c ^ 8).
+        const u32x4 rsrc_x = raw_rsrc(p.x, p.x_bytes);
+        const u32x4 rsrc_y = raw_rsrc(p.dy, p.dy_bytes);
+        const int lrow = lane >> 4;
+        int relx[NLH], rely[NLD];
+        unsigned colbad_lo = 0, colbad_hi = 0;
+#pragma unroll
+        for (int i = 0; i < NLH; ++i) {
+            const int slot = 4 * i + lrow;
+            unsigned r, c;
+            p.div_wp.divmod((unsigned)slot, r, c);
+            relx[i] = ((int)r * p.W + (int)c) * 256 + (((lane & 15) ^ ((slot & 1) << 3)) * 16);
+            const unsigned bad = (unsigned)((int)c - p.pW) >= (unsigned)p.W || 4 * i >= p.hslots ? 1u : 0u;
+            if (i < 32) colbad_lo |= bad << i;
+            else colbad_hi |= bad << (i - 32);
+        }
+#pragma unroll
+        for (int j = 0; j < NLD; ++j) {
+            const int row = 4 * j + lrow;
+            const int n4 = 4 * ((lane & 15) ^ ((row & 1) << 3));
+            rely[j] = (row * p.D + n4) * 4;
+            if (n4 >= p.D || row >= p.slab_m) rely[j] = (int)0x80000000;
+        }
+        // every load is issued, without a branch; those past the slab have offsets outside the
+        // descriptors (no memory access, zeros into buffer space nobody reads)
+        auto fetch = [&](int slab, int buf) __attribute__((always_inline)) {
+            unsigned s_img, r_img;
+            p.div_spi.divmod((unsigned)slab, s_img, r_img);
+            const int R0 = (int)r_img * p.R - p.pH;                         // image row of padded row 0 of the slab
+            const int base = (((int)s_img * p.H + R0) * p.W - p.pW) * 256;
+            const int a0 = lrow + R0 * p.Wp;                                // slot - lo
+            const int b0 = (p.H - R0) * p.Wp - 1 - lrow;                    // hi - 1 - slot
+            const unsigned hb = lds_address(&halo[buf][0]), yb = lds_address(&dyb[buf][0]);
+#pragma unroll
+            for (int i = 0; i < NLH; ++i) {
+                const unsigned rowbad = (unsigned)((a0 + 4 * i) | (b0 - 4 * i)) & 0x80000000u;
+                const unsigned colbad = i < 32 ? (colbad_lo << (31 - i)) : (colbad_hi << (63 - i));
+                lds_direct_load16(rsrc_x, hb + (unsigned)i * 1024u,
+                                  (unsigned)(base + relx[i]) | rowbad | (colbad & 0x80000000u));
+            }
+            const int ybase = (((int)s_img * p.Ho + (int)r_img * p.R) * p.Wo) * p.D * 4;
+#pragma unroll
+            for (int j = 0; j < NLD; ++j)
+                lds_direct_load16(rsrc_y, yb + (unsigned)j * 1024u,
+                                  (unsigned)(ybase + rely[j]) | ((unsigned)rely[j] & 0x80000000u));
+        };
+        if (nsl > 0) fetch(sl0, 0);
+        __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
+        asm volatile("s_barrier" ::: "memory");
+        for (int t = 0; t < nsl; ++t) {
+            // the multiplying waves are done with slab t - 1, whose buffers take slab t + 1
+            if (t + 1 < nsl) fetch(sl0 + t + 1, (t + 1) & 1);
+            __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
+            asm volatile("s_barrier" ::: "memory");
+        }
+        return;
+    }
+
+    // ---- the multiplying waves ----
+    const int nb = wave & 1, kb0 = 3 * (wave >> 1);
+    // byte offsets of the lane's operand of pair 0: x[pixel lh][k block q, channel l32] and dy[row lh][32 nb + l32]
+    int offa[3];
+    bool live[3];
+#pragma unroll
+    for (int q = 0; q < 3; ++q) {
+        const int kb = kb0 + q;
+        live[q] = kb < 2 * T;                                              // wave-uniform
+        unsigned fx, fy;
+        p.div_fw.divmod((unsigned)min(kb >> 1, T - 1), fx, fy);
+        const int slot = lh + (int)fx * p.Wp + (int)fy;
+        offa[q] = (slot * 64 + ((32 * (kb & 1) + l32) ^ ((slot & 1) << 5))) * 4;
+    }
+    const int offb = (lh * 64 + ((32 * nb + l32) ^ (lh << 5))) * 4;
+    f16v acc[3];
+#pragma unroll
+    for (int q = 0; q < 3; ++q)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[q][v] = 0.f;
+    float db = 0.f;
+    const bool do_db = p.want_dbias && kb0 == 0;
+    asm volatile("s_barrier" ::: "memory");
+    for (int t = 0; t < nsl; ++t) {
+        const char* hb = reinterpret_cast<const char*>(halo[t & 1]);
+        const char* yb = reinterpret_cast<const char*>(dyb[t & 1]);
+        const char* pa[3] = {hb + offa[0], hb + offa[1], hb + offa[2]};
+        const char* pb = yb + offb;
+        float a[2][3], b[2];
+        auto read_pair = [&](int pr, int s) __attribute__((always_inline)) {
+#pragma unroll
+            for (int q = 0; q < 3; ++q) a[s][q] = *reinterpret_cast<const float*>(pa[q] + 512 * pr);
+            b[s] = *reinterpret_cast<const float*>(pb + 512 * pr);
+        };
+        read_pair(0, 0);
+#pragma unroll
+        for (int pr = 0; pr < NPAIRS; ++pr) {
+            if (pr + 1 < NPAIRS) read_pair(pr + 1, (pr + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int q = 0; q < 3; ++q)                                      // blocks past the last tap too: no branch in here
+                acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[pr & 1][q], b[pr & 1], acc[q], 0, 0, 0);
+            db += b[pr & 1];
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        asm volatile("s_barrier" ::: "memory");
+    }
+    if (do_db) {
+        // everyone is past the last barrier of the loop: the first dy buffer is free
+        float* red = dyb[0];
+        red[nb * 64 + lane] = db;
+        __builtin_amdgcn_s_waitcnt(0);
+        if (lh == 0 && 32 * nb + l32 < p.D) outp[(size_t)K * p.D + 32 * nb + l32] = red[nb * 64 + l32] + red[nb * 64 + 32 + l32];
+    }
+#pragma unroll
+    for (int q = 0; q < 3; ++q) {
+        if (live[q]) {
+            const int n = 32 * nb + l32;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int k = (kb0 + q) * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+                if (n < p.D) outp[(size_t)k * p.D + n] = acc[q][v];
+            }
+        }
+    }
+}
+
+// Fills the plan of wgrad_halo_f32 and returns the number of workgroups (= splits), or 0 when the
+// kernel does not apply: unit stride, 64 input channels, D a multiple of 4 up to 64, at most 9 taps,
+// an even Wo of 28, 32, 56 or 64 (the built pair counts), fH padded rows of Wo + fW - 1 slots in the
+// halo buffer, and at least 4 output rows per CU (AETHER_WGRAD_HALO=1 drops the last condition, =0 turns
+// the kernel off).
+static int plan_wgrad_halo_f32(WgradHaloParams& p, int C, int sH, int sW, int cus) {
+    if (sH != 1 || sW != 1 || C != 64 || p.D % 4 != 0 || p.D > 64 || p.fH * p.fW > 9) return 0;
+    bool force = false;
+    if (const char* f = getenv("AETHER_WGRAD_HALO")) {
+        if (atoi(f) == 0) return 0;
+        force = true;
+    }
+    if (p.Wo != 28 && p.Wo != 32 && p.Wo != 56 && p.Wo != 64) return 0;
+    p.R = 1;
+    p.slab_m = p.Wo;
+    p.Wp = p.Wo + p.fW - 1;
+    p.hslots = p.fH * p.Wp;
+    if (p.hslots > kFhSlots) return 0;
+    const int64_t nslabs = (int64_t)p.S * p.Ho;
+    if (nslabs > (1 << 24) || (!force && nslabs < 4 * (int64_t)cus)) return 0;
+    // byte offsets are formed in 32 bits from the pixel above and left of the image
+    if (((int64_t)p.S * p.H + p.fH) * p.W * 256 >= ((int64_t)1 << 31)) return 0;
+    p.nslabs = (int)nslabs;
+    const int wgs = (int)std::min<int64_t>(nslabs, cus);
+    p.per = cdiv(p.nslabs, wgs);
+    p.div_wp = FastDiv(p.Wp);
+    p.div_wo = FastDiv(p.Wo);
+    p.div_fw = FastDiv(p.fW);
+    p.div_spi = FastDiv(p.Ho);
+    return cdiv(p.nslabs, p.per);
+}
+
 template <typename T>
 int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* dbias,
                     int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW) {
@@ -3056,20 +3254,30 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     const bool dma16 = sizeof(T) == 2 && va && vy && fits;      // bf16 MFMA kernel, 64-row slabs
     p.x_bytes = (dma || dma16) ? (unsigned)xb : 0u;
     p.dy_bytes = (dma || dma16) ? (unsigned)yb : 0u;
-    if constexpr (sizeof(T) == 2) {
+    {
         WgradHaloParams hp;
         hp.x = x; hp.dy = dy;
         hp.x_bytes = p.x_bytes; hp.dy_bytes = p.dy_bytes;
         hp.S = S; hp.H = H; hp.W = W; hp.Ho = Ho; hp.Wo = Wo; hp.D = D; hp.fH = fH; hp.fW = fW; hp.pH = pH; hp.pW = pW;
         hp.want_dbias = dbias != nullptr;
-        const int splits = dma16 ? plan_wgrad_halo(hp, C, sH, sW, c.prop.multiProcessorCount) : 0;
+        int splits = 0;
+        if constexpr (sizeof(T) == 2) splits = dma16 ? plan_wgrad_halo(hp, C, sH, sW, c.prop.multiProcessorCount) : 0;
+        else splits = (dma && va) ? plan_wgrad_halo_f32(hp, C, sH, sW, c.prop.multiProcessorCount) : 0;
         if (splits > 0) {
             const int64_t kd = (int64_t)p.K * D;
             void* ws;
             rc = workspace((int64_t)splits * (kd + D) * sizeof(float), &ws);
             if (rc) return rc;
             hp.out = (float*)ws;
-            hipLaunchKernelGGL(wgrad_halo_bf16, dim3(splits), dim3(64 * (fH * fW + 1)), 0, c.stream, hp);
+            if constexpr (sizeof(T) == 2) {
+                hipLaunchKernelGGL(wgrad_halo_bf16, dim3(splits), dim3(64 * (fH * fW + 1)), 0, c.stream, hp);
+            } else {
+                const dim3 grid(splits), block(64 * kFhWaves);
+                if (Wo == 56) hipLaunchKernelGGL(wgrad_halo_f32<28>, grid, block, 0, c.stream, hp);
+                else if (Wo == 64) hipLaunchKernelGGL(wgrad_halo_f32<32>, grid, block, 0, c.stream, hp);
+                else if (Wo == 32) hipLaunchKernelGGL(wgrad_halo_f32<16>, grid, block, 0, c.stream, hp);
+                else hipLaunchKernelGGL(wgrad_halo_f32<14>, grid, block, 0, c.stream, hp);
+            }
             AETH_LAUNCH_CHECK();
             const int n = (int)(kd + (dbias ? D : 0));
             const bool r4 = (reinterpret_cast<uintptr_t>(dw) & 15) == 0 &&

@@ -224,3 +224,36 @@ def test_fprop_with_the_filter_resident_in_lds(case, monkeypatch):
     # the other kernels add the same products in the same order of k
     monkeypatch.setenv("AETHER_DENSE_RES", "0")
     assert np.array_equal(got, abi.fprop(x, w, b, stride, pad))
+
+
+# fp32 wgrad of a unit-stride filter of at most 9 taps on 64 input channels and at most 64 output
+# channels, on rows of 28, 32, 56 or 64 output pixels: one persistent workgroup per CU keeps the whole
+# K x N result in registers (12 multiplying waves of three 32 x 32 blocks) and a loading wave brings one
+# output row and the padded source rows under it at a time.  The library takes that kernel from 4 rows
+# per CU on; AETHER_WGRAD_HALO=1 lets small inputs reach it.
+WGRAD_HALO_F32_CASES = [
+    (2, 56, 56, 64, 64, 3, 3, 1, 1, "same"),      # the 56x56x64 layer
+    (3, 28, 28, 64, 64, 3, 3, 1, 1, "same"),
+    (2, 30, 34, 64, 48, 3, 3, 1, 1, "valid"),     # 32 pixels per row, no padding, 48 output channels
+    (2, 20, 65, 64, 64, 2, 2, 1, 1, "valid"),     # even filter: 8 k blocks of the 18 carry taps
+    (2, 8, 58, 64, 40, 1, 3, 1, 1, "valid"),      # one filter row
+    (7, 56, 56, 64, 64, 3, 3, 1, 1, "same"),      # 392 rows on 196 workgroups of 2
+    (2, 14, 14, 64, 64, 3, 3, 1, 1, "same"),      # rows of 14 pixels: other kernels
+    (2, 28, 28, 32, 64, 3, 3, 1, 1, "same"),      # 32 input channels: other kernels
+]
+
+
+@pytest.mark.parametrize("case", WGRAD_HALO_F32_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_wgrad_with_the_whole_result_in_registers(case, monkeypatch):
+    from tests import abi
+    monkeypatch.setenv("AETHER_WGRAD_HALO", "1")
+    x, w, b, dy = _case(case, 14)
+    stride, pad = (case[7], case[8]), case[9]
+    dw, db = abi.wgrad(x, dy, w.shape, stride, pad)
+    want = O.conv_wgrad(x, dy, w.shape[:2], stride, pad, dtype=np.float64)
+    abi.close(dw, want, rms_scaled=True)
+    abi.close(db, O.conv_dbias(dy, dtype=np.float64), rms_scaled=True)
+    ref32 = O.conv_wgrad(x, dy, w.shape[:2], stride, pad, dtype=np.float32)
+    assert np.abs(dw - want).max() <= 2.0 * np.abs(ref32 - want).max() + 1e-6
+    dw2, none = abi.wgrad(x, dy, w.shape, stride, pad, want_dbias=False)
+    assert none is None and np.array_equal(dw, dw2)       # deterministic
