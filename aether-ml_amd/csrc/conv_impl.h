@@ -3049,13 +3049,14 @@ static int plan_wgrad_halo(WgradHaloParams& p, int C, int sH, int sW, int cus) {
 // that the two pixels of a pair, read by the two halves of a wave, fall into different banks.
 // dbias: the waves of k blocks 0..2 add up the dy values they multiply.
 // ------------------------------------------------------------------------------
-constexpr int kFhSlots = 176;       // halo buffer: 176 pixel slots of 256 B (3 padded rows of 58)
+constexpr int kFhRowSlots = 68;     // slots per padded row in LDS: Wo + fW - 1 rounded up to a multiple of 4
+constexpr int kFhSlots = 3 * kFhRowSlots;   // halo buffer: at most 3 padded rows of 256-byte pixel slots
 constexpr int kFhRows = 64;         // dy buffer: 64 rows of 256 B
 constexpr int kFhWaves = 13;
 
 template <int NPAIRS>
 static __global__ __launch_bounds__(64 * kFhWaves, 1) void wgrad_halo_f32(const WgradHaloParams p) {
-    constexpr int NLH = kFhSlots / 4, NLD = kFhRows / 4;
+    constexpr int NLD = kFhRows / 4;
     __shared__ float halo[2][kFhSlots * 64];
     __shared__ float dyb[2][kFhRows * 64];
 
@@ -3073,52 +3074,59 @@ static __global__ __launch_bounds__(64 * kFhWaves, 1) void wgrad_halo_f32(const 
 
     if (wave == kFhWaves - 1) {
         // ---- the loading wave ----
-        // Halo load i brings the slots 4 i .. 4 i + 3, dy load j the rows 4 j .. 4 j + 3 (lane / 16 picks
-        // the slot or row, lane % 16 the 16-byte chunk position; odd slots and rows hold chunk c at c ^ 8).
+        // It shares a SIMD with three waves that issue 64-cycle MFMAs back to back, and a vector
+        // instruction of its own waits for a gap between them: with five vector instructions of
+        // address arithmetic per load it needed 18 500 cycles for the 58 loads of a slab, more than the
+        // slab's MFMAs take.  So a load is scalar work only: padded row r of the halo takes Wpl / 4
+        // loads of 4 slots (lane / 16 picks the slot, lane % 16 the 16-byte chunk position; odd slots
+        // hold chunk c at c ^ 8) whose per-lane byte offset inside an image row is a constant of the
+        // workgroup (padding columns: bit 31, outside the descriptor: zeros); the row's start comes
+        // in as the scalar offset, and a padded row above or below the image is read through an
+        // empty descriptor.  dy rows likewise.
+        __builtin_amdgcn_s_setprio(3);
         const u32x4 rsrc_x = raw_rsrc(p.x, p.x_bytes);
         const u32x4 rsrc_y = raw_rsrc(p.dy, p.dy_bytes);
+        const u32x4 rsrc_none = raw_rsrc(p.x, 0u);
         const int lrow = lane >> 4;
-        int relx[NLH], rely[NLD];
-        unsigned colbad_lo = 0, colbad_hi = 0;
+        constexpr int NLR = kFhRowSlots / 4;
+        unsigned voffx[NLR], voffy[NLD];
 #pragma unroll
-        for (int i = 0; i < NLH; ++i) {
-            const int slot = 4 * i + lrow;
-            unsigned r, c;
-            p.div_wp.divmod((unsigned)slot, r, c);
-            relx[i] = ((int)r * p.W + (int)c) * 256 + (((lane & 15) ^ ((slot & 1) << 3)) * 16);
-            const unsigned bad = (unsigned)((int)c - p.pW) >= (unsigned)p.W || 4 * i >= p.hslots ? 1u : 0u;
-            if (i < 32) colbad_lo |= bad << i;
-            else colbad_hi |= bad << (i - 32);
+        for (int g = 0; g < NLR; ++g) {
+            const int c = 4 * g + lrow;
+            const int lc = (lane & 15) ^ ((c & 1) << 3);                    // Wpl is a multiple of 4: slot parity = column parity
+            voffx[g] = (unsigned)(c - p.pW) < (unsigned)p.W ? (unsigned)(((c - p.pW) * 64 + 4 * lc) * 4) : 0x80000000u;
         }
 #pragma unroll
         for (int j = 0; j < NLD; ++j) {
             const int row = 4 * j + lrow;
             const int n4 = 4 * ((lane & 15) ^ ((row & 1) << 3));
-            rely[j] = (row * p.D + n4) * 4;
-            if (n4 >= p.D || row >= p.slab_m) rely[j] = (int)0x80000000;
+            voffy[j] = (n4 < p.D && row < p.slab_m) ? (unsigned)((row * p.D + n4) * 4) : 0x80000000u;
         }
-        // every load is issued, without a branch; those past the slab have offsets outside the
-        // descriptors (no memory access, zeros into buffer space nobody reads)
+        auto load = [&](const u32x4& rsrc, unsigned lds_base, unsigned voff, unsigned soff) __attribute__((always_inline)) {
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         :: "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
+        };
+        const int nlr = p.Wp >> 2;                                         // p.Wp is the padded row pitch Wpl here
         auto fetch = [&](int slab, int buf) __attribute__((always_inline)) {
             unsigned s_img, r_img;
             p.div_spi.divmod((unsigned)slab, s_img, r_img);
-            const int R0 = (int)r_img * p.R - p.pH;                         // image row of padded row 0 of the slab
-            const int base = (((int)s_img * p.H + R0) * p.W - p.pW) * 256;
-            const int a0 = lrow + R0 * p.Wp;                                // slot - lo
-            const int b0 = (p.H - R0) * p.Wp - 1 - lrow;                    // hi - 1 - slot
+            const int s_u = __builtin_amdgcn_readfirstlane((int)s_img), r_u = __builtin_amdgcn_readfirstlane((int)r_img);
             const unsigned hb = lds_address(&halo[buf][0]), yb = lds_address(&dyb[buf][0]);
 #pragma unroll
-            for (int i = 0; i < NLH; ++i) {
-                const unsigned rowbad = (unsigned)((a0 + 4 * i) | (b0 - 4 * i)) & 0x80000000u;
-                const unsigned colbad = i < 32 ? (colbad_lo << (31 - i)) : (colbad_hi << (63 - i));
-                lds_direct_load16(rsrc_x, hb + (unsigned)i * 1024u,
-                                  (unsigned)(base + relx[i]) | rowbad | (colbad & 0x80000000u));
-            }
-            const int ybase = (((int)s_img * p.Ho + (int)r_img * p.R) * p.Wo) * p.D * 4;
+            for (int r = 0; r < 3; ++r) {
+                if (r < p.fH) {
+                    const int row = r_u - p.pH + r;                         // image row of padded row r
+                    const bool ok = (unsigned)row < (unsigned)p.H;
+                    const unsigned soff = ok ? (unsigned)((s_u * p.H + row) * p.W) * 256u : 0u;
+                    const u32x4 rs = ok ? rsrc_x : rsrc_none;
 #pragma unroll
-            for (int j = 0; j < NLD; ++j)
-                lds_direct_load16(rsrc_y, yb + (unsigned)j * 1024u,
-                                  (unsigned)(ybase + rely[j]) | ((unsigned)rely[j] & 0x80000000u));
+                    for (int g = 0; g < NLR; ++g)
+                        if (g < nlr) load(rs, hb + (unsigned)((r * p.Wp + 4 * g) * 256), voffx[g], soff);
+                }
+            }
+            const unsigned ybase = (unsigned)((s_u * p.Ho + r_u) * p.Wo) * (unsigned)(p.D * 4);
+#pragma unroll
+            for (int j = 0; j < NLD; ++j) load(rsrc_y, yb + (unsigned)j * 1024u, voffy[j], ybase);
         };
         if (nsl > 0) fetch(sl0, 0);
         __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
@@ -3201,8 +3209,8 @@ static __global__ __launch_bounds__(64 * kFhWaves, 1) void wgrad_halo_f32(const 
 
 // Fills the plan of wgrad_halo_f32 and returns the number of workgroups (= splits), or 0 when the
 // kernel does not apply: unit stride, 64 input channels, D a multiple of 4 up to 64, at most 9 taps,
-// an even Wo of 28, 32, 56 or 64 (the built pair counts), fH padded rows of Wo + fW - 1 slots in the
-// halo buffer, and at least 4 output rows per CU (AETHER_WGRAD_HALO=1 drops the last condition, =0 turns
+// an even Wo of 28, 32, 56 or 64 (the built pair counts), at most 3 filter rows of at most 68 padded
+// columns, and at least 4 output rows per CU (AETHER_WGRAD_HALO=1 drops the last condition, =0 turns
 // the kernel off).
 static int plan_wgrad_halo_f32(WgradHaloParams& p, int C, int sH, int sW, int cus) {
     if (sH != 1 || sW != 1 || C != 64 || p.D % 4 != 0 || p.D > 64 || p.fH * p.fW > 9) return 0;
@@ -3214,9 +3222,9 @@ static int plan_wgrad_halo_f32(WgradHaloParams& p, int C, int sH, int sW, int cu
     if (p.Wo != 28 && p.Wo != 32 && p.Wo != 56 && p.Wo != 64) return 0;
     p.R = 1;
     p.slab_m = p.Wo;
-    p.Wp = p.Wo + p.fW - 1;
+    p.Wp = (int)round_up(p.Wo + p.fW - 1, 4);            // row pitch of the halo in LDS: whole loads of 4 slots
     p.hslots = p.fH * p.Wp;
-    if (p.hslots > kFhSlots) return 0;
+    if (p.fH > 3 || p.Wp > kFhRowSlots) return 0;
     const int64_t nslabs = (int64_t)p.S * p.Ho;
     if (nslabs > (1 << 24) || (!force && nslabs < 4 * (int64_t)cus)) return 0;
     // byte offsets are formed in 32 bits from the pixel above and left of the image
