@@ -727,6 +727,240 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
 }
 
 // ------------------------------------------------------------------------------
+// gather_gemm_persist: the uniform-tap, 8-chunk-slab form of gather_gemm_dma for launches of many
+// rounds of tiles.  A one-tile workgroup spends a sixth of its life outside the slab loop (row decode,
+// the first slab's memory latency, the epilogue), and the workgroups that share a CU start together and
+// stay in step, so those gaps reach the matrix pipe.  Here 3 workgroups per CU stay resident and walk
+// tiles; the slab loop runs through the tile boundaries: the last slab of a tile issues the loads of the
+// next tile's first slab, the next tile's row table is worked out by the threads of slab 1 and picked up
+// at the last slab, and a finished tile stays in the accumulators until the next tile's first slab has
+// begun: it is stored there, behind that slab's loads, and the accumulators start again from the bias.  Slab order, operand reads and MFMA order are those of gather_gemm_dma: the
+// results are bit-identical.
+// Round i gives workgroup b the tile i * G + (b's place in an XCD-contiguous order), so that one XCD works
+// on neighbouring image rows at the same time; the last, partial round goes to the first workgroups in
+// launch order, which are spread over all XCDs.
+// ------------------------------------------------------------------------------
+constexpr int kPersistMaxN = 512;
+
+template <typename T, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(kThreads, 3) void gather_gemm_persist(const GatherParams p, const int tiles) {
+    static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
+    constexpr int KC = 8;
+    constexpr int CE = Elem<T>::CE;
+    constexpr int BK = KC * CE;
+    constexpr int RPL = 64 / KC;
+    constexpr int G = KC / 2;
+    constexpr int AL = BM / (4 * RPL);
+    constexpr int BL = BN / (4 * RPL);
+    static_assert(AL >= 2 && AL % 2 == 0 && BL >= 1, "8-row load blocks of a wave alternate even/odd");
+    static_assert(BM <= kThreads, "one thread per row of the table");
+    constexpr int TM = WM / 32;
+    constexpr int TN = WN / 32;
+
+    __shared__ f4 lds_a0[BM * KC];
+    __shared__ f4 lds_a1[BM * KC];
+    __shared__ f4 lds_b0[BN * KC];
+    __shared__ f4 lds_b1[BN * KC];
+    __shared__ int2 rowtab[BM];
+    __shared__ __attribute__((aligned(16))) float lds_bias[kPersistMaxN];   // zeros past N and without a bias
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int l32 = lane & 31;
+    const int lh = lane >> 5;
+    const int wm0 = (wave % (BM / WM)) * WM;
+    const int wn0 = (wave / (BM / WM)) * WN;
+    const int ntile = (p.N + BN - 1) / BN;
+    const int nwg = (int)gridDim.x;
+    const int rounds = tiles / nwg, rest = tiles - rounds * nwg;
+    const int my_count = rounds + ((int)blockIdx.x < rest ? 1 : 0);
+    if (my_count == 0) return;
+    const int lid = xcd_contiguous_id((int)blockIdx.x, nwg);
+    auto tile_of = [&](int i) { return i < rounds ? i * nwg + lid : rounds * nwg + (int)blockIdx.x; };
+
+    const int lr = lane / KC;
+    const int k4e = (lane & 7) ^ (lane >> 4);
+    // (element offset of tap (0,0), one bit per tap that says "outside the image") of row m0 + tid
+    auto decode_rows = [&](int m0) {
+        if (tid < BM) {
+            const int m = m0 + tid;
+            int off = 0, br = kInvalidRow, bc = 0;
+            if (m < p.M) {
+                unsigned s_, rem, ii, jj;
+                p.div_hw.divmod((unsigned)m, s_, rem);
+                p.div_w.divmod(rem, ii, jj);
+                br = (int)ii * p.sh + p.rh0;
+                bc = (int)jj * p.sw + p.rw0;
+                off = (((int)s_ * p.Hs + br) * p.Ws + bc) * p.Cs;
+            }
+            auto span = [](int lo, int hi) -> unsigned {
+                const unsigned upto_hi = hi > 0 ? ~0u >> (32 - hi) : 0u;
+                const unsigned upto_lo = lo > 0 ? ~0u >> (32 - lo) : 0u;
+                return hi > lo ? upto_hi & ~upto_lo : 0u;
+            };
+            const int lo_r = min(max(-br, 0), 32), hi_r = min(max(p.Hs - br, 0), p.Th);
+            const int lo_c = min(max(-bc, 0), 32), hi_c = min(max(p.Ws - bc, 0), p.Tw);
+            const unsigned rmask = span(lo_r, hi_r), cmask = span(lo_c, hi_c);
+            unsigned valid = 0;
+            for (int th = 0; th < p.Th; ++th) valid |= (((rmask >> th) & 1u) ? cmask : 0u) << (th * p.Tw);
+            rowtab[tid] = int2{off, (int)~valid};
+        }
+    };
+    unsigned a_byte[AL], a_inv[AL], b_off[BL];
+    auto take_rows = [&]() {
+#pragma unroll
+        for (int i = 0; i < AL; ++i) {
+            const int2 e = rowtab[(wave * AL + i) * RPL + lr];
+            a_inv[i] = (unsigned)e.y;
+            a_byte[i] = (unsigned)(e.x + CE * (k4e ^ ((i & 1) ? 4 : 0))) * (unsigned)sizeof(T);
+        }
+    };
+    auto set_b_off = [&](int n0) {
+#pragma unroll
+        for (int i = 0; i < BL; ++i) {
+            const int k4 = k4e ^ (((wave * BL + i) & 1) ? 4 : 0);
+            b_off[i] = (unsigned)(((n0 + (wave * BL + i) * RPL + lr) * p.Kpad + CE * k4) * (int)sizeof(T));
+        }
+    };
+    const __amdgpu_buffer_rsrc_t rsrc_a =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.src), 0, (int)p.src_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.bt), 0, (int)p.bt_bytes, 0x00020000);
+
+    unsigned ut_tap = 0, ut_tap_bytes = 0;
+    auto prep = [&](int k0) {
+        unsigned c0, th, tw;
+        p.div_c.divmod((unsigned)k0, ut_tap, c0);
+        p.div_tw.divmod(ut_tap, th, tw);
+        ut_tap_bytes = (unsigned)(((int)th * p.Ws + (int)tw) * p.Cs + (int)c0) * (unsigned)sizeof(T);
+    };
+    auto issue_load = [&](int j, int k0, f4* la, f4* lb) {
+        if (j >= AL) {
+            const int i = j - AL;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(lb + (wave * BL + i) * 64), 16,
+                                                     (int)(b_off[i] + (unsigned)k0 * (unsigned)sizeof(T)), 0, 0, 0);
+            return;
+        }
+        const unsigned bad = (a_inv[j] >> ut_tap) & 1u;
+        const unsigned voff = (a_byte[j] + ut_tap_bytes) | (bad << 31);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(la + (wave * AL + j) * 64), 16, (int)voff, 0, 0, 0);
+    };
+    constexpr int NL = AL + BL;
+    constexpr int LPG = (NL + G - 2) / (G - 1);
+    auto issue_part = [&](int g, int k0, f4* la, f4* lb) {
+#pragma unroll
+        for (int j = g * LPG; j < (g + 1) * LPG && j < NL; ++j) issue_load(j, k0, la, lb);
+    };
+
+    f16v acc[TM][TN];
+    const int sw7 = (l32 >> 1) & (KC - 1);
+    f4 fa[2][TM], fb[2][TN];
+    auto read_frags = [&](const f4* la, const f4* lb, int g, int slot) {
+        const int pc = (2 * g + lh) ^ sw7;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[slot][i] = la[(wm0 + 32 * i + l32) * KC + pc];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[slot][j] = lb[(wn0 + 32 * j + l32) * KC + pc];
+    };
+    auto mma_group = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) mma_chunk<T>(fb[slot][j], fa[slot][i], acc[i][j]);
+    };
+
+    // the first tile: as a one-tile workgroup starts
+    const int nslabs = p.Kpad / BK;
+    int ti = 0, s = 0;
+    int m0, n0;
+    {
+        const int t = tile_of(0);
+        m0 = (t / ntile) * BM;
+        n0 = (t % ntile) * BN;
+    }
+    for (int n = tid; n < kPersistMaxN; n += kThreads) lds_bias[n] = (p.bias != nullptr && n < p.N) ? p.bias[n] : 0.f;
+    decode_rows(m0);
+    __syncthreads();
+    take_rows();
+    set_b_off(n0);
+    prep(0);
+#pragma unroll
+    for (int j = 0; j < NL; ++j) issue_load(j, 0, lds_a0, lds_b0);
+    // a tile's accumulators start from the bias of its channels
+    auto start_acc = [&](int nw0) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const f4 v = *reinterpret_cast<const f4*>(lds_bias + nw0 + 32 * j + 8 * q + 4 * lh);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = v[e];
+            }
+    };
+    int done_m0 = 0, done_n0 = 0;
+    bool have_done = false;
+
+    auto step = [&](const f4* la, const f4* lb, f4* na, f4* nb) __attribute__((always_inline)) {
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        read_frags(la, lb, 0, 0);
+        const bool last = s == nslabs - 1;
+        const bool more_tiles = ti + 1 < my_count;
+        bool has_next = true;
+        int next_k0 = (s + 1) * BK;
+        int nm0 = 0, nn0 = 0;
+        if (last) {
+            next_k0 = 0;
+            has_next = more_tiles;
+            if (more_tiles) {
+                // from here on this wave's loads belong to the next tile
+                const int t = tile_of(ti + 1);
+                nm0 = (t / ntile) * BM;
+                nn0 = (t % ntile) * BN;
+                take_rows();
+                set_b_off(nn0);
+            }
+        }
+        if (has_next) prep(next_k0);
+        if (s == 0) {
+            // the finished tile is still in the accumulators: it is stored here, behind the loads of this
+            // tile's first slab, and the accumulators then start again from the bias
+            if (have_done) store_tile<TM, TN, true>(p, p.out, acc, done_m0 + wm0, done_n0 + wn0, l32, lh);
+            start_acc(n0 + wn0);
+        }
+        if (s == 1 && more_tiles) decode_rows((tile_of(ti + 1) / ntile) * BM);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            if (g < G - 1) read_frags(la, lb, g + 1, (g + 1) & 1);
+            if (has_next && g < G - 1) issue_part(g, next_k0, na, nb);
+            __builtin_amdgcn_sched_barrier(0);
+            mma_group(g & 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (last) {
+            done_m0 = m0;
+            done_n0 = n0;
+            have_done = true;
+            m0 = nm0;
+            n0 = nn0;
+            ++ti;
+            s = 0;
+        } else {
+            ++s;
+        }
+    };
+    const int total = my_count * nslabs;
+    for (int f = 0; f < total; f += 2) {
+        step(lds_a0, lds_b0, lds_a1, lds_b1);
+        if (f + 1 < total) step(lds_a1, lds_b1, lds_a0, lds_b0);
+    }
+    store_tile<TM, TN, true>(p, p.out, acc, done_m0 + wm0, done_n0 + wn0, l32, lh);
+}
+
+// ------------------------------------------------------------------------------
 // gather_halo_bf16: unit-stride gathers with several filter taps on bf16 inputs
 // (3x3 stride-1 fprop, every dgrad class with 2 taps or more).
 // The bf16 MFMAs of a slab take a fifth of the time its LDS-direct loads need to
@@ -1535,6 +1769,24 @@ static bool plan_halo_res(GatherParams& gp, bool dma, int cus, int* mtiles) {
     return true;
 }
 
+// gather_gemm_persist applies to fp32 launches of 128 x 64 tiles whose slabs lie inside one tap (channels
+// in whole slabs of 32, at most 32 taps), with 3 slabs or more, no split of K, 16-byte stores and at most
+// 512 output channels, from 4 rounds of the
+// 3 * cus resident workgroups on (AETHER_GATHER_PERSIST=1 drops the last condition, =0 turns the kernel off).
+static bool plan_persist(const GatherParams& gp, bool dma, int cus, int* tiles) {
+    if (!dma || gp.split_slabs != 0 || gp.Cs % 32 != 0 || gp.K != gp.Kpad || gp.K / gp.Cs > 32 || gp.Kpad / 32 < 3) return false;
+    if (gp.N > kPersistMaxN || gp.out_bytes == 0) return false;
+    bool force = false;
+    if (const char* f = getenv("AETHER_GATHER_PERSIST")) {
+        if (atoi(f) == 0) return false;
+        force = true;
+    }
+    const int64_t n = (int64_t)cdiv(gp.M, 128) * cdiv(gp.N, 64);
+    if (n > (1 << 30) || (!force && n < (int64_t)12 * cus)) return false;
+    *tiles = (int)n;
+    return true;
+}
+
 template <typename T>
 static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t st) {
     const int bn = gather_bn(gp.N);
@@ -1559,6 +1811,16 @@ static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t
         }
     }
     const int bm = gather_bm(gp.M, gp.N, cus, dma, (int)sizeof(T));
+    if constexpr (sizeof(T) == 4) {
+        int tiles = 0;
+        if (bm == 128 && bn == 64 && plan_persist(gp, dma, cus, &tiles)) {
+            int wgs = std::min(tiles, 3 * cus);
+            // AETHER_GATHER_PERSIST_WGS: fewer workgroups, so that small inputs give each of them several tiles
+            if (const char* f = getenv("AETHER_GATHER_PERSIST_WGS")) wgs = std::max(1, std::min(wgs, atoi(f)));
+            hipLaunchKernelGGL((gather_gemm_persist<T, 128, 64, 32, 64>), dim3((unsigned)wgs), dim3(kThreads), 0, st, gp, tiles);
+            return;
+        }
+    }
     // shallow slabs measure the same as deep ones on the 56x56 layers (within 2 % either
     // way), so they stay a tuning switch: AETHER_GATHER_KC=4
     bool kc4 = false;

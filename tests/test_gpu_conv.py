@@ -226,6 +226,43 @@ def test_fprop_with_the_filter_resident_in_lds(case, monkeypatch):
     assert np.array_equal(got, abi.fprop(x, w, b, stride, pad))
 
 
+# fp32 gathers over many rounds of 128 x 64 tiles: three resident workgroups per CU walk the tiles and the
+# slab loop runs through the tile boundaries.  The library takes that kernel from 4 rounds of tiles on;
+# AETHER_GATHER_BM=128 with AETHER_GATHER_PERSIST=1 lets small inputs reach it and
+# AETHER_GATHER_PERSIST_WGS gives a workgroup several tiles.
+PERSIST_CASES = [
+    ((4, 56, 56, 64, 64, 3, 3, 1, 1, "same"), 24),      # 98 tiles on 24 workgroups: 4 each and 2 more
+    ((4, 56, 56, 64, 64, 3, 3, 1, 1, "same"), 1000),    # one tile each
+    ((3, 28, 28, 128, 128, 3, 3, 1, 1, "same"), 7),     # two n tiles per m tile, 36 slabs
+    ((3, 27, 29, 64, 72, 3, 3, 1, 1, "valid"), 5),      # ragged last m tile, 8 channels in the last n tile
+    ((2, 20, 20, 32, 64, 5, 5, 1, 1, "same"), 3),       # 25 taps = 25 slabs: the tiles change LDS buffer parity
+    ((8, 24, 24, 128, 64, 1, 1, 1, 1, "valid"), 9),     # 1x1: 4 slabs
+    ((4, 28, 28, 64, 64, 3, 3, 2, 2, "same"), 2),       # stride 2 (dgrad: four classes of dx, strided output rows)
+    ((2, 40, 40, 96, 64, 3, 3, 1, 1, "same"), 8),       # 3 slabs per tap
+    ((2, 20, 20, 16, 64, 3, 3, 1, 1, "same"), 8),       # 16 channels: the one-tile kernels
+]
+
+
+@pytest.mark.parametrize("case,wgs", PERSIST_CASES, ids=lambda c: "x".join(str(v) for v in c) if isinstance(c, tuple) else "wgs%d" % c)
+def test_fprop_dgrad_with_resident_workgroups_walking_tiles(case, wgs, monkeypatch):
+    from tests import abi
+    monkeypatch.setenv("AETHER_GATHER_BM", "128")
+    monkeypatch.setenv("AETHER_GATHER_PERSIST", "1")
+    monkeypatch.setenv("AETHER_GATHER_PERSIST_WGS", str(wgs))
+    x, w, b, dy = _case(case, 15)
+    stride, pad = (case[7], case[8]), case[9]
+    y = abi.fprop(x, w, b, stride, pad)
+    abi.close(y, O.conv_fprop(x, w, b, stride, pad, dtype=np.float64))
+    y0 = abi.fprop(x, w, None, stride, pad)
+    abi.close(y0, O.conv_fprop(x, w, None, stride, pad, dtype=np.float64))
+    dx = abi.dgrad(dy, w, x.shape, stride, pad)
+    abi.close(dx, O.conv_dgrad(dy, w, x.shape[1:3], stride, pad, dtype=np.float64))
+    # the one-tile kernel adds the same products in the same order
+    monkeypatch.setenv("AETHER_GATHER_PERSIST", "0")
+    assert np.array_equal(y, abi.fprop(x, w, b, stride, pad))
+    assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
+
+
 # fp32 wgrad of a unit-stride filter of at most 9 taps on 64 input channels and at most 64 output
 # channels, on rows of 28, 32, 56 or 64 output pixels: one persistent workgroup per CU keeps the whole
 # K x N result in registers (12 multiplying waves of three 32 x 32 blocks) and a loading wave brings one
