@@ -226,10 +226,9 @@ def test_fprop_with_the_filter_resident_in_lds(case, monkeypatch):
     assert np.array_equal(got, abi.fprop(x, w, b, stride, pad))
 
 
-# fp32 gathers over many rounds of 128 x 64 tiles: three resident workgroups per CU walk the tiles and the
-# slab loop runs through the tile boundaries.  The library takes that kernel from 4 rounds of tiles on;
-# AETHER_GATHER_BM=128 with AETHER_GATHER_PERSIST=1 lets small inputs reach it and
-# AETHER_GATHER_PERSIST_WGS gives a workgroup several tiles.
+# fp32 gathers as resident workgroups that walk 128 x 64 tiles, the slab loop running through the tile
+# boundaries.  The kernel is a tuning switch (AETHER_GATHER_PERSIST=1, with AETHER_GATHER_BM=128 for
+# inputs that would get other tiles); AETHER_GATHER_PERSIST_WGS gives a workgroup several tiles.
 PERSIST_CASES = [
     ((4, 56, 56, 64, 64, 3, 3, 1, 1, "same"), 24),      # 98 tiles on 24 workgroups: 4 each and 2 more
     ((4, 56, 56, 64, 64, 3, 3, 1, 1, "same"), 1000),    # one tile each
