@@ -385,6 +385,45 @@ __global__ __launch_bounds__(kThreads, 3) void gather_gemm(const GatherParams p)
 // ------------------------------------------------------------------------------
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
+// A 16-byte-per-lane LDS-direct load the compiler does not see as one.  It orders every LDS
+// read behind the LDS-direct loads it knows to be in flight unless it can prove where they
+// land, and with a ring of buffers in a loop it cannot: the reads of a step then wait for the
+// slabs fetched for later steps.  The caller waits (vmcnt + barrier) before reading what a
+// load brings.  lds_base: wave-uniform LDS byte address; the lanes land at lds_base + 16 * lane.
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void lds_direct_load16(const u32x4& rsrc, unsigned lds_base, unsigned voff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :: "s"(lds_base), "v"(voff), "s"(rsrc) : "memory", "m0");
+}
+// the same with a scalar byte offset added to every lane's (the range check looks at `voff` alone)
+__device__ __forceinline__ void lds_direct_load16_s(const u32x4& rsrc, unsigned lds_base, unsigned voff, unsigned soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
+}
+__device__ __forceinline__ u32x4 raw_rsrc(const void* base, unsigned bytes) {
+    const unsigned long long a = reinterpret_cast<unsigned long long>(base);
+    return u32x4{(unsigned)a, (unsigned)(a >> 32) & 0xffffu, bytes, 0x00020000u};
+}
+__device__ __forceinline__ unsigned lds_address(const void* q) {
+    return (unsigned)reinterpret_cast<uintptr_t>((lds_ptr_t)const_cast<void*>(q));
+}
+
+// bit b of an 8-bit wave-uniform mask to lanes 8b .. 8b+7, on the scalar unit
+__device__ __forceinline__ unsigned long long spread8(unsigned m8) {
+    unsigned long long r;
+    asm("s_bitreplicate_b64_b32 %0, %1" : "=s"(r) : "s"(m8));
+    asm("s_bitreplicate_b64_b32 %0, %1" : "=s"(r) : "s"((unsigned)r));
+    asm("s_bitreplicate_b64_b32 %0, %1" : "=s"(r) : "s"((unsigned)r));
+    return r;
+}
+// lane l gets b where bit l of the wave-uniform mask is set, else a
+__device__ __forceinline__ unsigned select_by_mask(unsigned a, unsigned b, unsigned long long mask) {
+    unsigned v;
+    asm("v_cndmask_b32 %0, %1, %2, %3" : "=v"(v) : "v"(a), "v"(b), "s"(mask));
+    return v;
+}
+
+
 //   * UT ("uniform tap"): when the channel count is a multiple of the slab width and
 //     the filter has at most 32 taps, a slab lies inside one tap.  fp32 MFMA shares
 //     the FP32 lanes with ordinary vector instructions, so every address instruction
@@ -400,9 +439,18 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 //     channels: the HBM-bound case, where a one-tile workgroup is mostly set-up).  The
 //     workgroup keeps its A tile, both slabs, in the two A buffers and walks over all n
 //     tiles: one set-up and one fetch of A per m tile instead of one per output tile.
-template <typename T, int BM, int BN, int WM, int WN, bool UT, int KC, bool NLOOP>
+//   * SA ("scalar addressing", uniform-tap fp32 tiles of 128 rows with at most 9 taps): the loads of the slab
+//     loop use no vector instruction at all.  A lane's offset is a constant of the tile (its row's tap (0,0)
+//     plus its chunk, from a base moved down by the padding so that it is never negative: the range check
+//     looks at the vector offset alone), the tap and the channel block go into the scalar offset, and what
+//     lies outside the image at the slab's tap is one ballot per slab over the wave's 32 rows: a load whose
+//     8 rows are all inside, nearly all of them, is issued as it is; else the 8 bits are spread over the
+//     lanes on the scalar unit and one v_cndmask sends the outside lanes beyond the descriptor.
+
+template <typename T, int BM, int BN, int WM, int WN, bool UT, int KC, bool NLOOP, bool SA = false>
 __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p) {
     static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
+    static_assert(!SA || (UT && KC == 8 && !NLOOP && BM == 128 && sizeof(T) == 4), "scalar addressing: the fp32 128-row uniform-tap tile");
     static_assert(KC == 8 || KC == 4, "slab rows of 8 or 4 chunks");
     constexpr int CE = Elem<T>::CE;
     constexpr int BK = KC * CE;          // elements of k per slab
@@ -494,6 +542,20 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
         a_inv[i] = (unsigned)e.y;
         a_byte[i] = (unsigned)(e.x + CE * (k4e ^ ((i & 1) ? ODD : 0))) * (unsigned)sizeof(T);
     }
+    // SA: lane l (and l + 32) keeps the outside-the-image bits, one per tap, of row 32 * wave + l; a ballot
+    // over the slab's tap bit gives the 32 rows' mask in a scalar register (three vector instructions per
+    // slab; nine masks held in scalar registers and selected by the tap made the compiler keep the
+    // kernel's whole state in memory)
+    unsigned aux_row = 0, cur_mask = 0;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const unsigned sa_bias = SA ? (unsigned)((max(-p.rh0, 0) * p.Ws + max(-p.rw0, 0)) * p.Cs) * (unsigned)sizeof(T) : 0u;
+    if constexpr (SA) {
+        aux_row = (unsigned)rowtab[wave * (AL * RPL) + (lane & 31)].y;
+#pragma unroll
+        for (int i = 0; i < AL; ++i) a_byte[i] += sa_bias;
+    }
+    const u32x4 sa_rsrc_a = raw_rsrc(static_cast<const char*>(p.src) - sa_bias, (unsigned)p.src_bytes + sa_bias);
+    const u32x4 sa_rsrc_b = raw_rsrc(p.bt, (unsigned)p.bt_bytes);
     unsigned b_off[BL];
     auto set_b_off = [&]() {
 #pragma unroll
@@ -523,6 +585,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
             p.div_c.divmod((unsigned)k0, ut_tap, c0);
             p.div_tw.divmod(ut_tap, th, tw);
             ut_tap_bytes = (unsigned)(((int)th * p.Ws + (int)tw) * p.Cs + (int)c0) * (unsigned)sizeof(T);
+            if constexpr (SA) cur_mask = (unsigned)__builtin_amdgcn_ballot_w64(((aux_row >> ut_tap) & 1u) != 0u);
             return;
         }
         // tap decode for the two chunk columns a lane serves (even / odd 8-row blocks)
@@ -539,6 +602,19 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
         }
     };
     auto issue_load = [&](int j, int k0, f4* la, f4* lb) {
+        if constexpr (SA) {
+            if (j >= AL) {
+                const int i = j - AL;
+                lds_direct_load16_s(sa_rsrc_b, lds_address(lb) + (unsigned)(wave_u * BL + i) * 1024u, b_off[i],
+                                    (unsigned)k0 * (unsigned)sizeof(T));
+                return;
+            }
+            const unsigned m8 = (cur_mask >> (8 * j)) & 0xffu;
+            const unsigned dst = lds_address(la) + (unsigned)(wave_u * AL + j) * 1024u;
+            if (m8 != 0u) lds_direct_load16_s(sa_rsrc_a, dst, select_by_mask(a_byte[j], 0x80000000u, spread8(m8)), ut_tap_bytes);
+            else lds_direct_load16_s(sa_rsrc_a, dst, a_byte[j], ut_tap_bytes);
+            return;
+        }
         if (j >= AL) {
             const int i = j - AL;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(lb + (wave * BL + i) * 64), 16,
@@ -987,24 +1063,6 @@ __global__ __launch_bounds__(kThreads, 3) void gather_gemm_persist(const GatherP
 //     slab rows of gather_gemm_dma: 16 consecutive pixels cover the 64 banks once;
 //   * channel blocks beyond the first reload the halo (Cs = 64 j: j passes over the taps).
 // ------------------------------------------------------------------------------
-// A 16-byte-per-lane LDS-direct load the compiler does not see as one.  It orders every LDS
-// read behind the LDS-direct loads it knows to be in flight unless it can prove where they
-// land, and with a ring of buffers in a loop it cannot: the reads of a step then wait for the
-// slabs fetched for later steps.  The caller waits (vmcnt + barrier) before reading what a
-// load brings.  lds_base: wave-uniform LDS byte address; the lanes land at lds_base + 16 * lane.
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ void lds_direct_load16(const u32x4& rsrc, unsigned lds_base, unsigned voff) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                 :: "s"(lds_base), "v"(voff), "s"(rsrc) : "memory", "m0");
-}
-__device__ __forceinline__ u32x4 raw_rsrc(const void* base, unsigned bytes) {
-    const unsigned long long a = reinterpret_cast<unsigned long long>(base);
-    return u32x4{(unsigned)a, (unsigned)(a >> 32) & 0xffffu, bytes, 0x00020000u};
-}
-__device__ __forceinline__ unsigned lds_address(const void* q) {
-    return (unsigned)reinterpret_cast<uintptr_t>((lds_ptr_t)const_cast<void*>(q));
-}
-
 // STAGES ring buffers of 8 KB and the rest of 80 KB (two workgroups per CU) for the halo:
 // 4 stages (three taps ahead) and 384 slots where every span fits that, else 3 and 448
 // (56x56x64: 0.098 ms with 4 stages, 0.102 with 3).
@@ -1632,6 +1690,16 @@ static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
             grid.x = (unsigned)cdiv(gp.M, BM);
             if (ut) hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, true>), grid, dim3(kThreads), 0, st, gp);
             else hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, false, KC, true>), grid, dim3(kThreads), 0, st, gp);
+            return;
+        }
+    }
+    if constexpr (BM == 128 && KC == 8 && sizeof(T) == 4) {
+        // scalar addressing (AETHER_GATHER_SA=0 turns it off); the moved base must stay a 32-bit extent
+        const int taps = gp.Cs > 0 ? gp.K / gp.Cs : 0;
+        const int64_t bias = ((int64_t)std::max(-gp.rh0, 0) * gp.Ws + std::max(-gp.rw0, 0)) * gp.Cs * (int64_t)sizeof(T);
+        const char* f = getenv("AETHER_GATHER_SA");
+        if (ut && taps <= 32 && (int64_t)gp.src_bytes + bias < ((int64_t)1 << 31) && (f == nullptr || atoi(f) != 0)) {
+            hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, true>), grid, dim3(kThreads), 0, st, gp);
             return;
         }
     }
