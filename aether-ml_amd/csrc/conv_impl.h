@@ -439,18 +439,18 @@ __device__ __forceinline__ unsigned select_by_mask(unsigned a, unsigned b, unsig
 //     channels: the HBM-bound case, where a one-tile workgroup is mostly set-up).  The
 //     workgroup keeps its A tile, both slabs, in the two A buffers and walks over all n
 //     tiles: one set-up and one fetch of A per m tile instead of one per output tile.
-//   * SA ("scalar addressing", uniform-tap fp32 tiles of 128 rows with at most 9 taps): the loads of the slab
+//   * SA ("scalar addressing", uniform-tap fp32 tiles of 64 or 128 rows): the loads of the slab
 //     loop use no vector instruction at all.  A lane's offset is a constant of the tile (its row's tap (0,0)
 //     plus its chunk, from a base moved down by the padding so that it is never negative: the range check
 //     looks at the vector offset alone), the tap and the channel block go into the scalar offset, and what
-//     lies outside the image at the slab's tap is one ballot per slab over the wave's 32 rows: a load whose
+//     lies outside the image at the slab's tap is one ballot per slab over the wave's 16 or 32 rows: a load whose
 //     8 rows are all inside, nearly all of them, is issued as it is; else the 8 bits are spread over the
 //     lanes on the scalar unit and one v_cndmask sends the outside lanes beyond the descriptor.
 
 template <typename T, int BM, int BN, int WM, int WN, bool UT, int KC, bool NLOOP, bool SA = false>
 __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p) {
     static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
-    static_assert(!SA || (UT && KC == 8 && !NLOOP && BM == 128 && sizeof(T) == 4), "scalar addressing: the fp32 128-row uniform-tap tile");
+    static_assert(!SA || (UT && KC == 8 && !NLOOP && (BM == 128 || BM == 64) && sizeof(T) == 4), "scalar addressing: fp32 uniform-tap tiles of 64 or 128 rows");
     static_assert(KC == 8 || KC == 4, "slab rows of 8 or 4 chunks");
     constexpr int CE = Elem<T>::CE;
     constexpr int BK = KC * CE;          // elements of k per slab
@@ -542,15 +542,15 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
         a_inv[i] = (unsigned)e.y;
         a_byte[i] = (unsigned)(e.x + CE * (k4e ^ ((i & 1) ? ODD : 0))) * (unsigned)sizeof(T);
     }
-    // SA: lane l (and l + 32) keeps the outside-the-image bits, one per tap, of row 32 * wave + l; a ballot
-    // over the slab's tap bit gives the 32 rows' mask in a scalar register (three vector instructions per
+    // SA: lane l keeps the outside-the-image bits, one per tap, of the wave's row l (modulo its 32 or 16 rows);
+    // a ballot over the slab's tap bit gives the rows' mask in a scalar register (three vector instructions per
     // slab; nine masks held in scalar registers and selected by the tap made the compiler keep the
     // kernel's whole state in memory)
     unsigned aux_row = 0, cur_mask = 0;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const unsigned sa_bias = SA ? (unsigned)((max(-p.rh0, 0) * p.Ws + max(-p.rw0, 0)) * p.Cs) * (unsigned)sizeof(T) : 0u;
     if constexpr (SA) {
-        aux_row = (unsigned)rowtab[wave * (AL * RPL) + (lane & 31)].y;
+        aux_row = (unsigned)rowtab[wave * (AL * RPL) + (lane & (AL * RPL - 1))].y;
 #pragma unroll
         for (int i = 0; i < AL; ++i) a_byte[i] += sa_bias;
     }
@@ -1693,7 +1693,7 @@ static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
             return;
         }
     }
-    if constexpr (BM == 128 && KC == 8 && sizeof(T) == 4) {
+    if constexpr ((BM == 128 || BM == 64) && KC == 8 && sizeof(T) == 4) {
         // scalar addressing (AETHER_GATHER_SA=0 turns it off); the moved base must stay a 32-bit extent
         const int taps = gp.Cs > 0 ? gp.K / gp.Cs : 0;
         const int64_t bias = ((int64_t)std::max(-gp.rh0, 0) * gp.Ws + std::max(-gp.rw0, 0)) * gp.Cs * (int64_t)sizeof(T);
