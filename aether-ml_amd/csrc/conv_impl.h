@@ -408,12 +408,14 @@ __device__ __forceinline__ unsigned lds_address(const void* q) {
     return (unsigned)reinterpret_cast<uintptr_t>((lds_ptr_t)const_cast<void*>(q));
 }
 
-// bit b of an 8-bit wave-uniform mask to lanes 8b .. 8b+7, on the scalar unit
-__device__ __forceinline__ unsigned long long spread8(unsigned m8) {
+// bit b of a wave-uniform mask of 64 / LANES bits to lanes LANES * b .. LANES * b + LANES - 1, on the scalar unit
+template <int LANES>
+__device__ __forceinline__ unsigned long long spread_rows(unsigned m) {
+    static_assert(LANES == 8 || LANES == 4, "8 or 4 lanes per row");
     unsigned long long r;
-    asm("s_bitreplicate_b64_b32 %0, %1" : "=s"(r) : "s"(m8));
+    asm("s_bitreplicate_b64_b32 %0, %1" : "=s"(r) : "s"(m));
     asm("s_bitreplicate_b64_b32 %0, %1" : "=s"(r) : "s"((unsigned)r));
-    asm("s_bitreplicate_b64_b32 %0, %1" : "=s"(r) : "s"((unsigned)r));
+    if (LANES == 8) asm("s_bitreplicate_b64_b32 %0, %1" : "=s"(r) : "s"((unsigned)r));
     return r;
 }
 // lane l gets b where bit l of the wave-uniform mask is set, else a
@@ -450,7 +452,7 @@ __device__ __forceinline__ unsigned select_by_mask(unsigned a, unsigned b, unsig
 template <typename T, int BM, int BN, int WM, int WN, bool UT, int KC, bool NLOOP, bool SA = false>
 __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p) {
     static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
-    static_assert(!SA || (UT && KC == 8 && !NLOOP && (BM == 128 || BM == 64) && sizeof(T) == 4), "scalar addressing: fp32 uniform-tap tiles of 64 or 128 rows");
+    static_assert(!SA || (UT && !NLOOP && (BM == 128 || BM == 64) && sizeof(T) == 4), "scalar addressing: fp32 uniform-tap tiles of 64 or 128 rows");
     static_assert(KC == 8 || KC == 4, "slab rows of 8 or 4 chunks");
     constexpr int CE = Elem<T>::CE;
     constexpr int BK = KC * CE;          // elements of k per slab
@@ -609,9 +611,10 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
                                     (unsigned)k0 * (unsigned)sizeof(T));
                 return;
             }
-            const unsigned m8 = (cur_mask >> (8 * j)) & 0xffu;
+            // the load's 8 (16 with half-depth slabs) rows of the mask, a bit per row
+            const unsigned m8 = (cur_mask >> (RPL * j)) & ((1u << RPL) - 1u);
             const unsigned dst = lds_address(la) + (unsigned)(wave_u * AL + j) * 1024u;
-            if (m8 != 0u) lds_direct_load16_s(sa_rsrc_a, dst, select_by_mask(a_byte[j], 0x80000000u, spread8(m8)), ut_tap_bytes);
+            if (m8 != 0u) lds_direct_load16_s(sa_rsrc_a, dst, select_by_mask(a_byte[j], 0x80000000u, spread_rows<KC>(m8)), ut_tap_bytes);
             else lds_direct_load16_s(sa_rsrc_a, dst, a_byte[j], ut_tap_bytes);
             return;
         }
@@ -680,12 +683,30 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             if (g < G - 1) read_frags(la, lb, g + 1, (g + 1) & 1);
-            if (has_next && g < G - 1) issue_part(g, next_k0, na, nb);
-            // keep the prefetch ahead of the MFMAs (the scheduler would otherwise sink
-            // the reads next to their first use and expose the LDS latency)
-            __builtin_amdgcn_sched_barrier(0);
-            mma_group(g & 1);
-            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (SA && TM * TN * (G - 1) >= NL) {
+                // one load in front of each run of 4 MFMAs; consecutive MFMAs go to different accumulator blocks
+                __builtin_amdgcn_sched_barrier(0);
+                static_assert(TM * TN == 2 || TM * TN == 1 || TM * TN == 4, "blocks per wave");
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int c = g * TM * TN + (t * TM * TN) / 4;
+                    if (has_next && c < NL && (t * TM * TN) % 4 == 0) issue_load(c, next_k0, na, nb);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[g & 1][j][t], fa[g & 1][i][t], acc[i][j], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+                if (has_next && g < G - 1) issue_part(g, next_k0, na, nb);
+                // keep the prefetch ahead of the MFMAs (the scheduler would otherwise sink
+                // the reads next to their first use and expose the LDS latency)
+                __builtin_amdgcn_sched_barrier(0);
+                mma_group(g & 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
     };
 
@@ -1693,7 +1714,7 @@ static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
             return;
         }
     }
-    if constexpr ((BM == 128 || BM == 64) && KC == 8 && sizeof(T) == 4) {
+    if constexpr ((BM == 128 || BM == 64) && sizeof(T) == 4) {
         // scalar addressing (AETHER_GATHER_SA=0 turns it off); the moved base must stay a 32-bit extent
         const int taps = gp.Cs > 0 ? gp.K / gp.Cs : 0;
         const int64_t bias = ((int64_t)std::max(-gp.rh0, 0) * gp.Ws + std::max(-gp.rw0, 0)) * gp.Cs * (int64_t)sizeof(T);
