@@ -480,8 +480,11 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
     const int wn0 = (wave / (BM / WM)) * WN;
     const int ntile = (p.N + BN - 1) / BN;
     const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
-    const int m0 = NLOOP ? lid * BM : (lid / ntile) * BM;
-    int n0 = NLOOP ? 0 : (lid % ntile) * BN;
+    // (one n tile: no division; the compiler divides scalars by way of the vector unit's reciprocal, some 20
+    // vector instructions that a workgroup starting next to busy ones waits for one by one)
+    const int mt = (NLOOP || ntile == 1) ? lid : lid / ntile;
+    const int m0 = mt * BM;
+    int n0 = (NLOOP || ntile == 1) ? 0 : (lid - mt * ntile) * BN;
 
     // The bias is fetched first: its latency passes behind the row decode.
     const int split = (int)blockIdx.y;
