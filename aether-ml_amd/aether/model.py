@@ -37,6 +37,54 @@ class _ArrayOnlyUnpickler(pickle.Unpickler):
         raise pickle.UnpicklingError("parameter files may only contain NumPy arrays (found %s.%s)" % (module, name))
 
 
+def _cupy_array(a):
+    """Stands for `cupy._core.core.array` in parameter files written for the reference's CuPy model."""
+    raise RuntimeError("a marker for the pickler, never called")
+
+
+class _CupyWrapped:
+    """Pickles as `cupy._core.core.array(ndarray)`, which is how the reference's CuPy model's
+    `save_parameters` stores an array (CNN/models/CNN_model_cupy.py:320-323 pickles
+    `get_parameters()`, a list of tuples of cupy arrays)."""
+
+    def __init__(self, a):
+        self.a = a
+
+    def __reduce__(self):
+        return (_cupy_array, (self.a,))
+
+
+class _CupyStylePickler(pickle._Pickler):
+    """The pure-Python pickler with one global written under another name: cupy is not importable
+    here, and the stock pickler refuses a global it cannot import."""
+
+    def save_global(self, obj, name=None):
+        if obj is _cupy_array:
+            self.save("cupy._core.core")
+            self.save("array")
+            self.write(pickle.STACK_GLOBAL)
+            self.memoize(obj)
+            return
+        super().save_global(obj, name)
+
+    dispatch = dict(pickle._Pickler.dispatch)
+    dispatch[type(_cupy_array)] = save_global
+
+
+def write_parameters(params, path, cupy_arrays=False):
+    """Writes a list of per-layer tuples of host arrays as the reference's parameter files are
+    written: pickle protocol 4 of the list.  With `cupy_arrays` every array is stored as
+    `cupy._core.core.array(ndarray)`, so that the reference's CuPy model can `load_parameters`
+    the file (its checkpoints under CNN/saved_models have exactly this stream); without, as plain
+    NumPy arrays, which `pickle.load` reads anywhere."""
+    host = [tuple(np.ascontiguousarray(a) for a in tup) for tup in params]
+    with open(path, 'wb') as f:
+        if cupy_arrays:
+            _CupyStylePickler(f, protocol=4).dump([tuple(_CupyWrapped(a) for a in tup) for tup in host])
+        else:
+            pickle.dump(host, f, protocol=4)
+
+
 class Model:
     def __init__(self):
         self.layers = []
@@ -317,10 +365,8 @@ class Model:
         for parameter_set, layer in zip(parameters, self.trainable_layers):
             layer.set_parameters(*parameter_set)
 
-    def save_parameters(self, path):
-        host = [tuple(np.asarray(a) for a in tup) for tup in self.get_parameters()]
-        with open(path, 'wb') as f:
-            pickle.dump(host, f)
+    def save_parameters(self, path, cupy_arrays=False):
+        write_parameters([tuple(np.asarray(a) for a in tup) for tup in self.get_parameters()], path, cupy_arrays)
 
     def load_parameters(self, path):
         with open(path, 'rb') as f:

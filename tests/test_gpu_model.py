@@ -162,6 +162,15 @@ def test_train_prints_reference_format_and_parameters_round_trip(tmp_path, capsy
     assert other.layers[0].weights is other.layers[0].filter_weights
     after = other.predict(X)
     assert np.array_equal(before, after)
+    # the same through a file written the way the reference's CuPy model writes its checkpoints
+    path2 = str(tmp_path / "params_cupy.pkl")
+    model.save_parameters(path2, cupy_arrays=True)
+    assert b"cupy._core.core" in open(path2, "rb").read()
+    np.random.seed(5)
+    third = build_model(aether, hw=16)
+    third.forward(X[:4], training=False)
+    third.load_parameters(path2)
+    assert np.array_equal(before, third.predict(X))
     with pytest.raises(Exception):
         bad = tmp_path / "bad.pkl"
         import pickle
