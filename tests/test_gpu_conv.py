@@ -226,6 +226,39 @@ def test_fprop_with_the_filter_resident_in_lds(case, monkeypatch):
     assert np.array_equal(got, abi.fprop(x, w, b, stride, pad))
 
 
+# fp32 gathers whose slabs lie inside one tap load with addresses made on the scalar unit: lane offsets
+# that are constants of the tile, counted from a base the padding below the tensor, the tap in the scalar
+# offset, rows outside the image told by one ballot per slab.  AETHER_GATHER_SA=0 is the form with vector
+# address arithmetic; both must give the same bits.
+SA_CASES = [
+    (2, 12, 12, 32, 64, 5, 5, 1, 1, "same"),      # padding 2: the base lies 2 rows and 2 pixels below the tensor
+    (1, 9, 9, 64, 64, 3, 3, 1, 1, "same"),        # one small image: most rows of a tile touch a border
+    (3, 10, 14, 32, 40, 1, 3, 1, 1, "same"),      # fH = 1: no padding at all under the reference's rule, columns run out
+    (3, 10, 14, 32, 40, 3, 1, 1, 1, "same"),      # padding 1 on both axes with a filter one pixel wide
+    (2, 17, 17, 64, 64, 3, 3, 2, 2, "same"),      # stride 2
+    (2, 16, 16, 96, 72, 3, 3, 1, 1, "valid"),     # 3 slabs per tap, ragged n tile, no padding
+    (5, 7, 7, 128, 128, 3, 3, 1, 1, "same"),      # 245 rows: tiles run over image boundaries
+    (2, 13, 11, 32, 64, 4, 4, 1, 1, "same"),      # even filter: padding 1, the last taps run out at the far side
+]
+
+
+@pytest.mark.parametrize("bm", ["64", "128"])
+@pytest.mark.parametrize("case", SA_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_fprop_dgrad_with_scalar_addressed_loads(case, bm, monkeypatch):
+    from tests import abi
+    monkeypatch.setenv("AETHER_GATHER_BM", bm)
+    monkeypatch.setenv("AETHER_GATHER_SPLIT_OFF", "1")
+    x, w, b, dy = _case(case, 16)
+    stride, pad = (case[7], case[8]), case[9]
+    y = abi.fprop(x, w, b, stride, pad)
+    abi.close(y, O.conv_fprop(x, w, b, stride, pad, dtype=np.float64))
+    dx = abi.dgrad(dy, w, x.shape, stride, pad)
+    abi.close(dx, O.conv_dgrad(dy, w, x.shape[1:3], stride, pad, dtype=np.float64))
+    monkeypatch.setenv("AETHER_GATHER_SA", "0")
+    assert np.array_equal(y, abi.fprop(x, w, b, stride, pad))
+    assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
+
+
 # fp32 gathers as resident workgroups that walk 128 x 64 tiles, the slab loop running through the tile
 # boundaries.  The kernel is a tuning switch (AETHER_GATHER_PERSIST=1, with AETHER_GATHER_BM=128 for
 # inputs that would get other tiles); AETHER_GATHER_PERSIST_WGS gives a workgroup several tiles.
