@@ -450,8 +450,10 @@ __device__ __forceinline__ unsigned select_by_mask(unsigned a, unsigned b, unsig
 //     lanes on the scalar unit and one v_cndmask sends the outside lanes beyond the descriptor.
 
 template <typename T, int BM, int BN, int WM, int WN, bool UT, int KC, bool NLOOP, bool SA = false>
-__global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p) {
-    static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
+__global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(const GatherParams p) {
+    // 4 waves, or 8 for the widest bf16 tiles (256 x 128 and 256 x 256: one workgroup per CU)
+    constexpr int NW = (BM / WM) * (BN / WN);
+    static_assert(NW == 4 || (NW == 8 && !NLOOP && !SA), "4 or 8 waves per workgroup");
     static_assert(!SA || (UT && !NLOOP && (BM == 128 || BM == 64) && sizeof(T) == 4), "scalar addressing: fp32 uniform-tap tiles of 64 or 128 rows");
     static_assert(KC == 8 || KC == 4, "slab rows of 8 or 4 chunks");
     constexpr int CE = Elem<T>::CE;
@@ -459,9 +461,9 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
     constexpr int RPL = 64 / KC;         // slab rows per wave-level load
     constexpr int SH = KC == 8 ? 1 : 2;  // swizzle: chunk position = chunk ^ ((row >> SH) & (KC - 1))
     constexpr int G = KC / 2;            // MFMA groups per slab (one 16-byte chunk per lane half each)
-    constexpr int AL = BM / (4 * RPL);   // wave-level A loads per wave per slab
-    constexpr int BL = BN / (4 * RPL);
-    static_assert(AL >= 1 && BL >= 1 && BM % (4 * RPL) == 0 && BN % (4 * RPL) == 0, "tile too small for KC");
+    constexpr int AL = BM / (NW * RPL);  // wave-level A loads per wave per slab
+    constexpr int BL = BN / (NW * RPL);
+    static_assert(AL >= 1 && BL >= 1 && BM % (NW * RPL) == 0 && BN % (NW * RPL) == 0, "tile too small for KC");
     static_assert(KC == 4 || AL % 2 == 0, "8-row load blocks of a wave alternate even/odd");
     constexpr int TM = WM / 32;
     constexpr int TN = WN / 32;
@@ -504,7 +506,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_dma(const GatherParams p
     // that says "outside the image" (all ones for rows past M), else (row << 16 | column).
     // The table sits in the second B buffer, which is first written after the first
     // barrier of the K loop.
-    static_assert(BM <= kThreads && BM * sizeof(int2) <= BN * KC * sizeof(f4), "row table fits the B buffer");
+    static_assert(BM <= 64 * NW && BM * sizeof(int2) <= BN * KC * sizeof(f4), "row table fits the B buffer");
     int2* rowtab = reinterpret_cast<int2*>(lds_b1);
     if (tid < BM) {
         const int m = m0 + tid;
@@ -1718,6 +1720,7 @@ __global__ void pack_filter(const PackParams p) {
 
 template <typename T, int BM, int BN, int WM, int WN, int KC>
 static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
+    constexpr int kThreads = 64 * (BM / WM) * (BN / WN);     // of this tile shape (shadows the 256 of the others)
     dim3 grid(cdiv(gp.M, BM) * cdiv(gp.N, BN));
     if (gp.split_slabs > 0) grid.y = (unsigned)cdiv(gp.Kpad / (KC * Elem<T>::CE), gp.split_slabs);
     const bool ut = gp.Cs % (KC * Elem<T>::CE) == 0 && gp.K == gp.Kpad && gp.K / gp.Cs <= 32;
@@ -1910,6 +1913,27 @@ static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t
             if (stages == 4) hipLaunchKernelGGL(gather_halo_bf16<4>, grid, dim3(kThreads), 0, st, hp);
             else hipLaunchKernelGGL(gather_halo_bf16<3>, grid, dim3(kThreads), 0, st, hp);
             return;
+        }
+    }
+    if constexpr (sizeof(T) == 2) {
+        // Wide tiles for bf16 launches that the halo kernels do not take (strides, 1x1, long filters): the
+        // slab kernel with 256 x 64 tiles fetches (256 + 64) rows of k per 256 x 64 outputs, 11.5 TB/s from
+        // L2 on the 28x28x128 -> 256 stride-2 layer, and that rate is what bounds it; 256 x 256 tiles on 8 waves
+        // (one workgroup per CU, 128 KB of slabs) fetch 2.5 times less per output, 256 x 128 tiles 1.7 times.
+        // From 2 (256 wide) or 4 (128 wide) tiles per CU on (AETHER_GATHER_WIDE=1: always, =0: never).
+        const char* f = getenv("AETHER_GATHER_WIDE");
+        const bool force = f != nullptr && atoi(f) != 0;
+        if (dma && gp.split_slabs == 0 && !(f != nullptr && atoi(f) == 0)) {
+            const int64_t mt = cdiv(gp.M, 256);
+            if (gp.N > 192 && (force || mt * cdiv(gp.N, 256) >= 2 * (int64_t)cus)) {
+                launch_gather_dma<T, 256, 256, 64, 128, 8>(gp, st);
+                return;
+            }
+            // (the stride-2 layer's dgrad classes, 784 tiles of 1 to 4 taps each, are 4 % slower on them)
+            if (gp.N > 64 && (force || mt * cdiv(gp.N, 128) >= 4 * (int64_t)cus)) {
+                launch_gather_dma<T, 256, 128, 64, 64, 8>(gp, st);
+                return;
+            }
         }
     }
     if constexpr (sizeof(T) == 4) {

@@ -208,6 +208,37 @@ def test_bf16_fprop_dgrad_with_the_filter_resident_in_lds(case, monkeypatch):
     abi.close(abi.fprop_bf16(x, w, b, stride, pad), got, rtol=1e-5, atol=1e-5)
 
 
+# bf16 launches outside the halo kernels (strides, 1x1, more than 64 channels in) with more than 64 output
+# channels use tiles of 256 x 128 or 256 x 256 on 8 waves.  The library takes them from 2 tiles per CU on;
+# AETHER_GATHER_WIDE=1 lets small inputs reach them, =0 gives the 4-wave tiles: the same sums in the same order.
+WIDE_CASES = [
+    (4, 28, 28, 128, 256, 3, 3, 2, 2, "valid"),   # the stride-2 layer: 256 x 256 tiles; dgrad: 256 x 128 per class
+    (3, 15, 15, 64, 200, 3, 3, 2, 2, "same"),     # ragged n tile of 256 (channels 200 .. 255 read as zero)
+    (2, 20, 20, 96, 128, 1, 1, 1, 1, "valid"),    # 1x1, 96 channels: K is not a whole slab
+    (5, 9, 11, 128, 100, 3, 3, 1, 1, "same"),     # unit stride on 128 channels: 256 x 128 tiles, rows past M
+    (2, 12, 12, 48, 192, 5, 5, 1, 1, "same"),     # 25 taps of 48 channels: slabs run over tap boundaries
+    (300, 1, 1, 512, 160, 1, 1, 1, 1, "valid"),   # a dense layer: two n tiles of 128, the second of 32
+]
+
+
+@pytest.mark.parametrize("case", WIDE_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_bf16_fprop_dgrad_with_wide_tiles_on_eight_waves(case, monkeypatch):
+    from tests import abi
+    monkeypatch.setenv("AETHER_GATHER_SPLIT_OFF", "1")
+    monkeypatch.setenv("AETHER_GATHER_WIDE", "1")
+    x, w, b, dy = _case(case, 13)
+    stride, pad = (case[7], case[8]), case[9]
+    xr, wr, dyr = O.round_to_bf16(x), O.round_to_bf16(w), O.round_to_bf16(dy)
+    y = abi.fprop_bf16(x, w, b, stride, pad)
+    abi.close(y, O.conv_fprop(xr, wr, b, stride, pad, dtype=np.float64))
+    abi.close(abi.fprop_bf16(x, w, None, stride, pad), O.conv_fprop(xr, wr, None, stride, pad, dtype=np.float64))
+    dx = abi.dgrad_bf16(dy, w, x.shape, stride, pad)
+    abi.close(dx, O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
+    monkeypatch.setenv("AETHER_GATHER_WIDE", "0")
+    assert np.array_equal(y, abi.fprop_bf16(x, w, b, stride, pad))
+    assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
+
+
 # wgrad of a unit-stride filter of at most 9 taps on 64 input channels and at most 64 output channels:
 # one persistent workgroup per CU keeps the whole K x N result in registers (a wave per tap) and a
 # loading wave brings slabs of whole output rows with the padded source rows under them.  The library
