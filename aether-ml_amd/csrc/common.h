@@ -16,18 +16,18 @@ struct Context {
     int device = -1;
     hipStream_t stream = nullptr;
     hipDeviceProp_t prop;
-    // scratch owned by the library (packed filters, split partial sums)
-    void* ws = nullptr;
-    int64_t ws_bytes = 0;
     // small always-present buffer for counters used by single-pass reductions
     unsigned int* counters = nullptr;
 };
 
 Context& ctx();
 int fail(int code, const char* fmt, ...);
-// Returns a pointer to at least `bytes` of scratch; grows the buffer when
-// needed (synchronises the stream before freeing the old one).
+// Returns a pointer to at least `bytes` of library-owned scratch (packed filters, split
+// partial sums); grows the buffer when needed.  A buffer that a recorded step may still
+// replay into is kept until the last recording is destroyed; otherwise the old one is
+// freed after the stream has drained.  Fails with AETH_E_STATE while a step is being recorded.
 int workspace(int64_t bytes, void** out);
+
 
 #define AETH_REQUIRE_INIT()                                                     \
     do {                                                                        \

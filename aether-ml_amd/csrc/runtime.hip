@@ -1,8 +1,10 @@
 // Context, memory, copies, events: the part of the C ABI that owns device state.
 #include "common.h"
+#include "ws_ledger.h"
 
 #include <string.h>
 #include <map>
+#include <set>
 #include <unordered_map>
 #include <vector>
 
@@ -23,25 +25,26 @@ int fail(int code, const char* fmt, ...) {
     return code;
 }
 
-static bool g_recording = false;                       // a step is being recorded on the stream
-static bool recording_open() { return g_recording; }
+static WorkspaceLedger g_ws;                            // the scratch workspace and who may still use old ones
+static bool recording_open() { return g_ws.recording_open; }
 
 int workspace(int64_t bytes, void** out) {
-    Context& c = ctx();
-    if (bytes > c.ws_bytes) {
-        if (recording_open())
-            return fail(AETH_E_STATE, "the workspace would have to grow while a step is being recorded: run the step once first");
-        int64_t want = round_up(bytes + bytes / 4, 1 << 20);
-        if (c.ws) {
-            AETH_HIP(hipStreamSynchronize(c.stream));
-            AETH_HIP(hipFree(c.ws));
-            c.ws = nullptr;
-            c.ws_bytes = 0;
-        }
-        AETH_HIP(hipMalloc(&c.ws, (size_t)want));
-        c.ws_bytes = want;
-    }
-    *out = c.ws;
+    hipError_t err = hipSuccess;
+    const WorkspaceLedger::Result r = g_ws.acquire(
+        bytes, out,
+        [&](int64_t want) -> void* {
+            void* p = nullptr;
+            err = hipMalloc(&p, (size_t)want);
+            if (err != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+            return p;
+        },
+        [](void* p) { (void)hipFree(p); },
+        [] { (void)hipStreamSynchronize(ctx().stream); });
+    if (r == WorkspaceLedger::kWhileRecording)
+        return fail(AETH_E_STATE, "the workspace would have to grow while a step is being recorded: run the step once first");
+    if (r == WorkspaceLedger::kAllocFailed)
+        return fail(err == hipErrorOutOfMemory ? AETH_E_NOMEM : AETH_E_HIP, "workspace: hipMalloc(%lld bytes) -> %s",
+                    (long long)WorkspaceLedger::grown_size(bytes), hipGetErrorString(err));
     return AETH_OK;
 }
 
@@ -62,6 +65,8 @@ struct Pool {
         size_t b = bytes <= 0 ? 256 : (size_t)bytes;
         return (b + 255) & ~(size_t)255;
     }
+    // Frees every idle block.  Waits for the stream first, so it must not run while a step
+    // is being recorded (a synchronisation invalidates the capture).
     hipError_t release_cached() {
         hipError_t st = hipStreamSynchronize(ctx().stream);
         for (auto& kv : free_blocks)
@@ -83,6 +88,14 @@ __global__ void fill_u32_kernel(unsigned int* __restrict__ dst, unsigned int v, 
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) dst[i] = v;
 }
+
+// A recorded step: the instantiated graph and the blocks handed out while it was recorded.
+struct Recording {
+    hipGraphExec_t exec = nullptr;
+    std::vector<void*> blocks;
+};
+static Recording* g_open_recording = nullptr;          // being captured right now
+static std::set<Recording*> g_live_recordings;          // every handle given out and not yet destroyed
 
 }  // namespace aeth
 
@@ -118,10 +131,28 @@ int aeth_init(int device) {
 int aeth_shutdown(void) {
     Context& c = ctx();
     if (!c.ready) return AETH_OK;
+    // a recording left open: end the capture and drop what it collected
+    if (g_open_recording) {
+        hipGraph_t graph = nullptr;
+        if (hipStreamEndCapture(c.stream, &graph) == hipSuccess && graph) (void)hipGraphDestroy(graph);
+        (void)hipGetLastError();
+        g_live_recordings.erase(g_open_recording);
+        delete g_open_recording;
+        g_open_recording = nullptr;
+    }
+    (void)hipStreamSynchronize(c.stream);
+    // graphs the caller never destroyed: their handles become invalid with the context
+    for (Recording* r : g_live_recordings) {
+        if (r->exec) (void)hipGraphExecDestroy(r->exec);
+        delete r;
+    }
+    g_live_recordings.clear();
+    g_pool.recording = nullptr;
+    g_pool.reserved.clear();
     g_pool.release_cached();
     for (auto& kv : g_pool.live) (void)hipFree(kv.first);
     g_pool.live.clear();
-    if (c.ws) hipFree(c.ws);
+    g_ws.reset([](void* p) { (void)hipFree(p); });
     if (c.counters) hipFree(c.counters);
     hipStreamDestroy(c.stream);
     c = Context();
@@ -157,9 +188,9 @@ int aeth_malloc(void** host_out_ptr, int64_t bytes) {
     }
     void* p = nullptr;
     hipError_t e = hipMalloc(&p, sz);
-    if (e == hipErrorOutOfMemory && g_pool.cached_bytes > 0) {
+    if (e == hipErrorOutOfMemory && g_pool.cached_bytes > 0 && !recording_open()) {
         (void)hipGetLastError();
-        g_pool.release_cached();
+        g_pool.release_cached();                        // waits for the stream: never inside a recording
         e = hipMalloc(&p, sz);
     }
     if (e != hipSuccess) {
@@ -236,11 +267,6 @@ int aeth_fill_f32(float* dst, float value, int64_t n) {
 }
 
 // ---- recorded steps (HIP graphs) -----------------------------------------------------
-struct Recording {
-    hipGraphExec_t exec = nullptr;
-    std::vector<void*> blocks;
-};
-static Recording* g_open_recording = nullptr;
 #define AETH_NOT_RECORDING(fn)                                                                    \
     do {                                                                                          \
         if (g_open_recording) return fail(AETH_E_STATE, fn ": waits for the device, not possible while recording"); \
@@ -259,7 +285,7 @@ int aeth_graph_begin(void) {
         return fail(AETH_E_HIP, "aeth_graph_begin: hipStreamBeginCapture -> %s", hipGetErrorString(e));
     }
     g_open_recording = r;
-    g_recording = true;
+    g_ws.recording_open = true;
     g_pool.recording = &r->blocks;
     return AETH_OK;
 }
@@ -290,7 +316,7 @@ int aeth_graph_end(void** host_out_graph) {
     if (!g_open_recording) return fail(AETH_E_STATE, "aeth_graph_end: no recording is open");
     Recording* r = g_open_recording;
     g_open_recording = nullptr;
-    g_recording = false;
+    g_ws.recording_open = false;
     g_pool.recording = nullptr;
     hipGraph_t graph = nullptr;
     hipError_t e = hipStreamEndCapture(ctx().stream, &graph);
@@ -304,6 +330,8 @@ int aeth_graph_end(void** host_out_graph) {
         delete r;
         return fail(AETH_E_HIP, "aeth_graph_end: %s", hipGetErrorString(e));
     }
+    g_ws.recording_ended_ok();
+    g_live_recordings.insert(r);
     *host_out_graph = r;
     return AETH_OK;
 }
@@ -312,6 +340,8 @@ int aeth_graph_launch(void* graph) {
     AETH_REQUIRE_INIT();
     AETH_CHECK_ARG(graph != nullptr);
     if (g_open_recording) return fail(AETH_E_STATE, "aeth_graph_launch: a recording is open");
+    if (!g_live_recordings.count(static_cast<Recording*>(graph)))
+        return fail(AETH_E_INVALID, "aeth_graph_launch: %p is not a live recording", graph);
     AETH_HIP(hipGraphLaunch(static_cast<Recording*>(graph)->exec, ctx().stream));
     return AETH_OK;
 }
@@ -320,9 +350,13 @@ int aeth_graph_destroy(void* graph) {
     AETH_REQUIRE_INIT();
     if (!graph) return AETH_OK;
     Recording* r = static_cast<Recording*>(graph);
+    if (g_open_recording) return fail(AETH_E_STATE, "aeth_graph_destroy: a recording is open");
+    if (!g_live_recordings.count(r)) return fail(AETH_E_INVALID, "aeth_graph_destroy: %p is not a live recording", graph);
     AETH_HIP(hipStreamSynchronize(ctx().stream));
     if (r->exec) (void)hipGraphExecDestroy(r->exec);
     release_recording_blocks(r);
+    g_live_recordings.erase(r);
+    g_ws.recording_destroyed([](void* p) { (void)hipFree(p); });
     delete r;
     return AETH_OK;
 }
@@ -353,6 +387,7 @@ int aeth_event_destroy(void* event) {
 int aeth_event_record(void* event) {
     AETH_REQUIRE_INIT();
     AETH_CHECK_ARG(event != nullptr);
+    AETH_NOT_RECORDING("aeth_event_record");
     AETH_HIP(hipEventRecord((hipEvent_t)event, ctx().stream));
     return AETH_OK;
 }
@@ -360,6 +395,7 @@ int aeth_event_record(void* event) {
 int aeth_event_elapsed_ms(void* start, void* stop, float* host_out_ms) {
     AETH_REQUIRE_INIT();
     AETH_CHECK_ARG(start != nullptr && stop != nullptr && host_out_ms != nullptr);
+    AETH_NOT_RECORDING("aeth_event_elapsed_ms");
     AETH_HIP(hipEventSynchronize((hipEvent_t)stop));
     AETH_HIP(hipEventElapsedTime(host_out_ms, (hipEvent_t)start, (hipEvent_t)stop));
     return AETH_OK;

@@ -295,6 +295,41 @@ def test_recorded_steps_equal_eager_steps():
     assert eager.train_step(Xs[0], ys[0]) == rec.train_step(Xs[0], ys[0])
 
 
+def test_recorded_steps_survive_a_workspace_that_grows():
+    """A recorded step has the address of the library's scratch workspace in its kernel
+    arguments.  Eager work that needs a larger workspace after the recording was made
+    (here a wgrad whose split partials take tens of MB) replaces the workspace; the old
+    one must stay valid for the replays that follow."""
+    import aether
+    from tests import abi
+
+    def make():
+        np.random.seed(4)
+        m = build_model(aether, hw=16)
+        m.loss.new_pass()
+        m.accuracy.new_pass()
+        return m
+
+    rng = np.random.RandomState(6)
+    X, y = rng.rand(32, 16, 16, 3).astype(np.float32), rng.randint(0, 10, 32)
+    eager, rec = make(), make()
+    rec.record_steps(True)
+    for step in range(3):                                    # normal, recorded, replayed
+        assert eager.train_step(X, y) == rec.train_step(X, y)
+    assert any(r.get("graph") for r in rec._recordings.values())
+    xb = rng.randn(64, 56, 56, 64).astype(np.float32)
+    dyb = rng.randn(64, 56, 56, 64).astype(np.float32)
+    dw1, _ = abi.wgrad(xb, dyb, (3, 3, 64, 64), (1, 1), "same")      # grows the workspace
+    for step in range(3):
+        a, b = eager.train_step(X, y), rec.train_step(X, y)
+        assert a == b, "replay %d after the workspace grew: eager %r, recorded %r" % (step, a, b)
+        for la, lb in zip(eager.trainable_layers, rec.trainable_layers):
+            assert np.array_equal(np.asarray(la.weights), np.asarray(lb.weights))
+        dw2, _ = abi.wgrad(xb, dyb, (3, 3, 64, 64), (1, 1), "same")  # eager work in the new workspace between replays
+        assert np.array_equal(dw1, dw2)
+    rec.record_steps(False)
+
+
 def test_recording_refuses_calls_that_wait_for_the_device():
     import ctypes as C
     import aether
@@ -308,6 +343,8 @@ def test_recording_refuses_calls_that_wait_for_the_device():
         host = np.zeros(8, np.float32)
         assert lib.aeth_memcpy_d2h(host.ctypes.data, t.ptr, 32) == _lib.AETH_E_STATE
         assert lib.aeth_graph_begin() == _lib.AETH_E_STATE
+        ev = _lib.Event()
+        assert lib.aeth_event_record(ev._h) == _lib.AETH_E_STATE
         _lib.check(lib.aeth_fill_f32(t.ptr, 2.0, 8))
     finally:
         g = C.c_void_p()

@@ -1,0 +1,20 @@
+"""The workspace rules of the library (which scratch buffer a recorded step may keep
+using, when an old one may be freed) are plain bookkeeping in
+aether-ml_amd/csrc/ws_ledger.h; tests/cpu/ws_ledger_check.cpp drives them on the host
+with a fake allocator."""
+import os
+import subprocess
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_workspace_ledger_rules(tmp_path):
+    exe = str(tmp_path / "ws_ledger_check")
+    src = os.path.join(ROOT, "tests", "cpu", "ws_ledger_check.cpp")
+    inc = os.path.join(ROOT, "aether-ml_amd", "csrc")
+    subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-Werror", "-I", inc, src, "-o", exe], check=True)
+    r = subprocess.run([exe], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    names = [line.split()[1] for line in r.stdout.splitlines() if line.startswith("ok ")]
+    assert names == ["reuse", "grow_frees_old", "no_growth_while_recording", "live_recordings_keep_their_workspace",
+                     "retired_freed_with_last_recording", "alloc_failure", "reset"]
