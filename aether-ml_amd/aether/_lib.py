@@ -18,6 +18,7 @@ SIGNATURES = {
     "aeth_init": [_i],
     "aeth_shutdown": [],
     "aeth_device_info": [C.c_char_p, _i],
+    "aeth_debug_set": [C.c_char_p, _i],
     "aeth_malloc": [C.POINTER(_p), _i64],
     "aeth_free": [_p],
     "aeth_memcpy_h2d": [_p, _p, _i64],
@@ -118,6 +119,11 @@ def lib():
         check(L.aeth_init(int(os.environ.get("AETHER_DEVICE", "0"))))
         _initialised = True
     return L
+
+
+def debug_set(name=None, value=-1):
+    """Kernel-choice override for tests and measurements (aeth_debug_set); no name resets all."""
+    check(load().aeth_debug_set(name.encode() if name is not None else None, int(value)))
 
 
 def device_info():

@@ -1,7 +1,6 @@
-// bf16-input / fp32-accumulate / fp32-output entry points of the convolution path.
-// fprop and dgrad run on v_mfma_f32_32x32x16_bf16; wgrad widens its bf16 operands
-// to fp32 on the way into LDS (exact) and accumulates on the fp32 MFMA.
-#include "conv_impl.h"
+// bf16-input / fp32-accumulate / fp32-output entry points of the gather-GEMM path
+// (fprop and dgrad on v_mfma_f32_32x32x16_bf16).
+#include "gather_dispatch.h"
 
 using namespace aeth;
 
@@ -19,13 +18,6 @@ int aeth_conv_dgrad_bf16(const uint16_t* dy, const uint16_t* w, float* dx,
     AETH_REQUIRE_INIT();
     AETH_CHECK_ARG(dy != nullptr && w != nullptr && dx != nullptr);
     return conv_dgrad_impl<uint16_t>(__func__, dy, w, dx, S, H, W, C, D, fH, fW, sH, sW, pH, pW);
-}
-
-int aeth_conv_wgrad_bf16(const uint16_t* x, const uint16_t* dy, float* dw, float* dbias,
-                         int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW) {
-    AETH_REQUIRE_INIT();
-    AETH_CHECK_ARG(x != nullptr && dy != nullptr && dw != nullptr);
-    return conv_wgrad_impl<uint16_t>(__func__, x, dy, dw, dbias, S, H, W, C, D, fH, fW, sH, sW, pH, pW);
 }
 
 }  // extern "C"

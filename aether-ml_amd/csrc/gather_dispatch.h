@@ -1,0 +1,483 @@
+// Host side of the gather-GEMM path: which kernel a problem gets, split K, and the fprop / dgrad
+// entry points' shared implementation.
+#pragma once
+#include "gather_kernels.h"
+#include "tuning.h"
+
+namespace aeth {
+
+// dense_res_f32 applies to fp32 gathers that are plain matrix products (one tap, unit stride, no
+// padding), K = 32 or 64 whole, N a multiple of 4 up to 256 with more than one 64-wide tile, a dense
+// output with 16-byte stores, and at least 4 tiles of 128 rows per CU (tuning: dense_res = 1 drops the
+// last condition, =0 turns the kernel off).
+static bool plan_dense_res(const GatherParams& gp, bool dma, int cus, int* mtiles) {
+    if (!dma || gp.sh != 1 || gp.sw != 1 || gp.rh0 != 0 || gp.rw0 != 0 || gp.Hs != gp.Hg || gp.Ws != gp.Wg) return false;
+    if (gp.K != gp.Cs || gp.K != gp.Kpad || (gp.K != 32 && gp.K != 64) || gp.split_slabs != 0) return false;
+    if (gp.N <= 64 || gp.N > kD1MaxN || !gp.dense_out || gp.out_bytes == 0) return false;
+    if (tuning().dense_res == 0) return false;
+    const bool force = tuning().dense_res > 0;
+    const int n = cdiv(gp.M, kD1BM);
+    if (!force && n < 4 * cus) return false;
+    *mtiles = n;
+    return true;
+}
+
+template <typename T, int BM, int BN, int WM, int WN, int KC>
+static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
+    constexpr int kThreads = 64 * (BM / WM) * (BN / WN);     // of this tile shape (shadows the 256 of the others)
+    dim3 grid(cdiv(gp.M, BM) * cdiv(gp.N, BN));
+    if (gp.split_slabs > 0) grid.y = (unsigned)cdiv(gp.Kpad / (KC * Elem<T>::CE), gp.split_slabs);
+    const bool ut = gp.Cs % (KC * Elem<T>::CE) == 0 && gp.K == gp.Kpad && gp.K / gp.Cs <= 32;
+    // short K, several n tiles: one workgroup per m tile walks the n tiles (128 x 64 tiles only)
+    if constexpr (BM == 128 && BN == 64 && KC == 8) {
+        if (gp.split_slabs == 0 && gp.Kpad / (KC * Elem<T>::CE) <= 2 && gp.N > BN && gp.N <= kNloopMaxN && gp.out_bytes != 0 &&
+            tuning().gather_nloop != 0) {
+            grid.x = (unsigned)cdiv(gp.M, BM);
+            if (ut) hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, true>), grid, dim3(kThreads), 0, st, gp);
+            else hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, false, KC, true>), grid, dim3(kThreads), 0, st, gp);
+            return;
+        }
+    }
+    if constexpr ((BM == 128 || BM == 64) && sizeof(T) == 4) {
+        // scalar addressing (tuning: gather_sa = 0 turns it off); the moved base must stay a 32-bit extent
+        const int taps = gp.Cs > 0 ? gp.K / gp.Cs : 0;
+        const int64_t bias = ((int64_t)std::max(-gp.rh0, 0) * gp.Ws + std::max(-gp.rw0, 0)) * gp.Cs * (int64_t)sizeof(T);
+        if (ut && taps <= 32 && (int64_t)gp.src_bytes + bias < ((int64_t)1 << 31) && tuning().gather_sa != 0) {
+            hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, true>), grid, dim3(kThreads), 0, st, gp);
+            return;
+        }
+    }
+    if (ut) hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false>), grid, dim3(kThreads), 0, st, gp);
+    else hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, false, KC, false>), grid, dim3(kThreads), 0, st, gp);
+}
+
+// kc4: shallow slabs (4 chunks of k per row) for the LDS-direct kernel where the tile allows it
+template <typename T, int BM, int BN, int WM, int WN>
+static void launch_gather_cfg(const GatherParams& gp, bool vec, bool kc4, hipStream_t st) {
+    dim3 grid(cdiv(gp.M, BM) * cdiv(gp.N, BN));
+    if (vec && gp.src_bytes != 0 && gp.bt_bytes != 0) {
+        if constexpr (BM >= 64 && BN >= 64) {
+            if (kc4) {
+                launch_gather_dma<T, BM, BN, WM, WN, 4>(gp, st);
+                return;
+            }
+        }
+        launch_gather_dma<T, BM, BN, WM, WN, 8>(gp, st);
+    }
+    else if (vec)
+        hipLaunchKernelGGL((gather_gemm<T, BM, BN, WM, WN, Elem<T>::CE>), grid, dim3(kThreads), 0, st, gp);
+    else
+        hipLaunchKernelGGL((gather_gemm<T, BM, BN, WM, WN, 1>), grid, dim3(kThreads), 0, st, gp);
+}
+
+static inline int gather_bn(int N) { return N <= 32 ? 32 : 64; }
+
+// Tile height.  The LDS-direct kernel keeps two slabs per operand in LDS, so a
+// 128-row tile (48 KB) lets three workgroups share a CU where a 256-row tile
+// (80 KB) allows one or two; measured on the 56x56x64 shape, 128 rows is 11 %
+// faster.  64-row tiles (32 KB, five per CU) run at the same rate and leave a
+// smaller last round, so fp32 takes 128 rows only from about 8 rounds of tiles on
+// (6272 tiles, 56x56x64: 0.483 ms either way; 1568 tiles, 56x56x256 batch 64: 0.503 ms
+// with 128 rows, 0.488 with 64).  The register-staged kernel prefers 256 rows.
+static inline int gather_bm(int M, int N, int cus, bool dma, int elem_bytes = 4) {
+    const int bn = gather_bn(N);
+    {                                                       // tuning override: 256, 128 or 64
+        const int v = tuning().gather_bm;
+        if (v == 256 || v == 128 || (v == 64 && bn == 64)) return v;
+    }
+    const int ntiles = cdiv(N, bn);
+    const int want = elem_bytes == 2 ? cus : 2 * cus;   // bf16: the taller tile pays off from one tile per CU on
+    const int cands[3] = {256, 128, 64};
+    // bf16 MFMAs are 8x shorter per slab: there the larger wave tile of the 256-row shape wins
+    for (int i = (dma && elem_bytes == 4) ? 1 : 0; i < 3; ++i) {
+        int bm = cands[i];
+        if (bn == 32 && bm == 64) break;
+        const int64_t tiles = (int64_t)cdiv(M, bm) * ntiles;
+        if (dma && elem_bytes == 4 && bm == 128 && bn == 64 && tiles < 24 * (int64_t)cus) continue;
+        if (tiles >= want) return bm;
+    }
+    return bn == 32 ? 128 : 64;
+}
+
+// gather_halo_bf16 applies to unit-stride gathers of 2 to 32 taps over whole 64-channel blocks
+// when the span of every tile fits its buffer: with tiles cut per image (at most 10 % of empty
+// rows) or, failing that, running over image boundaries.  Fills the halo fields of gp and the
+// number of 256-row tiles when it does.
+static bool plan_halo(GatherParams& gp, bool dma, int* mtiles, int* stages) {
+    if (!dma || gp.sh != 1 || gp.sw != 1 || gp.Cs % 64 != 0 || gp.K != gp.Kpad || gp.split_slabs != 0) return false;
+    const int taps = gp.Th * gp.Tw;
+    if (taps < 2 || taps > 32 || gp.N <= 32 || gp.Cs <= 0 || gp.K != taps * gp.Cs) return false;
+    if (tuning().gather_halo == 0) return false;
+    const int hw = gp.Hg * gp.Wg;
+    const int wp = gp.Wg + gp.Tw - 1, hp = gp.Hg + gp.Th - 1;
+    if ((int64_t)gp.S * hp * wp >= ((int64_t)1 << 30)) return false;
+    auto slot0 = [&](int64_t m) {
+        const int64_t s = m / hw, rem = m % hw;
+        return (s * hp + rem / gp.Wg) * wp + rem % gp.Wg;
+    };
+    int64_t longest = 0;
+    auto fits = [&](int64_t first, int64_t last) {
+        const int64_t span = slot0(last) + (int64_t)(gp.Th - 1) * wp + gp.Tw - slot0(first);
+        longest = std::max(longest, span);
+        return span <= kHaloSlotsMax;
+    };
+    // tiles cut per image: every image has the same tiles
+    const int per_img = cdiv(hw, kHaloBM);
+    bool ok = (int64_t)per_img * kHaloBM * 10 <= (int64_t)hw * 11;
+    for (int t = 0; ok && t < per_img; ++t) ok = fits((int64_t)t * kHaloBM, std::min((t + 1) * kHaloBM, hw) - 1);
+    if (!ok) longest = 0;
+    if (ok) {
+        gp.halo_tiles = per_img;
+        *mtiles = gp.S * per_img;
+    } else {
+        const int n = cdiv(gp.M, kHaloBM);
+        if (n > (1 << 20)) return false;
+        ok = true;
+        for (int t = 0; ok && t < n; ++t)
+            ok = fits((int64_t)t * kHaloBM, std::min<int64_t>((int64_t)(t + 1) * kHaloBM, gp.M) - 1);
+        if (!ok) return false;
+        gp.halo_tiles = 0;
+        *mtiles = n;
+    }
+    *stages = longest <= halo_slots(4) ? 4 : 3;
+    gp.halo_wp = wp;
+    gp.halo_hp = hp;
+    gp.div_halo_wp = FastDiv(wp);
+    gp.div_halo_hp = FastDiv(hp);
+    gp.div_halo_tiles = FastDiv(gp.halo_tiles > 0 ? gp.halo_tiles : 1);
+    return true;
+}
+
+// gather_halo_res_bf16 applies to unit-stride gathers of 2 to 9 taps over one 64-channel block
+// with N in one tile, when 224-row tiles are whole rows of one image (Wg divides 224, at most
+// 15 % of empty rows in an image's last tile), a tile's rows and its halo fit a halo buffer and
+// there are at least 4 tiles per CU to walk (tuning: gather_res = 1 drops the last condition,
+// 0 turns the kernel off).
+static bool plan_halo_res(GatherParams& gp, bool dma, int cus, int* mtiles) {
+    if (!dma || gp.sh != 1 || gp.sw != 1 || gp.Cs != 64 || gp.K != gp.Kpad || gp.split_slabs != 0) return false;
+    const int taps = gp.Th * gp.Tw;
+    if (taps < 2 || taps > kResMaxTaps || gp.N <= 32 || gp.N > 64 || gp.K != taps * gp.Cs) return false;
+    if (tuning().gather_res == 0 || tuning().gather_halo == 0) return false;
+    const bool force = tuning().gather_res > 0;
+    if (gp.Wg <= 0 || kResBM % gp.Wg != 0) return false;
+    const int hw = gp.Hg * gp.Wg;
+    const int wp = gp.Wg + gp.Tw - 1, hp = gp.Hg + gp.Th - 1;
+    const int rows = kResBM / gp.Wg;                                     // image rows per tile
+    if ((int64_t)(rows + gp.Th - 1) * wp > kResSlots) return false;      // the tile's rows and the halo below them
+    const int per_img = cdiv(hw, kResBM);
+    if ((int64_t)per_img * kResBM * 100 > (int64_t)hw * 115) return false;
+    const int64_t n = (int64_t)gp.S * per_img;
+    if (n > (1 << 24) || (!force && n < 4 * (int64_t)cus)) return false;
+    // byte offsets are formed in 32 bits from the pixel above and left of the image
+    if (((int64_t)gp.S * gp.Hs + hp) * gp.Ws * 128 >= ((int64_t)1 << 31)) return false;
+    *mtiles = (int)n;
+    gp.halo_tiles = per_img;
+    gp.halo_wp = wp;
+    gp.halo_hp = hp;
+    gp.div_halo_wp = FastDiv(wp);
+    gp.div_halo_hp = FastDiv(hp);
+    gp.div_halo_tiles = FastDiv(per_img);
+    return true;
+}
+
+template <typename T>
+static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t st) {
+    const int bn = gather_bn(gp.N);
+    const bool dma = vec && gp.src_bytes != 0 && gp.bt_bytes != 0;
+    if constexpr (sizeof(T) == 2) {
+        GatherParams hp = gp;
+        int mtiles = 0, stages = 0;
+        if (plan_halo(hp, dma, &mtiles, &stages)) {
+            dim3 grid((unsigned)(mtiles * cdiv(gp.N, 64)));
+            if (stages == 4) hipLaunchKernelGGL(gather_halo_bf16<4>, grid, dim3(kThreads), 0, st, hp);
+            else hipLaunchKernelGGL(gather_halo_bf16<3>, grid, dim3(kThreads), 0, st, hp);
+            return;
+        }
+    }
+    if constexpr (sizeof(T) == 2) {
+        // Wide tiles for bf16 launches that the halo kernels do not take (strides, 1x1, long filters): the
+        // slab kernel with 256 x 64 tiles fetches (256 + 64) rows of k per 256 x 64 outputs, 11.5 TB/s from
+        // L2 on the 28x28x128 -> 256 stride-2 layer, and that rate is what bounds it; 256 x 256 tiles on 8 waves
+        // (one workgroup per CU, 128 KB of slabs) fetch 2.5 times less per output, 256 x 128 tiles 1.7 times.
+        // From 2 (256 wide) or 4 (128 wide) tiles per CU on (tuning: gather_wide = 1 always, 0 never).
+        const bool force = tuning().gather_wide > 0;
+        if (dma && gp.split_slabs == 0 && tuning().gather_wide != 0) {
+            const int64_t mt = cdiv(gp.M, 256);
+            if (gp.N > 192 && (force || mt * cdiv(gp.N, 256) >= 2 * (int64_t)cus)) {
+                launch_gather_dma<T, 256, 256, 64, 128, 8>(gp, st);
+                return;
+            }
+            // (the stride-2 layer's dgrad classes, 784 tiles of 1 to 4 taps each, are 4 % slower on them)
+            if (gp.N > 64 && (force || mt * cdiv(gp.N, 128) >= 4 * (int64_t)cus)) {
+                launch_gather_dma<T, 256, 128, 64, 64, 8>(gp, st);
+                return;
+            }
+        }
+    }
+    if constexpr (sizeof(T) == 4) {
+        int mtiles = 0;
+        if (plan_dense_res(gp, dma, cus, &mtiles)) {
+            const dim3 grid((unsigned)std::min(mtiles, cus));
+            if (gp.Kpad == 64) hipLaunchKernelGGL(dense_res_f32<2>, grid, dim3(kD1Threads), 0, st, gp, mtiles);
+            else hipLaunchKernelGGL(dense_res_f32<1>, grid, dim3(kD1Threads), 0, st, gp, mtiles);
+            return;
+        }
+    }
+    const int bm = gather_bm(gp.M, gp.N, cus, dma, (int)sizeof(T));
+    // shallow slabs measure the same as deep ones on the 56x56 layers (within 2 % either
+    // way), so they stay a tuning switch: gather_kc = 4
+    const bool kc4 = tuning().gather_kc == 4;
+    if (bn == 32) {
+        if (bm == 256) launch_gather_cfg<T, 256, 32, 64, 32>(gp, vec, false, st);
+        else launch_gather_cfg<T, 128, 32, 32, 32>(gp, vec, false, st);
+    } else {
+        if (bm == 256) launch_gather_cfg<T, 256, 64, 64, 64>(gp, vec, kc4, st);
+        else if (bm == 128) launch_gather_cfg<T, 128, 64, 32, 64>(gp, vec, kc4, st);
+        else launch_gather_cfg<T, 64, 64, 32, 32>(gp, vec, kc4, st);
+    }
+}
+
+// One gather-GEMM problem: pack the filter into the workspace at `ws_off`, launch.
+struct GatherSetup {
+    GatherParams gp;
+    PackParams pp;
+    int64_t bt_bytes;
+    int nsplit = 1;          // > 1: split K, partial products behind the packed filter in the workspace
+    int64_t part_bytes = 0;
+};
+
+// Split K when the tiles alone would leave most of the chip idle: at most one tile per
+// two CUs and at least 8 slabs of K.  Only for the LDS-direct kernel with 16-byte stores
+// to a dense [M, N] output.  Aim: about two workgroups per CU, at least 4 slabs each.
+template <typename T>
+static void plan_split(GatherSetup& gs, bool vec, int cus) {
+    const GatherParams& g = gs.gp;
+    gs.nsplit = 1;
+    gs.part_bytes = 0;
+    const int64_t lim = (int64_t)1 << 31;
+    const int64_t sb = (int64_t)g.S * g.Hs * g.Ws * g.Cs * (int64_t)sizeof(T);
+    const int64_t ob = (int64_t)g.M * g.N * (int64_t)sizeof(float);
+    const bool dma = vec && sb < lim && gs.bt_bytes < lim;
+    if (!dma || !g.dense_out || g.N % 4 != 0 || ob >= lim || (reinterpret_cast<uintptr_t>(g.out) & 15) != 0) return;
+    if (tuning().gather_kc != -1) return;                    // the tuning switch changes the slab depth
+    if (tuning().gather_split == 0) return;                  // lets small inputs reach the kernels of large ones
+    const int bn = gather_bn(g.N), bm = gather_bm(g.M, g.N, cus, true, (int)sizeof(T));
+    const int64_t tiles = (int64_t)cdiv(g.M, bm) * cdiv(g.N, bn);
+    const int nslabs = g.Kpad / Elem<T>::BK;
+    if (tiles * 2 > cus || nslabs < 8) return;
+    int n = (int)((2 * (int64_t)cus) / tiles);
+    if (n > nslabs / 4) n = nslabs / 4;
+    if (n > 64) n = 64;
+    if (n < 2) return;
+    const int per = cdiv(nslabs, n);
+    gs.gp.split_slabs = per;
+    gs.nsplit = cdiv(nslabs, per);
+    gs.part_bytes = round_up((int64_t)gs.nsplit * ob, 256);
+}
+
+template <typename T>
+static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
+    Context& c = ctx();
+    void* bt = ws + ws_off;
+    gs.gp.bt = bt;
+    gs.pp.bt = bt;
+    int total = gs.pp.Npad * gs.pp.Kpad;
+    {
+        const GatherParams& g = gs.gp;
+        int64_t sb = (int64_t)g.S * g.Hs * g.Ws * g.Cs * (int64_t)sizeof(T);
+        int64_t bb = (int64_t)total * (int64_t)sizeof(T);
+        const int64_t lim = (int64_t)1 << 31;
+        gs.gp.Th = (g.Tw > 0 && g.Cs > 0) ? (g.K / g.Cs) / g.Tw : 0;
+        gs.gp.src_bytes = (sb < lim && bb < lim) ? (unsigned)sb : 0u;
+        gs.gp.bt_bytes = (sb < lim && bb < lim) ? (unsigned)bb : 0u;
+        const int64_t ob = (g.dense_out ? (int64_t)g.M : (int64_t)g.S * g.Hof * g.Wof) * g.N * (int64_t)sizeof(float);
+        const bool ovec = ob < lim && g.N % 4 == 0 && (reinterpret_cast<uintptr_t>(g.out) & 15) == 0;
+        gs.gp.out_bytes = ovec ? (unsigned)ob : 0u;
+    }
+    if constexpr (sizeof(T) == 2) {
+        // the kernel that keeps the whole filter in LDS reads it from w itself
+        GatherParams hp = gs.gp;
+        int mtiles = 0;
+        const bool dma = vec && hp.src_bytes != 0 && gs.pp.w_elems * 2 < ((int64_t)1 << 31) && gs.pp.N % 2 == 0;
+        if (gs.nsplit == 1 && hp.M > 0 && plan_halo_res(hp, dma, c.prop.multiProcessorCount, &mtiles)) {
+            hipLaunchKernelGGL(gather_halo_res_bf16, dim3((unsigned)std::min(mtiles, c.prop.multiProcessorCount)),
+                               dim3(kResThreads), 0, c.stream, hp, gs.pp, mtiles);
+            AETH_LAUNCH_CHECK();
+            return AETH_OK;
+        }
+    }
+    if (total > 0) {
+        hipLaunchKernelGGL(pack_filter<T>, dim3(cdiv(total, 256)), dim3(256), 0, c.stream, gs.pp);
+        AETH_LAUNCH_CHECK();
+    }
+    if (gs.gp.M > 0 && gs.gp.N > 0) {
+        float* real_out = gs.gp.out;
+        if (gs.nsplit > 1) gs.gp.out = reinterpret_cast<float*>(ws + ws_off + round_up(gs.bt_bytes, 256));
+        launch_gather<T>(gs.gp, vec, c.prop.multiProcessorCount, c.stream);
+        AETH_LAUNCH_CHECK();
+        if (gs.nsplit > 1) {
+            const int n = gs.gp.M * gs.gp.N;
+            hipLaunchKernelGGL(reduce_splits4, dim3(cdiv(n, 64)), dim3(kThreads), 0, c.stream,
+                               (const float*)gs.gp.out, real_out, (float*)nullptr, n, n, n, gs.nsplit);
+            AETH_LAUNCH_CHECK();
+        }
+    }
+    return AETH_OK;
+}
+
+static inline void set_out_divs(GatherParams& g) {
+    g.div_hw = FastDiv(g.Hg * g.Wg > 0 ? g.Hg * g.Wg : 1);
+    g.div_w = FastDiv(g.Wg > 0 ? g.Wg : 1);
+    g.div_c = FastDiv(g.Cs);
+    g.div_tw = FastDiv(g.Tw > 0 ? g.Tw : 1);
+}
+
+template <typename T>
+static bool launch_direct(DirectParams& dp, bool dgrad, hipStream_t st) {
+    if (tuning().direct == 0) return false;
+    const int chunks = dp.D / 4;
+    if (dp.C > 3 || dp.D % 4 != 0 || chunks < 4 || chunks > 64 || (chunks & (chunks - 1)) != 0) return false;
+    if ((int64_t)dp.fH * dp.fW * dp.C * dp.D > kDirectMaxW || (int64_t)dp.M * chunks >= ((int64_t)1 << 31)) return false;
+    if ((reinterpret_cast<uintptr_t>(dp.a) & 15) != 0 || (reinterpret_cast<uintptr_t>(dp.out) & 15) != 0 ||
+        (dp.bias != nullptr && (reinterpret_cast<uintptr_t>(dp.bias) & 15) != 0))
+        return false;
+    dp.q_shift = 0;
+    while ((1 << dp.q_shift) < chunks) ++dp.q_shift;
+    const dim3 grid((unsigned)cdiv((int64_t)dp.M * chunks, kThreads));
+    const size_t lds = (size_t)dp.fH * dp.fW * dp.C * dp.D * sizeof(float);
+#define AETH_DIRECT_CASE(FH_, FW_, C_)                                                                              \
+    if (dp.fH == FH_ && dp.fW == FW_ && dp.C == C_) {                                                               \
+        if (dgrad) hipLaunchKernelGGL((direct_dgrad_smallc<T, FH_, FW_, C_>), grid, dim3(kThreads), lds, st, dp);   \
+        else hipLaunchKernelGGL((direct_fprop_smallc<T, FH_, FW_, C_>), grid, dim3(kThreads), lds, st, dp);         \
+        return true;                                                                                                \
+    }
+    AETH_DIRECT_CASE(3, 3, 1)
+    AETH_DIRECT_CASE(3, 3, 2)
+    AETH_DIRECT_CASE(3, 3, 3)
+    AETH_DIRECT_CASE(5, 5, 1)
+    AETH_DIRECT_CASE(5, 5, 3)
+#undef AETH_DIRECT_CASE
+    return false;
+}
+
+template <typename T>
+int conv_fprop_impl(const char* fn, const T* x, const T* w, const float* bias, float* y,
+                    int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW) {
+    int Ho, Wo;
+    int rc = check_conv_dims(fn, S, H, W, C, D, fH, fW, sH, sW, pH, pW, &Ho, &Wo);
+    if (rc) return rc;
+    if (C <= 3) {
+        DirectParams dp;
+        dp.a = x; dp.w = w; dp.bias = bias; dp.out = y;
+        dp.S = S; dp.H = H; dp.W = W; dp.C = C; dp.Ho = Ho; dp.Wo = Wo; dp.D = D;
+        dp.fH = fH; dp.fW = fW; dp.sH = sH; dp.sW = sW; dp.pH = pH; dp.pW = pW;
+        dp.M = S * Ho * Wo;
+        dp.div_hw = FastDiv(Ho * Wo);
+        dp.div_w = FastDiv(Wo);
+        if (launch_direct<T>(dp, false, ctx().stream)) {
+            AETH_LAUNCH_CHECK();
+            return AETH_OK;
+        }
+    }
+    constexpr int BK = Elem<T>::BK;
+    GatherSetup gs;
+    GatherParams& g = gs.gp;
+    g.src = x; g.bias = bias; g.out = y;
+    g.S = S; g.Hs = H; g.Ws = W; g.Cs = C;
+    g.Hg = Ho; g.Wg = Wo; g.M = S * Ho * Wo; g.N = D; g.K = fH * fW * C;
+    g.Kpad = (int)round_up(g.K, BK);
+    g.Tw = fW; g.sh = sH; g.sw = sW; g.rh0 = -pH; g.rw0 = -pW;
+    g.Hof = Ho; g.Wof = Wo; g.oh0 = 0; g.ow0 = 0; g.ohs = 1; g.ows = 1; g.dense_out = 1;
+    set_out_divs(g);
+    PackParams& pk = gs.pp;
+    pk.w = w; pk.fW = fW; pk.C = C; pk.D = D; pk.Tw = fW; pk.Ck = C; pk.w_elems = (int64_t)fH * fW * C * D;
+    pk.xa = 0; pk.xs = 1; pk.ya = 0; pk.ys = 1; pk.transposed = 0;
+    pk.N = D; pk.K = g.K; pk.Npad = (int)round_up(D, 64); pk.Kpad = g.Kpad;
+    gs.bt_bytes = (int64_t)pk.Npad * pk.Kpad * sizeof(T);
+    g.split_slabs = 0;
+    plan_split<T>(gs, C % Elem<T>::CE == 0, ctx().prop.multiProcessorCount);
+    void* ws;
+    rc = workspace(round_up(gs.bt_bytes, 256) + gs.part_bytes, &ws);
+    if (rc) return rc;
+    return run_gather<T>(gs, (char*)ws, 0, C % Elem<T>::CE == 0);
+}
+
+// dgrad: for input row i the contributing taps are x with (i + pH - x) % sH == 0 and
+// 0 <= (i + pH - x)/sH < Ho.  Rows are split by a = i % sH; inside a class the taps
+// are x_t = xmax - sH*t (xmax = largest x < fH with x == (a+pH) mod sH), and the
+// source row for class-row i' (i = a + sH*i') and tap t is i' + (a + pH - xmax)/sH + t:
+// a unit-stride gather over dy with Th = number of such taps.
+template <typename T>
+int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
+                    int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW) {
+    int Ho, Wo;
+    int rc = check_conv_dims(fn, S, H, W, C, D, fH, fW, sH, sW, pH, pW, &Ho, &Wo);
+    if (rc) return rc;
+    constexpr int BK = Elem<T>::BK;
+    const int nclass = sH * sW;
+    if (nclass > 64) return fail(AETH_E_INVALID, "%s: stride too large", fn);
+    if (C <= 3) {
+        DirectParams dp;
+        dp.a = dy; dp.w = w; dp.bias = nullptr; dp.out = dx;
+        dp.S = S; dp.H = H; dp.W = W; dp.C = C; dp.Ho = Ho; dp.Wo = Wo; dp.D = D;
+        dp.fH = fH; dp.fW = fW; dp.sH = sH; dp.sW = sW; dp.pH = pH; dp.pW = pW;
+        dp.M = S * H * W;
+        dp.div_hw = FastDiv(H * W);
+        dp.div_w = FastDiv(W);
+        if (launch_direct<T>(dp, true, ctx().stream)) {
+            AETH_LAUNCH_CHECK();
+            return AETH_OK;
+        }
+    }
+    std::vector<GatherSetup> sets;
+    int64_t total_bytes = 0;
+    for (int a = 0; a < sH; ++a) {
+        if (a >= H) continue;
+        int ra = (a + pH) % sH;
+        int Th = ra < fH ? (fH - 1 - ra) / sH + 1 : 0;
+        int xmax = ra + (Th - 1) * sH;
+        int offh = Th > 0 ? (a + pH - xmax) / sH : 0;   // exact: (a+pH-xmax) is a multiple of sH
+        int Hg = (H - a + sH - 1) / sH;
+        for (int b = 0; b < sW; ++b) {
+            if (b >= W) continue;
+            int rb = (b + pW) % sW;
+            int Tw = rb < fW ? (fW - 1 - rb) / sW + 1 : 0;
+            int ymax = rb + (Tw - 1) * sW;
+            int offw = Tw > 0 ? (b + pW - ymax) / sW : 0;
+            int Wg = (W - b + sW - 1) / sW;
+            GatherSetup gs;
+            GatherParams& g = gs.gp;
+            g.src = dy; g.bias = nullptr; g.out = dx;
+            g.S = S; g.Hs = Ho; g.Ws = Wo; g.Cs = D;
+            g.Hg = Hg; g.Wg = Wg; g.M = S * Hg * Wg; g.N = C;
+            g.K = Th * Tw * D;
+            g.Kpad = (int)round_up(g.K, BK);
+            g.Tw = Tw; g.sh = 1; g.sw = 1; g.rh0 = offh; g.rw0 = offw;
+            g.Hof = H; g.Wof = W; g.oh0 = a; g.ow0 = b; g.ohs = sH; g.ows = sW;
+            g.dense_out = (nclass == 1);
+            set_out_divs(g);
+            PackParams& pk = gs.pp;
+            pk.w = w; pk.fW = fW; pk.C = C; pk.D = D; pk.Tw = Tw > 0 ? Tw : 1; pk.Ck = D; pk.w_elems = (int64_t)fH * fW * C * D;
+            pk.xa = xmax; pk.xs = -sH; pk.ya = ymax; pk.ys = -sW; pk.transposed = 1;
+            pk.N = C; pk.K = g.K; pk.Npad = (int)round_up(C, 64); pk.Kpad = g.Kpad;
+            gs.bt_bytes = round_up((int64_t)pk.Npad * pk.Kpad * sizeof(T), 256);
+            g.split_slabs = 0;
+            plan_split<T>(gs, D % Elem<T>::CE == 0, ctx().prop.multiProcessorCount);
+            total_bytes += gs.bt_bytes + gs.part_bytes;
+            sets.push_back(gs);
+        }
+    }
+    void* ws;
+    rc = workspace(total_bytes > 0 ? total_bytes : 256, &ws);
+    if (rc) return rc;
+    int64_t off = 0;
+    for (auto& gs : sets) {
+        rc = run_gather<T>(gs, (char*)ws, off, D % Elem<T>::CE == 0);
+        if (rc) return rc;
+        off += gs.bt_bytes + gs.part_bytes;
+    }
+    return AETH_OK;
+}
+
+
+}  // namespace aeth

@@ -1,7 +1,7 @@
-// fp32 entry points of the convolution path and of the dense layer (the dense
-// products are the 1x1 cases of the same kernels: x [M,n_in] is an [M,1,1,n_in]
-// image and w [n_in,n_out] a [1,1,n_in,n_out] filter).
-#include "conv_impl.h"
+// fp32 entry points of the gather-GEMM path: convolution fprop / dgrad and the dense layer's
+// forward and input-gradient products (the 1x1 cases of the same kernels: x [M,n_in] is an
+// [M,1,1,n_in] image and w [n_in,n_out] a [1,1,n_in,n_out] filter).
+#include "gather_dispatch.h"
 
 using namespace aeth;
 
@@ -21,13 +21,6 @@ int aeth_conv_dgrad_f32(const float* dy, const float* w, float* dx,
     return conv_dgrad_impl<float>(__func__, dy, w, dx, S, H, W, C, D, fH, fW, sH, sW, pH, pW);
 }
 
-int aeth_conv_wgrad_f32(const float* x, const float* dy, float* dw, float* dbias,
-                        int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW) {
-    AETH_REQUIRE_INIT();
-    AETH_CHECK_ARG(x != nullptr && dy != nullptr && dw != nullptr);
-    return conv_wgrad_impl<float>(__func__, x, dy, dw, dbias, S, H, W, C, D, fH, fW, sH, sW, pH, pW);
-}
-
 int aeth_dense_fprop_f32(const float* x, const float* w, const float* bias, float* y, int M, int n_in, int n_out) {
     AETH_REQUIRE_INIT();
     AETH_CHECK_ARG(x != nullptr && w != nullptr && y != nullptr);
@@ -38,12 +31,6 @@ int aeth_dense_dgrad_f32(const float* dy, const float* w, float* dx, int M, int 
     AETH_REQUIRE_INIT();
     AETH_CHECK_ARG(dy != nullptr && w != nullptr && dx != nullptr);
     return conv_dgrad_impl<float>(__func__, dy, w, dx, M, 1, 1, n_in, n_out, 1, 1, 1, 1, 0, 0);
-}
-
-int aeth_dense_wgrad_f32(const float* x, const float* dy, float* dw, float* dbias, int M, int n_in, int n_out) {
-    AETH_REQUIRE_INIT();
-    AETH_CHECK_ARG(x != nullptr && dy != nullptr && dw != nullptr);
-    return conv_wgrad_impl<float>(__func__, x, dy, dw, dbias, M, 1, 1, n_in, n_out, 1, 1, 1, 1, 0, 0);
 }
 
 }  // extern "C"

@@ -1,7 +1,9 @@
 // Context, memory, copies, events: the part of the C ABI that owns device state.
 #include "common.h"
+#include "tuning.h"
 #include "ws_ledger.h"
 
+#include <stdlib.h>
 #include <string.h>
 #include <map>
 #include <set>
@@ -23,6 +25,56 @@ int fail(int code, const char* fmt, ...) {
     vsnprintf(g_err, sizeof(g_err), fmt, ap);
     va_end(ap);
     return code;
+}
+
+Tuning& tuning() {
+    static Tuning t;
+    return t;
+}
+
+bool tuning_set(const char* name, int value) {
+    Tuning& t = tuning();
+    if (name == nullptr) {
+        t = Tuning();
+        return true;
+    }
+    struct Field { const char* name; int Tuning::*member; };
+    static const Field fields[] = {
+        {"gather_bm", &Tuning::gather_bm},       {"gather_kc", &Tuning::gather_kc},
+        {"gather_nloop", &Tuning::gather_nloop}, {"gather_halo", &Tuning::gather_halo},
+        {"gather_split", &Tuning::gather_split}, {"gather_sa", &Tuning::gather_sa},
+        {"gather_wide", &Tuning::gather_wide},   {"gather_res", &Tuning::gather_res},
+        {"dense_res", &Tuning::dense_res},       {"direct", &Tuning::direct},
+        {"wgrad_halo", &Tuning::wgrad_halo},     {"wgrad_cw", &Tuning::wgrad_cw},
+        {"wgrad_br", &Tuning::wgrad_br},         {"wgrad_rounds", &Tuning::wgrad_rounds},
+    };
+    for (const Field& f : fields)
+        if (strcmp(f.name, name) == 0) {
+            t.*(f.member) = value;
+            return true;
+        }
+    return false;
+}
+
+void tuning_parse(const char* spec, const char** bad) {
+    if (bad) *bad = nullptr;
+    if (spec == nullptr) return;
+    static thread_local char unknown[64];
+    const char* p = spec;
+    while (*p) {
+        char name[64];
+        size_t n = 0;
+        while (*p && *p != '=' && *p != ',' && n + 1 < sizeof(name)) name[n++] = *p++;
+        name[n] = 0;
+        int value = 1;
+        if (*p == '=') value = atoi(++p);
+        while (*p && *p != ',') ++p;
+        if (*p == ',') ++p;
+        if (n > 0 && !tuning_set(name, value) && bad && *bad == nullptr) {
+            snprintf(unknown, sizeof(unknown), "%s", name);
+            *bad = unknown;
+        }
+    }
 }
 
 static WorkspaceLedger g_ws;                            // the scratch workspace and who may still use old ones
@@ -111,6 +163,11 @@ int aeth_init(int device) {
         if (c.device == device) return AETH_OK;
         return fail(AETH_E_STATE, "aeth_init: already bound to device %d", c.device);
     }
+    {   // the one place the library looks at the environment: kernel-choice overrides for measurements
+        const char* bad = nullptr;
+        tuning_parse(getenv("AETHER_TUNE"), &bad);
+        if (bad) return fail(AETH_E_INVALID, "aeth_init: AETHER_TUNE names an unknown switch '%s'", bad);
+    }
     int n = 0;
     AETH_HIP(hipGetDeviceCount(&n));
     if (device < 0 || device >= n) return fail(AETH_E_INVALID, "aeth_init: device %d out of range (%d present)", device, n);
@@ -156,6 +213,11 @@ int aeth_shutdown(void) {
     if (c.counters) hipFree(c.counters);
     hipStreamDestroy(c.stream);
     c = Context();
+    return AETH_OK;
+}
+
+int aeth_debug_set(const char* host_name, int value) {
+    if (!tuning_set(host_name, value)) return fail(AETH_E_INVALID, "aeth_debug_set: unknown switch '%s'", host_name);
     return AETH_OK;
 }
 

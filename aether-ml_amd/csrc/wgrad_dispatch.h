@@ -1,0 +1,202 @@
+// Host side of wgrad: kernel choice, number of splits, the fixed-order reduction of the partials.
+#pragma once
+#include "wgrad_kernels.h"
+#include "tuning.h"
+
+namespace aeth {
+
+// Fills the plan of wgrad_halo_bf16 and returns the number of workgroups (= splits), or 0 when the
+// kernel does not apply: unit stride, 64 input channels, D a multiple of 8 up to 64, at most 9 taps,
+// slabs of whole output rows (R rows with R * Wo a multiple of 16 up to 128, R dividing Ho) whose
+// padded source rows fit the halo buffer, and at least 4 slabs per CU (tuning: wgrad_halo = 1 drops
+// the last condition, 0 turns the kernel off).
+static int plan_wgrad_halo(WgradHaloParams& p, int C, int sH, int sW, int cus) {
+    if (sH != 1 || sW != 1 || C != 64 || p.D % 8 != 0 || p.D > 64 || p.fH * p.fW > kWhMaxTaps) return 0;
+    if (tuning().wgrad_halo == 0) return 0;
+    const bool force = tuning().wgrad_halo > 0;
+    int R = 0;
+    for (int r = 1; r * p.Wo <= kWhRows; ++r)
+        if ((r * p.Wo) % 16 == 0 && p.Ho % r == 0) R = r;                  // the tallest slab that fits
+    if (R == 0) return 0;
+    p.R = R;
+    p.slab_m = R * p.Wo;
+    p.Wp = p.Wo + p.fW - 1;
+    p.hslots = (R + p.fH - 1) * p.Wp;
+    if (p.hslots > kWhSlots) return 0;
+    const int64_t nslabs = (int64_t)p.S * (p.Ho / R);
+    if (nslabs > (1 << 24) || (!force && nslabs < 4 * (int64_t)cus)) return 0;
+    // byte offsets are formed in 32 bits from the pixel above and left of the image
+    if (((int64_t)p.S * p.H + p.fH) * p.W * 128 >= ((int64_t)1 << 31)) return 0;
+    p.nslabs = (int)nslabs;
+    const int wgs = (int)std::min<int64_t>(nslabs, cus);
+    p.per = cdiv(p.nslabs, wgs);
+    p.div_wp = FastDiv(p.Wp);
+    p.div_wo = FastDiv(p.Wo);
+    p.div_fw = FastDiv(p.fW);
+    p.div_spi = FastDiv(p.Ho / R);
+    return cdiv(p.nslabs, p.per);
+}
+
+// Fills the plan of wgrad_halo_f32 and returns the number of workgroups (= splits), or 0 when the
+// kernel does not apply: unit stride, 64 input channels, D a multiple of 4 up to 64, at most 9 taps,
+// an even Wo of 28, 32, 56 or 64 (the built pair counts), at most 3 filter rows of at most 68 padded
+// columns, and at least 4 output rows per CU (tuning: wgrad_halo = 1 drops the last condition, =0 turns
+// the kernel off).
+static int plan_wgrad_halo_f32(WgradHaloParams& p, int C, int sH, int sW, int cus) {
+    if (sH != 1 || sW != 1 || C != 64 || p.D % 4 != 0 || p.D > 64 || p.fH * p.fW > 9) return 0;
+    if (tuning().wgrad_halo == 0) return 0;
+    const bool force = tuning().wgrad_halo > 0;
+    if (p.Wo != 28 && p.Wo != 32 && p.Wo != 56 && p.Wo != 64) return 0;
+    p.R = 1;
+    p.slab_m = p.Wo;
+    p.Wp = (int)round_up(p.Wo + p.fW - 1, 4);            // row pitch of the halo in LDS: whole loads of 4 slots
+    p.hslots = p.fH * p.Wp;
+    if (p.fH > 3 || p.Wp > kFhRowSlots) return 0;
+    const int64_t nslabs = (int64_t)p.S * p.Ho;
+    if (nslabs > (1 << 24) || (!force && nslabs < 4 * (int64_t)cus)) return 0;
+    // byte offsets are formed in 32 bits from the pixel above and left of the image
+    if (((int64_t)p.S * p.H + p.fH) * p.W * 256 >= ((int64_t)1 << 31)) return 0;
+    p.nslabs = (int)nslabs;
+    const int wgs = (int)std::min<int64_t>(nslabs, cus);
+    p.per = cdiv(p.nslabs, wgs);
+    p.div_wp = FastDiv(p.Wp);
+    p.div_wo = FastDiv(p.Wo);
+    p.div_fw = FastDiv(p.fW);
+    p.div_spi = FastDiv(p.Ho);
+    return cdiv(p.nslabs, p.per);
+}
+
+template <typename T>
+int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* dbias,
+                    int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW) {
+    int Ho, Wo;
+    int rc = check_conv_dims(fn, S, H, W, C, D, fH, fW, sH, sW, pH, pW, &Ho, &Wo);
+    if (rc) return rc;
+    Context& c = ctx();
+    WgradParams p;
+    p.x = x; p.dy = dy;
+    p.S = S; p.H = H; p.W = W; p.C = C; p.Ho = Ho; p.Wo = Wo; p.D = D;
+    p.M = S * Ho * Wo; p.K = fH * fW * C;
+    p.fW = fW; p.sH = sH; p.sW = sW; p.pH = pH; p.pW = pW;
+    p.want_dbias = dbias != nullptr;
+    p.div_howo = FastDiv(Ho * Wo); p.div_wo = FastDiv(Wo); p.div_c = FastDiv(C); p.div_fw = FastDiv(fW);
+    constexpr int CE = Elem<T>::CE;
+    const bool va = (C % CE == 0), vy = (D % CE == 0);
+    const int64_t xb = (int64_t)S * H * W * C * (int64_t)sizeof(T), yb = (int64_t)p.M * D * (int64_t)sizeof(T);
+    const bool fits = xb < ((int64_t)1 << 31) && yb < ((int64_t)1 << 31);
+    // fp32: the LDS-direct kernel takes any C (one float per lane and load when C % 4 != 0)
+    const bool dma = sizeof(T) == 4 && vy && fits;
+    const bool dma16 = sizeof(T) == 2 && va && vy && fits;      // bf16 MFMA kernel, 64-row slabs
+    p.x_bytes = (dma || dma16) ? (unsigned)xb : 0u;
+    p.dy_bytes = (dma || dma16) ? (unsigned)yb : 0u;
+    {
+        WgradHaloParams hp;
+        hp.x = x; hp.dy = dy;
+        hp.x_bytes = p.x_bytes; hp.dy_bytes = p.dy_bytes;
+        hp.S = S; hp.H = H; hp.W = W; hp.Ho = Ho; hp.Wo = Wo; hp.D = D; hp.fH = fH; hp.fW = fW; hp.pH = pH; hp.pW = pW;
+        hp.want_dbias = dbias != nullptr;
+        int splits = 0;
+        if constexpr (sizeof(T) == 2) splits = dma16 ? plan_wgrad_halo(hp, C, sH, sW, c.prop.multiProcessorCount) : 0;
+        else splits = (dma && va) ? plan_wgrad_halo_f32(hp, C, sH, sW, c.prop.multiProcessorCount) : 0;
+        if (splits > 0) {
+            const int64_t kd = (int64_t)p.K * D;
+            void* ws;
+            rc = workspace((int64_t)splits * (kd + D) * sizeof(float), &ws);
+            if (rc) return rc;
+            hp.out = (float*)ws;
+            if constexpr (sizeof(T) == 2) {
+                hipLaunchKernelGGL(wgrad_halo_bf16, dim3(splits), dim3(64 * (fH * fW + 1)), 0, c.stream, hp);
+            } else {
+                const dim3 grid(splits), block(64 * kFhWaves);
+                if (Wo == 56) hipLaunchKernelGGL(wgrad_halo_f32<28>, grid, block, 0, c.stream, hp);
+                else if (Wo == 64) hipLaunchKernelGGL(wgrad_halo_f32<32>, grid, block, 0, c.stream, hp);
+                else if (Wo == 32) hipLaunchKernelGGL(wgrad_halo_f32<16>, grid, block, 0, c.stream, hp);
+                else hipLaunchKernelGGL(wgrad_halo_f32<14>, grid, block, 0, c.stream, hp);
+            }
+            AETH_LAUNCH_CHECK();
+            const int n = (int)(kd + (dbias ? D : 0));
+            const bool r4 = (reinterpret_cast<uintptr_t>(dw) & 15) == 0 &&
+                            (dbias == nullptr || (reinterpret_cast<uintptr_t>(dbias) & 15) == 0);
+            if (r4)
+                hipLaunchKernelGGL(reduce_splits4, dim3(cdiv(n, 64)), dim3(kThreads), 0, c.stream, (const float*)ws, dw,
+                                   dbias, (int)kd, n, (int)(kd + D), splits);
+            else
+                hipLaunchKernelGGL(reduce_splits, dim3(cdiv(n, 64)), dim3(kThreads), 0, c.stream, (const float*)ws, dw,
+                                   dbias, (int)kd, n, (int)(kd + D), splits);
+            AETH_LAUNCH_CHECK();
+            return AETH_OK;
+        }
+    }
+    // operand width of the fp32 LDS-direct kernel: 192-wide k tiles where they pad fewer rows than 128-wide ones
+    p.cw = !va ? 1 : (p.K <= 64 ? 2 : 4);
+    if (dma && p.cw == 4 && cdiv(p.K, 192) * 192 < cdiv(p.K, kWgBK) * kWgBK) p.cw = 6;
+    if (dma && va && p.K > 64 && (tuning().wgrad_cw == 4 || tuning().wgrad_cw == 6)) p.cw = tuning().wgrad_cw;
+    // slab height of the 192-wide kernel: 16 rows (three workgroups per CU) where a workgroup walks at
+    // least 64 of them (56x56x64: 0.481 ms against 0.487 with 32 rows; 8x8x64 -> 128, batch 128, 8 slabs of
+    // 32 per workgroup: 27.2 us with 32 rows, 28.3 with 16); tuning: wgrad_br overrides
+    int br = kWgBR;
+    if (dma && p.cw == 6) {
+        const int kt6 = cdiv(p.K, 192), nt6 = cdiv(D, kWgBN);
+        const int64_t wgs = (int64_t)3 * c.prop.multiProcessorCount;
+        if ((int64_t)cdiv(p.M, 32) * kt6 * nt6 >= 32 * wgs) br = 16;
+        if (tuning().wgrad_br == 32 || tuning().wgrad_br == 16) br = tuning().wgrad_br;
+    }
+    {
+        const int qs = br / (Ho * Wo), rem = br % (Ho * Wo), qh = rem / Wo, qw = rem % Wo;
+        p.step_c = qw * sW;
+        p.step_r = qh * sH;
+        p.inc0 = 4 * C * (qw * sW + qh * sH * W + qs * H * W);
+        p.inc1 = 4 * C * (-Wo * sW + sH * W);
+        p.inc2 = 4 * C * (-Ho * sH * W + H * W);
+    }
+    const int tkw = !dma ? kWgBK : (p.cw == 1 ? 32 : (p.cw == 6 ? 192 : kWgBK));
+    const int kt = cdiv(p.K, tkw), nt = cdiv(D, kWgBN);
+    const int slab_rows = dma16 ? 64 : kWgBR;
+    const int slabs = cdiv(p.M, slab_rows);           // fp32: counted in 32-row units for both tile shapes
+    // one round of resident workgroups (3 per CU for the LDS-direct kernels, 2 for the 192-wide
+    // one and the register-staged one), rounded down so that no second, nearly empty round follows.
+    // Every further round costs a set-up, an epilogue and a share of the reduction per workgroup
+    // (56x56x64: 0.485 ms with one round, 0.493 with two, 0.509 with four).
+    int rounds = 1;
+    if (tuning().wgrad_rounds >= 1 && tuning().wgrad_rounds <= 4) rounds = tuning().wgrad_rounds;
+    const int per_cu2 = (((dma && (p.cw != 6 || br == 16)) || dma16) ? 3 : 2) * rounds;
+    int splits = (per_cu2 * c.prop.multiProcessorCount) / (kt * nt);
+    // a workgroup's set-up, epilogue and its share of the reduction are worth several slabs
+    // (training step of the 3-block CNN: 0.672 ms with 1, 0.642 with 4, 0.611 with 8, 0.658 with 16)
+    const int min_slabs = 8;
+    if (splits > cdiv(slabs, min_slabs)) splits = cdiv(slabs, min_slabs);
+    if (splits < 1) splits = 1;
+    int slabs_per = cdiv(slabs, splits);
+    splits = cdiv(slabs, slabs_per);
+    p.m_per_split = slabs_per * slab_rows;
+    const int64_t kd = (int64_t)p.K * D;
+    void* ws;
+    rc = workspace((int64_t)splits * (kd + D) * sizeof(float), &ws);
+    if (rc) return rc;
+    p.out = (float*)ws;
+    p.kt = kt; p.nt = nt;
+    dim3 grid(kt * nt * splits);
+    if (dma16) hipLaunchKernelGGL(wgrad_gemm_dma_bf16, grid, dim3(kThreads), 0, c.stream, p);
+    else if (dma && p.cw == 6 && br == 16) hipLaunchKernelGGL(wgrad_gemm_dma192h, grid, dim3(kThreads), 0, c.stream, p);
+    else if (dma && p.cw == 6) hipLaunchKernelGGL(wgrad_gemm_dma192, grid, dim3(kThreads), 0, c.stream, p);
+    else if (dma) hipLaunchKernelGGL(wgrad_gemm_dma, grid, dim3(kThreads), 0, c.stream, p);
+    else if (va && vy) hipLaunchKernelGGL((wgrad_gemm<T, CE, CE>), grid, dim3(kThreads), 0, c.stream, p);
+    else if (va) hipLaunchKernelGGL((wgrad_gemm<T, CE, 1>), grid, dim3(kThreads), 0, c.stream, p);
+    else if (vy) hipLaunchKernelGGL((wgrad_gemm<T, 1, CE>), grid, dim3(kThreads), 0, c.stream, p);
+    else hipLaunchKernelGGL((wgrad_gemm<T, 1, 1>), grid, dim3(kThreads), 0, c.stream, p);
+    AETH_LAUNCH_CHECK();
+    const int n = (int)(kd + (dbias ? D : 0));
+    const bool r4 = kd % 4 == 0 && D % 4 == 0 && (reinterpret_cast<uintptr_t>(dw) & 15) == 0 &&
+                    (dbias == nullptr || (reinterpret_cast<uintptr_t>(dbias) & 15) == 0);
+    if (r4)
+        hipLaunchKernelGGL(reduce_splits4, dim3(cdiv(n, 64)), dim3(kThreads), 0, c.stream, (const float*)ws, dw, dbias,
+                           (int)kd, n, (int)(kd + D), splits);
+    else
+        hipLaunchKernelGGL(reduce_splits, dim3(cdiv(n, 64)), dim3(kThreads), 0, c.stream, (const float*)ws, dw, dbias,
+                           (int)kd, n, (int)(kd + D), splits);
+    AETH_LAUNCH_CHECK();
+    return AETH_OK;
+}
+
+
+}  // namespace aeth

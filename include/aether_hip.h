@@ -47,6 +47,17 @@ const char* aeth_last_error(void);
 /* "arch=gfx950;cus=256;clock_mhz=2400;mem_clock_mhz=...;hbm_bytes=...;lds_bytes=..." */
 int aeth_device_info(char* host_buf, int n);
 
+/* Kernel-choice overrides for tests and measurements; no counterpart in the reference.
+ * Every dispatch decision follows from the problem's shape; a switch lets a test reach a
+ * kernel with an input smaller than the shapes it is chosen for, or run a problem on a
+ * second, independently scheduled kernel.  -1 restores "decide from the shape";
+ * host_name == NULL resets every switch.  Names: gather_bm, gather_kc, gather_nloop,
+ * gather_halo, gather_split, gather_sa, gather_wide, gather_res, dense_res, direct,
+ * wgrad_halo, wgrad_cw, wgrad_br, wgrad_rounds.  May be called before aeth_init.  The
+ * same switches can be given once through the environment variable AETHER_TUNE
+ * ("name=value,name=value"), read by aeth_init; the library reads no other variable. */
+int aeth_debug_set(const char* host_name, int value);
+
 /* ---- memory (replaces cp.zeros / cp.asarray / .get(), cupy array ownership) - */
 int aeth_malloc(void** host_out_ptr, int64_t bytes);
 int aeth_free(void* p);

@@ -24,3 +24,17 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture
+def tune():
+    """Kernel-choice overrides of the library for one test (aeth_debug_set): `tune(gather_bm=128)`.
+    Every switch goes back to "decide from the shape" when the test ends."""
+    from aether import _lib
+
+    def set_switches(**switches):
+        for name, value in switches.items():
+            _lib.debug_set(name, value)
+
+    yield set_switches
+    _lib.debug_set(None)

@@ -113,9 +113,9 @@ HALO_CASES = [
 
 
 @pytest.mark.parametrize("case", HALO_CASES, ids=lambda c: "x".join(str(v) for v in c))
-def test_bf16_fprop_dgrad_without_split_k(case, monkeypatch):
+def test_bf16_fprop_dgrad_without_split_k(case, tune):
     from tests import abi
-    monkeypatch.setenv("AETHER_GATHER_SPLIT_OFF", "1")
+    tune(gather_split=0)
     x, w, b, dy = _case(case, 5)
     stride, pad = (case[7], case[8]), case[9]
     xr, wr, dyr = O.round_to_bf16(x), O.round_to_bf16(w), O.round_to_bf16(dy)
@@ -160,9 +160,9 @@ def _random_halo_cases(n, seed):
 
 
 @pytest.mark.parametrize("case", _random_halo_cases(28, 777), ids=lambda c: "x".join(str(v) for v in c))
-def test_bf16_random_geometries_without_split_k(case, monkeypatch):
+def test_bf16_random_geometries_without_split_k(case, tune):
     from tests import abi
-    monkeypatch.setenv("AETHER_GATHER_SPLIT_OFF", "1")
+    tune(gather_split=0)
     x, w, b, dy = _case(case, 9)
     stride, pad = (case[7], case[8]), case[9]
     xr, wr, dyr = O.round_to_bf16(x), O.round_to_bf16(w), O.round_to_bf16(dy)
@@ -175,7 +175,7 @@ def test_bf16_random_geometries_without_split_k(case, monkeypatch):
 # A filter of at most 9 taps on 64 channels and at most 64 output channels stays in LDS whole: one
 # persistent workgroup per CU, one wave fetching the source pixels of the next 224-row tile while
 # seven multiply the current one.  Tiles are whole image rows (the width divides 224).  The library
-# takes that kernel from 4 tiles per CU on; AETHER_GATHER_RES=1 lets small inputs reach it.
+# takes that kernel from 4 tiles per CU on; the gather_res switch lets small inputs reach it.
 RES_CASES = [
     (2, 56, 56, 64, 64, 3, 3, 1, 1, "same"),      # the 56x56x64 layer: 14 tiles of 4 image rows per image
     (3, 28, 28, 64, 64, 3, 3, 1, 1, "same"),      # 784 pixels per image: the fourth tile is half empty
@@ -191,10 +191,10 @@ RES_CASES = [
 
 
 @pytest.mark.parametrize("case", RES_CASES, ids=lambda c: "x".join(str(v) for v in c))
-def test_bf16_fprop_dgrad_with_the_filter_resident_in_lds(case, monkeypatch):
+def test_bf16_fprop_dgrad_with_the_filter_resident_in_lds(case, tune):
     from tests import abi
-    monkeypatch.setenv("AETHER_GATHER_SPLIT_OFF", "1")
-    monkeypatch.setenv("AETHER_GATHER_RES", "1")
+    tune(gather_split=0)
+    tune(gather_res=1)
     x, w, b, dy = _case(case, 11)
     stride, pad = (case[7], case[8]), case[9]
     xr, wr, dyr = O.round_to_bf16(x), O.round_to_bf16(w), O.round_to_bf16(dy)
@@ -204,13 +204,13 @@ def test_bf16_fprop_dgrad_with_the_filter_resident_in_lds(case, monkeypatch):
     dx = abi.dgrad_bf16(dy, w, x.shape, stride, pad)
     abi.close(dx, O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
     # the same sums of the same products in another order of taps and tiles
-    monkeypatch.setenv("AETHER_GATHER_RES", "0")
+    tune(gather_res=0)
     abi.close(abi.fprop_bf16(x, w, b, stride, pad), got, rtol=1e-5, atol=1e-5)
 
 
 # bf16 launches outside the halo kernels (strides, 1x1, more than 64 channels in) with more than 64 output
 # channels use tiles of 256 x 128 or 256 x 256 on 8 waves.  The library takes them from 2 tiles per CU on;
-# AETHER_GATHER_WIDE=1 lets small inputs reach them, =0 gives the 4-wave tiles: the same sums in the same order.
+# the gather_wide switch lets small inputs reach them, at 0 it gives the 4-wave tiles: the same sums in the same order.
 WIDE_CASES = [
     (4, 28, 28, 128, 256, 3, 3, 2, 2, "valid"),   # the stride-2 layer: 256 x 256 tiles; dgrad: 256 x 128 per class
     (3, 15, 15, 64, 200, 3, 3, 2, 2, "same"),     # ragged n tile of 256 (channels 200 .. 255 read as zero)
@@ -222,10 +222,10 @@ WIDE_CASES = [
 
 
 @pytest.mark.parametrize("case", WIDE_CASES, ids=lambda c: "x".join(str(v) for v in c))
-def test_bf16_fprop_dgrad_with_wide_tiles_on_eight_waves(case, monkeypatch):
+def test_bf16_fprop_dgrad_with_wide_tiles_on_eight_waves(case, tune):
     from tests import abi
-    monkeypatch.setenv("AETHER_GATHER_SPLIT_OFF", "1")
-    monkeypatch.setenv("AETHER_GATHER_WIDE", "1")
+    tune(gather_split=0)
+    tune(gather_wide=1)
     x, w, b, dy = _case(case, 13)
     stride, pad = (case[7], case[8]), case[9]
     xr, wr, dyr = O.round_to_bf16(x), O.round_to_bf16(w), O.round_to_bf16(dy)
@@ -234,7 +234,7 @@ def test_bf16_fprop_dgrad_with_wide_tiles_on_eight_waves(case, monkeypatch):
     abi.close(abi.fprop_bf16(x, w, None, stride, pad), O.conv_fprop(xr, wr, None, stride, pad, dtype=np.float64))
     dx = abi.dgrad_bf16(dy, w, x.shape, stride, pad)
     abi.close(dx, O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
-    monkeypatch.setenv("AETHER_GATHER_WIDE", "0")
+    tune(gather_wide=0)
     assert np.array_equal(y, abi.fprop_bf16(x, w, b, stride, pad))
     assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
 
@@ -242,7 +242,7 @@ def test_bf16_fprop_dgrad_with_wide_tiles_on_eight_waves(case, monkeypatch):
 # wgrad of a unit-stride filter of at most 9 taps on 64 input channels and at most 64 output channels:
 # one persistent workgroup per CU keeps the whole K x N result in registers (a wave per tap) and a
 # loading wave brings slabs of whole output rows with the padded source rows under them.  The library
-# takes that kernel from 4 slabs per CU on; AETHER_WGRAD_HALO=1 lets small inputs reach it.
+# takes that kernel from 4 slabs per CU on; the wgrad_halo switch lets small inputs reach it.
 WGRAD_HALO_CASES = [
     (2, 56, 56, 64, 64, 3, 3, 1, 1, "same"),      # slabs of 2 rows of 56
     (3, 28, 28, 64, 64, 3, 3, 1, 1, "same"),      # 4 rows of 28
@@ -257,9 +257,9 @@ WGRAD_HALO_CASES = [
 
 
 @pytest.mark.parametrize("case", WGRAD_HALO_CASES, ids=lambda c: "x".join(str(v) for v in c))
-def test_bf16_wgrad_with_the_whole_result_in_registers(case, monkeypatch):
+def test_bf16_wgrad_with_the_whole_result_in_registers(case, tune):
     from tests import abi
-    monkeypatch.setenv("AETHER_WGRAD_HALO", "1")
+    tune(wgrad_halo=1)
     x, w, b, dy = _case(case, 13)
     stride, pad = (case[7], case[8]), case[9]
     xr, dyr = O.round_to_bf16(x), O.round_to_bf16(dy)
@@ -269,7 +269,7 @@ def test_bf16_wgrad_with_the_whole_result_in_registers(case, monkeypatch):
     dw2, db2 = abi.wgrad_bf16(x, dy, w.shape, stride, pad)
     assert np.array_equal(dw, dw2) and np.array_equal(db, db2)            # deterministic
     # the same sums of the same products in another order
-    monkeypatch.setenv("AETHER_WGRAD_HALO", "0")
+    tune(wgrad_halo=0)
     dw3, db3 = abi.wgrad_bf16(x, dy, w.shape, stride, pad)
     abi.close(dw3, dw, rtol=1e-4, atol=1e-5, rms_scaled=True)
     abi.close(db3, db, rtol=1e-4, atol=1e-5, rms_scaled=True)

@@ -186,9 +186,9 @@ NLOOP_CASES = [
 
 
 @pytest.mark.parametrize("case", NLOOP_CASES, ids=lambda c: "x".join(str(v) for v in c))
-def test_fprop_parity_with_128_row_tiles(case, monkeypatch):
+def test_fprop_parity_with_128_row_tiles(case, tune):
     from tests import abi
-    monkeypatch.setenv("AETHER_GATHER_BM", "128")
+    tune(gather_bm=128)
     x, w, b, dy = _case(case, 11)
     stride, pad = (case[7], case[8]), case[9]
     want = O.conv_fprop(x, w, b, stride, pad, dtype=np.float64)
@@ -199,7 +199,7 @@ def test_fprop_parity_with_128_row_tiles(case, monkeypatch):
 
 # Plain matrix products with a short K (32 or 64) and a wide output (up to 256 columns, e.g. the 1x1
 # convolution 64 -> 256): one persistent workgroup per CU with the whole filter in LDS.  The library
-# takes that kernel from 4 tiles of 128 rows per CU on; AETHER_DENSE_RES=1 lets small inputs reach it.
+# takes that kernel from 4 tiles of 128 rows per CU on; the dense_res switch lets small inputs reach it.
 DENSE_RES_CASES = [
     (8, 48, 48, 64, 256, 1, 1, 1, 1, "valid"),    # 144 tiles: one each
     (8, 48, 48, 32, 192, 1, 1, 1, 1, "valid"),    # one slab, 3 n tiles: two waves have nothing to multiply
@@ -213,22 +213,22 @@ DENSE_RES_CASES = [
 
 
 @pytest.mark.parametrize("case", DENSE_RES_CASES, ids=lambda c: "x".join(str(v) for v in c))
-def test_fprop_with_the_filter_resident_in_lds(case, monkeypatch):
+def test_fprop_with_the_filter_resident_in_lds(case, tune):
     from tests import abi
-    monkeypatch.setenv("AETHER_DENSE_RES", "1")
+    tune(dense_res=1)
     x, w, b, dy = _case(case, 12)
     stride, pad = (case[7], case[8]), case[9]
     got = abi.fprop(x, w, b, stride, pad)
     abi.close(got, O.conv_fprop(x, w, b, stride, pad, dtype=np.float64))
     abi.close(abi.fprop(x, w, None, stride, pad), O.conv_fprop(x, w, None, stride, pad, dtype=np.float64))
     # the other kernels add the same products in the same order of k
-    monkeypatch.setenv("AETHER_DENSE_RES", "0")
+    tune(dense_res=0)
     assert np.array_equal(got, abi.fprop(x, w, b, stride, pad))
 
 
 # fp32 gathers whose slabs lie inside one tap load with addresses made on the scalar unit: lane offsets
 # that are constants of the tile, counted from a base the padding below the tensor, the tap in the scalar
-# offset, rows outside the image told by one ballot per slab.  AETHER_GATHER_SA=0 is the form with vector
+# offset, rows outside the image told by one ballot per slab.  the gather_sa switch at 0 is the form with vector
 # address arithmetic; both must give the same bits.
 SA_CASES = [
     (2, 12, 12, 32, 64, 5, 5, 1, 1, "same"),      # padding 2: the base lies 2 rows and 2 pixels below the tensor
@@ -244,53 +244,17 @@ SA_CASES = [
 
 @pytest.mark.parametrize("bm", ["64", "128"])
 @pytest.mark.parametrize("case", SA_CASES, ids=lambda c: "x".join(str(v) for v in c))
-def test_fprop_dgrad_with_scalar_addressed_loads(case, bm, monkeypatch):
+def test_fprop_dgrad_with_scalar_addressed_loads(case, bm, tune):
     from tests import abi
-    monkeypatch.setenv("AETHER_GATHER_BM", bm)
-    monkeypatch.setenv("AETHER_GATHER_SPLIT_OFF", "1")
+    tune(gather_bm=int(bm))
+    tune(gather_split=0)
     x, w, b, dy = _case(case, 16)
     stride, pad = (case[7], case[8]), case[9]
     y = abi.fprop(x, w, b, stride, pad)
     abi.close(y, O.conv_fprop(x, w, b, stride, pad, dtype=np.float64))
     dx = abi.dgrad(dy, w, x.shape, stride, pad)
     abi.close(dx, O.conv_dgrad(dy, w, x.shape[1:3], stride, pad, dtype=np.float64))
-    monkeypatch.setenv("AETHER_GATHER_SA", "0")
-    assert np.array_equal(y, abi.fprop(x, w, b, stride, pad))
-    assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
-
-
-# fp32 gathers as resident workgroups that walk 128 x 64 tiles, the slab loop running through the tile
-# boundaries.  The kernel is a tuning switch (AETHER_GATHER_PERSIST=1, with AETHER_GATHER_BM=128 for
-# inputs that would get other tiles); AETHER_GATHER_PERSIST_WGS gives a workgroup several tiles.
-PERSIST_CASES = [
-    ((4, 56, 56, 64, 64, 3, 3, 1, 1, "same"), 24),      # 98 tiles on 24 workgroups: 4 each and 2 more
-    ((4, 56, 56, 64, 64, 3, 3, 1, 1, "same"), 1000),    # one tile each
-    ((3, 28, 28, 128, 128, 3, 3, 1, 1, "same"), 7),     # two n tiles per m tile, 36 slabs
-    ((3, 27, 29, 64, 72, 3, 3, 1, 1, "valid"), 5),      # ragged last m tile, 8 channels in the last n tile
-    ((2, 20, 20, 32, 64, 5, 5, 1, 1, "same"), 3),       # 25 taps = 25 slabs: the tiles change LDS buffer parity
-    ((8, 24, 24, 128, 64, 1, 1, 1, 1, "valid"), 9),     # 1x1: 4 slabs
-    ((4, 28, 28, 64, 64, 3, 3, 2, 2, "same"), 2),       # stride 2 (dgrad: four classes of dx, strided output rows)
-    ((2, 40, 40, 96, 64, 3, 3, 1, 1, "same"), 8),       # 3 slabs per tap
-    ((2, 20, 20, 16, 64, 3, 3, 1, 1, "same"), 8),       # 16 channels: the one-tile kernels
-]
-
-
-@pytest.mark.parametrize("case,wgs", PERSIST_CASES, ids=lambda c: "x".join(str(v) for v in c) if isinstance(c, tuple) else "wgs%d" % c)
-def test_fprop_dgrad_with_resident_workgroups_walking_tiles(case, wgs, monkeypatch):
-    from tests import abi
-    monkeypatch.setenv("AETHER_GATHER_BM", "128")
-    monkeypatch.setenv("AETHER_GATHER_PERSIST", "1")
-    monkeypatch.setenv("AETHER_GATHER_PERSIST_WGS", str(wgs))
-    x, w, b, dy = _case(case, 15)
-    stride, pad = (case[7], case[8]), case[9]
-    y = abi.fprop(x, w, b, stride, pad)
-    abi.close(y, O.conv_fprop(x, w, b, stride, pad, dtype=np.float64))
-    y0 = abi.fprop(x, w, None, stride, pad)
-    abi.close(y0, O.conv_fprop(x, w, None, stride, pad, dtype=np.float64))
-    dx = abi.dgrad(dy, w, x.shape, stride, pad)
-    abi.close(dx, O.conv_dgrad(dy, w, x.shape[1:3], stride, pad, dtype=np.float64))
-    # the one-tile kernel adds the same products in the same order
-    monkeypatch.setenv("AETHER_GATHER_PERSIST", "0")
+    tune(gather_sa=0)
     assert np.array_equal(y, abi.fprop(x, w, b, stride, pad))
     assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
 
@@ -299,7 +263,7 @@ def test_fprop_dgrad_with_resident_workgroups_walking_tiles(case, wgs, monkeypat
 # channels, on rows of 28, 32, 56 or 64 output pixels: one persistent workgroup per CU keeps the whole
 # K x N result in registers (12 multiplying waves of three 32 x 32 blocks) and a loading wave brings one
 # output row and the padded source rows under it at a time.  The library takes that kernel from 4 rows
-# per CU on; AETHER_WGRAD_HALO=1 lets small inputs reach it.
+# per CU on; the wgrad_halo switch lets small inputs reach it.
 WGRAD_HALO_F32_CASES = [
     (2, 56, 56, 64, 64, 3, 3, 1, 1, "same"),      # the 56x56x64 layer
     (3, 28, 28, 64, 64, 3, 3, 1, 1, "same"),
@@ -313,9 +277,9 @@ WGRAD_HALO_F32_CASES = [
 
 
 @pytest.mark.parametrize("case", WGRAD_HALO_F32_CASES, ids=lambda c: "x".join(str(v) for v in c))
-def test_wgrad_with_the_whole_result_in_registers(case, monkeypatch):
+def test_wgrad_with_the_whole_result_in_registers(case, tune):
     from tests import abi
-    monkeypatch.setenv("AETHER_WGRAD_HALO", "1")
+    tune(wgrad_halo=1)
     x, w, b, dy = _case(case, 14)
     stride, pad = (case[7], case[8]), case[9]
     dw, db = abi.wgrad(x, dy, w.shape, stride, pad)
