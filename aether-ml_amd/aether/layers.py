@@ -12,7 +12,10 @@ Departures from the reference, each deliberate:
     "same" (the reference slices ``[:, 0:-0]`` to an empty array, :149-151);
   * ``Conv_Layer.set_parameters`` refreshes the ``weights`` alias (:159-161 does not);
   * ``Pooling(padding="same")`` raises ValueError (the reference reads ``H_out``
-    before assigning it, :226-228).
+    before assigning it, :226-228);
+  * 2-D ``y_true`` must be one-hot rows (they are reduced to class indices for the
+    loss kernels).  The reference multiplies a 2-D ``y_true`` in as given (:622-626,
+    :672-676), so soft or pre-smoothed targets work there; here they raise ValueError.
 """
 import os
 
@@ -542,10 +545,18 @@ class SoftMax:
 # Loss  (CNN_classes_cupy.py:565-680)
 # ----------------------------------------------------------------------------------
 def _sparse_labels(y_true):
-    """int32 class indices; one-hot rows are reduced with argmax."""
+    """int32 class indices; one-hot rows are reduced with argmax.  Rows that are not
+    one-hot (soft or already smoothed targets) are refused rather than silently
+    replaced by their argmax."""
     y = np.asarray(y_true)
     if y.ndim == 2:
-        y = np.argmax(y, axis=1)
+        idx = np.argmax(y, axis=1)
+        onehot = np.zeros(y.shape, dtype=y.dtype)
+        onehot[np.arange(y.shape[0]), idx] = 1
+        if not np.array_equal(y, onehot):
+            raise ValueError("2-D y_true must hold one-hot rows: soft or pre-smoothed targets are not supported "
+                             "(use class indices and the loss's label_smoothing)")
+        y = idx
     return np.ascontiguousarray(y, dtype=np.int32)
 
 

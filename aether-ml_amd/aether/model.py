@@ -1,8 +1,9 @@
-"""Model orchestrator with the reference's method names and behaviour
-(CNN/models/CNN_model_cupy.py:5-392): layer chain, batching loop, loss/accuracy
-bookkeeping and the printed progress lines.  Batches are sliced on the host and
-uploaded once; every activation then stays in HBM until the three printed
-scalars are read back.
+"""Model orchestrator with the reference's method names, signatures, attribute
+protocol and printed progress lines (CNN/models/CNN_model_cupy.py:5-392).  How the
+layer chain is linked and how batches are cut is this module's own: one batch
+iterator serves train / evaluate / predict, one step function serves eager and
+recorded steps.  Batches are sliced on the host and uploaded once; every activation
+then stays in HBM until the three printed scalars are read back.
 
 Parameter files written by ``save_parameters`` hold plain NumPy arrays (a list
 of per-layer tuples, the reference's structure).  ``load_parameters`` reads them
@@ -13,6 +14,7 @@ anything else from it.
 """
 import io
 import pickle
+import warnings
 
 import numpy as np
 
@@ -85,6 +87,28 @@ def write_parameters(params, path, cupy_arrays=False):
             pickle.dump(host, f, protocol=4)
 
 
+def _batches(n_rows, batch_size):
+    """Row ranges of one pass over `n_rows` samples: the whole set when no batch size is
+    given, else consecutive batches with a shorter last one (CNN_model_cupy.py:81-92)."""
+    if batch_size is None:
+        yield slice(None)
+        return
+    for start in range(0, n_rows, batch_size):
+        yield slice(start, start + batch_size)
+
+
+def _rows(a, span):
+    """`a[span]`, or `a` itself for the whole set (which may then be a DeviceTensor)."""
+    return a if span == slice(None) else a[span]
+
+
+def _progress(prefix, accuracy, loss, data_loss, regularization_loss, lr):
+    """The reference's training line (CNN_model_cupy.py:127-133, :142-147), unbalanced
+    bracket and doubled colon included."""
+    return (f'{prefix}acc: {accuracy:.3f}, loss: {loss:.3f} (data_loss: {data_loss:.3f}, '
+            f'reg_loss: {regularization_loss:.3f}, lr:: {lr}')
+
+
 class Model:
     def __init__(self):
         self.layers = []
@@ -94,75 +118,44 @@ class Model:
         self.layers.append(layer)
 
     def set(self, *, loss=None, optimizer=None, accuracy=None):
-        if loss is not None:
-            self.loss = loss
-        if optimizer is not None:
-            self.optimizer = optimizer
-        if accuracy is not None:
-            self.accuracy = accuracy
+        for name, value in (("loss", loss), ("optimizer", optimizer), ("accuracy", accuracy)):
+            if value is not None:
+                setattr(self, name, value)
 
     def finalize(self):
+        """Links the chain (CNN_model_cupy.py:33-64): every layer gets .prev / .next, the
+        first hangs on a Layer_Input, the last points at the loss; layers with `weights`
+        are trainable; SoftMax + categorical cross-entropy get the fused backward."""
         self.input_layer = Layer_Input()
-        layer_count = len(self.layers)
-        self.trainable_layers = []
-        for i in range(layer_count):
-            if i == 0:
-                self.layers[i].prev = self.input_layer
-                self.layers[i].next = self.layers[i + 1]
-            elif i < layer_count - 1:
-                self.layers[i].prev = self.layers[i - 1]
-                self.layers[i].next = self.layers[i + 1]
-            else:
-                self.layers[i].prev = self.layers[i - 1]
-                self.layers[i].next = self.loss
-                self.output_layer_activation = self.layers[i]
-            if hasattr(self.layers[i], 'weights'):
-                self.trainable_layers.append(self.layers[i])
+        chain = [self.input_layer] + self.layers + [self.loss]
+        for before, layer, after in zip(chain, chain[1:], chain[2:]):
+            layer.prev, layer.next = before, after
+        self.output_layer_activation = self.layers[-1]
+        self.trainable_layers = [layer for layer in self.layers if hasattr(layer, 'weights')]
         if self.loss is not None:
             self.loss.remember_trainable_layers(self.trainable_layers)
-        if isinstance(self.layers[-1], SoftMax) and isinstance(self.loss, Loss_CategoricalCrossEntropy):
+        fused = isinstance(self.layers[-1], SoftMax) and isinstance(self.loss, Loss_CategoricalCrossEntropy)
+        if fused:
             self.softmax_classifier_output = \
                 Activation_Softmax_Loss_CategoricalCrossEntropy(self.loss.label_smoothing)
 
     def train(self, X, y, *, epochs=1, batch_size=None, print_every=1, validation_data=None):
         self.accuracy.init(y)
-        train_steps = 1
-        if validation_data is not None:
-            X_val, y_val = validation_data
-        if batch_size is not None:
-            train_steps = len(X) // batch_size
-            if train_steps * batch_size < len(X):
-                train_steps += 1
+        spans = list(_batches(len(X), batch_size))
         print("Training")
         for epoch in range(1, epochs + 1):
             print(f' epoch: {epoch}')
             self.loss.new_pass()
             self.accuracy.new_pass()
-            for step in range(train_steps):
-                if batch_size is None:
-                    batch_X = X
-                    batch_y = y
-                else:
-                    batch_X = X[step * batch_size:(step + 1) * batch_size]
-                    batch_y = y[step * batch_size:(step + 1) * batch_size]
-                loss, data_loss, regularization_loss, accuracy = self.train_step(batch_X, batch_y)
-                if not step % print_every or step == train_steps - 1:
-                    print(f'epoch: {epoch}, ' +
-                          f'acc: {accuracy:.3f}, ' +
-                          f'loss: {loss:.3f} (' +
-                          f'data_loss: {data_loss:.3f}, ' +
-                          f'reg_loss: {regularization_loss:.3f}, ' +
-                          f'lr:: {self.optimizer.current_learning_rate}')
-        epoch_data_loss, epoch_regularization_loss = \
-            self.loss.calculate_accumulated(include_regularization=True)
-        epoch_loss = epoch_data_loss + epoch_regularization_loss
-        epoch_accuracy = self.accuracy.calculate_accumulated()
-        print(f' training, ' +
-              f'acc: {epoch_accuracy:.3f}, ' +
-              f'loss: {epoch_loss:.3f} (' +
-              f'data_loss: {epoch_data_loss:.3f}, ' +
-              f'reg_loss: {epoch_regularization_loss:.3f}, ' +
-              f'lr:: {self.optimizer.current_learning_rate}')
+            for step, rows in enumerate(spans):
+                loss, data_loss, regularization_loss, accuracy = self.train_step(_rows(X, rows), _rows(y, rows))
+                if step % print_every == 0 or step == len(spans) - 1:
+                    print(_progress(f'epoch: {epoch}, ', accuracy, loss, data_loss, regularization_loss,
+                                    self.optimizer.current_learning_rate))
+        # the summary and the validation pass come once, after the last epoch (:135-151)
+        data_loss, regularization_loss = self.loss.calculate_accumulated(include_regularization=True)
+        print(_progress(' training, ', self.accuracy.calculate_accumulated(), data_loss + regularization_loss,
+                        data_loss, regularization_loss, self.optimizer.current_learning_rate))
         if validation_data is not None:
             self.evaluate(*validation_data, batch_size=batch_size)
 
@@ -178,6 +171,15 @@ class Model:
         self._record = bool(enabled)
         if not enabled:
             self._drop_recordings()
+        elif not self._can_record():
+            warnings.warn("record_steps: this model cannot be recorded (dropout masks from the host, an active "
+                          "regulariser, or no Adam / fused softmax cross-entropy); steps run eagerly",
+                          RuntimeWarning, stacklevel=2)
+
+    @property
+    def recording_active(self):
+        """True when recording was asked for AND this model's steps can be recorded."""
+        return bool(getattr(self, "_record", False)) and self._can_record()
 
     def _drop_recordings(self):
         from . import _lib
@@ -194,7 +196,7 @@ class Model:
             return False
         if any(isinstance(layer, (Layer_Dropout, Layer_Dropout_Spatial)) for layer in self.layers):
             return False                                 # their masks are drawn and uploaded by the host every step
-        return all(hasattr(l, "weight_cache") for l in self.trainable_layers)     # Adam state exists
+        return True
 
     def _recorded_step(self, batch_X, batch_y):
         import ctypes as C
@@ -204,8 +206,9 @@ class Model:
         key = (tuple(batch_X.shape), labels.shape[0])
         recs = self.__dict__.setdefault("_recordings", {})
         rec = recs.get(key)
-        if rec is None:
-            # first step of this shape: a normal one (lazy initialisations, workspace sizes)
+        if rec is None or not all(hasattr(l, "weight_cache") for l in self.trainable_layers):
+            # first step of this shape, or no Adam state yet: a normal one (lazy initialisations,
+            # workspace sizes)
             recs[key] = {"graph": None}
             return None
         lib = _lib.lib()
@@ -263,17 +266,17 @@ class Model:
         """One iteration of the loop body of ``train`` (CNN_model_cupy.py:107-126):
         forward, loss, accuracy, backward, Adam.  Returns (loss, data_loss,
         regularization_loss, accuracy)."""
-        if getattr(self, "_record", False) and self._can_record():
+        if self.recording_active:
             result = self._recorded_step(batch_X, batch_y)
             if result is not None:
                 return result
         output = self.forward(batch_X, training=True)
         # The loss kernel is queued here and read after backward and the update have been
         # queued too, so the device never idles while the host prepares the backward pass.
-        defer = self.loss.can_defer()
-        if defer:
-            pending = self.loss.launch(output, batch_y, training=True)
-        else:
+        # With an active regulariser its sums must see the weights before the update, so
+        # the loss is then read first, as the reference does.
+        pending = self.loss.launch(output, batch_y, training=True) if self.loss.can_defer() else None
+        if pending is None:
             data_loss, regularization_loss = self.loss.calculate(output, batch_y, include_regularization=True,
                                                                  training=True)
         self.backward(output, batch_y)
@@ -281,88 +284,53 @@ class Model:
         for layer in self.trainable_layers:
             self.optimizer.update_parameters(layer)
         self.optimizer.post_update_parameters()
-        if defer:
+        if pending is not None:
             data_loss, regularization_loss = self.loss.finish(pending, include_regularization=True)
-        loss = data_loss + regularization_loss
         predictions = self.output_layer_activation.predictions(output)
         accuracy = self.accuracy.calculate(predictions, batch_y)
-        return loss, data_loss, regularization_loss, accuracy
+        return data_loss + regularization_loss, data_loss, regularization_loss, accuracy
 
     def forward(self, X, training):
+        """Every layer reads its predecessor's `.output` (CNN_model_cupy.py:153-163)."""
         self.input_layer.forward(X, training)
         for layer in self.layers:
             layer.forward(layer.prev.output, training)
-        return layer.output
+        return self.layers[-1].output
 
     def backward(self, output, y):
-        if self.softmax_classifier_output is not None:
+        """Every layer reads its successor's `.dinputs` (CNN_model_cupy.py:165-193).  With the
+        fused softmax / cross-entropy the last layer's dinputs come from the fused object."""
+        if self.softmax_classifier_output is None:
+            self.loss.backward(output, y)
+            walk = self.layers
+        else:
             self.softmax_classifier_output.backward(output, y, training=True)
             self.layers[-1].dinputs = self.softmax_classifier_output.dinputs
-            for layer in reversed(self.layers[:-1]):
-                layer.backward(layer.next.dinputs)
-            return
-        self.loss.backward(output, y)
-        for layer in reversed(self.layers):
+            walk = self.layers[:-1]
+        for layer in reversed(walk):
             layer.backward(layer.next.dinputs)
-
-    def backward_debug(self, X, y):
-        out = X
-        print("Forward pass:")
-        for i, layer in enumerate(self.layers):
-            layer.forward(out, training=True)
-            out = layer.output
-            print(f"Layer {i} ({layer.__class__.__name__}) output: {out.shape}")
-        print("\nBackward pass:")
-        if self.softmax_classifier_output is not None:
-            self.softmax_classifier_output.backward(out, y)
-            self.layers[-1].dinputs = self.softmax_classifier_output.dinputs
-            chain = list(enumerate(reversed(self.layers[:-1])))
-            first = -2
-        else:
-            self.loss.backward(out, y)
-            chain = list(enumerate(reversed(self.layers)))
-            first = -1
-        for i, layer in chain:
-            layer.backward(layer.next.dinputs)
-            print(f"Layer {first - i} ({layer.__class__.__name__}) dinputs: {layer.dinputs.shape}")
-            if hasattr(layer, 'dweights'):
-                print(f"             dweights: {layer.dweights.shape}")
-            if hasattr(layer, 'dbiases'):
-                print(f"             dbiases: {layer.dbiases.shape}")
 
     def evaluate(self, X_val, y_val, *, batch_size=None):
-        validation_steps = 1
-        if batch_size is not None:
-            validation_steps = len(X_val) // batch_size
-            if validation_steps * batch_size < len(X_val):
-                validation_steps += 1
         self.loss.new_pass()
         self.accuracy.new_pass()
-        for step in range(validation_steps):
-            if batch_size is None:
-                batch_X = X_val
-                batch_y = y_val
-            else:
-                batch_X = X_val[step * batch_size:(step + 1) * batch_size]
-                batch_y = y_val[step * batch_size:(step + 1) * batch_size]
-            output = self.forward(batch_X, training=False)
+        for rows in _batches(len(X_val), batch_size):
+            batch_y = _rows(y_val, rows)
+            output = self.forward(_rows(X_val, rows), training=False)
             self.loss.calculate(output, batch_y, training=False)
-            predictions = self.output_layer_activation.predictions(output)
-            self.accuracy.calculate(predictions, batch_y)
+            self.accuracy.calculate(self.output_layer_activation.predictions(output), batch_y)
         validation_loss = self.loss.calculate_accumulated()
         validation_accuracy = self.accuracy.calculate_accumulated()
-        print(f'Valdiation, ' +
-              f'acc: {validation_accuracy:.3f}, ' +
-              f'loss: {validation_loss:.3f}')
+        print(f'Valdiation, acc: {validation_accuracy:.3f}, loss: {validation_loss:.3f}')
+
+    def predict(self, X, *, batch_size=None):
+        parts = [np.asarray(self.forward(_rows(X, rows), training=False)) for rows in _batches(len(X), batch_size)]
+        return np.vstack(parts)
 
     def get_parameters(self):
-        parameters = []
-        for layer in self.trainable_layers:
-            parameters.append(layer.get_parameters())
-        return parameters
+        return [layer.get_parameters() for layer in self.trainable_layers]
 
     def set_parameters(self, parameters):
-        for parameter_set, layer in zip(parameters, self.trainable_layers):
+        for layer, parameter_set in zip(self.trainable_layers, parameters):
             layer.set_parameters(*parameter_set)
 
     def save_parameters(self, path, cupy_arrays=False):
@@ -381,50 +349,23 @@ class Model:
         raise NotImplementedError(
             "whole-model pickles are not supported (device buffers cannot be pickled); use load_parameters")
 
-    def predict(self, X, *, batch_size=None):
-        prediction_steps = 1
-        if batch_size is not None:
-            prediction_steps = len(X) // batch_size
-            if prediction_steps * batch_size < len(X):
-                prediction_steps += 1
-        output = []
-        for step in range(prediction_steps):
-            if batch_size is None:
-                batch_X = X
-            else:
-                batch_X = X[step * batch_size:(step + 1) * batch_size]
-            batch_output = self.forward(batch_X, training=False)
-            output.append(np.asarray(batch_output))
-        return np.vstack(output)
-
 
 class Accuracy:
-    def calculate(self, predictions, y):
-        comparisons = self.compare(predictions, y)
-        accuracy = np.mean(comparisons)
-        self.accumulated_sum += np.sum(comparisons)
-        self.accumulated_count += len(comparisons)
-        return accuracy
-
-    def calculate_accumulated(self):
-        accuracy = self.accumulated_sum / self.accumulated_count
-        return accuracy
+    """Running share of correct predictions (CNN_model_cupy.py:344-366): subclasses say
+    what "correct" means through ``compare``."""
 
     def new_pass(self):
         self.accumulated_sum = 0
         self.accumulated_count = 0
 
+    def calculate(self, predictions, y):
+        hits = self.compare(predictions, y)
+        self.accumulated_sum += np.sum(hits)
+        self.accumulated_count += len(hits)
+        return np.mean(hits)
 
-class Accuracy_Regression(Accuracy):
-    def __init__(self):
-        self.precision = None
-
-    def init(self, y, reinit=False):
-        if self.precision is None or reinit:
-            self.precision = np.std(np.asarray(y)) / 250
-
-    def compare(self, predictions, y):
-        return np.absolute(np.asarray(predictions) - np.asarray(y)) < self.precision
+    def calculate_accumulated(self):
+        return self.accumulated_sum / self.accumulated_count
 
 
 class Accuracy_Categorical(Accuracy):
@@ -433,9 +374,8 @@ class Accuracy_Categorical(Accuracy):
 
     def compare(self, predictions, y):
         y = np.asarray(y)
-        if len(y.shape) == 2:
-            y = np.argmax(y, axis=1)
-        return np.asarray(predictions) == y
+        labels = np.argmax(y, axis=1) if y.ndim == 2 else y
+        return np.asarray(predictions) == labels
 
 
 class Layer_Input:

@@ -94,3 +94,18 @@ def test_product_package_does_not_import_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text, os.path.join(dirpath, f)
+
+
+def test_two_dimensional_targets_must_be_one_hot():
+    """Host logic of the loss: one-hot rows become class indices, anything softer is refused
+    (the loss kernels take indices; the reference would use the rows as given)."""
+    import numpy as np
+    import pytest
+    from aether.layers import _sparse_labels
+    y = np.array([2, 0, 1])
+    assert _sparse_labels(y).dtype == np.int32 and list(_sparse_labels(y)) == [2, 0, 1]
+    assert list(_sparse_labels(np.eye(3)[y])) == [2, 0, 1]
+    with pytest.raises(ValueError):
+        _sparse_labels(np.eye(3)[y] * 0.9 + 0.1 / 3)
+    with pytest.raises(ValueError):
+        _sparse_labels(np.array([[1.0, 1.0, 0.0]]))
