@@ -25,6 +25,10 @@ What pins each function (see tests/test_oracle_*.py):
   batch norm  -- torch batch_norm + invariants
   softmax/CCE -- torch cross_entropy(label_smoothing)
   adam        -- torch.optim.Adam(eps=1e-7), step-1 closed form
+  dropout, regularization_loss, learning-rate decay, the L2 terms of dense_backward
+              -- three steps of OracleCNN with masks, L2 and decay against a torch
+                 graph (masks as multiplications, the penalty as a term of the loss,
+                 torch.optim.Adam stepped at lr/(1+decay*t))
 """
 from __future__ import annotations
 
@@ -443,34 +447,86 @@ def bf16_bits(a):
 
 
 # ----------------------------------------------------------------------------
+# dropout and the regulariser term of the loss
+# ----------------------------------------------------------------------------
+def dropout_forward(x, mask):
+    """Layer_Dropout / Layer_Dropout_Spatial in training (cupy:375-377, :396-399):
+    output = inputs * mask, where the mask already holds Bernoulli(keep)/keep.
+    Elementwise dropout passes a mask of the input's shape, spatial dropout one of
+    shape (1,1,1,C) that every sample and pixel shares."""
+    return x * np.asarray(mask, dtype=x.dtype)
+
+
+def dropout_backward(dy, mask):
+    """dinputs = dvalues * mask (cupy:381-382, :402-403)."""
+    return dy * np.asarray(mask, dtype=dy.dtype)
+
+
+def regularization_loss(weights, biases, wl1=0.0, wl2=0.0, bl1=0.0, bl2=0.0):
+    """One layer's share of Loss.regularization_loss (cupy:593-609):
+    l1*sum|w| + l2*sum w^2 for weights and biases, each term only when its
+    coefficient is positive."""
+    w = np.asarray(weights)
+    b = np.asarray(biases)
+    r = 0.0
+    if wl1 > 0:
+        r += wl1 * np.sum(np.abs(w))
+    if wl2 > 0:
+        r += wl2 * np.sum(w * w)
+    if bl1 > 0:
+        r += bl1 * np.sum(np.abs(b))
+    if bl2 > 0:
+        r += bl2 * np.sum(b * b)
+    return float(r)
+
+
+# ----------------------------------------------------------------------------
 # The three-block CNN of the headline training step, as a plain function chain
-# (topology: CNN/architectures/CNN_cifar1.py:19-47 without the dropout layers)
+# (topology: CNN/architectures/CNN_cifar1.py:19-47; the dropout layers and the
+# regulariser of that script are optional)
 # ----------------------------------------------------------------------------
 class OracleCNN:
-    """Conv(32)-BN-ReLU-Pool, Conv(64)-BN-ReLU-Pool, Conv(128)-BN-ReLU-Pool,
-    Flatten, Dense(256) LeakyReLU(0.01), Dense(10), softmax CCE, Adam.
+    """Conv(32)-BN-ReLU-Pool, Conv(64)-BN-ReLU-[SpatialDropout]-Pool,
+    Conv(128)-BN-ReLU-[SpatialDropout]-Pool, Flatten, Dense(256) LeakyReLU(0.01)
+    [Dropout], Dense(10), softmax CCE, Adam.
 
     ``params`` is the list of per-layer tuples in trainable-layer order
     (conv W,b / bn gamma,beta,rm,rv / dense W,b), all float arrays of
     ``dtype``.  ``step`` performs forward, loss, backward and the Adam update
     and returns a dict of every intermediate a parity test wants.
+
+    The shipped recipe (CNN_cifar1.py:30,38,43,45,51) adds spatial dropout behind
+    the ReLU of blocks 2 and 3, elementwise dropout behind the leaky ReLU, an L2
+    penalty on Dense-1's weights and biases and learning-rate decay.  Masks are
+    passed per step as ``masks={"spatial1": (1,1,1,64), "spatial2": (1,1,1,128),
+    "dense": (S,256)}`` (values Bernoulli(keep)/keep, any of them optional); the
+    L2 coefficients as ``dense1_l2=(weight_l2, bias_l2)``.
     """
 
     def __init__(self, params, label_smoothing=0.01, lr=1e-3, decay=0.0, dtype=np.float32,
-                 eps_bn=1e-5, momentum=0.9):
+                 eps_bn=1e-5, momentum=0.9, dense1_l2=(0.0, 0.0)):
         self.dt = dtype
         self.p = [[np.array(a, dtype=dtype) for a in tup] for tup in params]
         self.ls = label_smoothing
         self.lr = lr
         self.decay = decay
         self.iterations = 0
+        self.current_lr = lr
         self.eps_bn = eps_bn
         self.momentum = momentum
+        self.dense1_l2 = tuple(dense1_l2)
         self.m = [[np.zeros_like(a) for a in tup[:2]] for tup in self.p]
         self.v = [[np.zeros_like(a) for a in tup[:2]] for tup in self.p]
 
-    def forward(self, X, training=True):
+    def regularization_loss(self):
+        """Loss.regularization_loss over the trainable layers (cupy:593-609): only
+        Dense-1 carries coefficients in this network."""
+        W, b = self.p[6]
+        return regularization_loss(W, b, wl2=self.dense1_l2[0], bl2=self.dense1_l2[1])
+
+    def forward(self, X, training=True, masks=None):
         dt = self.dt
+        masks = masks or {}
         a = np.asarray(X, dtype=dt)
         cache = {}
         li = 0
@@ -491,6 +547,10 @@ class OracleCNN:
             cache[f"bn{blk}_out"] = a
             cache[f"relu{blk}_in"] = a
             a = relu_forward(a)
+            mask = masks.get(f"spatial{blk}") if training else None
+            cache[f"spatial{blk}"] = mask
+            if mask is not None:
+                a = dropout_forward(a, np.asarray(mask).reshape(1, 1, 1, -1)).astype(dt)
             pooled, idx = maxpool_forward(a, dtype=dt)
             cache[f"pool{blk}"] = (idx, a.shape)
             a = pooled.astype(dt)
@@ -503,6 +563,10 @@ class OracleCNN:
         a = dense_forward(a, W, b, dtype=dt)
         cache["leaky_in"] = a
         a = leaky_relu_forward(a, 0.01).astype(dt)
+        mask = masks.get("dense") if training else None
+        cache["dense_mask"] = mask
+        if mask is not None:
+            a = dropout_forward(a, mask).astype(dt)
         W, b = self.p[li + 1]
         cache["d1_in"] = a
         a = dense_forward(a, W, b, dtype=dt)
@@ -511,11 +575,12 @@ class OracleCNN:
         cache["probs"] = probs
         return probs, cache
 
-    def step(self, X, y):
+    def step(self, X, y, masks=None):
         dt = self.dt
-        probs, c = self.forward(X, training=True)
+        probs, c = self.forward(X, training=True, masks=masks)
         losses = cce_forward(probs, y, self.ls, training=True)
         loss = float(np.mean(losses))
+        reg_loss = self.regularization_loss()            # with the parameters before the update (model_cupy:113-115)
         acc = float(np.mean(np.argmax(probs, axis=1) == y))
         grads = [None] * len(self.p)
         d = softmax_cce_backward(probs, y, self.ls).astype(dt)
@@ -524,16 +589,20 @@ class OracleCNN:
         W, b = self.p[li]
         dw, db, d = dense_backward(c["d1_in"], W, b, d, dtype=dt)
         grads[li] = (dw, db)
+        if c["dense_mask"] is not None:
+            d = dropout_backward(d, c["dense_mask"]).astype(dt)
         d = leaky_relu_backward(c["leaky_in"], d, 0.01)
         li -= 1
         W, b = self.p[li]
-        dw, db, d = dense_backward(c["d0_in"], W, b, d, dtype=dt)
+        dw, db, d = dense_backward(c["d0_in"], W, b, d, wl2=self.dense1_l2[0], bl2=self.dense1_l2[1], dtype=dt)
         grads[li] = (dw, db)
         d = d.reshape(c["flat_shape"])
         dinputs = {}
         for blk in (2, 1, 0):
             idx, shp = c[f"pool{blk}"]
             d = maxpool_backward(d, idx, shp, dtype=dt)
+            if c[f"spatial{blk}"] is not None:
+                d = dropout_backward(d, np.asarray(c[f"spatial{blk}"]).reshape(1, 1, 1, -1)).astype(dt)
             d = relu_backward(c[f"relu{blk}_in"], d)
             li -= 1
             g = self.p[li][0]
@@ -549,7 +618,8 @@ class OracleCNN:
             dinputs[f"conv{blk}"] = d
         lr = self.lr
         if self.decay:
-            lr = self.lr * (1.0 / (1.0 + self.decay * self.iterations))
+            lr = self.lr * (1.0 / (1.0 + self.decay * self.iterations))      # pre_update_parameters, cupy:695-697
+        self.current_lr = lr
         for i, tup in enumerate(self.p):
             for j in range(2):
                 gj = grads[i][j].reshape(tup[j].shape)
@@ -558,7 +628,8 @@ class OracleCNN:
                 self.m[i][j] = m.astype(dt)
                 self.v[i][j] = v.astype(dt)
         self.iterations += 1
-        return {"loss": loss, "acc": acc, "probs": probs, "grads": grads, "dinputs": dinputs, "cache": c}
+        return {"loss": loss, "reg_loss": reg_loss, "acc": acc, "probs": probs, "grads": grads, "dinputs": dinputs,
+                "cache": c, "lr": lr}
 
 
 def make_cnn_params(rng_module=np.random, dtype=np.float32, in_ch=3, hw=32):

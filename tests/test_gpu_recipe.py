@@ -1,0 +1,130 @@
+"""Whole training steps of the reference's shipped CIFAR recipe
+(CNN/architectures/CNN_cifar1.py:19-55) on the GPU against the float64 oracle:
+Conv(32)-BN-ReLU-Pool, Conv(64)-BN-ReLU-SpatialDropout(0.075)-Pool,
+Conv(128)-BN-ReLU-SpatialDropout(0.1)-Pool, Flatten, Dense(2048,256; L2 2e-5 on weights
+and biases)-LeakyReLU(0.01)-Dropout(0.075), Dense(256,10), softmax cross-entropy with
+label smoothing 0.01, Adam(lr 1e-3, decay 5e-5), batch 128.
+
+Dropout masks are drawn on the host with the reference's shapes ((1,1,1,C)/keep and
+elementwise/keep) and handed to both sides (`fixed_mask` on the layers, `masks=` on the
+oracle), a fresh set every step.  Tolerances as in tests/test_gpu_model.py."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from tests.test_gpu_model import host_params, outside_share, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def cifar1_model(aether):
+    m = aether.Model()
+    m.add(aether.Conv_Layer(input_shape=(32, 32, 3), num_filters=32, filter_size=(3, 3), strides=(1, 1), padding="same"))
+    m.add(aether.Batch_Norm(epsilon=1e-5, momentum=0.9))
+    m.add(aether.ReLU())
+    m.add(aether.Pooling(filter_size=(2, 2), strides=(2, 2), padding="valid", pooling_type="max"))
+    m.add(aether.Conv_Layer(input_shape=(16, 16, 32), num_filters=64, filter_size=(3, 3), strides=(1, 1), padding="same"))
+    m.add(aether.Batch_Norm(epsilon=1e-5, momentum=0.9))
+    m.add(aether.ReLU())
+    m.add(aether.Layer_Dropout_Spatial(rate=0.075))
+    m.add(aether.Pooling(filter_size=(2, 2), strides=(2, 2), padding="valid", pooling_type="max"))
+    m.add(aether.Conv_Layer(input_shape=(8, 8, 64), num_filters=128, filter_size=(3, 3), strides=(1, 1), padding="same"))
+    m.add(aether.Batch_Norm(epsilon=1e-5, momentum=0.9))
+    m.add(aether.ReLU())
+    m.add(aether.Layer_Dropout_Spatial(rate=0.1))
+    m.add(aether.Pooling(filter_size=(2, 2), strides=(2, 2), padding="valid", pooling_type="max"))
+    m.add(aether.Flatten())
+    m.add(aether.Layer_Dense(4 * 4 * 128, n_neurons=256, weight_regularizer_l2=2e-5, bias_regularizer_l2=2e-5))
+    m.add(aether.Leaky_ReLU(alpha=0.01))
+    m.add(aether.Layer_Dropout(rate=0.075))
+    m.add(aether.Layer_Dense(256, 10))
+    m.add(aether.SoftMax())
+    m.set(loss=aether.Loss_CategoricalCrossEntropy(label_smoothing=0.01),
+          optimizer=aether.Optimizer_Adam(learning_rate=0.001, decay=5e-5),
+          accuracy=aether.Accuracy_Categorical())
+    m.finalize()
+    return m
+
+
+def draw_masks(rng, S):
+    """Bernoulli(keep)/keep with the reference's shapes (CNN_classes_cupy.py:375-376, :397-398)."""
+    return {"spatial1": (rng.binomial(1, 1 - 0.075, size=(1, 1, 1, 64)) / (1 - 0.075)).astype(np.float32),
+            "spatial2": (rng.binomial(1, 1 - 0.1, size=(1, 1, 1, 128)) / (1 - 0.1)).astype(np.float32),
+            "dense": (rng.binomial(1, 1 - 0.075, size=(S, 256)) / (1 - 0.075)).astype(np.float32)}
+
+
+def test_cifar1_recipe_steps_match_oracle():
+    import aether
+    from tests import abi
+    np.random.seed(0)
+    S = 128
+    X = np.random.rand(S, 32, 32, 3).astype(np.float32)
+    y = np.random.randint(0, 10, S)
+    model = cifar1_model(aether)
+    # Dense-1's fresh weights are ~1e-4 (the reference's 0.01 factor): its penalty would be
+    # 2e-5 * 0.03 and invisible next to the data loss.  Scale them so that the L2 terms matter.
+    d1 = [l for l in model.layers if isinstance(l, aether.Layer_Dense)][0]
+    d1.set_parameters(np.asarray(d1.weights) * 200, np.full((1, 256), 0.5, np.float32))
+    spatial = [l for l in model.layers if isinstance(l, aether.Layer_Dropout_Spatial)]
+    dense_drop = [l for l in model.layers if isinstance(l, aether.Layer_Dropout)][0]
+    params = host_params(model)
+    net = O.OracleCNN(params, label_smoothing=0.01, lr=1e-3, decay=5e-5, dtype=np.float64, dense1_l2=(2e-5, 2e-5))
+
+    model.record_steps(True)                                # this model cannot be recorded: the request must say so
+    assert model.recording_active is False
+    model.loss.new_pass()
+    model.accuracy.new_pass()
+    rng = np.random.RandomState(9)
+    for step in range(3):
+        masks = draw_masks(rng, S)
+        spatial[0].fixed_mask, spatial[1].fixed_mask, dense_drop.fixed_mask = \
+            masks["spatial1"], masks["spatial2"], masks["dense"]
+        ref = net.step(X, y, masks=masks)
+        loss, data_loss, reg_loss, acc = model.train_step(X, y)
+        assert ref["reg_loss"] > 1e-3                       # the penalty is visible at the printed precision
+        assert abs(data_loss - ref["loss"]) <= 1e-5 + 1e-4 * abs(ref["loss"]), (step, data_loss, ref["loss"])
+        assert abs(reg_loss - ref["reg_loss"]) <= 1e-6 + 1e-4 * ref["reg_loss"], (step, reg_loss, ref["reg_loss"])
+        assert abs(loss - (ref["loss"] + ref["reg_loss"])) <= 2e-5 + 1e-4 * abs(loss)
+        assert abs(acc - ref["acc"]) <= 1.0 / S + 1e-9
+        assert model.optimizer.current_learning_rate == pytest.approx(1e-3 / (1 + 5e-5 * step), rel=1e-12)
+        assert model.optimizer.current_learning_rate == pytest.approx(ref["lr"], rel=1e-12)
+        # the masks the layers used are the ones handed in, in the reference's shapes
+        assert np.array_equal(spatial[0].channel_mask.get(), masks["spatial1"])
+        assert np.array_equal(spatial[1].channel_mask.get(), masks["spatial2"])
+        assert np.array_equal(dense_drop.binary_mask.get(), masks["dense"])
+        probs = model.layers[-1].output.get()
+        assert rel_l2(probs, ref["probs"]) <= (1e-4 if step == 0 else 2e-3)
+        if step == 0:
+            abi.close(probs, ref["probs"])
+            for i, layer in enumerate(model.trainable_layers):
+                gw, gb = ref["grads"][i]
+                name = "%d:%s" % (i, type(layer).__name__)
+                assert rel_l2(layer.dweights.get(), gw.reshape(layer.dweights.shape)) <= 2e-4, name
+                assert outside_share(layer.dweights.get(), gw.reshape(layer.dweights.shape)) <= 1e-3, name
+                if np.linalg.norm(gb) > 1e-12:
+                    assert rel_l2(layer.dbiases.get(), gb.reshape(layer.dbiases.shape)) <= 2e-4, name
+                else:
+                    assert np.abs(layer.dbiases.get()).max() <= 1e-5, name
+            # Dense-1's gradient carries 2*lambda*W: without it the comparison above fails
+            gw = ref["grads"][6][0]
+            assert rel_l2(gw - 2 * 2e-5 * params[6][0].astype(np.float64), gw) > 1e-3
+            convs = [l for l in model.layers if isinstance(l, aether.Conv_Layer)]
+            for blk, conv in enumerate(convs):
+                want = ref["dinputs"]["conv%d" % blk]
+                assert rel_l2(conv.dinputs.get(), want) <= 2e-4, blk
+                assert outside_share(conv.dinputs.get(), want) <= 1e-3, blk
+        lr_allow = 2e-3 * (step + 1)
+        for i, layer in enumerate(model.trainable_layers):
+            got = [np.asarray(a) for a in layer.get_parameters()]
+            for j, want in enumerate(net.p[i]):
+                g = got[j].reshape(want.shape)
+                if j < 2:
+                    assert np.all(np.abs(g - want) <= lr_allow + 1e-3 * np.abs(want)), (step, i, j)
+                else:
+                    assert np.all(np.abs(g - want) <= 1e-5 + 1e-3 * np.abs(want)), (step, i, j)
+    assert model.optimizer.iterations == 3
+
+    # evaluation: dropout layers pass their input through, no smoothing
+    probs_eval, _ = net.forward(X, training=False)
+    pred = model.predict(X, batch_size=64)
+    assert rel_l2(pred, probs_eval) <= 5e-3

@@ -183,3 +183,71 @@ def test_oracle_cnn_step_matches_torch_autograd():
         for j in range(2):
             got = out["grads"][i][j].reshape(tup[j].shape)
             np.testing.assert_allclose(got, tup[j].grad.numpy(), rtol=1e-6, atol=1e-10)
+
+
+def test_oracle_cnn_recipe_step_matches_torch_autograd_and_adam():
+    """The shipped recipe (CNN/architectures/CNN_cifar1.py:19-55): spatial dropout behind
+    the ReLU of blocks 2 and 3, elementwise dropout behind the leaky ReLU, L2 on Dense-1
+    and learning-rate decay.  Pinned by a torch graph that the oracle did not write: the
+    masks enter as plain multiplications, the L2 penalty as a TERM OF THE LOSS (so autograd
+    must produce the 2*lambda*W the oracle adds to dweights by hand, and the penalty value
+    must be the oracle's regularization_loss), and the update is torch.optim.Adam stepped
+    with the decayed learning rate lr/(1 + decay*t)."""
+    np.random.seed(1)
+    S = 6
+    X = np.random.rand(S, 8, 8, 3)
+    y = np.random.randint(0, 10, S)
+    params = O.make_cnn_params(dtype=np.float64, hw=8)
+    params[6] = (params[6][0] * 100, params[6][1] + 0.3)
+    params[7] = (params[7][0] * 100, params[7][1])
+    wl2, bl2, decay, lr = 2e-2, 3e-2, 0.5, 1e-3         # large on purpose: a dropped term must show
+    net = O.OracleCNN(params, label_smoothing=0.01, lr=lr, decay=decay, dtype=np.float64, dense1_l2=(wl2, bl2))
+    r = np.random.RandomState(2)
+
+    t = lambda a: torch.from_numpy(np.array(a, dtype=np.float64)).requires_grad_(True)
+    tp = [[t(a) for a in tup[:2]] for tup in params]
+    flat = [p for tup in tp for p in tup]
+    opt = torch.optim.Adam(flat, lr=lr, betas=(0.9, 0.999), eps=1e-7)
+    for step in range(3):
+        masks = {"spatial1": r.binomial(1, 0.7, (1, 1, 1, 64)) / 0.7,
+                 "spatial2": r.binomial(1, 0.6, (1, 1, 1, 128)) / 0.6,
+                 "dense": r.binomial(1, 0.8, (S, 256)) / 0.8}
+        out = net.step(X, y, masks=masks)
+
+        a = torch.from_numpy(X).permute(0, 3, 1, 2)
+        li = 0
+        for blk in range(3):
+            W, b = tp[li]
+            a = F.conv2d(a, W.permute(3, 2, 0, 1), b, padding=1)
+            g, be = tp[li + 1]
+            a = F.relu(F.batch_norm(a, None, None, g, be, training=True, eps=1e-5))
+            if blk > 0:
+                a = a * torch.from_numpy(masks["spatial%d" % blk]).reshape(1, -1, 1, 1)
+            a = F.max_pool2d(a, 2)
+            li += 2
+        a = a.permute(0, 2, 3, 1).reshape(S, -1)
+        a = F.leaky_relu(a @ tp[6][0] + tp[6][1], 0.01) * torch.from_numpy(masks["dense"])
+        logits = a @ tp[7][0] + tp[7][1]
+        data = F.cross_entropy(logits, torch.from_numpy(y), label_smoothing=0.01)
+        penalty = wl2 * (tp[6][0] ** 2).sum() + bl2 * (tp[6][1] ** 2).sum()
+        opt.zero_grad()
+        (data + penalty).backward()
+        assert abs(out["loss"] - data.item()) < 1e-9
+        assert abs(out["reg_loss"] - penalty.item()) < 1e-12 and out["reg_loss"] > 1e-3
+        for i, tup in enumerate(tp):
+            for j in range(2):
+                got = out["grads"][i][j].reshape(tup[j].shape)
+                np.testing.assert_allclose(got, tup[j].grad.numpy(), rtol=1e-6, atol=1e-10)
+        want_lr = lr / (1.0 + decay * step)
+        assert abs(out["lr"] - want_lr) < 1e-15
+        for grp in opt.param_groups:
+            grp["lr"] = want_lr
+        opt.step()
+        for i, tup in enumerate(tp):
+            for j in range(2):
+                np.testing.assert_allclose(net.p[i][j], tup[j].detach().numpy().reshape(net.p[i][j].shape),
+                                           rtol=1e-7, atol=1e-10)
+    # evaluation ignores the masks
+    p_eval, _ = net.forward(X, training=False, masks=masks)
+    p_eval2, _ = net.forward(X, training=False)
+    assert np.array_equal(p_eval, p_eval2)
