@@ -1,15 +1,37 @@
-"""The benchmark's full-size shapes on the GPU, checked without a full-size CPU
-run: convolution is independent per sample, so fprop/dgrad of individual samples
-of the big batch are compared with the oracle directly; wgrad is linear in the
-upstream gradient, so a gradient that is zero outside one sample must reproduce
-the oracle's wgrad of that sample; and the adjoint identities
-<y - b, dy> = <x, dx> = <W, dW> tie the three full-size results together."""
+"""The benchmark's full-size shapes on the GPU.
+
+Every output element of fprop and dgrad is compared with the float64 oracle (the
+oracle runs over the batch in chunks on a few host threads: convolution is independent
+per sample), and bit for bit with a second, independently scheduled kernel of the
+library (other loads, other tiles, other store schedule, same order of k): a handful of
+wrong elements among tens of millions cannot hide in a global sum.  wgrad is linear in
+the upstream gradient, so a gradient that is zero outside one sample must reproduce the
+oracle's wgrad of that sample; and the adjoint identities <y - b, dy> = <x, dx> = <W, dW>
+tie the three full-size results together."""
+from concurrent.futures import ThreadPoolExecutor
+
 import numpy as np
 import pytest
 
 from oracle import oracle as O
 
 pytestmark = pytest.mark.gpu
+
+# the second kernel each full-size result is compared with, bit for bit
+OTHER_KERNELS = dict(gather_sa=0, gather_res=0, dense_res=0, gather_wide=0)
+
+
+def whole_tensor_close(got, oracle_of_rows, S, chunk=8, threads=8):
+    """abi.close(got[rows], oracle_of_rows(lo, hi)) for every chunk of the batch."""
+    from tests import abi
+    spans = [(lo, min(lo + chunk, S)) for lo in range(0, S, chunk)]
+
+    def check(span):
+        lo, hi = span
+        return abi.close(got[lo:hi], oracle_of_rows(lo, hi))
+
+    with ThreadPoolExecutor(max_workers=threads) as pool:
+        return max(pool.map(check, spans))
 
 FULL = [
     # name, S, H, W, C, D, fH, fW, stride, padding
@@ -20,7 +42,7 @@ FULL = [
 
 
 @pytest.mark.parametrize("cfg", FULL, ids=lambda c: c[0])
-def test_full_size_conv(cfg):
+def test_full_size_conv(cfg, tune):
     from aether import _lib
     from aether.tensor import DeviceTensor
     from tests import abi
@@ -44,10 +66,20 @@ def test_full_size_conv(cfg):
     y_h, dx_h, dw_h, db_h = y.get(), dx.get(), dw.get(), db.get()
     assert np.all(np.isfinite(y_h)) and np.all(np.isfinite(dx_h))
 
-    # per-sample parity at the real launch geometry (first, middle, last sample)
-    for s in (0, S // 2 + 1, S - 1):
-        abi.close(y_h[s:s + 1], O.conv_fprop(x[s:s + 1], w, b, stride, pad, dtype=np.float64))
-        abi.close(dx_h[s:s + 1], O.conv_dgrad(dy[s:s + 1], w, (H, W), stride, pad, dtype=np.float64))
+    # every element against the oracle
+    whole_tensor_close(y_h, lambda lo, hi: O.conv_fprop(x[lo:hi], w, b, stride, pad, dtype=np.float64), S)
+    whole_tensor_close(dx_h, lambda lo, hi: O.conv_dgrad(dy[lo:hi], w, (H, W), stride, pad, dtype=np.float64), S)
+    # and bit for bit against the library's other kernels for these shapes
+    tune(**OTHER_KERNELS)
+    y2 = DeviceTensor.full(yshape, np.nan)
+    _lib.check(L.aeth_conv_fprop_f32(xd.ptr, wd.ptr, bd.ptr, y2.ptr, *dims))
+    assert np.array_equal(y_h, y2.get()), "fprop: the two kernels disagree"
+    del y2
+    dx2 = DeviceTensor.full(x.shape, np.nan)
+    _lib.check(L.aeth_conv_dgrad_f32(dyd.ptr, wd.ptr, dx2.ptr, *dims))
+    assert np.array_equal(dx_h, dx2.get()), "dgrad: the two kernels disagree"
+    del dx2
+    tune(**{k: -1 for k in OTHER_KERNELS})
     if name == "wide_s2":
         # 28x28, 3x3 stride 2 valid: row/column 27 is never read, so its gradient is exactly 0
         assert np.all(dx_h[:, 27] == 0) and np.all(dx_h[:, :, 27] == 0)
@@ -86,7 +118,7 @@ def test_full_size_conv(cfg):
 
 
 @pytest.mark.parametrize("cfg", FULL, ids=lambda c: c[0] + "_bf16")
-def test_full_size_conv_bf16(cfg):
+def test_full_size_conv_bf16(cfg, tune):
     """The bf16-input kernels at the same full-size shapes.  Inputs are rounded to bf16
     on the device; the oracle gets the same rounded values, so the fp32 tolerance
     applies (bf16 products are exact in fp32, accumulation is fp32).  The adjoint
@@ -117,9 +149,18 @@ def test_full_size_conv_bf16(cfg):
     y_h, dx_h, dw_h, db_h = y.get(), dx.get(), dw.get(), db.get()
     assert np.all(np.isfinite(y_h)) and np.all(np.isfinite(dx_h)) and np.all(np.isfinite(dw_h))
 
-    for s in (0, S // 2 + 1, S - 1):
-        abi.close(y_h[s:s + 1], O.conv_fprop(xr[s:s + 1], wr, b, stride, pad, dtype=np.float64))
-        abi.close(dx_h[s:s + 1], O.conv_dgrad(dyr[s:s + 1], wr, (H, W), stride, pad, dtype=np.float64))
+    whole_tensor_close(y_h, lambda lo, hi: O.conv_fprop(xr[lo:hi], wr, b, stride, pad, dtype=np.float64), S)
+    whole_tensor_close(dx_h, lambda lo, hi: O.conv_dgrad(dyr[lo:hi], wr, (H, W), stride, pad, dtype=np.float64), S)
+    tune(**OTHER_KERNELS)
+    y2 = DeviceTensor.full(yshape, np.nan)
+    _lib.check(L.aeth_conv_fprop_bf16(xd.ptr, wd.ptr, bd.ptr, y2.ptr, *dims))
+    assert np.array_equal(y_h, y2.get()), "fprop: the two kernels disagree"
+    del y2
+    dx2 = DeviceTensor.full(x.shape, np.nan)
+    _lib.check(L.aeth_conv_dgrad_bf16(dyd.ptr, wd.ptr, dx2.ptr, *dims))
+    assert np.array_equal(dx_h, dx2.get()), "dgrad: the two kernels disagree"
+    del dx2
+    tune(**{k: -1 for k in OTHER_KERNELS})
 
     lhs = float(np.sum((y_h.astype(np.float64) - b.astype(np.float64)) * dyr))
     rhs_x = float(np.sum(xr.astype(np.float64) * dx_h))
