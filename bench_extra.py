@@ -158,8 +158,53 @@ def train_step(steps, warmup):
                     "includes the per-step scalar read-backs"}
 
 
+def cpu_table():
+    """The NumPy einsum oracle on the other benchmark configurations, one core: 1 warm-up +
+    3 runs (median) for the small layers, one run of one training step of the three-block
+    CNN, one run of a batch-16 sample of the stride-2 layer.  Seconds and GFLOP/s per
+    direction, next to which the GPU figures of `conv_shapes` stand."""
+    from oracle import oracle as O
+    out = {"numpy": np.__version__, "host_cores": os.cpu_count(), "threads_used": 1}
+    rng = np.random.RandomState(0)
+
+    def layer(S, H, W, C, D, f, st, pad, runs):
+        x = rng.randn(S, H, W, C).astype(np.float32)
+        w = (rng.randn(f, f, C, D) * np.sqrt(2.0 / (f * f * C))).astype(np.float32)
+        b = np.zeros(D, np.float32)
+        y = O.conv_fprop(x, w, b, (st, st), pad)
+        dy = rng.randn(*y.shape).astype(np.float32)
+        flops = 2.0 * y.size * f * f * C
+        res = {"batch": S}
+        for name, fn in (("fprop", lambda: O.conv_fprop(x, w, b, (st, st), pad)),
+                         ("dgrad", lambda: O.conv_dgrad(dy, w, (H, W), (st, st), pad)),
+                         ("wgrad", lambda: (O.conv_wgrad(x, dy, (f, f), (st, st), pad), O.conv_dbias(dy)))):
+            ts = []
+            for _ in range(runs):
+                t0 = time.perf_counter()
+                fn()
+                ts.append(time.perf_counter() - t0)
+            sec = float(np.median(ts))
+            res[name] = {"seconds": round(sec, 4), "gflops": round(flops / sec / 1e9, 2)}
+        return res
+
+    for name, S, H, W, C, D, f, st, P, _ in SHAPES[:3]:
+        layer(S, H, W, C, D, f, st, "same", 1)                                   # warm-up
+        out[name] = layer(S, H, W, C, D, f, st, "same", 3)
+    out["cfg5_28x28x128_to256_s2"] = dict(layer(16, 28, 28, 128, 256, 3, 2, "valid", 1),
+                                          note="batch 16 of 1024; time is linear in the batch")
+    np.random.seed(0)
+    X = np.random.rand(128, 32, 32, 3).astype(np.float32)
+    y = np.random.randint(0, 10, 128)
+    net = O.OracleCNN(O.make_cnn_params(dtype=np.float32), dtype=np.float32)
+    t0 = time.perf_counter()
+    net.step(X, y)
+    sec = time.perf_counter() - t0
+    out["train_step_cnn3"] = {"seconds_per_step": round(sec, 3), "images_per_sec": round(128.0 / sec, 2), "batch": 128}
+    return out
+
+
 def run(steps, warmup):
-    return {"conv_shapes": conv_table(max(5, steps // 2), 2), "train_step_cnn3": train_step(max(steps, 20), warmup)}
+    return {"conv_shapes": conv_table(max(20, steps), 2), "train_step_cnn3": train_step(max(steps, 20), warmup)}
 
 
 if __name__ == "__main__":
@@ -168,6 +213,6 @@ if __name__ == "__main__":
         print(json.dumps(train_step(50, 10), indent=1))
     elif "--shape" in sys.argv:
         # one shape of the list only, e.g. --shape cfg4_1x1_64_to256 (for profiler runs)
-        print(json.dumps(conv_table(10, 2, only=sys.argv[sys.argv.index("--shape") + 1]), indent=1))
+        print(json.dumps(conv_table(20, 2, only=sys.argv[sys.argv.index("--shape") + 1]), indent=1))
     else:
         print(json.dumps(run(20, 5), indent=1))
