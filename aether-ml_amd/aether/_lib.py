@@ -31,6 +31,7 @@ SIGNATURES = {
     "aeth_event_record": [_p],
     "aeth_event_elapsed_ms": [_p, _p, C.POINTER(_f)],
     "aeth_conv_fprop_f32": [_p, _p, _p, _p] + _conv_dims,
+    "aeth_conv_fprop_f32_noalloc": [_p, _p, _p, _p] + _conv_dims,
     "aeth_conv_dgrad_f32": [_p, _p, _p] + _conv_dims,
     "aeth_conv_wgrad_f32": [_p, _p, _p, _p] + _conv_dims,
     "aeth_cast_f32_to_bf16": [_p, _p, _i64],

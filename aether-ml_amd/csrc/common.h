@@ -27,7 +27,9 @@ int fail(int code, const char* fmt, ...);
 // replay into is kept until the last recording is destroyed; otherwise the old one is
 // freed after the stream has drained.  Fails with AETH_E_STATE while a step is being recorded.
 int workspace(int64_t bytes, void** out);
-
+// Resolves the device address of the fixed scratch array of the entry point that
+// allocates nothing (gather_f32.hip); called by aeth_init with the device current.
+int conv_scratch_init(int device);
 
 #define AETH_REQUIRE_INIT()                                                     \
     do {                                                                        \

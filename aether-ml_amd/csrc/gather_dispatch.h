@@ -360,9 +360,13 @@ static bool launch_direct(DirectParams& dp, bool dgrad, hipStream_t st) {
     return false;
 }
 
+// `fixed_scratch` (with its capacity) replaces the library's growing workspace: the call then
+// allocates nothing and fails with AETH_E_INVALID when the packed filter and the split
+// partials do not fit.
 template <typename T>
 int conv_fprop_impl(const char* fn, const T* x, const T* w, const float* bias, float* y,
-                    int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW) {
+                    int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW,
+                    char* fixed_scratch = nullptr, int64_t fixed_capacity = 0) {
     int Ho, Wo;
     int rc = check_conv_dims(fn, S, H, W, C, D, fH, fW, sH, sW, pH, pW, &Ho, &Wo);
     if (rc) return rc;
@@ -397,8 +401,16 @@ int conv_fprop_impl(const char* fn, const T* x, const T* w, const float* bias, f
     g.split_slabs = 0;
     plan_split<T>(gs, C % Elem<T>::CE == 0, ctx().prop.multiProcessorCount);
     void* ws;
-    rc = workspace(round_up(gs.bt_bytes, 256) + gs.part_bytes, &ws);
-    if (rc) return rc;
+    const int64_t need = round_up(gs.bt_bytes, 256) + gs.part_bytes;
+    if (fixed_scratch != nullptr) {
+        if (need > fixed_capacity)
+            return fail(AETH_E_INVALID, "%s: needs %lld bytes of scratch, this entry point holds %lld", fn,
+                        (long long)need, (long long)fixed_capacity);
+        ws = fixed_scratch;
+    } else {
+        rc = workspace(need, &ws);
+        if (rc) return rc;
+    }
     return run_gather<T>(gs, (char*)ws, 0, C % Elem<T>::CE == 0);
 }
 

@@ -180,6 +180,8 @@ int aeth_init(int device) {
     hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(256), 0, c.stream, c.counters, 0u, 256);
     AETH_LAUNCH_CHECK();
     AETH_HIP(hipStreamSynchronize(c.stream));
+    int rc = conv_scratch_init(device);
+    if (rc) return rc;
     c.device = device;
     c.ready = true;
     return AETH_OK;

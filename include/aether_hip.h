@@ -94,6 +94,20 @@ int aeth_conv_wgrad_f32(const float* x, const float* dy, float* dw, float* dbias
                         int S, int H, int W, int C, int D,
                         int fH, int fW, int sH, int sW, int pH, int pW);
 
+/* aeth_conv_fprop_f32 for callers that cannot allocate (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments, same kernels, bit-identical results; the packed filter and
+ * the split-K partial tiles go to a fixed array of AETH_NOALLOC_SCRATCH_BYTES that each
+ * GPU holds until the process ends, instead of the library's growing workspace, and the
+ * call makes no hipMalloc / hipFree.  Shapes whose scratch does not fit fail with
+ * AETH_E_INVALID (the message states both sizes).  Every call on a GPU shares that
+ * GPU's array: calls that overlap on one GPU race (the library's single stream
+ * serialises its own). */
+#define AETH_NOALLOC_SCRATCH_BYTES (8 << 20)
+int aeth_conv_fprop_f32_noalloc(const float* x, const float* w, const float* bias, float* y,
+                                int S, int H, int W, int C, int D,
+                                int fH, int fW, int sH, int sW, int pH, int pW);
+
 /* ---- convolution, bf16 in / fp32 accumulate / fp32 out --------------------------
  * Same three contractions with x, w, dy given as bf16.  No reference counterpart
  * (the reference is fp32 only); the inputs are produced by aeth_cast_f32_to_bf16.
