@@ -35,6 +35,21 @@ def _ck(rc):
     _lib.check(rc)
 
 
+_recording = [False]        # a training step is being recorded (Model sets it around the capture)
+
+
+def _wants_bf16(layer):
+    """True for a convolution that runs on bf16 inputs: the kernel that produces its input
+    (or its upstream gradient) then leaves a bfloat16 copy beside the float32 tensor."""
+    return isinstance(layer, Conv_Layer) and layer.precision == "bf16"
+
+
+def _twin(t):
+    """Attach an empty bfloat16 copy to a float32 tensor and return it."""
+    t._bf16 = DeviceTensor(t.shape, np.uint16)
+    return t._bf16
+
+
 # ----------------------------------------------------------------------------------
 # Conv_Layer  (CNN_classes_cupy.py:37-161)
 # ----------------------------------------------------------------------------------
@@ -76,9 +91,24 @@ class Conv_Layer:
 
     @staticmethod
     def _bf16(t):
+        """The tensor's bfloat16 copy: the one its producing kernel left beside it, else a cast."""
+        if t._bf16 is not None:
+            return t._bf16
         out = DeviceTensor(t.shape, np.uint16)
         _ck(_L().aeth_cast_f32_to_bf16(t.ptr, out.ptr, t.size))
         return out
+
+    def _filter_bf16(self):
+        """bfloat16 filter, cast once per version of the weights (the optimizer and
+        set_parameters change the version).  While a step is being recorded the cast always
+        runs, so that it is part of the recording."""
+        w = self.filter_weights
+        key = (w.ptr, w._version)
+        if _recording[0] or getattr(self, "_w16_key", None) != key:
+            out = DeviceTensor(w.shape, np.uint16)
+            _ck(_L().aeth_cast_f32_to_bf16(w.ptr, out.ptr, w.size))
+            self._w16, self._w16_key = out, key
+        return self._w16
 
     def forward(self, inputs, training):
         inputs = as_device(inputs, _F32)
@@ -92,7 +122,7 @@ class Conv_Layer:
         dims = self._dims(S, H_in, W_in, D_in)
         if self.precision == "bf16":
             self._x_bf16 = self._bf16(inputs)
-            w16 = self._bf16(self.filter_weights)
+            w16 = self._filter_bf16()
             _ck(_L().aeth_conv_fprop_bf16(self._x_bf16.ptr, w16.ptr, self.biases.ptr, self.output.ptr, *dims))
         else:
             _ck(_L().aeth_conv_fprop_f32(inputs.ptr, self.filter_weights.ptr, self.biases.ptr,
@@ -109,7 +139,7 @@ class Conv_Layer:
         self.dinputs = DeviceTensor(self.inputs.shape, _F32)
         if self.precision == "bf16":
             dy16 = self._bf16(dvalues)
-            w16 = self._bf16(self.filter_weights)
+            w16 = self._filter_bf16()
             _ck(_L().aeth_conv_wgrad_bf16(self._x_bf16.ptr, dy16.ptr, self.dweights.ptr, self.dbiases.ptr, *dims))
             _ck(_L().aeth_conv_dgrad_bf16(dy16.ptr, w16.ptr, self.dinputs.ptr, *dims))
         else:
@@ -183,10 +213,11 @@ class Pooling:
                 bn.dinputs = DeviceTensor(self.inputs.shape, _F32)
                 bn.dweights = DeviceTensor(C, _F32)
                 bn.dbiases = DeviceTensor(C, _F32)
+                dx16 = _twin(bn.dinputs).ptr if _wants_bf16(getattr(bn, "prev", None)) else None
                 _ck(_L().aeth_maxpool2_relu_bn_bwd_f32(
                     dvalues.ptr, self.max_indicies.ptr, relu.inputs.ptr, bn.inputs.ptr, bn.gamma.ptr,
                     bn.batch_mean.ptr, bn.batch_invstd.ptr, self.dinputs.ptr, relu.dinputs.ptr, bn.dinputs.ptr,
-                    bn.dweights.ptr, bn.dbiases.ptr, S, H_in, W_in, C, _relu_alpha(relu)))
+                    bn.dweights.ptr, bn.dbiases.ptr, S, H_in, W_in, C, _relu_alpha(relu), dx16))
                 bn._bwd_prefilled_for = relu.dinputs
             else:
                 _ck(_L().aeth_maxpool2_relu_bwd_f32(dvalues.ptr, self.max_indicies.ptr, relu.inputs.ptr,
@@ -352,7 +383,10 @@ class ReLU:
         inputs = as_device(inputs, _F32)
         self.inputs = inputs
         self.output = DeviceTensor(inputs.shape, _F32)
-        _ck(_L().aeth_relu_fwd_f32(inputs.ptr, self.output.ptr, 0.0, inputs.size))
+        if _wants_bf16(getattr(self, "next", None)):
+            _ck(_L().aeth_relu_fwd_twin_f32(inputs.ptr, self.output.ptr, _twin(self.output).ptr, 0.0, inputs.size))
+        else:
+            _ck(_L().aeth_relu_fwd_f32(inputs.ptr, self.output.ptr, 0.0, inputs.size))
         return self.output
 
     def backward(self, dvalues):
@@ -373,7 +407,10 @@ class Leaky_ReLU:
         inputs = as_device(inputs, _F32)
         self.inputs = inputs
         self.output = DeviceTensor(inputs.shape, _F32)
-        _ck(_L().aeth_relu_fwd_f32(inputs.ptr, self.output.ptr, self.alpha, inputs.size))
+        if _wants_bf16(getattr(self, "next", None)):
+            _ck(_L().aeth_relu_fwd_twin_f32(inputs.ptr, self.output.ptr, _twin(self.output).ptr, self.alpha, inputs.size))
+        else:
+            _ck(_L().aeth_relu_fwd_f32(inputs.ptr, self.output.ptr, self.alpha, inputs.size))
         return self.output
 
     def backward(self, dvalues):
@@ -470,10 +507,11 @@ class Batch_Norm:
         pool.inputs = act.output
         pool.output = DeviceTensor((S, H // 2, W // 2, C), _F32)
         pool.max_indicies = DeviceTensor((S, H // 2, W // 2, C), np.uint8)
+        out16 = _twin(pool.output).ptr if _wants_bf16(getattr(pool, "next", None)) else None
         _ck(_L().aeth_bn_relu_maxpool2_fwd_f32(
             inputs.ptr, self.gamma.ptr, self.beta.ptr, self.running_mean.ptr, self.running_var.ptr,
             self.batch_mean.ptr, self.batch_invstd.ptr, self.output.ptr, act.output.ptr, pool.output.ptr,
-            pool.max_indicies.ptr, S, H, W, C, self.epsilon, self.momentum, _relu_alpha(act)))
+            pool.max_indicies.ptr, S, H, W, C, self.epsilon, self.momentum, _relu_alpha(act), out16))
         act._prefilled_for = self.output
         pool._prefilled_for = act.output
         pool._fused_relu = act
@@ -488,9 +526,14 @@ class Batch_Norm:
         self.dinputs = DeviceTensor(self.inputs.shape, _F32)
         self.dweights = DeviceTensor(C, _F32)
         self.dbiases = DeviceTensor(C, _F32)
-        _ck(_L().aeth_bn_bwd_f32(self.inputs.ptr, dvalues.ptr, self.gamma.ptr, self.batch_mean.ptr,
-                                 self.batch_invstd.ptr, self.dinputs.ptr, self.dweights.ptr, self.dbiases.ptr,
-                                 rows, C))
+        if _wants_bf16(getattr(self, "prev", None)):
+            _ck(_L().aeth_bn_bwd_twin_f32(self.inputs.ptr, dvalues.ptr, self.gamma.ptr, self.batch_mean.ptr,
+                                          self.batch_invstd.ptr, self.dinputs.ptr, _twin(self.dinputs).ptr,
+                                          self.dweights.ptr, self.dbiases.ptr, rows, C))
+        else:
+            _ck(_L().aeth_bn_bwd_f32(self.inputs.ptr, dvalues.ptr, self.gamma.ptr, self.batch_mean.ptr,
+                                     self.batch_invstd.ptr, self.dinputs.ptr, self.dweights.ptr, self.dbiases.ptr,
+                                     rows, C))
         return self.dinputs
 
     def get_parameters(self):
@@ -736,6 +779,8 @@ class Optimizer_Adam:
                     raise ValueError("gradient shape %s does not match parameter shape %s" % (t[1].shape, t[0].shape))
             _ck(_L().aeth_adam_multi_f32(n, arr(0), arr(1), arr(2), arr(3), sizes, self.current_learning_rate,
                                          self.beta_1, self.beta_2, self.epsilon, self.iterations))
+            for t in batch:
+                t[0].touched()                               # the parameters changed in place
 
     def post_update_parameters(self):
         self._flush()
@@ -760,6 +805,7 @@ class Optimizer_Adam:
         that can be replayed: learning rate and bias corrections come from device_state()."""
         import ctypes as C
         state = self._state
+        self._recorded_params = [t for layer in layers for t in (layer.weights, layer.biases)]
         b1, b2 = float(np.float32(self.beta_1)), float(np.float32(self.beta_2))
         _ck(_L().aeth_adam_state_step(state.ptr, float(self.learning_rate), float(self.decay), b1, b2))
         batch = []
@@ -780,3 +826,5 @@ class Optimizer_Adam:
             self.current_learning_rate = self.learning_rate * (1. / (1. + self.decay * self.iterations))
         self.iterations += 1
         self._state_iterations = self.iterations
+        for t in getattr(self, "_recorded_params", ()):
+            t.touched()

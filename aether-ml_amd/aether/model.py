@@ -224,6 +224,7 @@ class Model:
             self.optimizer.device_state()
             _lib.check(lib.aeth_graph_begin())
             L._label_buffer[0] = rec["labels"]
+            L._recording[0] = True
             try:
                 output = self.forward(rec["x"], training=True)
                 rec["pending"] = self.loss.launch(output, batch_y, training=True)
@@ -232,6 +233,7 @@ class Model:
                 self.optimizer.record_update(self.trainable_layers)
             finally:
                 L._label_buffer[0] = None
+                L._recording[0] = False
                 handle = C.c_void_p()
                 rc = lib.aeth_graph_end(C.byref(handle))
             _lib.check(rc)

@@ -11,7 +11,7 @@ from . import _lib
 
 
 class DeviceTensor:
-    __slots__ = ("ptr", "shape", "dtype", "_base", "_cache", "__weakref__")
+    __slots__ = ("ptr", "shape", "dtype", "_base", "_cache", "_bf16", "_version", "__weakref__")
 
     def __init__(self, shape, dtype=np.float32, _ptr=None, _base=None):
         if isinstance(shape, (int, np.integer)):
@@ -20,6 +20,8 @@ class DeviceTensor:
         self.dtype = np.dtype(dtype)
         self._base = _base
         self._cache = None      # host-side values derived from this tensor by a kernel (e.g. row argmax)
+        self._bf16 = None       # a bfloat16 copy of the contents left by the kernel that wrote them, if any
+        self._version = 0       # bumped by everything that rewrites the contents in place
         if _ptr is None:
             p = C.c_void_p()
             _lib.check(_lib.lib().aeth_malloc(C.byref(p), self.nbytes))
@@ -88,7 +90,14 @@ class DeviceTensor:
             a = a.reshape(self.shape)
         if a.nbytes:
             _lib.check(_lib.lib().aeth_memcpy_h2d(self.ptr, a.ctypes.data, a.nbytes))
+        self.touched()
         return self
+
+    def touched(self):
+        """The contents were rewritten in place: copies derived from them are stale."""
+        self._version += 1
+        self._bf16 = None
+        self._cache = None
 
     # -- device ops -----------------------------------------------------------------------
     def fill(self, value):
@@ -96,6 +105,7 @@ class DeviceTensor:
             return self
         if self.dtype == np.float32:
             _lib.check(_lib.lib().aeth_fill_f32(self.ptr, float(value), self.size))
+            self.touched()
         else:
             self.set(np.full(self.shape, value, dtype=self.dtype))
         return self

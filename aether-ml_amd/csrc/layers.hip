@@ -254,13 +254,21 @@ __global__ void bn_bwd_final(const float* __restrict__ part, int nblk, int rows,
     coef[2 * C + c] = -g * is * s1 * inv_n;
 }
 
+// dx16 (may be null): a bfloat16 copy of dx for a bf16 convolution that takes it as its upstream gradient
 __global__ void bn_bwd_apply(const float* __restrict__ x, const float* __restrict__ dy, const float* __restrict__ mean,
-                             const float* __restrict__ coef, float* __restrict__ dx, int64_t n, int C) {
+                             const float* __restrict__ coef, float* __restrict__ dx, uint16_t* __restrict__ dx16,
+                             int64_t n, int C) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (; i < n; i += stride) {
         int c = (int)(i % C);
-        dx[i] = coef[c] * dy[i] + coef[C + c] * (x[i] - mean[c]) + coef[2 * C + c];
+        const float v = coef[c] * dy[i] + coef[C + c] * (x[i] - mean[c]) + coef[2 * C + c];
+        dx[i] = v;
+        if (dx16 != nullptr) {
+            const unsigned u = __float_as_uint(v);
+            dx16[i] = (uint16_t)(((u & 0x7fffffffu) > 0x7f800000u) ? ((u >> 16) | 0x40u)
+                                                                   : ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16));
+        }
     }
 }
 
@@ -300,15 +308,62 @@ __global__ void l1_grad_kernel(float lambda, const float* __restrict__ w, float*
     for (; i < n; i += stride) dw[i] += w[i] < 0.f ? -lambda : lambda;
 }
 
+// float32 -> bfloat16 bits, round to nearest even; NaN stays NaN
+__device__ __forceinline__ unsigned bf16_bits(float f) {
+    const unsigned u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+typedef unsigned ew_u2 __attribute__((ext_vector_type(2)));
+typedef unsigned ew_u4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ ew_u2 pack_bf16x4(const ew_f4& v) {
+    return ew_u2{bf16_bits(v[0]) | (bf16_bits(v[1]) << 16), bf16_bits(v[2]) | (bf16_bits(v[3]) << 16)};
+}
+
 __global__ void cast_bf16_kernel(const float* __restrict__ src, uint16_t* __restrict__ dst, int64_t n) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) dst[i] = (uint16_t)bf16_bits(src[i]);
+}
+
+// 8 elements per thread: two 16-byte loads, one 16-byte store (n8 = n / 8 groups)
+__global__ __launch_bounds__(kEwThreads) void cast_bf16_kernel8(const ew_f4* __restrict__ src, ew_u4* __restrict__ dst,
+                                                               int64_t n8) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n8; i += stride) {
+        const ew_f4 a = src[2 * i], b = src[2 * i + 1];
+        const ew_u2 lo = pack_bf16x4(a), hi = pack_bf16x4(b);
+        dst[i] = ew_u4{lo[0], lo[1], hi[0], hi[1]};
+    }
+}
+
+// ReLU / leaky ReLU on groups of 4 that also leaves a bfloat16 copy of its output (for a
+// bf16 convolution that reads it next: the copy costs 2 bytes per element here instead of a
+// cast pass of 6)
+__global__ __launch_bounds__(kEwThreads) void relu_fwd_twin_kernel4(const ew_f4* __restrict__ x, ew_f4* __restrict__ y,
+                                                                   ew_u2* __restrict__ y16, float alpha, int64_t n4) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n4; i += stride) {
+        const ew_f4 v = x[i];
+        ew_f4 r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = v[e] > 0.f ? v[e] : alpha * v[e];
+        y[i] = r;
+        y16[i] = pack_bf16x4(r);
+    }
+}
+
+__global__ void relu_fwd_twin_kernel(const float* __restrict__ x, float* __restrict__ y, uint16_t* __restrict__ y16,
+                                     float alpha, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (; i < n; i += stride) {
-        unsigned u = __float_as_uint(src[i]);
-        unsigned r;
-        if ((u & 0x7fffffffu) > 0x7f800000u) r = (u >> 16) | 0x40u;   // NaN stays NaN
-        else r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-        dst[i] = (uint16_t)r;
+        const float v = x[i];
+        const float r = v > 0.f ? v : alpha * v;
+        y[i] = r;
+        y16[i] = (uint16_t)bf16_bits(r);
     }
 }
 
@@ -628,8 +683,8 @@ struct Pool2Params {
 __global__ __launch_bounds__(kEwThreads) void bn_relu_maxpool2_fwd_kernel(
     const ew_f4* __restrict__ x, const ew_f4* __restrict__ gamma, const ew_f4* __restrict__ beta,
     const ew_f4* __restrict__ mean, const ew_f4* __restrict__ invstd, ew_f4* __restrict__ bn_out,
-    ew_f4* __restrict__ relu_out, ew_f4* __restrict__ pool_out, uint32_t* __restrict__ idx, float alpha,
-    Pool2Params p, unsigned n) {
+    ew_f4* __restrict__ relu_out, ew_f4* __restrict__ pool_out, ew_u2* __restrict__ pool_out16,
+    uint32_t* __restrict__ idx, float alpha, Pool2Params p, unsigned n) {
     const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     unsigned t, c4, u, wo, s, ho;
@@ -664,6 +719,7 @@ __global__ __launch_bounds__(kEwThreads) void bn_relu_maxpool2_fwd_kernel(
         }
     }
     pool_out[i] = best;
+    if (pool_out16 != nullptr) pool_out16[i] = pack_bf16x4(best);
     idx[i] = bi;
 }
 
@@ -753,12 +809,15 @@ __global__ __launch_bounds__(kEwThreads) void maxpool2_relu_bnpart_bwd_kernel(
 // dx = coef0 * dy + A * (x - mean) + B on groups of 4 channels
 __global__ __launch_bounds__(kEwThreads) void bn_bwd_apply4(const ew_f4* __restrict__ x, const ew_f4* __restrict__ dy,
                                                            const ew_f4* __restrict__ mean, const float* __restrict__ coef,
-                                                           ew_f4* __restrict__ dx, unsigned n4, int C4) {
+                                                           ew_f4* __restrict__ dx, ew_u2* __restrict__ dx16,
+                                                           unsigned n4, int C4) {
     const unsigned stride = gridDim.x * blockDim.x;
     const ew_f4* c0 = reinterpret_cast<const ew_f4*>(coef);
     for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
         const unsigned c4 = i % (unsigned)C4;
-        dx[i] = c0[c4] * dy[i] + c0[C4 + c4] * (x[i] - mean[c4]) + c0[2 * C4 + c4];
+        const ew_f4 v = c0[c4] * dy[i] + c0[C4 + c4] * (x[i] - mean[c4]) + c0[2 * C4 + c4];
+        dx[i] = v;
+        if (dx16 != nullptr) dx16[i] = pack_bf16x4(v);
     }
 }
 
@@ -814,7 +873,7 @@ static inline bool aligned16(const void* q) { return (reinterpret_cast<uintptr_t
 int aeth_bn_relu_maxpool2_fwd_f32(const float* x, const float* gamma, const float* beta, float* running_mean,
                                   float* running_var, float* save_mean, float* save_invstd, float* bn_out,
                                   float* relu_out, float* pool_out, uint8_t* idx, int S, int H, int W, int C,
-                                  float eps, float momentum, float alpha) {
+                                  float eps, float momentum, float alpha, uint16_t* pool_out_bf16) {
     AETH_REQUIRE_INIT();
     AETH_CHECK_ARG(x && gamma && beta && running_mean && running_var && save_mean && save_invstd);
     AETH_CHECK_ARG(bn_out && relu_out && pool_out && idx);
@@ -824,7 +883,7 @@ int aeth_bn_relu_maxpool2_fwd_f32(const float* x, const float* gamma, const floa
         return fail(AETH_E_INVALID, "%s: needs even H and W, C %% 4 == 0 and fewer than 2^31 elements", __func__);
     AETH_CHECK_ARG(aligned16(x) && aligned16(gamma) && aligned16(beta) && aligned16(save_mean) &&
                    aligned16(save_invstd) && aligned16(bn_out) && aligned16(relu_out) && aligned16(pool_out) &&
-                   aligned16(idx));
+                   aligned16(idx) && aligned16(pool_out_bf16));
     const int rows = S * H * W;
     int nblk, rpb;
     dim3 grid;
@@ -845,8 +904,8 @@ int aeth_bn_relu_maxpool2_fwd_f32(const float* x, const float* gamma, const floa
     AETH_LAUNCH_CHECK();
     hipLaunchKernelGGL(bn_relu_maxpool2_fwd_kernel, dim3(cdiv(n, kEwThreads)), dim3(kEwThreads), 0, st,
                        (const ew_f4*)x, (const ew_f4*)gamma, (const ew_f4*)beta, (const ew_f4*)save_mean,
-                       (const ew_f4*)save_invstd, (ew_f4*)bn_out, (ew_f4*)relu_out, (ew_f4*)pool_out, (uint32_t*)idx,
-                       alpha, p, n);
+                       (const ew_f4*)save_invstd, (ew_f4*)bn_out, (ew_f4*)relu_out, (ew_f4*)pool_out, (ew_u2*)pool_out_bf16,
+                       (uint32_t*)idx, alpha, p, n);
     AETH_LAUNCH_CHECK();
     return AETH_OK;
 }
@@ -870,7 +929,7 @@ int aeth_maxpool2_relu_bwd_f32(const float* dy, const uint8_t* idx, const float*
 int aeth_maxpool2_relu_bn_bwd_f32(const float* dy, const uint8_t* idx, const float* relu_in, const float* x,
                                   const float* gamma, const float* save_mean, const float* save_invstd,
                                   float* pool_dx, float* relu_dx, float* bn_dx, float* dgamma, float* dbeta,
-                                  int S, int H, int W, int C, float alpha) {
+                                  int S, int H, int W, int C, float alpha, uint16_t* bn_dx_bf16) {
     AETH_REQUIRE_INIT();
     AETH_CHECK_ARG(dy && idx && relu_in && x && gamma && save_mean && save_invstd);
     AETH_CHECK_ARG(pool_dx && relu_dx && bn_dx && dgamma && dbeta);
@@ -880,7 +939,7 @@ int aeth_maxpool2_relu_bn_bwd_f32(const float* dy, const uint8_t* idx, const flo
         return fail(AETH_E_INVALID, "%s: needs even H and W, C / 4 a divisor of %d and fewer than 2^31 elements",
                     __func__, kEwThreads);
     AETH_CHECK_ARG(aligned16(dy) && aligned16(idx) && aligned16(relu_in) && aligned16(x) && aligned16(save_mean) &&
-                   aligned16(pool_dx) && aligned16(relu_dx) && aligned16(bn_dx));
+                   aligned16(pool_dx) && aligned16(relu_dx) && aligned16(bn_dx) && aligned16(bn_dx_bf16));
     const int rows = S * H * W;
     int nblk = cdiv(n, kEwThreads);
     if (nblk > 256) nblk = 256;
@@ -899,7 +958,7 @@ int aeth_maxpool2_relu_bn_bwd_f32(const float* dy, const uint8_t* idx, const flo
     AETH_LAUNCH_CHECK();
     const unsigned n4 = (unsigned)((int64_t)rows * C / 4);
     hipLaunchKernelGGL(bn_bwd_apply4, dim3(ew_blocks(n4)), dim3(kEwThreads), 0, st, (const ew_f4*)x,
-                       (const ew_f4*)relu_dx, (const ew_f4*)save_mean, coef, (ew_f4*)bn_dx, n4, C / 4);
+                       (const ew_f4*)relu_dx, (const ew_f4*)save_mean, coef, (ew_f4*)bn_dx, (ew_u2*)bn_dx_bf16, n4, C / 4);
     AETH_LAUNCH_CHECK();
     return AETH_OK;
 }
@@ -914,8 +973,9 @@ int aeth_bn_fwd_infer_f32(const float* x, const float* gamma, const float* beta,
     return AETH_OK;
 }
 
-int aeth_bn_bwd_f32(const float* x, const float* dy, const float* gamma, const float* save_mean,
-                    const float* save_invstd, float* dx, float* dgamma, float* dbeta, int rows, int C) {
+static int bn_bwd_impl(const float* x, const float* dy, const float* gamma, const float* save_mean,
+                       const float* save_invstd, float* dx, uint16_t* dx_bf16, float* dgamma, float* dbeta, int rows,
+                       int C) {
     AETH_REQUIRE_INIT();
     AETH_CHECK_ARG(x && dy && gamma && save_mean && save_invstd && dx && dgamma && dbeta);
     AETH_CHECK_ARG(rows > 0 && C > 0 && (int64_t)rows * C < ((int64_t)1 << 31));
@@ -939,8 +999,27 @@ int aeth_bn_bwd_f32(const float* x, const float* dy, const float* gamma, const f
                        dgamma, dbeta, coef);
     AETH_LAUNCH_CHECK();
     int64_t n = (int64_t)rows * C;
-    EW_LAUNCH(bn_bwd_apply, n, x, dy, save_mean, coef, dx, n, C);
+    if (col_vec4(C, x, dy) && col_vec4(C, save_mean, dx) && aligned16(dx_bf16) && aligned16(coef)) {
+        const unsigned n4 = (unsigned)(n / 4);
+        hipLaunchKernelGGL(bn_bwd_apply4, dim3(ew_blocks(n4)), dim3(kEwThreads), 0, st, (const ew_f4*)x, (const ew_f4*)dy,
+                           (const ew_f4*)save_mean, coef, (ew_f4*)dx, (ew_u2*)dx_bf16, n4, C / 4);
+        AETH_LAUNCH_CHECK();
+    } else {
+        EW_LAUNCH(bn_bwd_apply, n, x, dy, save_mean, coef, dx, dx_bf16, n, C);
+    }
     return AETH_OK;
+}
+
+int aeth_bn_bwd_f32(const float* x, const float* dy, const float* gamma, const float* save_mean,
+                    const float* save_invstd, float* dx, float* dgamma, float* dbeta, int rows, int C) {
+    return bn_bwd_impl(x, dy, gamma, save_mean, save_invstd, dx, nullptr, dgamma, dbeta, rows, C);
+}
+
+int aeth_bn_bwd_twin_f32(const float* x, const float* dy, const float* gamma, const float* save_mean,
+                         const float* save_invstd, float* dx, uint16_t* dx_bf16, float* dgamma, float* dbeta,
+                         int rows, int C) {
+    AETH_CHECK_ARG(dx_bf16 != nullptr);
+    return bn_bwd_impl(x, dy, gamma, save_mean, save_invstd, dx, dx_bf16, dgamma, dbeta, rows, C);
 }
 
 int aeth_relu_fwd_f32(const float* x, float* y, float alpha, int64_t n) {
@@ -949,6 +1028,20 @@ int aeth_relu_fwd_f32(const float* x, float* y, float alpha, int64_t n) {
     if (n == 0) return AETH_OK;
     AETH_CHECK_ARG(x && y);
     EW_LAUNCH(relu_fwd_kernel, n, x, y, alpha, n);
+    return AETH_OK;
+}
+
+int aeth_relu_fwd_twin_f32(const float* x, float* y, uint16_t* y_bf16, float alpha, int64_t n) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(n >= 0);
+    if (n == 0) return AETH_OK;
+    AETH_CHECK_ARG(x && y && y_bf16);
+    if (n % 4 == 0 && aligned16(x) && aligned16(y) && (reinterpret_cast<uintptr_t>(y_bf16) & 7) == 0) {
+        const int64_t n4 = n / 4;
+        EW_LAUNCH(relu_fwd_twin_kernel4, n4, (const ew_f4*)x, (ew_f4*)y, (ew_u2*)y_bf16, alpha, n4);
+    } else {
+        EW_LAUNCH(relu_fwd_twin_kernel, n, x, y, y_bf16, alpha, n);
+    }
     return AETH_OK;
 }
 
@@ -1157,7 +1250,13 @@ int aeth_cast_f32_to_bf16(const float* src, uint16_t* dst, int64_t n) {
     AETH_CHECK_ARG(n >= 0);
     if (n == 0) return AETH_OK;
     AETH_CHECK_ARG(src && dst);
-    EW_LAUNCH(cast_bf16_kernel, n, src, dst, n);
+    int64_t done = 0;
+    if (n >= 8 && aligned16(src) && aligned16(dst)) {
+        const int64_t n8 = n / 8;
+        EW_LAUNCH(cast_bf16_kernel8, n8, (const ew_f4*)src, (ew_u4*)dst, n8);
+        done = 8 * n8;
+    }
+    if (done < n) EW_LAUNCH(cast_bf16_kernel, n - done, src + done, dst + done, n - done);
     return AETH_OK;
 }
 

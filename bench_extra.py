@@ -203,13 +203,64 @@ def cpu_table():
     return out
 
 
+def bf16_layer(steps, warmup):
+    """Conv_Layer.forward + backward on bf16 inputs THROUGH THE LAYER on the headline shape, next
+    to the sum of the three ABI calls: (a) a lone layer handed float32 tensors, which has to cast
+    x and dy itself (two passes of 308 MB each); (b) the same layer fed by producers that leave
+    bfloat16 copies beside their float32 outputs, as ReLU / the fused batch-norm block / batch
+    norm's backward pass do inside a model, so that only the filter is cast."""
+    import aether
+    from aether import _lib
+    from aether.tensor import DeviceTensor
+    L = _lib.lib()
+    S, H, W, C, D = 256, 56, 56, 64, 64
+    rng = np.random.default_rng(0)
+    x = DeviceTensor.from_numpy(rng.standard_normal((S, H, W, C), dtype=np.float32))
+    dy = DeviceTensor.from_numpy(rng.standard_normal((S, H, W, D), dtype=np.float32))
+    np.random.seed(0)
+    layer = aether.Conv_Layer((H, W, C), num_filters=D, filter_size=(3, 3), strides=(1, 1), padding="same")
+    layer.precision = "bf16"
+
+    def step():
+        layer.forward(x, True)
+        layer.backward(dy)
+
+    alone = _time(step, steps, warmup)
+    for t in (x, dy):
+        t._bf16 = DeviceTensor(t.shape, np.uint16)
+        _lib.check(L.aeth_cast_f32_to_bf16(t.ptr, t._bf16.ptr, t.size))
+    fed = _time(step, steps, warmup)
+    x16, dy16, w16 = x._bf16, dy._bf16, layer._filter_bf16()
+    dims = (S, H, W, C, D, 3, 3, 1, 1, 1, 1)
+    y, dx, dw, db = layer.output, layer.dinputs, layer.dweights, layer.dbiases
+
+    def abi():
+        _lib.check(L.aeth_conv_fprop_bf16(x16.ptr, w16.ptr, layer.biases.ptr, y.ptr, *dims))
+        _lib.check(L.aeth_conv_wgrad_bf16(x16.ptr, dy16.ptr, dw.ptr, db.ptr, *dims))
+        _lib.check(L.aeth_conv_dgrad_bf16(dy16.ptr, w16.ptr, dx.ptr, *dims))
+
+    calls = _time(abi, steps, warmup)
+    cast = _time(lambda: _lib.check(L.aeth_cast_f32_to_bf16(x.ptr, x16.ptr, x.size)), steps, warmup)
+    flops = 3 * 2.0 * S * H * W * 9 * C * D
+    return {"shape": "Conv_Layer fwd+bwd, bf16 inputs, NHWC [256,56,56,64] -> 64 filters 3x3",
+            "abi_calls_ms": round(calls, 4), "abi_calls_tflops": round(flops / calls / 1e9, 1),
+            "layer_fed_by_producers_ms": round(fed, 4), "layer_fed_by_producers_tflops": round(flops / fed / 1e9, 1),
+            "layer_alone_casting_x_and_dy_ms": round(alone, 4),
+            "layer_alone_casting_x_and_dy_tflops": round(flops / alone / 1e9, 1),
+            "cast_205MB_tensor_ms": round(cast, 4), "cast_tb_per_s": round(x.size * 6 / cast / 1e9, 2),
+            "layer_over_abi": round(fed / calls, 3)}
+
+
 def run(steps, warmup):
-    return {"conv_shapes": conv_table(max(20, steps), 2), "train_step_cnn3": train_step(max(steps, 20), warmup)}
+    return {"conv_shapes": conv_table(max(20, steps), 2), "bf16_through_the_layer": bf16_layer(max(20, steps), 3),
+            "train_step_cnn3": train_step(max(steps, 20), warmup)}
 
 
 if __name__ == "__main__":
     import json
-    if "--train-only" in sys.argv:
+    if "--bf16-layer" in sys.argv:
+        print(json.dumps(bf16_layer(20, 3), indent=1))
+    elif "--train-only" in sys.argv:
         print(json.dumps(train_step(50, 10), indent=1))
     elif "--shape" in sys.argv:
         # one shape of the list only, e.g. --shape cfg4_1x1_64_to256 (for profiler runs)

@@ -163,6 +163,16 @@ int aeth_bn_bwd_f32(const float* x, const float* dy, const float* gamma,
  * fwd: y = x > 0 ? x : alpha*x ;  bwd: dx = x < 0 ? alpha*dy : dy  (strict <). */
 int aeth_relu_fwd_f32(const float* x, float* y, float alpha, int64_t n);
 int aeth_relu_bwd_f32(const float* x, const float* dy, float* dx, float alpha, int64_t n);
+/* Producers that also leave a bfloat16 copy of what they write, for a bf16 convolution that
+ * reads it next (no counterpart in the reference, which is fp32 only): the copy costs 2
+ * bytes per element inside the producing kernel instead of a cast pass of 6.
+ * relu_fwd_twin = relu_fwd with y_bf16; bn_bwd_twin = bn_bwd with dx_bf16 (declared below,
+ * same arguments otherwise).  The fused block entry points take the same kind of optional
+ * last argument (pool_out_bf16, bn_dx_bf16; NULL = none). */
+int aeth_relu_fwd_twin_f32(const float* x, float* y, uint16_t* y_bf16, float alpha, int64_t n);
+int aeth_bn_bwd_twin_f32(const float* x, const float* dy, const float* gamma,
+                         const float* save_mean, const float* save_invstd,
+                         float* dx, uint16_t* dx_bf16, float* dgamma, float* dbeta, int rows, int C);
 /* Pooling "max"/"valid" :212-273 and :275-300.  idx holds the flat window index
  * fh*fW+fw of the FIRST maximum in row-major window order. */
 int aeth_maxpool_fwd_f32(const float* x, float* y, uint8_t* idx,
@@ -181,7 +191,8 @@ int aeth_bn_relu_maxpool2_fwd_f32(const float* x, const float* gamma, const floa
                                   float* running_mean, float* running_var,
                                   float* save_mean, float* save_invstd,
                                   float* bn_out, float* relu_out, float* pool_out, uint8_t* idx,
-                                  int S, int H, int W, int C, float eps, float momentum, float alpha);
+                                  int S, int H, int W, int C, float eps, float momentum, float alpha,
+                                  uint16_t* pool_out_bf16 /* may be NULL */);
 int aeth_maxpool2_relu_bwd_f32(const float* dy, const uint8_t* idx, const float* relu_in,
                                float* pool_dx, float* relu_dx,
                                int S, int H, int W, int C, float alpha);
@@ -193,7 +204,8 @@ int aeth_maxpool2_relu_bn_bwd_f32(const float* dy, const uint8_t* idx, const flo
                                   const float* save_mean, const float* save_invstd,
                                   float* pool_dx, float* relu_dx, float* bn_dx,
                                   float* dgamma, float* dbeta,
-                                  int S, int H, int W, int C, float alpha);
+                                  int S, int H, int W, int C, float alpha,
+                                  uint16_t* bn_dx_bf16 /* may be NULL */);
 /* Pooling "average" :267-268 and the scatter kernel :163-202. */
 int aeth_avgpool_fwd_f32(const float* x, float* y,
                          int S, int H, int W, int C, int fH, int fW, int sH, int sW);

@@ -273,3 +273,140 @@ def test_bf16_wgrad_with_the_whole_result_in_registers(case, tune):
     dw3, db3 = abi.wgrad_bf16(x, dy, w.shape, stride, pad)
     abi.close(dw3, dw, rtol=1e-4, atol=1e-5, rms_scaled=True)
     abi.close(db3, db, rtol=1e-4, atol=1e-5, rms_scaled=True)
+
+
+# ---- bfloat16 copies left by the producing kernels ------------------------------------------
+# A bf16 convolution reads bfloat16 x and dy.  The layers that produce them (ReLU / leaky ReLU,
+# the fused batch-norm block, batch norm's backward pass) can leave the bfloat16 copy beside the
+# float32 tensor they write anyway; the copy must be the round-to-nearest-even image of exactly
+# the float32 values written, bit for bit, so that a convolution fed by it computes what it
+# computes after a cast pass.
+@pytest.mark.parametrize("n", [4096 * 7, 1001])            # 16-byte groups, and a length that is not a multiple of 4
+def test_relu_twin_is_the_cast_of_what_relu_writes(n):
+    from aether import _lib
+    from aether.tensor import DeviceTensor
+    r = np.random.RandomState(2)
+    x = r.randn(n).astype(np.float32)
+    xd = DeviceTensor.from_numpy(x)
+    for alpha in (0.0, 0.01):
+        y, y2 = DeviceTensor.full(n, np.nan), DeviceTensor.full(n, np.nan)
+        y16 = DeviceTensor(n, np.uint16)
+        _lib.check(_lib.lib().aeth_relu_fwd_f32(xd.ptr, y.ptr, alpha, n))
+        _lib.check(_lib.lib().aeth_relu_fwd_twin_f32(xd.ptr, y2.ptr, y16.ptr, alpha, n))
+        assert np.array_equal(y.get(), y2.get())
+        assert np.array_equal(y.get(), np.where(x > 0, x, np.float32(alpha) * x))
+        assert np.array_equal(y16.get(), O.bf16_bits(y.get()))
+
+
+@pytest.mark.parametrize("shape", [(6, 10, 10, 32), (5, 7, 7, 6)])       # 16-byte path, scalar path
+def test_bn_bwd_twin_is_the_cast_of_what_bn_bwd_writes(shape):
+    from aether import _lib
+    from aether.tensor import DeviceTensor
+    from tests import abi
+    r = np.random.RandomState(3)
+    C = shape[-1]
+    rows = int(np.prod(shape[:-1]))
+    x = r.randn(*shape).astype(np.float32) * 2 + 1
+    dy = r.randn(*shape).astype(np.float32)
+    g = (r.rand(C) + 0.5).astype(np.float32)
+    mu = x.reshape(rows, C).mean(0).astype(np.float32)
+    var = x.reshape(rows, C).var(0)
+    invstd = (1.0 / np.sqrt(var + 1e-5)).astype(np.float32)
+    d = {k: DeviceTensor.from_numpy(v) for k, v in dict(x=x, dy=dy, g=g, mu=mu, invstd=invstd).items()}
+    dx, dx2 = DeviceTensor.full(shape, np.nan), DeviceTensor.full(shape, np.nan)
+    dx16 = DeviceTensor(shape, np.uint16)
+    dg, db, dg2, db2 = (DeviceTensor.full(C, np.nan) for _ in range(4))
+    L = _lib.lib()
+    _lib.check(L.aeth_bn_bwd_f32(d["x"].ptr, d["dy"].ptr, d["g"].ptr, d["mu"].ptr, d["invstd"].ptr, dx.ptr, dg.ptr,
+                                 db.ptr, rows, C))
+    _lib.check(L.aeth_bn_bwd_twin_f32(d["x"].ptr, d["dy"].ptr, d["g"].ptr, d["mu"].ptr, d["invstd"].ptr, dx2.ptr,
+                                      dx16.ptr, dg2.ptr, db2.ptr, rows, C))
+    assert np.array_equal(dg.get(), dg2.get()) and np.array_equal(db.get(), db2.get())
+    want, _, _ = O.bn_backward(x.astype(np.float64), dy.astype(np.float64), g.astype(np.float64),
+                               mu.astype(np.float64).reshape((1,) * (len(shape) - 1) + (C,)),
+                               var.reshape((1,) * (len(shape) - 1) + (C,)), 1e-5)
+    abi.close(dx2.get(), want, rtol=2e-4)
+    abi.close(dx.get(), want, rtol=2e-4)
+    assert np.array_equal(dx16.get(), O.bf16_bits(dx2.get()))
+
+
+def test_bf16_convolution_between_producers_uses_their_copies():
+    """ReLU -> Conv_Layer(bf16) -> Batch_Norm, linked as Model.finalize links them: the
+    convolution finds bfloat16 copies of its input and of its upstream gradient and casts
+    nothing but its filter; results equal, bit for bit, those of the same layers without
+    the links (where the convolution casts x and dy itself)."""
+    import aether
+
+    def chain(linked):
+        np.random.seed(8)
+        relu, conv, bn = aether.ReLU(), aether.Conv_Layer((12, 12, 64), num_filters=64), aether.Batch_Norm()
+        conv.precision = "bf16"
+        if linked:
+            relu.next, conv.prev, conv.next, bn.prev = conv, relu, bn, conv
+        return relu, conv, bn
+
+    r = np.random.RandomState(9)
+    x = r.randn(4, 12, 12, 64).astype(np.float32)
+    dy = r.randn(4, 12, 12, 64).astype(np.float32)
+    outs = []
+    for linked in (True, False):
+        relu, conv, bn = chain(linked)
+        relu.forward(x, True)
+        conv.forward(relu.output, True)
+        bn.forward(conv.output, True)
+        bn.backward(dy)
+        conv.backward(bn.dinputs)
+        if linked:
+            assert relu.output._bf16 is not None and conv._x_bf16 is relu.output._bf16
+            assert bn.dinputs._bf16 is not None
+            assert np.array_equal(relu.output._bf16.get(), O.bf16_bits(relu.output.get()))
+            assert np.array_equal(bn.dinputs._bf16.get(), O.bf16_bits(bn.dinputs.get()))
+        else:
+            assert relu.output._bf16 is None and bn.dinputs._bf16 is None
+        outs.append([t.get() for t in (conv.output, conv.dinputs, conv.dweights, conv.dbiases)])
+    for a, b in zip(*outs):
+        assert np.array_equal(a, b)
+    # the filter is cast once per version of the weights: set_parameters and an in-place change make it stale
+    relu, conv, bn = chain(True)
+    relu.forward(x, True)
+    conv.forward(relu.output, True)
+    first = conv._w16
+    conv.forward(relu.output, True)
+    assert conv._w16 is first
+    conv.filter_weights.set(conv.filter_weights.get() * 2)
+    y1 = conv.forward(relu.output, True).get()
+    assert conv._w16 is not first
+    np.testing.assert_allclose(y1, 2 * outs[0][0], rtol=1e-6, atol=1e-6)
+
+
+def test_bf16_training_steps_of_the_cnn_recorded_and_eager(monkeypatch):
+    """The three-block CNN with every convolution on bf16 inputs (AETHER_PRECISION=bf16): the
+    fused blocks hand their bfloat16 pooling output to the next convolution, the fused backward
+    pass its bfloat16 batch-norm gradient.  Loss within the bf16 tolerance of the float32
+    model's, and recorded steps equal eager ones bit for bit (the filter casts are part of the
+    recording)."""
+    import aether
+    from tests.test_gpu_model import build_model
+    rng = np.random.RandomState(4)
+    X, y = rng.rand(32, 16, 16, 3).astype(np.float32), rng.randint(0, 10, 32)
+
+    def make(precision):
+        monkeypatch.setenv("AETHER_PRECISION", precision)
+        np.random.seed(6)
+        m = build_model(aether, hw=16)
+        m.loss.new_pass()
+        m.accuracy.new_pass()
+        return m
+
+    f32, eager, rec = make("fp32"), make("bf16"), make("bf16")
+    rec.record_steps(True)
+    for step in range(5):
+        a, b, c = f32.train_step(X, y), eager.train_step(X, y), rec.train_step(X, y)
+        assert b == c, "step %d: eager %r, recorded %r" % (step, b, c)
+        assert abs(a[0] - b[0]) <= 2e-2 * abs(a[0]), (step, a, b)
+        for la, lb in zip(eager.trainable_layers, rec.trainable_layers):
+            assert np.array_equal(np.asarray(la.weights), np.asarray(lb.weights))
+    convs = [l for l in eager.layers if isinstance(l, aether.Conv_Layer)]
+    assert all(c.precision == "bf16" for c in convs)
+    assert convs[1].inputs._bf16 is not None and convs[1]._x_bf16 is convs[1].inputs._bf16
+    rec.record_steps(False)
