@@ -149,9 +149,24 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
         p.inc1 = 4 * C * (-Wo * sW + sH * W);
         p.inc2 = 4 * C * (-Ho * sH * W + H * W);
     }
-    const int tkw = !dma ? kWgBK : (p.cw == 1 ? 32 : (p.cw == 6 ? 192 : kWgBK));
-    const int kt = cdiv(p.K, tkw), nt = cdiv(D, kWgBN);
-    const int slab_rows = dma16 ? 64 : kWgBR;
+    // bf16: wide wave tiles (128 k x 256 n or 128 k x 128 n per workgroup) where they pad the output
+    // channels by at most a third more than 64-wide tiles do (tuning: wgrad_wide = 0 never, >= 1 wherever D > 64)
+    int wide_nb = 0;
+    if (dma16 && D > 64 && tuning().wgrad_wide != 0) {
+        const int64_t pad64 = round_up(D, 64), pad128 = round_up(D, 128), pad256 = round_up(D, 256);
+        const bool force = tuning().wgrad_wide > 0;
+        if (pad256 * 3 <= pad64 * 4) wide_nb = 4;
+        else if (pad128 * 3 <= pad64 * 4 || force) wide_nb = 2;
+    }
+    // 256 k rows per workgroup (8 waves, one workgroup per CU) where K has more than two 128-row tiles and
+    // the slabs are long enough to give every CU a share of m (tuning: wgrad_wide = 2 never, 3 always)
+    const int tile_n = wide_nb ? 64 * wide_nb : kWgBN;
+    bool wide_k = wide_nb == 4 && p.K > 256 && (int64_t)cdiv(p.M, kWwBR) * cdiv(p.K, 256) >= 8 * (int64_t)c.prop.multiProcessorCount;
+    if (tuning().wgrad_wide == 2) wide_k = false;
+    if (tuning().wgrad_wide == 3 && wide_nb == 4) wide_k = true;
+    const int tkw = wide_k ? 256 : (!dma ? kWgBK : (p.cw == 1 ? 32 : (p.cw == 6 ? 192 : kWgBK)));
+    const int kt = cdiv(p.K, tkw), nt = cdiv(D, tile_n);
+    const int slab_rows = wide_nb ? kWwBR : (dma16 ? 64 : kWgBR);
     const int slabs = cdiv(p.M, slab_rows);           // fp32: counted in 32-row units for both tile shapes
     // one round of resident workgroups (3 per CU for the LDS-direct kernels, 2 for the 192-wide
     // one and the register-staged one), rounded down so that no second, nearly empty round follows.
@@ -159,7 +174,7 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     // (56x56x64: 0.485 ms with one round, 0.493 with two, 0.509 with four).
     int rounds = 1;
     if (tuning().wgrad_rounds >= 1 && tuning().wgrad_rounds <= 4) rounds = tuning().wgrad_rounds;
-    const int per_cu2 = (((dma && (p.cw != 6 || br == 16)) || dma16) ? 3 : 2) * rounds;
+    const int per_cu2 = (wide_k ? 1 : wide_nb == 4 ? 2 : (((dma && (p.cw != 6 || br == 16)) || dma16) ? 3 : 2)) * rounds;
     int splits = (per_cu2 * c.prop.multiProcessorCount) / (kt * nt);
     // a workgroup's set-up, epilogue and its share of the reduction are worth several slabs
     // (training step of the 3-block CNN: 0.672 ms with 1, 0.642 with 4, 0.611 with 8, 0.658 with 16)
@@ -176,7 +191,10 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     p.out = (float*)ws;
     p.kt = kt; p.nt = nt;
     dim3 grid(kt * nt * splits);
-    if (dma16) hipLaunchKernelGGL(wgrad_gemm_dma_bf16, grid, dim3(kThreads), 0, c.stream, p);
+    if (wide_k) hipLaunchKernelGGL((wgrad_gemm_dma_bf16w<4, 4>), grid, dim3(512), 0, c.stream, p);
+    else if (wide_nb == 4) hipLaunchKernelGGL((wgrad_gemm_dma_bf16w<2, 4>), grid, dim3(kThreads), 0, c.stream, p);
+    else if (wide_nb == 2) hipLaunchKernelGGL((wgrad_gemm_dma_bf16w<2, 2>), grid, dim3(kThreads), 0, c.stream, p);
+    else if (dma16) hipLaunchKernelGGL(wgrad_gemm_dma_bf16, grid, dim3(kThreads), 0, c.stream, p);
     else if (dma && p.cw == 6 && br == 16) hipLaunchKernelGGL(wgrad_gemm_dma192h, grid, dim3(kThreads), 0, c.stream, p);
     else if (dma && p.cw == 6) hipLaunchKernelGGL(wgrad_gemm_dma192, grid, dim3(kThreads), 0, c.stream, p);
     else if (dma) hipLaunchKernelGGL(wgrad_gemm_dma, grid, dim3(kThreads), 0, c.stream, p);

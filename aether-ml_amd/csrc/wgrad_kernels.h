@@ -738,6 +738,231 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma_bf16(const Wgr
 }
 
 // ------------------------------------------------------------------------------
+// wgrad_gemm_dma_bf16w: the same product on wide wave tiles, for outputs of more than 64
+// channels.  With a wave tile of 32 k x 64 n an MFMA step needs three transposing 8-byte
+// reads per MFMA, 1536 B of LDS traffic for 32 MFMA cycles on each of the four SIMDs: the
+// LDS (128 B per clock and CU) is asked for 48 clocks of work per 32 of MFMA and bounds the
+// loop.  Here the four waves form a 2 x 2 grid of tiles of 64 k x (32 NB) n (NB = 4: 128 n,
+// workgroup tile 128 k x 256 n; NB = 2: 64 n, 128 k x 128 n): 2 + NB operand blocks feed
+// 2 NB MFMAs, 1.5 reads per MFMA for NB = 4 (24 clocks of LDS per 32 of MFMA).  One n tile
+// also means that x, the larger operand, is gathered once per k tile instead of once per
+// (k tile, n tile).
+//   slab = 32 rows of m in a ring of three LDS buffers of (8 + 4 NB) KB filled by LDS-direct
+//   loads two slabs ahead (one slab of 16 MFMAs per wave is 0.2 us, a fraction of the memory
+//   latency), one barrier per slab; 16-byte chunk c of slab row m sits at c ^ ((m & 3) << 2) in
+//   both operands: the 4 rows x 64 B that 32 lanes of a transposing read touch then fall into
+//   the four 64-byte quarters of the banks.  The loads are inline assembly so that the compiler
+//   does not order the LDS reads of a slab behind the loads of later slabs; the wave waits for
+//   its own loads of the slab with a partial vmcnt, the barrier covers the other waves'.
+// ------------------------------------------------------------------------------
+constexpr int kWwBR = 32;
+
+// KW x 2 waves of 64 k x (32 NB) n each: KW = 2 -> 128 k rows per workgroup, KW = 4 -> 256 (8 waves,
+// one workgroup per CU: every dy slab is read by half as many workgroups, and the slabs that the
+// workgroups pull out of L2 are what bounds this kernel: 1.17 GB per launch on the stride-2 layer with
+// 128 k rows, 8.4 TB/s).
+template <int KW, int NB>
+static __global__ __launch_bounds__(128 * KW, KW == 4 ? 1 : (NB == 4 ? 2 : 3)) void wgrad_gemm_dma_bf16w(const WgradParams p) {
+    constexpr int BR = kWwBR;
+    constexpr int NWAVES = 2 * KW;
+    constexpr int BK = 64 * KW;                          // k columns of the x slab
+    constexpr int BN = 64 * NB;                          // n columns of the dy slab
+    constexpr int XCH = BK / 8, YCH = BN / 8;            // 16-byte chunks per slab row
+    constexpr int XROWS = 64 / XCH, YROWS = 64 / YCH;    // slab rows per wave-level load
+    constexpr int XLOADS = BR / XROWS / NWAVES;          // loads per wave and slab
+    constexpr int YLOADS = BR / YROWS / NWAVES;
+    static_assert(XLOADS >= 1 && YLOADS >= 1 && XLOADS * XROWS * NWAVES == BR && YLOADS * YROWS * NWAVES == BR, "slab split");
+    constexpr int RING = KW == 4 ? 4 : 3;
+    __shared__ uint16_t lds_a[RING][BR * BK];
+    __shared__ uint16_t lds_y[RING][BR * BN];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kw = wave % KW, nw = wave / KW;            // the wave's place in the KW x 2 grid
+    const int l32 = lane & 31;
+    const int lh = lane >> 5;
+
+    const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
+    const int tiles = p.kt * p.nt;
+    const int split = lid / tiles;
+    const int tile = lid - split * tiles;
+    const int ktile = tile % p.kt;
+    const int kt0 = ktile * BK;
+    const int n0 = (tile / p.kt) * BN;
+    const int m_begin = split * p.m_per_split;
+    int m_end = m_begin + p.m_per_split;
+    if (m_end > p.M) m_end = p.M;
+    const bool do_db = p.want_dbias && (ktile == 0);
+
+    // ---- x: one wave-level load = XROWS slab rows x XCH chunks -----------------------------
+    // position pc of slab row r holds logical chunk pc ^ ((r & 3) << 2); XROWS divides 4, so the
+    // rows a lane loads all have r & 3 == (lane / XCH) + XROWS * (i & (4 / XROWS - 1)): the tap decode
+    // is done once per such row class
+    const int x_row = lane / XCH;
+    const int x_pc = lane % XCH;
+    constexpr int XCLS = 4 / XROWS;                      // row classes per lane: 1 or 2
+    int a_tap_off[XCLS], a_fx[XCLS], a_fy[XCLS];
+    bool a_kok[XCLS];
+#pragma unroll
+    for (int q = 0; q < XCLS; ++q) {
+        const int r3 = (x_row + XROWS * q) & 3;
+        const int kk = kt0 + 8 * (x_pc ^ (r3 << 2));
+        unsigned tap, c, fx, fy;
+        p.div_c.divmod((unsigned)kk, tap, c);
+        p.div_fw.divmod(tap, fx, fy);
+        a_kok[q] = kk < p.K;
+        a_fx[q] = (int)fx - p.pH;
+        a_fy[q] = (int)fy - p.pW;
+        a_tap_off[q] = (a_fx[q] * p.W + a_fy[q]) * p.C + (int)c;
+    }
+    // ---- dy: one wave-level load = YROWS slab rows x YCH chunks ------------------------------
+    const int y_row = lane / YCH;
+    const int y_pc = lane % YCH;
+
+    const u32x4 rsrc_x = raw_rsrc(p.x, p.x_bytes);
+    const u32x4 rsrc_y = raw_rsrc(p.dy, p.dy_bytes);
+
+    auto issue = [&](int mb, uint16_t* la, uint16_t* ly) {
+        const unsigned la_base = lds_address(la), ly_base = lds_address(ly);
+#pragma unroll
+        for (int i = 0; i < XLOADS; ++i) {
+            const int ld = wave * XLOADS + i;            // wave-level load number inside the slab
+            const int q = XCLS == 1 ? 0 : (i & (XCLS - 1));          // (ld * XROWS) & 3 == XROWS * (i & (XCLS - 1)): XLOADS is even
+            const int m = mb + ld * XROWS + x_row;
+            unsigned s, rem, ho, wo;
+            p.div_howo.divmod((unsigned)m, s, rem);
+            p.div_wo.divmod(rem, ho, wo);
+            const int r0 = (int)ho * p.sH, c0 = (int)wo * p.sW;
+            const int pix = (((int)s * p.H + r0) * p.W + c0) * p.C;
+            const unsigned bad = (unsigned)!((m < m_end) & a_kok[q] & ((unsigned)(r0 + a_fx[q]) < (unsigned)p.H) &
+                                             ((unsigned)(c0 + a_fy[q]) < (unsigned)p.W));
+            const unsigned voff = ((unsigned)(pix + a_tap_off[q]) * 2u) | (bad << 31);
+            lds_direct_load16(rsrc_x, la_base + (unsigned)ld * 1024u, voff);
+        }
+#pragma unroll
+        for (int i = 0; i < YLOADS; ++i) {
+            const int ld = wave * YLOADS + i;
+            const int row = ld * YROWS + y_row;          // slab row; the slab starts at a multiple of 32
+            const int m = mb + row;
+            const int y_n = n0 + 8 * (y_pc ^ ((row & 3) << 2));
+            const unsigned bad = (unsigned)!((m < m_end) & (y_n < p.D));
+            const unsigned voff = ((unsigned)(m * p.D + y_n) * 2u) | (bad << 31);
+            lds_direct_load16(rsrc_y, ly_base + (unsigned)ld * 1024u, voff);
+        }
+    };
+    constexpr int LOADS = XLOADS + YLOADS;               // per wave and slab
+    static_assert(XCLS == 1 || XLOADS % XCLS == 0, "row classes repeat with the loads of a wave");
+
+    // ---- transposing operand reads: 16-lane group G covers columns 16 (G & 1).., rows 8 (G >> 1)..;
+    // lane j of the group points at row j >> 2, elements 4 (j & 3)..+3
+    const int G = lane >> 4, j16 = lane & 15;
+    const int t_row = 8 * (G >> 1) + (j16 >> 2);         // row inside a 16-row step, first read (+4: second); & 3 == j16 >> 2
+    const int sw = (j16 >> 2) << 2;                      // chunk swizzle of that row (the same for row + 4)
+    int a_eo[2], y_eo[NB];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+        const int col = kw * 64 + kb * 32 + 16 * (G & 1) + 4 * (j16 & 3);
+        a_eo[kb] = (((col >> 3) ^ sw) << 3) + (col & 4);
+    }
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int col = nw * 32 * NB + nb * 32 + 16 * (G & 1) + 4 * (j16 & 3);
+        y_eo[nb] = (((col >> 3) ^ sw) << 3) + (col & 4);
+    }
+    auto tr = [&](const uint16_t* base) {
+        return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr_t)base);
+    };
+    typedef short s8v __attribute__((ext_vector_type(8)));
+
+    f16v acc[2][NB];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[kb][nb][v] = 0.f;
+    const bool active = kt0 + kw * 64 < p.K;             // wave-uniform
+
+    float dbsum = 0.f;                                   // thread t < BN sums column t of every dy slab
+    auto add_columns = [&](const uint16_t* ly) {
+        if (tid < BN) {
+#pragma unroll 8
+            for (int row = 0; row < BR; ++row) {
+                const int e = (((tid >> 3) ^ ((row & 3) << 2)) << 3) + (tid & 7);
+                dbsum += __uint_as_float((unsigned)ly[row * BN + e] << 16);
+            }
+        }
+    };
+
+    auto compute = [&](const uint16_t* la, const uint16_t* ly) {
+        if (do_db) add_columns(ly);
+        if (active) {
+#pragma unroll
+            for (int st = 0; st < BR / 16; ++st) {
+                const int r0 = st * 16 + t_row;
+                s8v av[2], bv[NB];
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+                    const s4v lo = tr(la + r0 * BK + a_eo[kb]);
+                    const s4v hi = tr(la + (r0 + 4) * BK + a_eo[kb]);
+                    av[kb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) {
+                    const s4v lo = tr(ly + r0 * BN + y_eo[nb]);
+                    const s4v hi = tr(ly + (r0 + 4) * BN + y_eo[nb]);
+                    bv[nb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) {
+                    acc[0][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av[0]),
+                                                                         __builtin_bit_cast(bf16x8, bv[nb]), acc[0][nb], 0, 0, 0);
+                    // (k rows past K were loaded as zeros: their products vanish without a branch between the MFMAs)
+                    acc[1][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av[1]),
+                                                                             __builtin_bit_cast(bf16x8, bv[nb]), acc[1][nb], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    // slab k of the split lives in buffer k % RING; its loads go out RING - 1 slabs earlier
+    const int nslab = m_begin < m_end ? (m_end - m_begin + BR - 1) / BR : 0;
+#pragma unroll
+    for (int k = 0; k < RING - 1; ++k)
+        if (k < nslab) issue(m_begin + k * BR, lds_a[k], lds_y[k]);
+    int cur = 0;
+    for (int k = 0; k < nslab; ++k) {
+        // this wave's loads of slab k have landed: everything but the loads of the slabs behind it (at most RING - 2)
+        const int behind = nslab - 1 - k;
+        if (RING >= 4 && behind >= 2) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * LOADS) : "memory");
+        else if (behind >= 1) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(LOADS) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();                                 // ... and so have the other waves'; slab k - 1 has been read by all
+        int nxt = cur + RING - 1;
+        if (nxt >= RING) nxt -= RING;
+        if (k + RING - 1 < nslab) issue(m_begin + (k + RING - 1) * BR, lds_a[nxt], lds_y[nxt]);
+        compute(lds_a[cur], lds_y[cur]);
+        cur = cur + 1 == RING ? 0 : cur + 1;
+    }
+
+    const size_t split_stride = (size_t)p.K * p.D + p.D;
+    float* outp = p.out + (size_t)split * split_stride;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const int n = n0 + nw * 32 * NB + nb * 32 + l32;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int k = kt0 + kw * 64 + kb * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+                if (k < p.K && n < p.D) outp[(size_t)k * p.D + n] = acc[kb][nb][v];
+            }
+        }
+    if (do_db && tid < BN && n0 + tid < p.D) outp[(size_t)p.K * p.D + n0 + tid] = dbsum;
+}
+
+// ------------------------------------------------------------------------------
 // wgrad_halo_bf16: bf16 wgrad of a unit-stride filter of at most 9 taps on 64 input channels and
 // at most 64 output channels, as one persistent workgroup per CU that holds the WHOLE K x N
 // result in registers: wave t owns filter tap t (64 k rows x 64 n columns, four 32 x 32

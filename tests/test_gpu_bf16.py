@@ -275,6 +275,40 @@ def test_bf16_wgrad_with_the_whole_result_in_registers(case, tune):
     abi.close(db3, db, rtol=1e-4, atol=1e-5, rms_scaled=True)
 
 
+# bf16 wgrad onto more than 64 output channels: wave tiles of 64 k x 128 n (workgroup 128 k x 256 n) or
+# 64 k x 64 n (128 x 128), where the library takes them from the channel padding they cost; the
+# wgrad_wide switch forces them (1: the narrower form wherever D > 64) or turns them off (0).
+WGRAD_WIDE_CASES = [
+    (3, 13, 13, 128, 256, 3, 3, 2, 2, "valid"),   # the stride-2 layer's shape: 9 k tiles, one n tile of 256
+    (2, 14, 14, 64, 256, 1, 1, 1, 1, "valid"),    # 1x1: K = 64, the wave's second k block is empty
+    (2, 9, 9, 72, 200, 3, 3, 1, 1, "same"),       # K = 648: ragged last k tile; 200 of 256 columns
+    (2, 12, 12, 32, 128, 3, 3, 1, 1, "same"),     # 128 columns: the 128 x 128 form
+    (2, 11, 11, 40, 96, 3, 3, 1, 1, "same"),      # 96 of 128 columns
+    (2, 10, 10, 16, 320, 2, 2, 1, 1, "valid"),    # two n tiles, the second a quarter full
+    (5, 7, 9, 24, 72, 3, 3, 1, 1, "same"),        # 72 columns: forced onto the 128-wide form
+    (40, 8, 8, 64, 128, 3, 3, 1, 1, "same"),      # 2560 rows: several slabs per split
+]
+
+
+@pytest.mark.parametrize("mode", [1, 3], ids=["wide", "wide_256k"])   # 3: also 256 k rows per workgroup (8 waves)
+@pytest.mark.parametrize("case", WGRAD_WIDE_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_bf16_wgrad_on_wide_wave_tiles(case, mode, tune):
+    from tests import abi
+    tune(wgrad_wide=mode, wgrad_halo=0)
+    x, w, b, dy = _case(case, 17)
+    stride, pad = (case[7], case[8]), case[9]
+    xr, dyr = O.round_to_bf16(x), O.round_to_bf16(dy)
+    dw, db = abi.wgrad_bf16(x, dy, w.shape, stride, pad)
+    abi.close(dw, O.conv_wgrad(xr, dyr, w.shape[:2], stride, pad, dtype=np.float64), rms_scaled=True)
+    abi.close(db, O.conv_dbias(dyr, dtype=np.float64), rms_scaled=True)
+    dw2, db2 = abi.wgrad_bf16(x, dy, w.shape, stride, pad)
+    assert np.array_equal(dw, dw2) and np.array_equal(db, db2)            # deterministic
+    tune(wgrad_wide=0)                                                    # 64-wide tiles: another order of the same sums
+    dw3, db3 = abi.wgrad_bf16(x, dy, w.shape, stride, pad)
+    abi.close(dw3, dw, rtol=1e-4, atol=1e-5, rms_scaled=True)
+    abi.close(db3, db, rtol=1e-4, atol=1e-5, rms_scaled=True)
+
+
 # ---- bfloat16 copies left by the producing kernels ------------------------------------------
 # A bf16 convolution reads bfloat16 x and dy.  The layers that produce them (ReLU / leaky ReLU,
 # the fused batch-norm block, batch norm's backward pass) can leave the bfloat16 copy beside the
