@@ -72,7 +72,7 @@ __device__ __forceinline__ void mma_chunk<uint16_t>(const f4& a, const f4& b, f1
 // ------------------------------------------------------------------------------
 struct GatherParams {
     const void* src;     // [S, Hs, Ws, Cs] of T
-    const void* bt;      // packed filter [Npad][Kpad] of T, zero filled
+    const void* bt;      // packed filter [Npad][Kpad] of T, zero filled (or the filter itself: bt_direct)
     const float* bias;   // [N] or nullptr
     float* out;
     int S, Hs, Ws, Cs;
@@ -88,6 +88,12 @@ struct GatherParams {
     unsigned bt_bytes;
     unsigned out_bytes;  // extent of out; 0: no 16-byte stores (too large, N not a multiple of 4, or unaligned)
     int split_slabs;     // 0, or slabs of K per blockIdx.y: split y writes its partial product at out + y*M*N
+    // B operand addressing of the slab kernels: row n of the B matrix starts bt_ld elements after row n - 1.
+    // bt_direct (dgrad on uniform-tap slabs): bt is the filter w[fH][fW][C][D] itself, whose rows (tap, c) are
+    // already contiguous in k = d; the slab of tap (th, tw), channel offset c0 starts at element
+    // ((bd_xa + bd_xs th) bd_fw + bd_ya + bd_ys tw) * bd_tap_elems + c0 of row 0: no packing launch.
+    int bt_ld, bt_direct;
+    int bd_xa, bd_xs, bd_ya, bd_ys, bd_fw, bd_tap_elems;
     // gather_halo_bf16: columns and rows of the padded source image, 256-row tiles per image (0: tiles
     // run over image boundaries)
     int halo_wp, halo_hp, halo_tiles;

@@ -306,6 +306,29 @@ static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
             return AETH_OK;
         }
     }
+    // dgrad whose slabs lie inside one tap reads its B operand from w itself: row (tap, c) of w is
+    // contiguous in d, which is dgrad's k.  fp32 slab kernel with at least three slabs (shorter K
+    // goes to the n-loop and resident kernels, which keep the packed layout); tuning: gather_direct_b = 0 packs.
+    gs.gp.bt_ld = gs.gp.Kpad;
+    gs.gp.bt_direct = 0;
+    if constexpr (sizeof(T) == 4) {
+        const GatherParams& g = gs.gp;
+        const PackParams& pk = gs.pp;
+        const int taps = g.Cs > 0 ? g.K / g.Cs : 0;
+        if (pk.transposed && vec && g.src_bytes != 0 && g.Cs % 32 == 0 && g.K == g.Kpad && taps >= 1 && taps <= 32 &&
+            g.Kpad / 32 >= 3 && g.Th * g.Tw == taps && pk.w_elems * 4 < ((int64_t)1 << 31) &&
+            g.N % gather_bn(g.N) == 0 &&                 // no B rows past C: such rows of the last tap would lie behind w
+                                                         // (loads with a scalar offset are not range-checked against it)
+            (reinterpret_cast<uintptr_t>(pk.w) & 15) == 0 && tuning().gather_direct_b != 0 && tuning().gather_kc == -1) {
+            gs.gp.bt = pk.w;
+            gs.gp.bt_bytes = (unsigned)(pk.w_elems * 4);
+            gs.gp.bt_ld = pk.D;
+            gs.gp.bt_direct = 1;
+            gs.gp.bd_xa = pk.xa; gs.gp.bd_xs = pk.xs; gs.gp.bd_ya = pk.ya; gs.gp.bd_ys = pk.ys;
+            gs.gp.bd_fw = pk.fW; gs.gp.bd_tap_elems = pk.C * pk.D;
+            total = 0;                                   // nothing to pack
+        }
+    }
     if (total > 0) {
         hipLaunchKernelGGL(pack_filter<T>, dim3(cdiv(total, 256)), dim3(256), 0, c.stream, gs.pp);
         AETH_LAUNCH_CHECK();

@@ -308,7 +308,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
 #pragma unroll
         for (int i = 0; i < BL; ++i) {
             const int k4 = k4e ^ (((wave * BL + i) & 1) ? ODD : 0);
-            b_off[i] = (unsigned)(((n0 + (wave * BL + i) * RPL + lr) * p.Kpad + CE * k4) * (int)sizeof(T));
+            b_off[i] = (unsigned)(((n0 + (wave * BL + i) * RPL + lr) * p.bt_ld + CE * k4) * (int)sizeof(T));
         }
     };
     set_b_off();
@@ -324,14 +324,19 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
     // `prep` decodes the slab's tap(s) once, `issue_part(j)` issues load j of the
     // wave (j < AL: 8 rows of A, else 8 rows of B).
     unsigned ut_tap = 0, ut_tap_bytes = 0;              // UT: wave-uniform, scalar registers
+    unsigned b_k_bytes = 0;                              // byte offset of the slab inside a B row (wave-uniform)
     int tap_off[2] = {0, 0}, tap_h[2] = {0, 0}, tap_w[2] = {0, 0};
     bool kvalid[2] = {false, false};
     auto prep = [&](int k0) {
+        b_k_bytes = (unsigned)k0 * (unsigned)sizeof(T);
         if (UT) {
             unsigned c0, th, tw;
             p.div_c.divmod((unsigned)k0, ut_tap, c0);
             p.div_tw.divmod(ut_tap, th, tw);
             ut_tap_bytes = (unsigned)(((int)th * p.Ws + (int)tw) * p.Cs + (int)c0) * (unsigned)sizeof(T);
+            if (p.bt_direct)                             // the filter itself: tap (th, tw) of this class, channels c0..
+                b_k_bytes = (unsigned)(((p.bd_xa + p.bd_xs * (int)th) * p.bd_fw + p.bd_ya + p.bd_ys * (int)tw) * p.bd_tap_elems +
+                                       (int)c0) * (unsigned)sizeof(T);
             if constexpr (SA) cur_mask = (unsigned)__builtin_amdgcn_ballot_w64(((aux_row >> ut_tap) & 1u) != 0u);
             return;
         }
@@ -352,8 +357,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
         if constexpr (SA) {
             if (j >= AL) {
                 const int i = j - AL;
-                lds_direct_load16_s(sa_rsrc_b, lds_address(lb) + (unsigned)(wave_u * BL + i) * 1024u, b_off[i],
-                                    (unsigned)k0 * (unsigned)sizeof(T));
+                lds_direct_load16_s(sa_rsrc_b, lds_address(lb) + (unsigned)(wave_u * BL + i) * 1024u, b_off[i], b_k_bytes);
                 return;
             }
             // the load's 8 (16 with half-depth slabs) rows of the mask, a bit per row
@@ -366,7 +370,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
         if (j >= AL) {
             const int i = j - AL;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(lb + (wave * BL + i) * 64), 16,
-                                                     (int)(b_off[i] + (unsigned)k0 * (unsigned)sizeof(T)), 0, 0, 0);
+                                                     (int)(b_off[i] + b_k_bytes), 0, 0, 0);
             return;
         }
         const int i = j;
@@ -478,6 +482,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
 #pragma unroll
             for (int j = 0; j < AL; ++j) issue_load(j, BK, lds_a1, lds_b1);
         }
+        b_k_bytes = 0;
 #pragma unroll
         for (int j = AL; j < NL; ++j) issue_load(j, 0, lds_a0, lds_b0);         // B of step 0
         fill_acc<TM, TN>(bv, acc);
@@ -517,6 +522,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
                 const int k0_next = nslabs == 2 ? (fn & 1) * BK : 0;
                 n0 = nt_next * BN;
                 set_b_off();
+                b_k_bytes = (unsigned)k0_next * (unsigned)sizeof(T);     // (the packed filter: this mode never reads w itself)
 #pragma unroll
                 for (int j = AL; j < NL; ++j) issue_load(j, k0_next, lds_a0, nb);
             }

@@ -259,6 +259,35 @@ def test_fprop_dgrad_with_scalar_addressed_loads(case, bm, tune):
     assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
 
 
+# dgrad whose slabs lie inside one filter tap (output channels in whole slabs of 32, input channels filling
+# their tiles) reads its B operand from the filter itself instead of a packed copy: row (tap, c) of
+# w[fH][fW][C][D] is contiguous in d, which is dgrad's k.  The gather_direct_b switch at 0 packs as before;
+# both must give the same bits (same slabs, same order).
+DIRECT_B_CASES = [
+    (4, 16, 16, 32, 64, 3, 3, 1, 1, "same"),      # 32 input channels: 32-wide tiles
+    (3, 8, 8, 64, 128, 3, 3, 1, 1, "same"),       # 4 slabs per tap
+    (2, 20, 20, 64, 64, 3, 3, 2, 2, "same"),      # stride 2: classes of 4, 2, 2 and 1 taps (the 1- and 2-tap ones keep packing: K < 3 slabs)
+    (2, 13, 11, 128, 96, 5, 5, 1, 1, "same"),     # 25 taps of 3 slabs, two n tiles
+    (2, 12, 12, 64, 32, 4, 4, 3, 3, "valid"),     # stride 3, even filter: taps differ per class
+    (128, 1, 1, 2048, 256, 1, 1, 1, 1, "valid"),  # a dense layer's input gradient: one tap, split K
+    (2, 12, 12, 48, 64, 3, 3, 1, 1, "same"),      # 48 input channels do not fill a 64-wide tile: packed
+    (2, 12, 12, 64, 40, 3, 3, 1, 1, "same"),      # 40 output channels: slabs straddle taps, packed
+]
+
+
+@pytest.mark.parametrize("case", DIRECT_B_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_dgrad_reading_the_filter_in_place(case, tune):
+    from tests import abi
+    x, w, b, dy = _case(case, 21)
+    stride, pad = (case[7], case[8]), case[9]
+    dx = abi.dgrad(dy, w, x.shape, stride, pad)
+    abi.close(dx, O.conv_dgrad(dy, w, x.shape[1:3], stride, pad, dtype=np.float64))
+    tune(gather_direct_b=0)
+    assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
+    tune(gather_direct_b=-1, gather_sa=0)             # vector-addressed loads: the other form of the B loads
+    assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
+
+
 # fp32 wgrad of a unit-stride filter of at most 9 taps on 64 input channels and at most 64 output
 # channels, on rows of 28, 32, 56 or 64 output pixels: one persistent workgroup per CU keeps the whole
 # K x N result in registers (12 multiplying waves of three 32 x 32 blocks) and a loading wave brings one
