@@ -464,6 +464,15 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
             return AETH_OK;
         }
     }
+    // Rows of dx beyond h_last and columns beyond w_last are reached by no output pixel (the largest
+    // index a tap touches is (Ho - 1) sH + fH - 1 - pH): the classes' pixel grids stop there and one small
+    // launch zeroes the strips, instead of multiplying rows of padding (tuning: gather_clip = 0 keeps the full grids).
+    int h_lim = H, w_lim = W;
+    if (tuning().gather_clip != 0) {
+        h_lim = std::min(H, (Ho - 1) * sH + fH - pH);
+        w_lim = std::min(W, (Wo - 1) * sW + fW - pW);
+        if (h_lim < 1 || w_lim < 1) { h_lim = H; w_lim = W; }
+    }
     std::vector<GatherSetup> sets;
     int64_t total_bytes = 0;
     for (int a = 0; a < sH; ++a) {
@@ -472,14 +481,14 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
         int Th = ra < fH ? (fH - 1 - ra) / sH + 1 : 0;
         int xmax = ra + (Th - 1) * sH;
         int offh = Th > 0 ? (a + pH - xmax) / sH : 0;   // exact: (a+pH-xmax) is a multiple of sH
-        int Hg = (H - a + sH - 1) / sH;
+        int Hg = (std::min(H, std::max(h_lim, a + 1)) - a + sH - 1) / sH;      // class rows i = a + sH i' below h_lim (at least one)
         for (int b = 0; b < sW; ++b) {
             if (b >= W) continue;
             int rb = (b + pW) % sW;
             int Tw = rb < fW ? (fW - 1 - rb) / sW + 1 : 0;
             int ymax = rb + (Tw - 1) * sW;
             int offw = Tw > 0 ? (b + pW - ymax) / sW : 0;
-            int Wg = (W - b + sW - 1) / sW;
+            int Wg = (std::min(W, std::max(w_lim, b + 1)) - b + sW - 1) / sW;
             GatherSetup gs;
             GatherParams& g = gs.gp;
             g.src = dy; g.bias = nullptr; g.out = dx;
@@ -510,6 +519,20 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
         rc = run_gather<T>(gs, (char*)ws, off, D % Elem<T>::CE == 0);
         if (rc) return rc;
         off += gs.bt_bytes + gs.part_bytes;
+    }
+    if (h_lim < H || w_lim < W) {
+        ZeroStripParams zp;
+        zp.dx = dx; zp.S = S; zp.H = H; zp.W = W; zp.C = C; zp.h0 = h_lim; zp.w0 = w_lim;
+        zp.per_image = (H - h_lim) * W + h_lim * (W - w_lim);
+        zp.vec = (C % 4 == 0 && (reinterpret_cast<uintptr_t>(dx) & 15) == 0) ? 1 : 0;
+        zp.cgroups = zp.vec ? C / 4 : C;
+        zp.div_cg = FastDiv(zp.cgroups);
+        zp.div_pi = FastDiv(zp.per_image);
+        zp.div_w = FastDiv(W);
+        zp.div_wt = FastDiv(W - w_lim > 0 ? W - w_lim : 1);
+        const int64_t n = (int64_t)S * zp.per_image * zp.cgroups;     // below 2^31: it is a part of dx
+        hipLaunchKernelGGL(zero_strips, dim3((unsigned)cdiv(n, kThreads)), dim3(kThreads), 0, ctx().stream, zp, (unsigned)n);
+        AETH_LAUNCH_CHECK();
     }
     return AETH_OK;
 }

@@ -1172,6 +1172,37 @@ static __global__ __launch_bounds__(kD1Threads, 1) void dense_res_f32(const Gath
     if (active && have_done) store_done();
 }
 
+// dx[s][i][j][:] = 0 for i >= h0 or j >= w0: the trailing rows and columns of a strided dgrad that
+// no output pixel reaches (a 28 x 28 input under a 3 x 3 stride-2 "valid" filter: row and column 27).
+// One thread per strip pixel and group of 4 channels (C % 4 == 0) or per channel.
+struct ZeroStripParams {
+    float* dx;
+    int S, H, W, C, h0, w0;
+    int per_image;       // strip pixels per image: (H - h0) * W + h0 * (W - w0)
+    int cgroups, vec;    // channel groups per pixel; 1: groups of 4 with 16-byte stores
+    FastDiv div_cg, div_pi, div_w, div_wt;
+};
+
+static __global__ __launch_bounds__(kThreads) void zero_strips(const ZeroStripParams p, const unsigned n) {
+    const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    unsigned t, cg, s, b;
+    p.div_cg.divmod(i, t, cg);
+    p.div_pi.divmod(t, s, b);
+    unsigned row, col;
+    const unsigned bottom = (unsigned)((p.H - p.h0) * p.W);
+    if (b < bottom) {                                    // the rows from h0 on, whole width
+        p.div_w.divmod(b, row, col);
+        row += (unsigned)p.h0;
+    } else {                                             // the columns from w0 on of the rows above
+        p.div_wt.divmod(b - bottom, row, col);
+        col += (unsigned)p.w0;
+    }
+    const size_t pix = ((size_t)s * p.H + row) * p.W + col;
+    if (p.vec) *reinterpret_cast<f4*>(p.dx + pix * p.C + 4 * cg) = f4{0.f, 0.f, 0.f, 0.f};
+    else p.dx[pix * p.C + cg] = 0.f;
+}
+
 template <typename T>
 __global__ void pack_filter(const PackParams p) {
     int idx = blockIdx.x * blockDim.x + threadIdx.x;

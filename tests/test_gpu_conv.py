@@ -288,6 +288,30 @@ def test_dgrad_reading_the_filter_in_place(case, tune):
     assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
 
 
+# Strided dgrad whose last rows / columns are reached by no output pixel: the classes' pixel grids stop
+# at the last reachable index and one small launch zeroes the strips.  The gather_clip switch at 0
+# multiplies the full grids (every tap of those pixels falls outside dy: zeros); same bits either way.
+CLIP_CASES = [
+    (3, 12, 12, 8, 16, 3, 3, 2, 2, "valid"),      # row and column 11 untouched
+    (2, 28, 28, 32, 64, 3, 3, 2, 2, "valid"),     # the stride-2 benchmark layer's geometry, fewer channels
+    (2, 14, 13, 6, 8, 2, 2, 3, 3, "valid"),       # filter smaller than the stride: gaps (classes without taps) and two untouched columns
+    (2, 11, 9, 5, 8, 5, 5, 3, 3, "valid"),        # 5 channels: scalar stores in the strip; one untouched column
+    (2, 10, 10, 4, 8, 3, 3, 2, 2, "same"),        # nothing to clip
+    (2, 9, 16, 64, 32, 3, 3, 1, 4, "valid"),      # stride (1, 4): three untouched columns, none of the rows
+]
+
+
+@pytest.mark.parametrize("case", CLIP_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_strided_dgrad_with_clipped_class_grids(case, tune):
+    from tests import abi
+    x, w, b, dy = _case(case, 22)
+    stride, pad = (case[7], case[8]), case[9]
+    dx = abi.dgrad(dy, w, x.shape, stride, pad)          # the output buffer starts as NaN: every element must be written
+    abi.close(dx, O.conv_dgrad(dy, w, x.shape[1:3], stride, pad, dtype=np.float64))
+    tune(gather_clip=0)
+    assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
+
+
 # fp32 wgrad of a unit-stride filter of at most 9 taps on 64 input channels and at most 64 output
 # channels, on rows of 28, 32, 56 or 64 output pixels: one persistent workgroup per CU keeps the whole
 # K x N result in registers (12 multiplying waves of three 32 x 32 blocks) and a loading wave brings one
