@@ -311,17 +311,20 @@ static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
     // goes to the n-loop and resident kernels, which keep the packed layout); tuning: gather_direct_b = 0 packs.
     gs.gp.bt_ld = gs.gp.Kpad;
     gs.gp.bt_direct = 0;
-    if constexpr (sizeof(T) == 4) {
+    {
         const GatherParams& g = gs.gp;
         const PackParams& pk = gs.pp;
+        constexpr int BK = Elem<T>::BK;
         const int taps = g.Cs > 0 ? g.K / g.Cs : 0;
-        if (pk.transposed && vec && g.src_bytes != 0 && g.Cs % 32 == 0 && g.K == g.Kpad && taps >= 1 && taps <= 32 &&
-            g.Kpad / 32 >= 3 && g.Th * g.Tw == taps && pk.w_elems * 4 < ((int64_t)1 << 31) &&
-            g.N % gather_bn(g.N) == 0 &&                 // no B rows past C: such rows of the last tap would lie behind w
-                                                         // (loads with a scalar offset are not range-checked against it)
+        // fp32: no B rows past C, such rows of the last tap would lie behind w and the fp32 kernel's loads carry the
+        // tap in a scalar offset, which the range check does not see; the bf16 kernels' loads are checked in full,
+        // their rows past C read zeros or other taps and feed only columns that are not stored
+        const bool rows_ok = sizeof(T) == 4 ? g.N % gather_bn(g.N) == 0 : g.N % 8 == 0;
+        if (pk.transposed && vec && g.src_bytes != 0 && g.Cs % BK == 0 && g.K == g.Kpad && taps >= 1 && taps <= 32 &&
+            g.Kpad / BK >= 3 && g.Th * g.Tw == taps && pk.w_elems * (int64_t)sizeof(T) < ((int64_t)1 << 31) && rows_ok &&
             (reinterpret_cast<uintptr_t>(pk.w) & 15) == 0 && tuning().gather_direct_b != 0 && tuning().gather_kc == -1) {
             gs.gp.bt = pk.w;
-            gs.gp.bt_bytes = (unsigned)(pk.w_elems * 4);
+            gs.gp.bt_bytes = (unsigned)(pk.w_elems * (int64_t)sizeof(T));
             gs.gp.bt_ld = pk.D;
             gs.gp.bt_direct = 1;
             gs.gp.bd_xa = pk.xa; gs.gp.bd_xs = pk.xs; gs.gp.bd_ya = pk.ya; gs.gp.bd_ys = pk.ys;

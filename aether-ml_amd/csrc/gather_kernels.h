@@ -700,7 +700,7 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_bf16(const Gat
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const int k4 = k4e ^ (((wave * 2 + i) & 1) ? 4 : 0);
-        b_off[i] = (unsigned)(((n0 + (wave * 2 + i) * 8 + (lane >> 3)) * p.Kpad + 8 * k4) * 2);
+        b_off[i] = (unsigned)(((n0 + (wave * 2 + i) * 8 + (lane >> 3)) * p.bt_ld + 8 * k4) * 2);
     }
     const u32x4 rsrc_a = raw_rsrc(p.src, p.src_bytes);
     const u32x4 rsrc_b = raw_rsrc(p.bt, p.bt_bytes);
@@ -722,9 +722,16 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_bf16(const Gat
     // (with conditional loads the compiler cannot tell which loads a count leaves in
     // flight and waits for all of them before the first LDS read).
     int pf_tap = 0, pf_cb = 0;
+    int pf_th = 0, pf_tw = 0;                            // the prefetched tap as (row, column) of the class
     auto pf_next = [&]() __attribute__((always_inline)) {
-        const unsigned k0_bytes = pf_cb < p.Cs / BK ? (unsigned)(pf_tap * p.Cs + pf_cb * BK) * 2u : 0x80000000u;
-        if (++pf_tap == T) { pf_tap = 0; ++pf_cb; }
+        // start of the slab inside a B row: packed filter k = tap * Cs + 64 * block; the filter itself (bt_direct):
+        // tap (th, tw) of this class is w's tap (bd_xa + bd_xs th, bd_ya + bd_ys tw), whose rows hold the Cs channels
+        const int k_elems = p.bt_direct
+            ? ((p.bd_xa + p.bd_xs * pf_th) * p.bd_fw + p.bd_ya + p.bd_ys * pf_tw) * p.bd_tap_elems + pf_cb * BK
+            : pf_tap * p.Cs + pf_cb * BK;
+        const unsigned k0_bytes = pf_cb < p.Cs / BK ? (unsigned)k_elems * 2u : 0x80000000u;
+        if (++pf_tw == p.Tw) { pf_tw = 0; ++pf_th; }
+        if (++pf_tap == T) { pf_tap = 0; pf_th = 0; pf_tw = 0; ++pf_cb; }
         return k0_bytes;
     };
     load_halo(0);

@@ -275,6 +275,33 @@ def test_bf16_wgrad_with_the_whole_result_in_registers(case, tune):
     abi.close(db3, db, rtol=1e-4, atol=1e-5, rms_scaled=True)
 
 
+# bf16 dgrad reads its filter operand from w itself where slabs lie inside one tap (output channels in whole
+# slabs of 64): the halo kernel, the slab kernel and its 8-wave tiles.  The gather_direct_b switch at 0 packs;
+# same bits either way.
+DIRECT_B_BF16_CASES = [
+    (2, 16, 16, 64, 64, 3, 3, 1, 1, "same", {}),                    # gather_halo_res_bf16 reads w itself anyway
+    (2, 16, 16, 64, 128, 3, 3, 1, 1, "same", {"gather_split": 0}),    # halo kernel, two slabs per tap
+    (3, 13, 13, 128, 256, 3, 3, 2, 2, "valid", {"gather_split": 0}),  # the stride-2 layer: classes of 4, 2, 2, 1 taps
+    (2, 14, 14, 64, 256, 1, 1, 1, 1, "valid", {"gather_split": 0}),   # 1x1: one tap of 4 slabs, slab kernel
+    (2, 9, 9, 40, 128, 3, 3, 1, 1, "same", {"gather_split": 0}),      # 40 input channels: rows past C in the tile
+    (2, 12, 12, 256, 192, 3, 3, 1, 1, "same", {"gather_split": 0, "gather_wide": 1}),   # 8-wave tiles
+    (2, 10, 10, 64, 96, 3, 3, 1, 1, "same", {"gather_split": 0}),     # 96 output channels: slabs straddle taps, packed
+]
+
+
+@pytest.mark.parametrize("case", DIRECT_B_BF16_CASES, ids=lambda c: "x".join(str(v) for v in c[:10]))
+def test_bf16_dgrad_reading_the_filter_in_place(case, tune):
+    from tests import abi
+    x, w, b, dy = _case(case[:10], 23)
+    stride, pad = (case[7], case[8]), case[9]
+    tune(**case[10])
+    dyr, wr = O.round_to_bf16(dy), O.round_to_bf16(w)
+    dx = abi.dgrad_bf16(dy, w, x.shape, stride, pad)
+    abi.close(dx, O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
+    tune(gather_direct_b=0)
+    assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
+
+
 # bf16 wgrad onto more than 64 output channels: wave tiles of 64 k x 128 n (workgroup 128 k x 256 n) or
 # 64 k x 64 n (128 x 128), where the library takes them from the channel padding they cost; the
 # wgrad_wide switch forces them (1: the narrower form wherever D > 64) or turns them off (0).
