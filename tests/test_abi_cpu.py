@@ -109,3 +109,21 @@ def test_two_dimensional_targets_must_be_one_hot():
         _sparse_labels(np.eye(3)[y] * 0.9 + 0.1 / 3)
     with pytest.raises(ValueError):
         _sparse_labels(np.array([[1.0, 1.0, 0.0]]))
+
+
+def test_debug_switches_are_known_by_name(lib):
+    """aeth_debug_set may be called before aeth_init: known names are accepted, -1 and NULL reset,
+    an unknown name is refused with a message that names it."""
+    for name in (b"gather_bm", b"gather_kc", b"gather_nloop", b"gather_halo", b"gather_split", b"gather_sa",
+                 b"gather_direct_b", b"gather_clip", b"gather_wide", b"gather_res", b"dense_res", b"direct",
+                 b"wgrad_halo", b"wgrad_wide", b"wgrad_cw", b"wgrad_br", b"wgrad_rounds"):
+        assert lib.aeth_debug_set(name, 1) == 0, name
+        assert lib.aeth_debug_set(name, -1) == 0, name
+    assert lib.aeth_debug_set(None, 0) == 0
+    assert lib.aeth_debug_set(b"no_such_switch", 1) == -1
+    assert b"no_such_switch" in lib.aeth_last_error()
+    # every name the header lists is one the library knows
+    text = open(HEADER).read()
+    doc = text[text.index("Names:"):text.index("May be called before aeth_init")]
+    for name in doc.replace("Names:", "").replace("*", " ").replace(".", " ").replace(",", " ").split():
+        assert lib.aeth_debug_set(name.encode(), -1) == 0, name
