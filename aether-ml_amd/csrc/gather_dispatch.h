@@ -103,10 +103,10 @@ static inline int gather_bm(int M, int N, int cus, bool dma, int elem_bytes = 4)
 // when the span of every tile fits its buffer: with tiles cut per image (at most 10 % of empty
 // rows) or, failing that, running over image boundaries.  Fills the halo fields of gp and the
 // number of 256-row tiles when it does.
-static bool plan_halo(GatherParams& gp, bool dma, int* mtiles, int* stages) {
+static bool plan_halo(GatherParams& gp, bool dma, int* mtiles, int* stages, int min_taps = 2, int max_slots = kHaloSlotsMax) {
     if (!dma || gp.sh != 1 || gp.sw != 1 || gp.Cs % 64 != 0 || gp.K != gp.Kpad || gp.split_slabs != 0) return false;
     const int taps = gp.Th * gp.Tw;
-    if (taps < 2 || taps > 32 || gp.N <= 32 || gp.Cs <= 0 || gp.K != taps * gp.Cs) return false;
+    if (taps < min_taps || taps > 32 || gp.N <= 32 || gp.Cs <= 0 || gp.K != taps * gp.Cs) return false;
     if (tuning().gather_halo == 0) return false;
     const int hw = gp.Hg * gp.Wg;
     const int wp = gp.Wg + gp.Tw - 1, hp = gp.Hg + gp.Th - 1;
@@ -119,7 +119,7 @@ static bool plan_halo(GatherParams& gp, bool dma, int* mtiles, int* stages) {
     auto fits = [&](int64_t first, int64_t last) {
         const int64_t span = slot0(last) + (int64_t)(gp.Th - 1) * wp + gp.Tw - slot0(first);
         longest = std::max(longest, span);
-        return span <= kHaloSlotsMax;
+        return span <= max_slots;
     };
     // tiles cut per image: every image has the same tiles
     const int per_img = cdiv(hw, kHaloBM);
@@ -246,6 +246,73 @@ struct GatherSetup {
     int64_t part_bytes = 0;
 };
 
+// The kernels that multiply two classes of one dgrad from one halo take 2 or 4 classes that gather_halo_bf16 would take
+// (`sets`, already filled in by plan_halo) when every tile of `bm` pixels has a span of the common padded source tensor that
+// fits `max_slots`.  The classes are paired (most taps with fewest) and given the common geometry.
+static bool plan_class_pairs(const std::vector<GatherSetup>& sets, GatherClasses& gc, int bm, int max_slots, int64_t* mtiles, int64_t* longest) {
+    const int n = (int)sets.size();
+    if (n != 2 && n != 4) return false;
+    const GatherParams& g0 = sets[0].gp;
+    if (g0.Cs % 64 != 0 || g0.M <= 0 || g0.out_bytes == 0 || g0.bias != nullptr) return false;
+    int rh_min = g0.rh0, rw_min = g0.rw0;
+    for (const GatherSetup& gs : sets) {
+        const GatherParams& g = gs.gp;
+        if (g.Hg != g0.Hg || g.Wg != g0.Wg || g.M != g0.M || g.N != g0.N || g.Cs != g0.Cs || g.src != g0.src || g.S != g0.S ||
+            g.Hs != g0.Hs || g.Ws != g0.Ws || g.Th < 1 || g.Tw < 1 || g.sh != 1 || g.sw != 1)
+            return false;
+        rh_min = std::min(rh_min, g.rh0);
+        rw_min = std::min(rw_min, g.rw0);
+    }
+    int hth = 1, htw = 1;
+    for (const GatherSetup& gs : sets) {
+        hth = std::max(hth, gs.gp.rh0 - rh_min + gs.gp.Th);
+        htw = std::max(htw, gs.gp.rw0 - rw_min + gs.gp.Tw);
+    }
+    const int hw = g0.Hg * g0.Wg;
+    const int wp = g0.Wg + htw - 1, hp = g0.Hg + hth - 1;
+    if ((int64_t)g0.S * hp * wp >= ((int64_t)1 << 30)) return false;
+    auto slot0 = [&](int64_t m) {
+        const int64_t s = m / hw, rem = m % hw;
+        return (s * hp + rem / g0.Wg) * wp + rem % g0.Wg;
+    };
+    const int64_t mt = cdiv(g0.M, bm);
+    if (mt > (1 << 20)) return false;
+    *longest = 0;
+    for (int64_t t = 0; t < mt; ++t) {
+        const int64_t first = t * bm, last = std::min<int64_t>((t + 1) * bm, g0.M) - 1;
+        const int64_t span = slot0(last) + (int64_t)(hth - 1) * wp + htw - slot0(first);
+        if (span > max_slots) return false;
+        *longest = std::max(*longest, span);
+    }
+    // most taps first; pairs (0, n - 1), (1, n - 2)
+    int order[kMaxClasses];
+    for (int i = 0; i < n; ++i) {
+        int j = i;
+        const int taps = sets[i].gp.Th * sets[i].gp.Tw;
+        for (; j > 0 && sets[order[j - 1]].gp.Th * sets[order[j - 1]].gp.Tw < taps; --j) order[j] = order[j - 1];
+        order[j] = i;
+    }
+    for (int i = 0; i < n; ++i) {
+        const int src = (i % 2 == 0) ? order[i / 2] : order[n - 1 - i / 2];
+        GatherParams g = sets[src].gp;
+        g.tap_dh = g.rh0 - rh_min;
+        g.tap_dw = g.rw0 - rw_min;
+        g.rh0 = rh_min;
+        g.rw0 = rw_min;
+        g.halo_th = hth;
+        g.halo_tw = htw;
+        g.halo_wp = wp;
+        g.halo_hp = hp;
+        g.halo_tiles = 0;
+        g.div_halo_wp = FastDiv(wp);
+        g.div_halo_hp = FastDiv(hp);
+        gc.cls[i] = g;
+    }
+    gc.ncls = n;
+    *mtiles = mt;
+    return mt * cdiv(g0.N, 64) * n < ((int64_t)1 << 30);
+}
+
 // Split K when the tiles alone would leave most of the chip idle: at most one tile per
 // two CUs and at least 8 slabs of K.  Only for the LDS-direct kernel with 16-byte stores
 // to a dense [M, N] output.  Aim: about two workgroups per CU, at least 4 slabs each.
@@ -275,25 +342,60 @@ static void plan_split(GatherSetup& gs, bool vec, int cus) {
     gs.part_bytes = round_up((int64_t)gs.nsplit * ob, 256);
 }
 
+// Where the B operand of a problem comes from and how far its tensors reach: the workspace slot at
+// `ws_off` for the packed filter, the byte extents for the buffer descriptors, the filter rows.
 template <typename T>
-static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
-    Context& c = ctx();
+static void fill_gather(GatherSetup& gs, char* ws, int64_t ws_off) {
     void* bt = ws + ws_off;
     gs.gp.bt = bt;
     gs.pp.bt = bt;
-    int total = gs.pp.Npad * gs.pp.Kpad;
-    {
-        const GatherParams& g = gs.gp;
-        int64_t sb = (int64_t)g.S * g.Hs * g.Ws * g.Cs * (int64_t)sizeof(T);
-        int64_t bb = (int64_t)total * (int64_t)sizeof(T);
-        const int64_t lim = (int64_t)1 << 31;
-        gs.gp.Th = (g.Tw > 0 && g.Cs > 0) ? (g.K / g.Cs) / g.Tw : 0;
-        gs.gp.src_bytes = (sb < lim && bb < lim) ? (unsigned)sb : 0u;
-        gs.gp.bt_bytes = (sb < lim && bb < lim) ? (unsigned)bb : 0u;
-        const int64_t ob = (g.dense_out ? (int64_t)g.M : (int64_t)g.S * g.Hof * g.Wof) * g.N * (int64_t)sizeof(float);
-        const bool ovec = ob < lim && g.N % 4 == 0 && (reinterpret_cast<uintptr_t>(g.out) & 15) == 0;
-        gs.gp.out_bytes = ovec ? (unsigned)ob : 0u;
+    const GatherParams& g = gs.gp;
+    const int64_t total = (int64_t)gs.pp.Npad * gs.pp.Kpad;
+    int64_t sb = (int64_t)g.S * g.Hs * g.Ws * g.Cs * (int64_t)sizeof(T);
+    int64_t bb = total * (int64_t)sizeof(T);
+    const int64_t lim = (int64_t)1 << 31;
+    gs.gp.Th = (g.Tw > 0 && g.Cs > 0) ? (g.K / g.Cs) / g.Tw : 0;
+    gs.gp.src_bytes = (sb < lim && bb < lim) ? (unsigned)sb : 0u;
+    gs.gp.bt_bytes = (sb < lim && bb < lim) ? (unsigned)bb : 0u;
+    const int64_t ob = (g.dense_out ? (int64_t)g.M : (int64_t)g.S * g.Hof * g.Wof) * g.N * (int64_t)sizeof(float);
+    const bool ovec = ob < lim && g.N % 4 == 0 && (reinterpret_cast<uintptr_t>(g.out) & 15) == 0;
+    gs.gp.out_bytes = ovec ? (unsigned)ob : 0u;
+    gs.gp.bt_ld = gs.gp.Kpad;
+    gs.gp.bt_direct = 0;
+}
+
+// dgrad whose slabs lie inside one tap reads its B operand from w itself: row (tap, c) of w is
+// contiguous in d, which is dgrad's k.  fp32 slab kernel with at least `min_slabs` = 3 slabs (shorter K
+// goes to the n-loop and resident kernels, which keep the packed layout); tuning: gather_direct_b = 0 packs.
+// Returns the number of elements pack_filter has to write (0: the filter is read in place).
+template <typename T>
+static int choose_b_operand(GatherSetup& gs, bool vec, int min_slabs = 3) {
+    const GatherParams& g = gs.gp;
+    const PackParams& pk = gs.pp;
+    constexpr int BK = Elem<T>::BK;
+    const int taps = g.Cs > 0 ? g.K / g.Cs : 0;
+    // fp32: no B rows past C, such rows of the last tap would lie behind w and the fp32 kernel's loads carry the
+    // tap in a scalar offset, which the range check does not see; the bf16 kernels' loads are checked in full,
+    // their rows past C read zeros or other taps and feed only columns that are not stored
+    const bool rows_ok = sizeof(T) == 4 ? g.N % gather_bn(g.N) == 0 : g.N % 8 == 0;
+    if (pk.transposed && vec && g.src_bytes != 0 && g.Cs % BK == 0 && g.K == g.Kpad && taps >= 1 && taps <= 32 &&
+        g.Kpad / BK >= min_slabs && g.Th * g.Tw == taps && pk.w_elems * (int64_t)sizeof(T) < ((int64_t)1 << 31) && rows_ok &&
+        (reinterpret_cast<uintptr_t>(pk.w) & 15) == 0 && tuning().gather_direct_b != 0 && tuning().gather_kc == -1) {
+        gs.gp.bt = pk.w;
+        gs.gp.bt_bytes = (unsigned)(pk.w_elems * (int64_t)sizeof(T));
+        gs.gp.bt_ld = pk.D;
+        gs.gp.bt_direct = 1;
+        gs.gp.bd_xa = pk.xa; gs.gp.bd_xs = pk.xs; gs.gp.bd_ya = pk.ya; gs.gp.bd_ys = pk.ys;
+        gs.gp.bd_fw = pk.fW; gs.gp.bd_tap_elems = pk.C * pk.D;
+        return 0;                                    // nothing to pack
     }
+    return pk.Npad * pk.Kpad;
+}
+
+template <typename T>
+static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
+    Context& c = ctx();
+    fill_gather<T>(gs, ws, ws_off);
     if constexpr (sizeof(T) == 2) {
         // the kernel that keeps the whole filter in LDS reads it from w itself
         GatherParams hp = gs.gp;
@@ -306,32 +408,7 @@ static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
             return AETH_OK;
         }
     }
-    // dgrad whose slabs lie inside one tap reads its B operand from w itself: row (tap, c) of w is
-    // contiguous in d, which is dgrad's k.  fp32 slab kernel with at least three slabs (shorter K
-    // goes to the n-loop and resident kernels, which keep the packed layout); tuning: gather_direct_b = 0 packs.
-    gs.gp.bt_ld = gs.gp.Kpad;
-    gs.gp.bt_direct = 0;
-    {
-        const GatherParams& g = gs.gp;
-        const PackParams& pk = gs.pp;
-        constexpr int BK = Elem<T>::BK;
-        const int taps = g.Cs > 0 ? g.K / g.Cs : 0;
-        // fp32: no B rows past C, such rows of the last tap would lie behind w and the fp32 kernel's loads carry the
-        // tap in a scalar offset, which the range check does not see; the bf16 kernels' loads are checked in full,
-        // their rows past C read zeros or other taps and feed only columns that are not stored
-        const bool rows_ok = sizeof(T) == 4 ? g.N % gather_bn(g.N) == 0 : g.N % 8 == 0;
-        if (pk.transposed && vec && g.src_bytes != 0 && g.Cs % BK == 0 && g.K == g.Kpad && taps >= 1 && taps <= 32 &&
-            g.Kpad / BK >= 3 && g.Th * g.Tw == taps && pk.w_elems * (int64_t)sizeof(T) < ((int64_t)1 << 31) && rows_ok &&
-            (reinterpret_cast<uintptr_t>(pk.w) & 15) == 0 && tuning().gather_direct_b != 0 && tuning().gather_kc == -1) {
-            gs.gp.bt = pk.w;
-            gs.gp.bt_bytes = (unsigned)(pk.w_elems * (int64_t)sizeof(T));
-            gs.gp.bt_ld = pk.D;
-            gs.gp.bt_direct = 1;
-            gs.gp.bd_xa = pk.xa; gs.gp.bd_xs = pk.xs; gs.gp.bd_ya = pk.ya; gs.gp.bd_ys = pk.ys;
-            gs.gp.bd_fw = pk.fW; gs.gp.bd_tap_elems = pk.C * pk.D;
-            total = 0;                                   // nothing to pack
-        }
-    }
+    const int total = choose_b_operand<T>(gs, vec);
     if (total > 0) {
         hipLaunchKernelGGL(pack_filter<T>, dim3(cdiv(total, 256)), dim3(256), 0, c.stream, gs.pp);
         AETH_LAUNCH_CHECK();
@@ -478,42 +555,129 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
     }
     std::vector<GatherSetup> sets;
     int64_t total_bytes = 0;
-    for (int a = 0; a < sH; ++a) {
-        if (a >= H) continue;
-        int ra = (a + pH) % sH;
-        int Th = ra < fH ? (fH - 1 - ra) / sH + 1 : 0;
-        int xmax = ra + (Th - 1) * sH;
-        int offh = Th > 0 ? (a + pH - xmax) / sH : 0;   // exact: (a+pH-xmax) is a multiple of sH
-        int Hg = (std::min(H, std::max(h_lim, a + 1)) - a + sH - 1) / sH;      // class rows i = a + sH i' below h_lim (at least one)
-        for (int b = 0; b < sW; ++b) {
-            if (b >= W) continue;
-            int rb = (b + pW) % sW;
-            int Tw = rb < fW ? (fW - 1 - rb) / sW + 1 : 0;
-            int ymax = rb + (Tw - 1) * sW;
-            int offw = Tw > 0 ? (b + pW - ymax) / sW : 0;
-            int Wg = (std::min(W, std::max(w_lim, b + 1)) - b + sW - 1) / sW;
-            GatherSetup gs;
-            GatherParams& g = gs.gp;
-            g.src = dy; g.bias = nullptr; g.out = dx;
-            g.S = S; g.Hs = Ho; g.Ws = Wo; g.Cs = D;
-            g.Hg = Hg; g.Wg = Wg; g.M = S * Hg * Wg; g.N = C;
-            g.K = Th * Tw * D;
-            g.Kpad = (int)round_up(g.K, BK);
-            g.Tw = Tw; g.sh = 1; g.sw = 1; g.rh0 = offh; g.rw0 = offw;
-            g.Hof = H; g.Wof = W; g.oh0 = a; g.ow0 = b; g.ohs = sH; g.ows = sW;
-            g.dense_out = (nclass == 1);
-            set_out_divs(g);
-            PackParams& pk = gs.pp;
-            pk.w = w; pk.fW = fW; pk.C = C; pk.D = D; pk.Tw = Tw > 0 ? Tw : 1; pk.Ck = D; pk.w_elems = (int64_t)fH * fW * C * D;
-            pk.xa = xmax; pk.xs = -sH; pk.ya = ymax; pk.ys = -sW; pk.transposed = 1;
-            pk.N = C; pk.K = g.K; pk.Npad = (int)round_up(C, 64); pk.Kpad = g.Kpad;
-            gs.bt_bytes = round_up((int64_t)pk.Npad * pk.Kpad * sizeof(T), 256);
-            g.split_slabs = 0;
-            plan_split<T>(gs, D % Elem<T>::CE == 0, ctx().prop.multiProcessorCount);
-            total_bytes += gs.bt_bytes + gs.part_bytes;
-            sets.push_back(gs);
+    auto build_sets = [&](int hl, int wl) {
+        sets.clear();
+        total_bytes = 0;
+        for (int a = 0; a < sH; ++a) {
+            if (a >= H) continue;
+            int ra = (a + pH) % sH;
+            int Th = ra < fH ? (fH - 1 - ra) / sH + 1 : 0;
+            int xmax = ra + (Th - 1) * sH;
+            int offh = Th > 0 ? (a + pH - xmax) / sH : 0;   // exact: (a+pH-xmax) is a multiple of sH
+            int Hg = (std::min(H, std::max(hl, a + 1)) - a + sH - 1) / sH;      // class rows i = a + sH i' below hl (at least one)
+            for (int b = 0; b < sW; ++b) {
+                if (b >= W) continue;
+                int rb = (b + pW) % sW;
+                int Tw = rb < fW ? (fW - 1 - rb) / sW + 1 : 0;
+                int ymax = rb + (Tw - 1) * sW;
+                int offw = Tw > 0 ? (b + pW - ymax) / sW : 0;
+                int Wg = (std::min(W, std::max(wl, b + 1)) - b + sW - 1) / sW;
+                GatherSetup gs;
+                GatherParams& g = gs.gp;
+                g.src = dy; g.bias = nullptr; g.out = dx;
+                g.S = S; g.Hs = Ho; g.Ws = Wo; g.Cs = D;
+                g.Hg = Hg; g.Wg = Wg; g.M = S * Hg * Wg; g.N = C;
+                g.K = Th * Tw * D;
+                g.Kpad = (int)round_up(g.K, BK);
+                g.Tw = Tw; g.sh = 1; g.sw = 1; g.rh0 = offh; g.rw0 = offw;
+                g.Hof = H; g.Wof = W; g.oh0 = a; g.ow0 = b; g.ohs = sH; g.ows = sW;
+                g.dense_out = (nclass == 1);
+                set_out_divs(g);
+                PackParams& pk = gs.pp;
+                pk.w = w; pk.fW = fW; pk.C = C; pk.D = D; pk.Tw = Tw > 0 ? Tw : 1; pk.Ck = D; pk.w_elems = (int64_t)fH * fW * C * D;
+                pk.xa = xmax; pk.xs = -sH; pk.ya = ymax; pk.ys = -sW; pk.transposed = 1;
+                pk.N = C; pk.K = g.K; pk.Npad = (int)round_up(C, 64); pk.Kpad = g.Kpad;
+                gs.bt_bytes = round_up((int64_t)pk.Npad * pk.Kpad * sizeof(T), 256);
+                g.split_slabs = 0;
+                plan_split<T>(gs, D % Elem<T>::CE == 0, ctx().prop.multiProcessorCount);
+                total_bytes += gs.bt_bytes + gs.part_bytes;
+                sets.push_back(gs);
+            }
+        }
+    };
+    // bf16, 2 or 4 classes with the same pixel grid, each of them a problem for gather_halo_bf16 with the same
+    // tiles: one launch for all classes (tuning: gather_merge = 0 keeps one launch per class).  The full grids
+    // are used, so that they are equal; the classes then write the zeros of the unreachable rows themselves.
+    if constexpr (sizeof(T) == 2) {
+        if (nclass > 1 && nclass <= kMaxClasses && H % sH == 0 && W % sW == 0 && tuning().gather_merge != 0) {
+            build_sets(H, W);
+            void* ws = nullptr;
+            bool ok = (int)sets.size() == nclass;
+            if (ok) {
+                rc = workspace(total_bytes > 0 ? total_bytes : 256, &ws);
+                if (rc) return rc;
+            }
+            const bool vec = D % Elem<T>::CE == 0;
+            const int cus = ctx().prop.multiProcessorCount;
+            GatherClasses gc;
+            gc.ncls = nclass;
+            int mtiles = 0, stages = 4;
+            std::vector<int> pack(sets.size(), 0);
+            int64_t off = 0;
+            for (size_t i = 0; ok && i < sets.size(); ++i) {
+                GatherSetup& gs = sets[i];
+                ok = gs.nsplit == 1 && gs.gp.M > 0 && gs.gp.N > 0 && gs.gp.K > 0;
+                if (!ok) break;
+                fill_gather<T>(gs, (char*)ws, off);
+                off += gs.bt_bytes + gs.part_bytes;
+                GatherParams probe = gs.gp;
+                int mt_res = 0;
+                const bool dma_res = vec && probe.src_bytes != 0 && gs.pp.w_elems * 2 < ((int64_t)1 << 31) && gs.pp.N % 2 == 0;
+                if (plan_halo_res(probe, dma_res, cus, &mt_res)) { ok = false; break; }   // that class has a faster kernel of its own
+                pack[i] = choose_b_operand<T>(gs, vec, 1);
+                const bool dma = vec && gs.gp.src_bytes != 0 && gs.gp.bt_bytes != 0;
+                int mt = 0, st = 0;
+                ok = plan_halo(gs.gp, dma, &mt, &st, 1) && (i == 0 || (mt == mtiles && gs.gp.halo_tiles == sets[0].gp.halo_tiles));
+                mtiles = mt;
+                stages = std::min(stages, st);
+                gc.cls[i] = gs.gp;
+            }
+            if (ok) {
+                for (size_t i = 0; i < sets.size(); ++i)
+                    if (pack[i] > 0) {
+                        hipLaunchKernelGGL(pack_filter<T>, dim3(cdiv(pack[i], 256)), dim3(256), 0, ctx().stream, sets[i].pp);
+                        AETH_LAUNCH_CHECK();
+                    }
+                // more than 64 channels out, several channel blocks in and at least two tiles per CU: the persistent form
+                // (tuning: gather_stream = 1 wherever its conditions hold, 0 never)
+                if (C > 64 && tuning().gather_stream > 0) {
+                    GatherClasses sc;
+                    int64_t smt = 0, longest = 0;
+                    if (plan_class_pairs(sets, sc, kStreamBM, kStreamSlots, &smt, &longest)) {
+                        const int64_t units = smt * cdiv(C, kStreamBN) * (nclass / 2);
+                        const dim3 sgrid((unsigned)std::min<int64_t>(units, cus));
+                        hipLaunchKernelGGL(gather_halo_stream_bf16<2>, sgrid, dim3(kStreamThreads), 0, ctx().stream, sc, (int)units);
+                        AETH_LAUNCH_CHECK();
+                        return AETH_OK;
+                    }
+                }
+                // two classes per workgroup from one halo, where all classes read the filter in place (tuning: gather_pairs = 0 never)
+                if (tuning().gather_pairs != 0) {
+                    bool direct = true;
+                    for (const GatherSetup& gs : sets) direct = direct && gs.gp.bt_direct != 0;
+                    GatherClasses pc;
+                    int64_t pmt = 0, longest = 0;
+                    if (direct && plan_class_pairs(sets, pc, kHaloBM, kHaloSlotsMax, &pmt, &longest)) {
+                        const dim3 pgrid((unsigned)(pmt * (nclass / 2) * cdiv(C, 64)));
+                        if (longest <= halo_slots(4)) hipLaunchKernelGGL(gather_halo_pairs_bf16<4>, pgrid, dim3(kThreads), 0, ctx().stream, pc);
+                        else hipLaunchKernelGGL(gather_halo_pairs_bf16<3>, pgrid, dim3(kThreads), 0, ctx().stream, pc);
+                        AETH_LAUNCH_CHECK();
+                        return AETH_OK;
+                    }
+                }
+                const dim3 grid((unsigned)((int64_t)mtiles * nclass * cdiv(C, 64)));
+                // no bias and a dx that the descriptor covers: tiles go out as whole lines (0.197 against 0.213 ms on the stride-2 layer)
+                const bool lines = sets[0].gp.bias == nullptr && sets[0].gp.out_bytes != 0;
+                if (stages == 4 && lines) hipLaunchKernelGGL((gather_halo_classes_bf16<4, true>), grid, dim3(kThreads), 0, ctx().stream, gc);
+                else if (stages == 4) hipLaunchKernelGGL((gather_halo_classes_bf16<4, false>), grid, dim3(kThreads), 0, ctx().stream, gc);
+                else if (lines) hipLaunchKernelGGL((gather_halo_classes_bf16<3, true>), grid, dim3(kThreads), 0, ctx().stream, gc);
+                else hipLaunchKernelGGL((gather_halo_classes_bf16<3, false>), grid, dim3(kThreads), 0, ctx().stream, gc);
+                AETH_LAUNCH_CHECK();
+                return AETH_OK;
+            }
         }
     }
+    build_sets(h_lim, w_lim);
     void* ws;
     rc = workspace(total_bytes > 0 ? total_bytes : 256, &ws);
     if (rc) return rc;

@@ -302,6 +302,46 @@ def test_bf16_dgrad_reading_the_filter_in_place(case, tune):
     assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
 
 
+# bf16 dgrad of a strided layer whose stride classes all have the same pixel grid (H and W multiples of the
+# strides) and all go to the halo kernel: one launch for the 2 or 4 classes, whose workgroups for one tile of
+# pixels run next to each other.  The gather_merge switch at 0 launches class by class (clipped grids, a
+# zeroed strip): same bits either way.
+MERGE_CASES = [
+    (3, 28, 28, 128, 256, 3, 3, 2, 2, "valid"),   # the stride-2 layer: classes of 4, 2, 2 and 1 taps, row and column 27 of dx unreachable
+    (2, 16, 16, 64, 64, 3, 3, 2, 2, "same"),      # one channel block; 'same' padding shifts the classes
+    (2, 20, 12, 40, 128, 4, 4, 2, 2, "valid"),    # 4 taps in every class, 40 channels of dx
+    (2, 16, 16, 36, 64, 2, 2, 2, 2, "valid"),     # one tap per class; 36 channels: the filter is packed
+    (2, 16, 16, 64, 128, 3, 3, 2, 1, "same"),     # two classes (rows only)
+    (2, 12, 18, 64, 64, 5, 5, 2, 2, "same"),      # 9, 6, 6 and 4 taps
+    (5, 8, 8, 128, 192, 3, 3, 2, 2, "same"),      # 16 pixels per class and image: tiles run over images
+    (1, 18, 12, 48, 64, 3, 2, 1, 2, "valid"),     # two classes (columns only), 3 x 2 filter
+    (40, 28, 28, 128, 128, 3, 3, 2, 2, "valid"),  # 31 tiles of 256 pixels per class: several units per workgroup when persistent
+    (9, 16, 16, 200, 64, 3, 3, 2, 2, "same"),     # 200 channels of dx: two n tiles of 128, the second ragged
+    (4, 16, 16, 96, 128, 3, 3, 2, 1, "same"),     # two classes and 96 channels of dx: one pair when persistent
+    (3, 12, 18, 72, 64, 5, 5, 2, 2, "same"),      # 9, 6, 6 and 4 taps on 72 channels of dx: windows of 3 x 3 in the common halo
+    (2, 24, 24, 128, 128, 4, 4, 2, 2, "valid"),   # 4 taps in every class
+]
+
+
+@pytest.mark.parametrize("case", MERGE_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_bf16_dgrad_with_all_stride_classes_in_one_launch(case, tune):
+    from tests import abi
+    x, w, b, dy = _case(case, 29)
+    stride, pad = (case[7], case[8]), case[9]
+    tune(gather_split=0, gather_pairs=0)
+    dyr, wr = O.round_to_bf16(dy), O.round_to_bf16(w)
+    dx = abi.dgrad_bf16(dy, w, x.shape, stride, pad)
+    abi.close(dx, O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
+    tune(gather_merge=0)
+    assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
+    # two classes per workgroup from one halo (what the library takes where all classes read the filter in place)
+    tune(gather_merge=-1, gather_pairs=-1)
+    assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
+    # the persistent form of the same (one workgroup per CU walks tiles and pairs; more than 64 channels of dx)
+    tune(gather_stream=1)
+    assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
+
+
 # bf16 wgrad onto more than 64 output channels: wave tiles of 64 k x 128 n (workgroup 128 k x 256 n) or
 # 64 k x 64 n (128 x 128), where the library takes them from the channel padding they cost; the
 # wgrad_wide switch forces them (1: the narrower form wherever D > 64) or turns them off (0).
