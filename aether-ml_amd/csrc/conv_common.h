@@ -97,7 +97,7 @@ struct GatherParams {
     // gather_halo_bf16: columns and rows of the padded source image, 256-row tiles per image (0: tiles
     // run over image boundaries)
     int halo_wp, halo_hp, halo_tiles;
-    // gather_halo_stream_bf16: the classes of a dgrad share one padded source tensor of halo_th x halo_tw windows per
+    // gather_halo_pairs_bf16: the classes of a dgrad share one padded source tensor of halo_th x halo_tw windows per
     // pixel; this class's tap (th, tw) is the window (th + tap_dh, tw + tap_dw)
     int halo_th, halo_tw, tap_dh, tap_dw;
     FastDiv div_hw, div_w, div_c, div_tw, div_halo_wp, div_halo_hp, div_halo_tiles;
@@ -242,16 +242,13 @@ __device__ __forceinline__ void store_tile(const GatherParams& p, float* out, co
 // instruction issue.  Every lane works out the row of one pixel of the block, the stores fetch the
 // rows of their two pixels from those lanes.  Needs p.out_bytes != 0 (the descriptor drops rows
 // past m_end and channels past N).
-// Blocks b0 <= 32-row block i, 32-column block j (numbered i TN + j) < b1 are stored, so that a caller can spread a
-// tile's stores over the steps of other work.
 template <int TM, int TN>
 __device__ __forceinline__ void store_tile_lines(const GatherParams& p, float* out, const f16v (&acc)[TM][TN], int mw0,
-                                                 int nw0, int l32, int lh, int m_end, int b0 = 0, int b1 = TM * TN) {
+                                                 int nw0, int l32, int lh, int m_end) {
     const __amdgpu_buffer_rsrc_t rsrc =
         __builtin_amdgcn_make_buffer_rsrc(out, 0, (int)p.out_bytes, 0x00020000);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-        if (b1 <= i * TN || b0 >= (i + 1) * TN) continue;            // wave-uniform
         const int m = mw0 + 32 * i + l32;
         const bool mok = m < m_end;
         unsigned row = (unsigned)m;
@@ -263,18 +260,50 @@ __device__ __forceinline__ void store_tile_lines(const GatherParams& p, float* o
         }
         const int rowbytes = (int)((row * (unsigned)p.N * 4u) | ((unsigned)!mok << 31));   // < 2^31: checked by the host
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            if (i * TN + j < b0 || i * TN + j >= b1) continue;
-            const int n = nw0 + 32 * j + l32;
-            const unsigned col = (unsigned)n * 4u, colbad = (unsigned)!(n < p.N) << 31;
+        for (int v = 0; v < 16; ++v) {
+            const int pix = 8 * (v >> 2) + (v & 3);
+            const unsigned base = (unsigned)__builtin_amdgcn_ds_bpermute(4 * pix + 16 * lh, rowbytes);
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int pix = 8 * (v >> 2) + (v & 3);
-                const int lo = __builtin_amdgcn_readlane(rowbytes, pix), hi = __builtin_amdgcn_readlane(rowbytes, pix + 4);
-                const unsigned off = ((unsigned)(lh ? hi : lo) + col) | colbad;   // bit 31 from either part: outside the descriptor
+            for (int j = 0; j < TN; ++j) {
+                const int n = nw0 + 32 * j + l32;
+                const unsigned off = (base + (unsigned)n * 4u) | ((unsigned)!(n < p.N) << 31);   // bit 31 from either part: outside the descriptor
                 const float value = acc[i][j][v];        // (a bit cast of the vector element itself reads element 0)
                 __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(value), rsrc, (int)off, 0, 0);
             }
+        }
+    }
+}
+
+// The same for a wave tile of two 32-column blocks whose columns are interleaved: column l of block j is channel
+// nw0 + 2 l + j (the kernel fetches the filter rows in that order), so a lane holds two neighbouring channels of a pixel
+// and 32 lanes write 256 contiguous bytes with 8-byte stores: half the store instructions of store_tile_lines.
+template <int TM>
+__device__ __forceinline__ void store_tile_lines2(const GatherParams& p, float* out, const f16v (&acc)[TM][2], int mw0,
+                                                  int nw0, int l32, int lh, int m_end) {
+    typedef unsigned u2 __attribute__((ext_vector_type(2)));
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(out, 0, (int)p.out_bytes, 0x00020000);
+    const int n = nw0 + 2 * l32;
+    const unsigned col = ((unsigned)n * 4u) | ((unsigned)!(n < p.N) << 31);      // N is even: both channels or neither
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int m = mw0 + 32 * i + l32;
+        const bool mok = m < m_end;
+        unsigned row = (unsigned)m;
+        if (!p.dense_out) {
+            unsigned s, rem, ii, jj;
+            p.div_hw.divmod(mok ? (unsigned)m : 0u, s, rem);
+            p.div_w.divmod(rem, ii, jj);
+            row = ((unsigned)s * p.Hof + p.oh0 + ii * p.ohs) * p.Wof + p.ow0 + jj * p.ows;
+        }
+        const int rowbytes = (int)((row * (unsigned)p.N * 4u) | ((unsigned)!mok << 31));   // < 2^31: checked by the host
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int pix = 8 * (v >> 2) + (v & 3);
+            const unsigned base = (unsigned)__builtin_amdgcn_ds_bpermute(4 * pix + 16 * lh, rowbytes);
+            const float a = acc[i][0][v], b = acc[i][1][v];    // (a bit cast of the vector element itself reads element 0)
+            const u2 value = {__float_as_uint(a), __float_as_uint(b)};
+            __builtin_amdgcn_raw_buffer_store_b64(value, rsrc, (int)((base + (col & 0x7fffffffu)) | (col & 0x80000000u)), 0, 0);
         }
     }
 }

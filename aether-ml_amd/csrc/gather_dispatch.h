@@ -638,19 +638,6 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
                         hipLaunchKernelGGL(pack_filter<T>, dim3(cdiv(pack[i], 256)), dim3(256), 0, ctx().stream, sets[i].pp);
                         AETH_LAUNCH_CHECK();
                     }
-                // more than 64 channels out, several channel blocks in and at least two tiles per CU: the persistent form
-                // (tuning: gather_stream = 1 wherever its conditions hold, 0 never)
-                if (C > 64 && tuning().gather_stream > 0) {
-                    GatherClasses sc;
-                    int64_t smt = 0, longest = 0;
-                    if (plan_class_pairs(sets, sc, kStreamBM, kStreamSlots, &smt, &longest)) {
-                        const int64_t units = smt * cdiv(C, kStreamBN) * (nclass / 2);
-                        const dim3 sgrid((unsigned)std::min<int64_t>(units, cus));
-                        hipLaunchKernelGGL(gather_halo_stream_bf16<2>, sgrid, dim3(kStreamThreads), 0, ctx().stream, sc, (int)units);
-                        AETH_LAUNCH_CHECK();
-                        return AETH_OK;
-                    }
-                }
                 // two classes per workgroup from one halo, where all classes read the filter in place (tuning: gather_pairs = 0 never)
                 if (tuning().gather_pairs != 0) {
                     bool direct = true;

@@ -903,7 +903,10 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_pairs_bf16(con
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const int k4 = k4e ^ (((wave * 2 + i) & 1) ? 4 : 0);
-        b_off[i] = (unsigned)(((n0 + (wave * 2 + i) * 8 + (lane >> 3)) * p0.bt_ld + 8 * k4) * 2);
+        // slab row r holds channel n0 + 2 (r % 32) + r / 32: a lane of the multiplying waves then owns two neighbouring
+        // channels, one in each of its 32-column blocks (store_tile_lines2)
+        const int r = (wave * 2 + i) * 8 + (lane >> 3);
+        b_off[i] = (unsigned)(((n0 + 2 * (r & 31) + (r >> 5)) * p0.bt_ld + 8 * k4) * 2);
     }
     const u32x4 rsrc_a = raw_rsrc(p0.src, p0.src_bytes);
     const u32x4 rsrc_b = raw_rsrc(p0.bt, p0.bt_bytes);
@@ -1003,407 +1006,8 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_pairs_bf16(con
         }
     }
     (void)nsteps;
-    store_tile_lines<TM, TN>(pa, pa.out, acc[0], m0 + wm0, n0, l32, lh, m_end);
-    store_tile_lines<TM, TN>(pb, pb.out, acc[1], m0 + wm0, n0, l32, lh, m_end);
-}
-
-// ------------------------------------------------------------------------------
-// gather_halo_stream_bf16: the halo gather as one persistent workgroup per CU for the stride classes of a
-// dgrad with several channel blocks and more than 64 output channels (28x28x128 -> 256, stride 2: four
-// classes of 4, 2, 2 and 1 taps over 256 source channels).  gather_halo_bf16 waits for the halo of every
-// channel block with nothing else to do in that workgroup, and with 1 to 4 taps per block the wait is
-// longer than the MFMAs: 213 us for the four classes of that layer, 27 % of them in the matrix pipe,
-// 2.4 TB/s, whichever way the classes are launched.  Here
-//   * the classes share one halo: their taps are windows of one padded source tensor (a class's tap
-//     (th, tw) is the window at (th + tap_dh, tw + tap_dw)), and a workgroup multiplies CPP = 2 classes
-//     of a tile from the same halo, 4 or 5 taps per channel block instead of 1 to 4;
-//   * waves 0..5 multiply a tile of 192 pixels x 128 channels (64 x 64 per wave and class) and never touch
-//     memory except to store a finished tile;
-//   * wave 6 fetches halos, two channel blocks ahead (three buffers);
-//   * wave 7 fetches filter slabs (64 k x 128 n = 16 KB) into a ring of four, three steps ahead;
-//   * one barrier per step (one tap of one channel block): the loading waves wait for their own loads
-//     before it, and after it the buffer of the step before belongs to them again.
-// A workgroup walks a contiguous run of units (m tile, n tile, pair of classes), pairs innermost: the
-// pairs of one tile read the same span of the source, which the L2 then still holds.
-// ------------------------------------------------------------------------------
-constexpr int kStreamBM = 192, kStreamBN = 128;
-constexpr int kStreamSlots = 248;        // 3 x 248 x 128 B of halo + 4 x 16 KB of filter slabs + the slot table = 158 KB
-constexpr int kStreamThreads = 512;
-
-template <int CPP>
-static __global__ __launch_bounds__(kStreamThreads, 1) void gather_halo_stream_bf16(const GatherClasses q, const int units) {
-    constexpr int BM = kStreamBM, BN = kStreamBN, TM = 2, TN = 2, KC = 8, BK = 64;
-    constexpr int NL = kStreamSlots / 8;                 // wave-level loads per halo (8 slots each)
-    constexpr int NB = BN / 8;                           // wave-level loads per filter slab (8 rows each)
-    static_assert(NL == 31 && NB == 16, "the loading waves' wait counts");
-    __shared__ f4 halo[3][kStreamSlots * KC];
-    __shared__ f4 ring[4][BN * KC];
-    __shared__ int tab[kStreamSlots];                    // the halo wave's slot table
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int l32 = lane & 31;
-    const int lh = lane >> 5;
-    const int G = (int)gridDim.x;
-    const int lid = xcd_contiguous_id((int)blockIdx.x, G);
-    const int u0 = (int)(((long long)lid * units) / G);
-    const int u1 = (int)(((long long)(lid + 1) * units) / G);
-    const int npass = q.ncls / CPP;
-    const GatherParams& p0 = q.cls[0];                   // what all classes have in common: source, pixel grid, halo geometry, N
-    const int ntile = (p0.N + BN - 1) / BN;
-    const int ncb = p0.Cs / BK;
-    const int Wp = p0.halo_wp, Hp = p0.halo_hp;
-
-    // unit -> pair of classes, n tile, m tile
-    auto decode = [&](int qi, int& pass, int& nt, int& mt) __attribute__((always_inline)) {
-        const int r = qi / npass;
-        pass = qi - r * npass;
-        mt = r / ntile;
-        nt = r - mt * ntile;
-    };
-    // slot of window (0,0) of output pixel m in the padded source tensor
-    auto slot0 = [&](int m) __attribute__((always_inline)) {
-        unsigned s_, rem, ii, jj;
-        p0.div_hw.divmod((unsigned)m, s_, rem);
-        p0.div_w.divmod(rem, ii, jj);
-        return ((int)s_ * Hp + (int)ii) * Wp + (int)jj;
-    };
-    auto steps_of = [&](int pass) __attribute__((always_inline)) {
-        int t = 0;
-#pragma unroll
-        for (int ci = 0; ci < CPP; ++ci) t += q.cls[pass * CPP + ci].Th * q.cls[pass * CPP + ci].Tw;
-        return t;
-    };
-
-    if (wave == 6) {
-        // ---- halos ----
-        const u32x4 rsrc_a = raw_rsrc(p0.src, p0.src_bytes);
-        unsigned offs[NL];
-        // byte offset of every slot's channel 0 (bit 31: padding or past the span), one or more slots per
-        // lane, through the table to the lanes that fetch them (lane / 8 picks the slot of a load, lane % 8 the chunk)
-        auto addresses = [&](int mt) __attribute__((always_inline)) {
-            const int m0 = mt * BM;
-            const int lfirst = slot0(m0);
-            const int span = slot0(min(m0 + BM, p0.M) - 1) + (p0.halo_th - 1) * Wp + p0.halo_tw - lfirst;
-            for (int sl = lane; sl < kStreamSlots; sl += 64) {
-                unsigned rg, cc, s_, rr;
-                p0.div_halo_wp.divmod((unsigned)(lfirst + sl), rg, cc);
-                p0.div_halo_hp.divmod(rg, s_, rr);
-                const int srow = (int)rr + p0.rh0, scol = (int)cc + p0.rw0;
-                const bool ok = sl < span && (unsigned)srow < (unsigned)p0.Hs && (unsigned)scol < (unsigned)p0.Ws && (int)s_ < p0.S;
-                const unsigned off = (unsigned)((((int)s_ * p0.Hs + srow) * p0.Ws + scol) * p0.Cs) * 2u;
-                tab[sl] = (int)(ok ? off : 0x80000000u);
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                      // the table is written (this wave only)
-#pragma unroll
-            for (int i = 0; i < NL; ++i) {
-                const int sl = i * 8 + (lane >> 3);
-                offs[i] = (unsigned)tab[sl] + (unsigned)((((lane & 7) ^ (sl >> 1)) & 7) * 16);
-            }
-        };
-        int gq = u0, gcb = 0, buf = 0, gmt = -1;         // the halo to fetch next: unit, channel block, buffer; the tile `offs` is for
-        auto fetch_next = [&]() __attribute__((always_inline)) {
-            const unsigned base = lds_address(&halo[buf][0]);
-            const bool live = gq < u1;                   // past the last unit: no memory access, the same count of loads
-            const unsigned add = (unsigned)(gcb * BK * 2);
-#pragma unroll
-            for (int i = 0; i < NL; ++i) lds_direct_load16(rsrc_a, base + (unsigned)i * 1024u, live ? offs[i] + add : 0x80000000u);
-            buf = buf == 2 ? 0 : buf + 1;
-            if (gq < u1 && ++gcb == ncb) {
-                gcb = 0;
-                if (++gq < u1) {
-                    int pass, nt, mt;
-                    decode(gq, pass, nt, mt);
-                    if (mt != gmt) { addresses(mt); gmt = mt; }      // worked out while the loads are in flight
-                }
-            }
-        };
-#pragma unroll
-        for (int i = 0; i < NL; ++i) offs[i] = 0x80000000u;
-        if (u0 < u1) {
-            int pass, nt, mt;
-            decode(u0, pass, nt, mt);
-            addresses(mt);
-            gmt = mt;
-        }
-        fetch_next();
-        fetch_next();
-        for (int qi = u0; qi < u1; ++qi) {
-            int pass, nt, mt;
-            decode(qi, pass, nt, mt);
-            const int T = steps_of(pass);
-            for (int cb = 0; cb < ncb; ++cb)
-                for (int t = 0; t < T; ++t) {
-                    if (t == 0) asm volatile("s_waitcnt vmcnt(31)" ::: "memory");   // all but the younger halo (NL loads)
-                    asm volatile("s_barrier" ::: "memory");
-                    if (t == 0) fetch_next();            // two blocks ahead, into the buffer of the block before this one
-                }
-        }
-        return;
-    }
-
-    if (wave == 7) {
-        // ---- filter slabs, in the order of the steps ----
-        int pq = u0, pcb = 0, pci = 0, pth = 0, ptw = 0; // the slab to fetch next: unit, channel block, class of the pair, tap
-        int p_pass = 0, p_nt = 0;
-        int p_th_n = 1, p_tw_n = 1, p_direct = 0;
-        int bd_xa = 0, bd_xs = 0, bd_ya = 0, bd_ys = 0, bd_fw = 0, bd_tap = 0;
-        u32x4 rsrc_b = raw_rsrc(nullptr, 0);
-        unsigned b_off[NB];
-        auto enter_class = [&]() __attribute__((always_inline)) {
-            const GatherParams& p = q.cls[p_pass * CPP + pci];
-            rsrc_b = raw_rsrc(p.bt, p.bt_bytes);
-            p_th_n = p.Th; p_tw_n = p.Tw; p_direct = p.bt_direct;
-            bd_xa = p.bd_xa; bd_xs = p.bd_xs; bd_ya = p.bd_ya; bd_ys = p.bd_ys; bd_fw = p.bd_fw; bd_tap = p.bd_tap_elems;
-            // rows of 8 chunks, chunk c of row r at c ^ ((r >> 1) & 7), as in gather_gemm_dma
-            const int k4e = (lane & 7) ^ (lane >> 4);
-#pragma unroll
-            for (int i = 0; i < NB; ++i) {
-                const int k4 = k4e ^ ((i & 1) ? 4 : 0);
-                b_off[i] = (unsigned)(((p_nt * BN + i * 8 + (lane >> 3)) * p.bt_ld + 8 * k4) * 2);
-            }
-        };
-        auto fetch_next = [&](int slot) __attribute__((always_inline)) {
-            const bool live = pq < u1;                   // past the last step: no memory access, the same count of loads
-            const int k_elems = p_direct ? ((bd_xa + bd_xs * pth) * bd_fw + bd_ya + bd_ys * ptw) * bd_tap + pcb * BK
-                                         : (pth * p_tw_n + ptw) * p0.Cs + pcb * BK;
-            const unsigned k0_bytes = (unsigned)k_elems * 2u;
-            const unsigned base = lds_address(&ring[slot][0]);
-#pragma unroll
-            for (int i = 0; i < NB; ++i) lds_direct_load16(rsrc_b, base + (unsigned)i * 1024u, live ? b_off[i] + k0_bytes : 0x80000000u);
-            if (pq < u1) {
-                if (++ptw == p_tw_n) { ptw = 0; ++pth; }
-                if (pth == p_th_n) {
-                    pth = 0;
-                    bool again = true;                   // the next class of the pair, channel block or unit
-                    if (++pci == CPP) {
-                        pci = 0;
-                        if (++pcb == ncb) {
-                            pcb = 0;
-                            if (++pq < u1) {
-                                int mt;
-                                decode(pq, p_pass, p_nt, mt);
-                            } else {
-                                again = false;
-                            }
-                        }
-                    }
-                    if (again) enter_class();
-                }
-            }
-        };
-#pragma unroll
-        for (int i = 0; i < NB; ++i) b_off[i] = 0;
-        if (u0 < u1) {
-            int mt;
-            decode(u0, p_pass, p_nt, mt);
-            enter_class();
-        }
-        fetch_next(0);
-        fetch_next(1);
-        fetch_next(2);
-        int u = 0;
-        for (int qi = u0; qi < u1; ++qi) {
-            int pass, nt, mt;
-            decode(qi, pass, nt, mt);
-            const int steps = steps_of(pass) * ncb;
-            for (int t = 0; t < steps; ++t, ++u) {
-                asm volatile("s_waitcnt vmcnt(32)" ::: "memory");          // all but the two youngest slabs (NB loads each)
-                asm volatile("s_barrier" ::: "memory");
-                fetch_next((u + 3) & 3);                 // the buffer of step u - 1
-            }
-        }
-        return;
-    }
-
-    // ---- the multiplying waves ----
-    // The pixels are the MFMAs' first operand: acc[ci][i][j][v] belongs to pixel 32 i + 8 (v/4) + 4 lh + v%4 and channel
-    // 32 j + l32, and a tile goes out in 4-byte stores of whole 128-byte lines: this kernel waits for its stores, and as
-    // 16-byte pieces of 32 lines per instruction they took 75 us of 206.
-    // The steps run as one flat loop, each in four k groups with two operand sets taking turns: the LDS reads of a
-    // group are issued before the MFMAs of the group before it, across the barrier between two steps as well.  With
-    // all reads of a step issued behind its barrier and all its MFMAs behind the reads, the LDS and the matrix pipe took
-    // turns (1040 + 1024 clocks per step).
-    const int wm0 = (wave % 3) * 64, wn0 = (wave / 3) * 64;
-    const int sw7 = (l32 >> 1) & 7;
-    f16v acc[CPP][TM][TN];
-    auto start_from_bias = [&](const GatherParams& p, int n0, f16v (&a)[TM][TN]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int n = n0 + 32 * j + l32;
-            const float bj = (p.bias != nullptr && n < p.N) ? p.bias[n] : 0.0f;
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) a[i][j][v] = bj;
-        }
-    };
-    // A cursor runs one step ahead of the multiplying loops below (unit, channel block, class of the pair, tap) and says
-    // where the reads of that step go: halo buffer, tap shift, the unit's pixel slots.
-    struct Cursor {
-        int qi, cb, ci, th, tw;
-        int pass, m0, n0;
-        int hb;                                          // halo buffer of the channel block
-        int Th, Tw, shift0;                              // of the class
-        int cTh[CPP], cTw[CPP], cshift0[CPP];            // of the unit's classes (kept here: a scalar load from the kernel
-                                                         // arguments waits for every LDS read in flight as well)
-        int pslot[TM];                                   // slot of window (0,0) for this lane's pixels (rows past the end: slot 0, never stored)
-    };
-    auto enter_class = [&](Cursor& c) __attribute__((always_inline)) {
-#pragma unroll
-        for (int cc = 0; cc < CPP; ++cc)
-            if (cc == c.ci) { c.Th = c.cTh[cc]; c.Tw = c.cTw[cc]; c.shift0 = c.cshift0[cc]; }
-    };
-    auto enter_unit = [&](Cursor& c) __attribute__((always_inline)) {
-        int nt, mt;
-        decode(c.qi, c.pass, nt, mt);
-#pragma unroll
-        for (int cc = 0; cc < CPP; ++cc) {
-            const GatherParams& p = q.cls[c.pass * CPP + cc];
-            c.cTh[cc] = p.Th; c.cTw[cc] = p.Tw;
-            c.cshift0[cc] = p.tap_dh * Wp + p.tap_dw;
-        }
-        c.m0 = mt * BM;
-        c.n0 = nt * BN + wn0;
-        const int lfirst = slot0(c.m0);
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int m = c.m0 + wm0 + 32 * i + l32;
-            c.pslot[i] = m < p0.M ? slot0(m) - lfirst : 0;
-        }
-        enter_class(c);
-    };
-    // to the next step; false past the last one
-    auto advance = [&](Cursor& c) __attribute__((always_inline)) {
-        if (++c.tw < c.Tw) return true;
-        c.tw = 0;
-        if (++c.th < c.Th) return true;
-        c.th = 0;
-        if (++c.ci < CPP) { enter_class(c); return true; }
-        c.ci = 0;
-        c.hb = c.hb == 2 ? 0 : c.hb + 1;
-        if (++c.cb < ncb) { enter_class(c); return true; }
-        c.cb = 0;
-        if (++c.qi < u1) { enter_unit(c); return true; }
-        return false;
-    };
-    // what the reads of one step need: the f4 index of k group 0 of each pixel in the halo buffers, and of the slab's rows
-    struct Reads {
-        int a[TM];
-        int b;
-    };
-    auto describe = [&](const Cursor& c, int step) __attribute__((always_inline)) {
-        Reads r;
-        const int shift = c.shift0 + c.th * Wp + c.tw;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int sl = c.pslot[i] + shift;
-            r.a[i] = c.hb * (kStreamSlots * KC) + sl * 8 + ((lh ^ (sl >> 1)) & 7);
-        }
-        r.b = (step & 3) * (BN * KC) + (wn0 + l32) * KC;
-        return r;
-    };
-    const f4* const halo0 = &halo[0][0];
-    const f4* const ring0 = &ring[0][0];
-    // the operands of k group kg (16 of the 64 k)
-    auto read_kg = [&](const Reads& r, int kg, f4 (&fa)[TM], f4 (&fb)[TN]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) fa[i] = halo0[r.a[i] ^ (kg << 1)];
-#pragma unroll
-        for (int j = 0; j < TN; ++j) fb[j] = ring0[r.b + 32 * j * KC + ((2 * kg + lh) ^ sw7)];
-    };
-    auto multiply = [&](f16v (&a)[TM][TN], const f4 (&fa)[TM], const f4 (&fb)[TN]) __attribute__((always_inline)) {
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) mma_chunk<uint16_t>(fa[i], fb[j], a[i][j]);
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    // Both classes of the pair at once: where a pixel's row of dx starts differs between the classes by a constant
-    // ((oh0 Wof + ow0) N), which rides in the stores' scalar offset; the rest is worked out once per 32-pixel
-    // block, every lane for one pixel, and fetched by the lanes that store that pixel.  No vector instruction per store
-    // but the store.
-    auto store_unit = [&](int pass, int m0, int n0) __attribute__((always_inline)) {
-        const GatherParams& pa = q.cls[pass * CPP];
-        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(pa.out, 0, (int)pa.out_bytes, 0x00020000);
-        const bool full_n = n0 + 32 * TN <= pa.N;        // wave-uniform
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int m = m0 + wm0 + 32 * i + l32;
-            const bool mok = m < p0.M;
-            unsigned s_, rem, ii, jj;
-            pa.div_hw.divmod(mok ? (unsigned)m : 0u, s_, rem);
-            pa.div_w.divmod(rem, ii, jj);
-            const unsigned row = pa.dense_out ? (unsigned)m : (s_ * pa.Hof + ii * pa.ohs) * pa.Wof + jj * pa.ows;
-            const int rowbytes = (int)((row * (unsigned)pa.N * 4u) | ((unsigned)!mok << 31));
-            int voff[16];
-#pragma unroll
-            for (int v = 0; v < 16; ++v)
-                voff[v] = __builtin_amdgcn_ds_bpermute(4 * (8 * (v >> 2) + (v & 3)) + 16 * lh, rowbytes) + (n0 + l32) * 4;
-#pragma unroll
-            for (int ci = 0; ci < CPP; ++ci) {
-                const GatherParams& pc = q.cls[pass * CPP + ci];
-                const int soff = pc.dense_out ? 0 : (pc.oh0 * pc.Wof + pc.ow0) * pc.N * 4;
-#pragma unroll
-                for (int v = 0; v < 16; ++v)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j) {
-                        const float value = acc[ci][i][j][v];    // (a bit cast of the vector element itself reads element 0)
-                        const unsigned bad = full_n ? 0u : (unsigned)!(n0 + 32 * j + l32 < pa.N) << 31;
-                        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(value), rsrc, (int)((unsigned)(voff[v] + 128 * j) | bad), soff, 0);
-                    }
-            }
-        }
-    };
-    auto start_unit = [&](int pass, int n0) __attribute__((always_inline)) {
-#pragma unroll
-        for (int ci = 0; ci < CPP; ++ci) start_from_bias(q.cls[pass * CPP + ci], n0, acc[ci]);
-    };
-
-    if (u0 >= u1) return;
-    Cursor nxt;                                          // one step ahead of the loops
-    nxt.qi = u0; nxt.cb = 0; nxt.ci = 0; nxt.th = 0; nxt.tw = 0; nxt.hb = 0;
-    enter_unit(nxt);
-    int u = 0;                                           // steps so far: the ring buffer
-    f4 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
-    Reads rd = describe(nxt, 0);
-    asm volatile("s_barrier" ::: "memory");              // the first step's halo and slab are there
-    read_kg(rd, 0, fa0, fb0);
-    bool more = true;
-    for (int qi = u0; qi < u1; ++qi) {
-        const int pass = nxt.pass, m0 = nxt.m0, n0 = nxt.n0;     // the cursor is at this unit's first step
-        int T[CPP];
-#pragma unroll
-        for (int ci = 0; ci < CPP; ++ci) T[ci] = nxt.cTh[ci] * nxt.cTw[ci];
-        start_unit(pass, n0);
-        for (int cb = 0; cb < ncb; ++cb) {
-#pragma unroll
-            for (int ci = 0; ci < CPP; ++ci) {
-                for (int t = 0; t < T[ci]; ++t) {
-                    read_kg(rd, 1, fa1, fb1);
-                    multiply(acc[ci], fa0, fb0);
-                    read_kg(rd, 2, fa0, fb0);
-                    multiply(acc[ci], fa1, fb1);
-                    read_kg(rd, 3, fa1, fb1);
-                    multiply(acc[ci], fa0, fb0);
-                    more = advance(nxt);
-                    ++u;
-                    if (more) {
-                        rd = describe(nxt, u);
-                        // every read of this step has come back (the slab wave refills its buffer after this barrier), and
-                        // the next step's halo and slab are there
-                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                        asm volatile("s_barrier" ::: "memory");
-                        read_kg(rd, 0, fa0, fb0);
-                    }
-                    multiply(acc[ci], fa1, fb1);
-                }
-            }
-        }
-        store_unit(pass, m0, n0);
-    }
+    store_tile_lines2<TM>(pa, pa.out, acc[0], m0 + wm0, n0, l32, lh, m_end);
+    store_tile_lines2<TM>(pb, pb.out, acc[1], m0 + wm0, n0, l32, lh, m_end);
 }
 
 struct PackParams {

@@ -48,7 +48,7 @@ bool tuning_set(const char* name, int value) {
         {"wgrad_halo", &Tuning::wgrad_halo},     {"wgrad_cw", &Tuning::wgrad_cw},
         {"wgrad_wide", &Tuning::wgrad_wide},     {"gather_direct_b", &Tuning::gather_direct_b},
         {"gather_clip", &Tuning::gather_clip},       {"gather_merge", &Tuning::gather_merge},
-        {"gather_stream", &Tuning::gather_stream}, {"gather_pairs", &Tuning::gather_pairs},
+        {"gather_pairs", &Tuning::gather_pairs},
         {"wgrad_br", &Tuning::wgrad_br},         {"wgrad_rounds", &Tuning::wgrad_rounds},
     };
     for (const Field& f : fields)

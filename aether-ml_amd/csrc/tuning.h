@@ -20,7 +20,6 @@ struct Tuning {
     int gather_direct_b = -1; // 0: dgrad always packs its filter (no reads from w itself)
     int gather_clip = -1;    // 0: strided dgrad multiplies its classes' full pixel grids (no zeroed strips)
     int gather_merge = -1;   // 0: bf16 strided dgrad launches its classes one by one
-    int gather_stream = -1;  // 1: the persistent halo kernel wherever its conditions hold (measurements)
     int gather_pairs = -1;   // 0: the merged launch keeps one class per workgroup
     int gather_wide = -1;    // bf16 8-wave tiles: 0 never, 1 also for few tiles
     int gather_res = -1;     // gather_halo_res_bf16: 0 off, 1 also for few tiles

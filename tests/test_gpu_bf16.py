@@ -315,9 +315,9 @@ MERGE_CASES = [
     (2, 12, 18, 64, 64, 5, 5, 2, 2, "same"),      # 9, 6, 6 and 4 taps
     (5, 8, 8, 128, 192, 3, 3, 2, 2, "same"),      # 16 pixels per class and image: tiles run over images
     (1, 18, 12, 48, 64, 3, 2, 1, 2, "valid"),     # two classes (columns only), 3 x 2 filter
-    (40, 28, 28, 128, 128, 3, 3, 2, 2, "valid"),  # 31 tiles of 256 pixels per class: several units per workgroup when persistent
-    (9, 16, 16, 200, 64, 3, 3, 2, 2, "same"),     # 200 channels of dx: two n tiles of 128, the second ragged
-    (4, 16, 16, 96, 128, 3, 3, 2, 1, "same"),     # two classes and 96 channels of dx: one pair when persistent
+    (40, 28, 28, 128, 128, 3, 3, 2, 2, "valid"),  # 31 tiles of 256 pixels per class
+    (9, 16, 16, 200, 64, 3, 3, 2, 2, "same"),     # 200 channels of dx: four n tiles, the last ragged
+    (4, 16, 16, 96, 128, 3, 3, 2, 1, "same"),     # two classes (one pair) and 96 channels of dx
     (3, 12, 18, 72, 64, 5, 5, 2, 2, "same"),      # 9, 6, 6 and 4 taps on 72 channels of dx: windows of 3 x 3 in the common halo
     (2, 24, 24, 128, 128, 4, 4, 2, 2, "valid"),   # 4 taps in every class
 ]
@@ -336,9 +336,6 @@ def test_bf16_dgrad_with_all_stride_classes_in_one_launch(case, tune):
     assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
     # two classes per workgroup from one halo (what the library takes where all classes read the filter in place)
     tune(gather_merge=-1, gather_pairs=-1)
-    assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
-    # the persistent form of the same (one workgroup per CU walks tiles and pairs; more than 64 channels of dx)
-    tune(gather_stream=1)
     assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
 
 
