@@ -308,6 +308,58 @@ __device__ __forceinline__ void store_tile_lines2(const GatherParams& p, float* 
     }
 }
 
+// The general form: a wave tile of TN 32-column blocks with interleaved columns (column l of block j is channel
+// nw0 + TN l + j; TN = 2 or 4): a lane holds TN neighbouring channels of a pixel and 32 lanes write 32 TN contiguous
+// floats per pixel with one 8- or 16-byte store each.  N is a multiple of 4 (p.out_bytes != 0).
+template <int TM, int TN>
+__device__ __forceinline__ void store_tile_runs(const GatherParams& p, float* out, const f16v (&acc)[TM][TN], int mw0,
+                                                int nw0, int l32, int lh, int m_end) {
+    static_assert(TN == 2 || TN == 4, "8- or 16-byte stores");
+    typedef unsigned u2 __attribute__((ext_vector_type(2)));
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(out, 0, (int)p.out_bytes, 0x00020000);
+    const int n = nw0 + TN * l32;
+    const unsigned col = (unsigned)n * 4u, colbad = (unsigned)!(n < p.N) << 31;   // N is a multiple of TN here: all channels or none
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int m = mw0 + 32 * i + l32;
+        const bool mok = m < m_end;
+        unsigned row = (unsigned)m;
+        if (!p.dense_out) {
+            unsigned s, rem, ii, jj;
+            p.div_hw.divmod(mok ? (unsigned)m : 0u, s, rem);
+            p.div_w.divmod(rem, ii, jj);
+            row = ((unsigned)s * p.Hof + p.oh0 + ii * p.ohs) * p.Wof + p.ow0 + jj * p.ows;
+        }
+        const int rowbytes = (int)((row * (unsigned)p.N * 4u) | ((unsigned)!mok << 31));   // < 2^31: checked by the host
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int pix = 8 * (v >> 2) + (v & 3);
+            const unsigned base = (unsigned)__builtin_amdgcn_ds_bpermute(4 * pix + 16 * lh, rowbytes);
+            const int off = (int)((base + col) | colbad);
+            float e[TN];                                 // (a bit cast of the vector element itself reads element 0)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) e[j] = acc[i][j][v];
+            if constexpr (TN == 2) {
+                const u2 value = {__float_as_uint(e[0]), __float_as_uint(e[1])};
+                __builtin_amdgcn_raw_buffer_store_b64(value, rsrc, off, 0, 0);
+            } else {
+                const u4 value = {__float_as_uint(e[0]), __float_as_uint(e[1]), __float_as_uint(e[2]), __float_as_uint(e[3])};
+                __builtin_amdgcn_raw_buffer_store_b128(value, rsrc, off, 0, 0);
+            }
+        }
+    }
+#if defined(__HIP_DEVICE_COMPILE__)                      // see store_tile: the stored registers stay untouched for a few cycles
+    if constexpr (TN == 4) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) asm volatile("s_nop 3" :: "v"(acc[i][j]));
+    }
+#endif
+}
+
 // ------------------------------------------------------------------------------
 // LDS-direct loads and wave-uniform mask helpers shared by the gather and the wgrad kernels
 // ------------------------------------------------------------------------------

@@ -189,11 +189,15 @@ __global__ __launch_bounds__(kThreads, 3) void gather_gemm(const GatherParams p)
 //     8 rows are all inside, nearly all of them, is issued as it is; else the 8 bits are spread over the
 //     lanes on the scalar unit and one v_cndmask sends the outside lanes beyond the descriptor.
 
-template <typename T, int BM, int BN, int WM, int WN, bool UT, int KC, bool NLOOP, bool SA = false>
+// RUNS (the 8-wave bf16 tiles, whose launches wait for their stores rather than for instruction issue): the pixels are the
+// MFMAs' first operand and the filter rows of a wave's columns are fetched interleaved (column l of block j is channel
+// TN l + j), so that the tile goes out in runs of 32 TN contiguous floats per pixel (store_tile_runs).
+template <typename T, int BM, int BN, int WM, int WN, bool UT, int KC, bool NLOOP, bool SA = false, bool RUNS = false>
 __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(const GatherParams p) {
     // 4 waves, or 8 for the widest bf16 tiles (256 x 128 and 256 x 256: one workgroup per CU)
     constexpr int NW = (BM / WM) * (BN / WN);
     static_assert(NW == 4 || (NW == 8 && !NLOOP && !SA), "4 or 8 waves per workgroup");
+    static_assert(!RUNS || (NW == 8 && sizeof(T) == 2 && (WN == 64 || WN == 128)), "runs: the 8-wave bf16 tiles");
     static_assert(!SA || (UT && !NLOOP && (BM == 128 || BM == 64) && sizeof(T) == 4), "scalar addressing: fp32 uniform-tap tiles of 64 or 128 rows");
     static_assert(KC == 8 || KC == 4, "slab rows of 8 or 4 chunks");
     constexpr int CE = Elem<T>::CE;
@@ -308,7 +312,9 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
 #pragma unroll
         for (int i = 0; i < BL; ++i) {
             const int k4 = k4e ^ (((wave * BL + i) & 1) ? ODD : 0);
-            b_off[i] = (unsigned)(((n0 + (wave * BL + i) * RPL + lr) * p.bt_ld + CE * k4) * (int)sizeof(T));
+            int r = (wave * BL + i) * RPL + lr;          // slab row; RUNS: it holds channel (r / WN) WN + TN (r % 32) + (r % WN) / 32
+            if constexpr (RUNS) r = (r / WN) * WN + (WN / 32) * (r & 31) + (r % WN) / 32;
+            b_off[i] = (unsigned)(((n0 + r) * p.bt_ld + CE * k4) * (int)sizeof(T));
         }
     };
     set_b_off();
@@ -419,7 +425,10 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) mma_chunk<T>(fb[slot][j], fa[slot][i], acc[i][j]);
+            for (int j = 0; j < TN; ++j) {
+                if constexpr (RUNS) mma_chunk<T>(fa[slot][i], fb[slot][j], acc[i][j]);
+                else mma_chunk<T>(fb[slot][j], fa[slot][i], acc[i][j]);
+            }
     };
     // One slab: the first operand reads go out right after the barrier, then the
     // loads of the next slab are issued (their address arithmetic overlaps the LDS
@@ -565,13 +574,27 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
         if (s_begin + p.split_slabs < nslabs) nslabs = s_begin + p.split_slabs;
     }
     if (s_begin < nslabs) issue(s_begin * BK, lds_a0, lds_b0);
-    fill_acc<TM, TN>(bv, acc);
+    if constexpr (RUNS) {
+        // a lane's accumulators of block j all belong to channel n0 + wn0 + TN l32 + j
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int n = n0 + wn0 + TN * l32 + j;
+            const float bj = (split == 0 && p.bias != nullptr && n < p.N) ? p.bias[n] : 0.0f;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = bj;
+        }
+    } else {
+        fill_acc<TM, TN>(bv, acc);
+    }
     for (int s = s_begin; s < nslabs; s += 2) {
         slab(lds_a0, lds_b0, lds_a1, lds_b1, (s + 1) * BK, s + 1 < nslabs);
         if (s + 1 < nslabs) slab(lds_a1, lds_b1, lds_a0, lds_b0, (s + 2) * BK, s + 2 < nslabs);
     }
 
-    store_tile<TM, TN>(p, p.out + (size_t)split * p.M * p.N, acc, m0 + wm0, n0 + wn0, l32, lh);
+    if constexpr (RUNS) store_tile_runs<TM, TN>(p, p.out + (size_t)split * p.M * p.N, acc, m0 + wm0, n0 + wn0, l32, lh, p.M);
+    else store_tile<TM, TN>(p, p.out + (size_t)split * p.M * p.N, acc, m0 + wm0, n0 + wn0, l32, lh);
 }
 
 // ------------------------------------------------------------------------------

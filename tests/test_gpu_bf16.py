@@ -224,7 +224,7 @@ WIDE_CASES = [
 @pytest.mark.parametrize("case", WIDE_CASES, ids=lambda c: "x".join(str(v) for v in c))
 def test_bf16_fprop_dgrad_with_wide_tiles_on_eight_waves(case, tune):
     from tests import abi
-    tune(gather_split=0)
+    tune(gather_split=0, gather_merge=0)          # (one launch per dgrad class: the merged launch has kernels of its own)
     tune(gather_wide=1)
     x, w, b, dy = _case(case, 13)
     stride, pad = (case[7], case[8]), case[9]
@@ -234,6 +234,9 @@ def test_bf16_fprop_dgrad_with_wide_tiles_on_eight_waves(case, tune):
     abi.close(abi.fprop_bf16(x, w, None, stride, pad), O.conv_fprop(xr, wr, None, stride, pad, dtype=np.float64))
     dx = abi.dgrad_bf16(dy, w, x.shape, stride, pad)
     abi.close(dx, O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
+    tune(gather_runs=0)                           # 16-byte pieces per pixel instead of runs of contiguous channels
+    assert np.array_equal(y, abi.fprop_bf16(x, w, b, stride, pad))
+    assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
     tune(gather_wide=0)
     assert np.array_equal(y, abi.fprop_bf16(x, w, b, stride, pad))
     assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
