@@ -226,8 +226,11 @@ static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t
         int mtiles = 0;
         if (plan_dense_res(gp, dma, cus, &mtiles)) {
             const dim3 grid((unsigned)std::min(mtiles, cus));
-            if (gp.Kpad == 64) hipLaunchKernelGGL(dense_res_f32<2>, grid, dim3(kD1Threads), 0, st, gp, mtiles);
-            else hipLaunchKernelGGL(dense_res_f32<1>, grid, dim3(kD1Threads), 0, st, gp, mtiles);
+            const bool runs = tuning().gather_runs != 0 && gp.N % 2 == 0;
+            if (gp.Kpad == 64 && runs) hipLaunchKernelGGL((dense_res_f32<2, true>), grid, dim3(kD1Threads), 0, st, gp, mtiles);
+            else if (gp.Kpad == 64) hipLaunchKernelGGL((dense_res_f32<2, false>), grid, dim3(kD1Threads), 0, st, gp, mtiles);
+            else if (runs) hipLaunchKernelGGL((dense_res_f32<1, true>), grid, dim3(kD1Threads), 0, st, gp, mtiles);
+            else hipLaunchKernelGGL((dense_res_f32<1, false>), grid, dim3(kD1Threads), 0, st, gp, mtiles);
             return;
         }
     }

@@ -1287,7 +1287,9 @@ constexpr int kD1BM = 128;
 constexpr int kD1Threads = 512;
 constexpr int kD1MaxN = 256;
 
-template <int NSLAB>                                   // K = 32 * NSLAB
+// RUNS: the pixels are the MFMAs' first operand and slab row r of the filter holds channel (r / 64) 64 + 2 (r % 32) + (r % 64) / 32,
+// so that a lane owns two neighbouring channels and a tile goes out in runs of 256 contiguous bytes per pixel (store_tile_runs).
+template <int NSLAB, bool RUNS>                        // K = 32 * NSLAB
 static __global__ __launch_bounds__(kD1Threads, 1) void dense_res_f32(const GatherParams p, const int mtiles) {
     constexpr int BM = kD1BM, KC = 8, TM = 2, TN = 2, nslab = NSLAB;
     __shared__ f4 filt[2][kD1MaxN * KC];                 // slab s: rows n of 128 B, chunk c at c ^ ((n >> 1) & 7)
@@ -1316,7 +1318,9 @@ static __global__ __launch_bounds__(kD1Threads, 1) void dense_res_f32(const Gath
         for (int q = wave; q < nslab * pieces; q += 8) {
             const int sl = q / pieces, part = q - sl * pieces;
             const int k4 = k4e ^ ((part & 1) ? 4 : 0);
-            const unsigned off = (unsigned)(((part * 8 + prow) * p.Kpad + 32 * sl + 4 * k4) * 4);
+            int r = part * 8 + prow;
+            if constexpr (RUNS) r = (r & ~63) + 2 * (r & 31) + ((r >> 5) & 1);
+            const unsigned off = (unsigned)((r * p.Kpad + 32 * sl + 4 * k4) * 4);
             lds_direct_load16(rsrc_b, lds_address(&filt[sl][0]) + (unsigned)part * 1024u, off);
         }
         if (tid < kD1MaxN / 4) {
@@ -1355,11 +1359,22 @@ static __global__ __launch_bounds__(kD1Threads, 1) void dense_res_f32(const Gath
     int done_m0 = 0;
     bool have_done = false;
     auto store_done = [&]() __attribute__((always_inline)) {
-        store_tile<TM, TN, true>(p, p.out, done, done_m0 + wm0, wn0, l32, lh);
+        if constexpr (RUNS) store_tile_runs<TM, TN>(p, p.out, done, done_m0 + wm0, wn0, l32, lh, p.M);
+        else store_tile<TM, TN, true>(p, p.out, done, done_m0 + wm0, wn0, l32, lh);
     };
     for (int t = 0; t < ntl; ++t) {
         if (wave == 0 && t + 1 < ntl) fetch(tile0 + t + 1, (t + 1) & 1);
         if (active) {
+            if constexpr (RUNS) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    const float bj = reinterpret_cast<const float*>(bias_lds)[wn0 + 2 * l32 + j];
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) acc[i][j][v] = bj;
+                }
+            } else {
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -1370,6 +1385,7 @@ static __global__ __launch_bounds__(kD1Threads, 1) void dense_res_f32(const Gath
 #pragma unroll
                         for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = b[e];
                 }
+            }
             // k groups u = 4 slab + g of 8 k each; the operands of group u + 1 are read during the MFMAs of group u
             f4 fa[2][TM], fb[2][TN];
             auto read_frags = [&](int u, int slot) __attribute__((always_inline)) {
@@ -1391,7 +1407,10 @@ static __global__ __launch_bounds__(kD1Threads, 1) void dense_res_f32(const Gath
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
 #pragma unroll
-                        for (int j = 0; j < TN; ++j) mma_chunk<float>(fb[u & 1][j], fa[u & 1][i], acc[i][j]);
+                        for (int j = 0; j < TN; ++j) {
+                            if constexpr (RUNS) mma_chunk<float>(fa[u & 1][i], fb[u & 1][j], acc[i][j]);
+                            else mma_chunk<float>(fb[u & 1][j], fa[u & 1][i], acc[i][j]);
+                        }
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 // the finished tile leaves after k group `wave` (a few 16-byte pieces after every group

@@ -221,6 +221,8 @@ def test_fprop_with_the_filter_resident_in_lds(case, tune):
     got = abi.fprop(x, w, b, stride, pad)
     abi.close(got, O.conv_fprop(x, w, b, stride, pad, dtype=np.float64))
     abi.close(abi.fprop(x, w, None, stride, pad), O.conv_fprop(x, w, None, stride, pad, dtype=np.float64))
+    tune(gather_runs=0)                           # tiles stored as 16-byte pieces per pixel instead of runs of contiguous channels
+    assert np.array_equal(got, abi.fprop(x, w, b, stride, pad))
     # the other kernels add the same products in the same order of k
     tune(dense_res=0)
     assert np.array_equal(got, abi.fprop(x, w, b, stride, pad))
