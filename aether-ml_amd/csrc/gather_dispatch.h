@@ -43,7 +43,20 @@ static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
         const int taps = gp.Cs > 0 ? gp.K / gp.Cs : 0;
         const int64_t bias = ((int64_t)std::max(-gp.rh0, 0) * gp.Ws + std::max(-gp.rw0, 0)) * gp.Cs * (int64_t)sizeof(T);
         if (ut && taps <= 32 && (int64_t)gp.src_bytes + bias < ((int64_t)1 << 31) && tuning().gather_sa != 0) {
+            if constexpr (KC == 8) {
+                if (gp.bt_kn) {
+                    hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, true, false, true>), grid, dim3(kThreads), 0, st, gp);
+                    return;
+                }
+            }
             hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, true>), grid, dim3(kThreads), 0, st, gp);
+            return;
+        }
+    }
+    if constexpr (sizeof(T) == 4 && KC == 8 && kThreads == 256) {
+        if (gp.bt_kn) {                                      // fprop reading the filter in place
+            if (ut) hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, false, false, true>), grid, dim3(kThreads), 0, st, gp);
+            else hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, false, KC, false, false, false, true>), grid, dim3(kThreads), 0, st, gp);
             return;
         }
     }
@@ -373,6 +386,7 @@ static void fill_gather(GatherSetup& gs, char* ws, int64_t ws_off) {
     gs.gp.out_bytes = ovec ? (unsigned)ob : 0u;
     gs.gp.bt_ld = gs.gp.Kpad;
     gs.gp.bt_direct = 0;
+    gs.gp.bt_kn = 0;
 }
 
 // dgrad whose slabs lie inside one tap reads its B operand from w itself: row (tap, c) of w is
@@ -399,6 +413,20 @@ static int choose_b_operand(GatherSetup& gs, bool vec, int min_slabs = 3) {
         gs.gp.bd_xa = pk.xa; gs.gp.bd_xs = pk.xs; gs.gp.bd_ya = pk.ya; gs.gp.bd_ys = pk.ys;
         gs.gp.bd_fw = pk.fW; gs.gp.bd_tap_elems = pk.C * pk.D;
         return 0;                                    // nothing to pack
+    }
+    // fp32 fprop with at least three slabs (the slab kernel): w[fH][fW][C][D] is the [K][N] matrix itself, rows of D floats.
+    // Whole n tiles only: with the slab's row in the scalar offset the range check does not see columns past the last row.
+    // (tuning: gather_direct_b = 0 packs)
+    if constexpr (sizeof(T) == 4) {
+        if (!pk.transposed && vec && g.src_bytes != 0 && g.Kpad / BK >= min_slabs && pk.D % 4 == 0 && g.N % gather_bn(g.N) == 0 &&
+            g.K == pk.K && pk.w_elems * 4 < ((int64_t)1 << 31) && (reinterpret_cast<uintptr_t>(pk.w) & 15) == 0 &&
+            tuning().gather_direct_b != 0 && tuning().gather_kc == -1 && tuning().gather_bkn != 0) {
+            gs.gp.bt = pk.w;
+            gs.gp.bt_bytes = (unsigned)(pk.w_elems * 4);
+            gs.gp.bt_ld = pk.D;
+            gs.gp.bt_kn = 1;
+            return 0;
+        }
     }
     return pk.Npad * pk.Kpad;
 }

@@ -192,8 +192,13 @@ __global__ __launch_bounds__(kThreads, 3) void gather_gemm(const GatherParams p)
 // RUNS (the 8-wave bf16 tiles, whose launches wait for their stores rather than for instruction issue): the pixels are the
 // MFMAs' first operand and the filter rows of a wave's columns are fetched interleaved (column l of block j is channel
 // TN l + j), so that the tile goes out in runs of 32 TN contiguous floats per pixel (store_tile_runs).
-template <typename T, int BM, int BN, int WM, int WN, bool UT, int KC, bool NLOOP, bool SA = false, bool RUNS = false>
+// BKN (fp32 fprop): the B operand is the filter w[fH][fW][C][D] itself, a [K][N] matrix with n contiguous: a slab is 32 rows of k
+// x BN floats (1 KB loads of 4 or 8 rows; with 64 columns the odd rows are stored with their halves swapped, so that the two
+// lane halves of a 4-byte operand read, which sit one row apart, use different banks), and an operand read is four 4-byte reads
+// from four rows instead of one 16-byte read.  No packing launch.
+template <typename T, int BM, int BN, int WM, int WN, bool UT, int KC, bool NLOOP, bool SA = false, bool RUNS = false, bool BKN = false>
 __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(const GatherParams p) {
+    static_assert(!BKN || (sizeof(T) == 4 && KC == 8 && !NLOOP && !RUNS && (BN == 64 || BN == 32)), "filter in place: fp32 slab tiles");
     // 4 waves, or 8 for the widest bf16 tiles (256 x 128 and 256 x 256: one workgroup per CU)
     constexpr int NW = (BM / WM) * (BN / WN);
     static_assert(NW == 4 || (NW == 8 && !NLOOP && !SA), "4 or 8 waves per workgroup");
@@ -311,6 +316,14 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
     auto set_b_off = [&]() {
 #pragma unroll
         for (int i = 0; i < BL; ++i) {
+            if constexpr (BKN) {
+                // load ld = wave BL + i brings rows RB ld .. of the slab, 16-byte chunks of BN floats each
+                constexpr int CPRB = BN / 4, RB = 64 / CPRB;
+                const int row = (wave * BL + i) * RB + lane / CPRB;
+                const int c = (lane % CPRB) ^ ((BN == 64 && (row & 1)) ? 8 : 0);
+                b_off[i] = (unsigned)((row * p.bt_ld + n0 + 4 * c) * 4);
+                continue;
+            }
             const int k4 = k4e ^ (((wave * BL + i) & 1) ? ODD : 0);
             int r = (wave * BL + i) * RPL + lr;          // slab row; RUNS: it holds channel (r / WN) WN + TN (r % 32) + (r % WN) / 32
             if constexpr (RUNS) r = (r / WN) * WN + (WN / 32) * (r & 31) + (r % WN) / 32;
@@ -334,13 +347,13 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
     int tap_off[2] = {0, 0}, tap_h[2] = {0, 0}, tap_w[2] = {0, 0};
     bool kvalid[2] = {false, false};
     auto prep = [&](int k0) {
-        b_k_bytes = (unsigned)k0 * (unsigned)sizeof(T);
+        b_k_bytes = BKN ? (unsigned)k0 * (unsigned)p.bt_ld * 4u : (unsigned)k0 * (unsigned)sizeof(T);
         if (UT) {
             unsigned c0, th, tw;
             p.div_c.divmod((unsigned)k0, ut_tap, c0);
             p.div_tw.divmod(ut_tap, th, tw);
             ut_tap_bytes = (unsigned)(((int)th * p.Ws + (int)tw) * p.Cs + (int)c0) * (unsigned)sizeof(T);
-            if (p.bt_direct)                             // the filter itself: tap (th, tw) of this class, channels c0..
+            if (!BKN && p.bt_direct)                     // the filter itself: tap (th, tw) of this class, channels c0..
                 b_k_bytes = (unsigned)(((p.bd_xa + p.bd_xs * (int)th) * p.bd_fw + p.bd_ya + p.bd_ys * (int)tw) * p.bd_tap_elems +
                                        (int)c0) * (unsigned)sizeof(T);
             if constexpr (SA) cur_mask = (unsigned)__builtin_amdgcn_ballot_w64(((aux_row >> ut_tap) & 1u) != 0u);
@@ -418,6 +431,17 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
         const int pc = (2 * g + lh) ^ sw7;
 #pragma unroll
         for (int i = 0; i < TM; ++i) fa[slot][i] = la[(wm0 + 32 * i + l32) * KC + pc];
+        if constexpr (BKN) {
+            // k = 8 g + 4 lh + t for t = 0..3: rows of BN floats; odd rows of a 64-wide slab have their halves swapped
+            const float* lbf = reinterpret_cast<const float*>(lb) + (8 * g + 4 * lh) * BN;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int n = wn0 + 32 * j + l32;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) fb[slot][j][t] = lbf[t * BN + (n ^ ((BN == 64 && (t & 1)) ? 32 : 0))];
+            }
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < TN; ++j) fb[slot][j] = lb[(wn0 + 32 * j + l32) * KC + pc];
     };

@@ -290,6 +290,34 @@ def test_dgrad_reading_the_filter_in_place(case, tune):
     assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
 
 
+# fp32 fprop with at least three slabs of K and whole n tiles reads its B operand from the filter itself too:
+# w[fH][fW][C][D] is the [K][N] matrix with n contiguous, fetched as slabs of 32 rows of k and read with 4-byte
+# operand reads.  The gather_bkn switch at 0 packs as before; same bits (same slabs, same order).
+BKN_CASES = [
+    (4, 16, 16, 32, 64, 3, 3, 1, 1, "same"),      # 9 slabs, 64-wide tiles: odd rows stored with their halves swapped
+    (4, 16, 16, 32, 32, 3, 3, 1, 1, "same"),      # 32-wide tiles: 8 rows per load
+    (3, 9, 9, 64, 128, 3, 3, 2, 2, "valid"),      # stride 2, two n tiles
+    (2, 10, 10, 3, 64, 5, 5, 1, 1, "same"),       # K = 75: the last slab has rows past K, taps decoded per lane
+    (2, 10, 10, 12, 32, 3, 3, 1, 1, "valid"),     # K = 108, 12 channels
+    (128, 1, 1, 2048, 256, 1, 1, 1, 1, "valid"),  # a dense layer on a small batch: split K
+    (40, 12, 12, 64, 64, 3, 3, 1, 1, "same"),     # 5760 rows: 128-row tiles
+    (2, 12, 12, 64, 40, 3, 3, 1, 1, "same"),      # 40 output channels are not whole n tiles: packed
+]
+
+
+@pytest.mark.parametrize("case", BKN_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_fprop_reading_the_filter_in_place(case, tune):
+    from tests import abi
+    x, w, b, dy = _case(case, 22)
+    stride, pad = (case[7], case[8]), case[9]
+    y = abi.fprop(x, w, b, stride, pad)
+    abi.close(y, O.conv_fprop(x, w, b, stride, pad, dtype=np.float64))
+    tune(gather_bkn=0)
+    assert np.array_equal(y, abi.fprop(x, w, b, stride, pad))
+    tune(gather_bkn=-1, gather_sa=0)                  # vector-addressed loads
+    assert np.array_equal(y, abi.fprop(x, w, b, stride, pad))
+
+
 # Strided dgrad whose last rows / columns are reached by no output pixel: the classes' pixel grids stop
 # at the last reachable index and one small launch zeroes the strips.  The gather_clip switch at 0
 # multiplies the full grids (every tap of those pixels falls outside dy: zeros); same bits either way.
