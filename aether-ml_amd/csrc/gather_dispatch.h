@@ -2,6 +2,7 @@
 // entry points' shared implementation.
 #pragma once
 #include "gather_kernels.h"
+#include "narrow_kernels.h"
 #include "tuning.h"
 
 namespace aeth {
@@ -512,6 +513,17 @@ int conv_fprop_impl(const char* fn, const T* x, const T* w, const float* bias, f
     int Ho, Wo;
     int rc = check_conv_dims(fn, S, H, W, C, D, fH, fW, sH, sW, pH, pW, &Ho, &Wo);
     if (rc) return rc;
+    if constexpr (sizeof(T) == 4) {
+        const int64_t M = (int64_t)S * H * W;
+        if (narrow_shape(D, fH, fW, sH, sW, pH, pW) && M > 0 && M * 64 < ((int64_t)1 << 31) && C <= 16384) {
+            NarrowParams np;
+            np.a = x; np.b = w; np.bias = bias; np.out = y; np.out2 = nullptr;
+            np.M = (int)M; np.K = C; np.N = D;
+            hipLaunchKernelGGL(narrow_fprop, dim3((unsigned)cdiv(M * 64, kThreads)), dim3(kThreads), 0, ctx().stream, np);
+            AETH_LAUNCH_CHECK();
+            return AETH_OK;
+        }
+    }
     if (C <= 3) {
         DirectParams dp;
         dp.a = x; dp.w = w; dp.bias = bias; dp.out = y;
@@ -570,6 +582,17 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
     constexpr int BK = Elem<T>::BK;
     const int nclass = sH * sW;
     if (nclass > 64) return fail(AETH_E_INVALID, "%s: stride too large", fn);
+    if constexpr (sizeof(T) == 4) {
+        const int64_t M = (int64_t)S * H * W;
+        if (narrow_shape(D, fH, fW, sH, sW, pH, pW) && M > 0 && M * C < ((int64_t)1 << 31)) {
+            NarrowParams np;
+            np.a = dy; np.b = w; np.bias = nullptr; np.out = dx; np.out2 = nullptr;
+            np.M = (int)M; np.K = C; np.N = D;
+            hipLaunchKernelGGL(narrow_dgrad, dim3((unsigned)cdiv(M * C, kThreads)), dim3(kThreads), 0, ctx().stream, np, (unsigned)(M * C));
+            AETH_LAUNCH_CHECK();
+            return AETH_OK;
+        }
+    }
     if (C <= 3) {
         DirectParams dp;
         dp.a = dy; dp.w = w; dp.bias = nullptr; dp.out = dx;

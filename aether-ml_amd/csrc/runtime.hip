@@ -49,7 +49,7 @@ bool tuning_set(const char* name, int value) {
         {"wgrad_wide", &Tuning::wgrad_wide},     {"gather_direct_b", &Tuning::gather_direct_b},
         {"gather_clip", &Tuning::gather_clip},       {"gather_merge", &Tuning::gather_merge},
         {"gather_pairs", &Tuning::gather_pairs},
-        {"gather_runs", &Tuning::gather_runs},   {"gather_bkn", &Tuning::gather_bkn},
+        {"gather_runs", &Tuning::gather_runs},   {"narrow", &Tuning::narrow},   {"gather_bkn", &Tuning::gather_bkn},
         {"wgrad_br", &Tuning::wgrad_br},         {"wgrad_rounds", &Tuning::wgrad_rounds},
     };
     for (const Field& f : fields)

@@ -1,6 +1,7 @@
 // Host side of wgrad: kernel choice, number of splits, the fixed-order reduction of the partials.
 #pragma once
 #include "wgrad_kernels.h"
+#include "narrow_kernels.h"
 #include "tuning.h"
 
 namespace aeth {
@@ -72,6 +73,18 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     int Ho, Wo;
     int rc = check_conv_dims(fn, S, H, W, C, D, fH, fW, sH, sW, pH, pW, &Ho, &Wo);
     if (rc) return rc;
+    if constexpr (sizeof(T) == 4) {
+        // at most 16 output channels and few rows: one thread per element of dw walks the rows
+        const int64_t M = (int64_t)S * H * W;
+        if (narrow_shape(D, fH, fW, sH, sW, pH, pW) && M > 0 && M <= 1024 && (int64_t)(C + 1) * 16 < ((int64_t)1 << 31)) {
+            NarrowParams np;
+            np.a = x; np.b = dy; np.bias = nullptr; np.out = dw; np.out2 = dbias;
+            np.M = (int)M; np.K = C; np.N = D;
+            hipLaunchKernelGGL(narrow_wgrad, dim3((unsigned)cdiv((int64_t)(C + 1) * 16, kThreads)), dim3(kThreads), 0, ctx().stream, np);
+            AETH_LAUNCH_CHECK();
+            return AETH_OK;
+        }
+    }
     Context& c = ctx();
     WgradParams p;
     p.x = x; p.dy = dy;

@@ -318,6 +318,41 @@ def test_fprop_reading_the_filter_in_place(case, tune):
     assert np.array_equal(y, abi.fprop(x, w, b, stride, pad))
 
 
+# Products with at most 16 output channels (a classifier head) and a 1x1 filter go to kernels with one thread
+# per output, one launch per direction and no scratch memory; wgrad only where the rows are few (at most 1024).
+# The narrow switch at 0 sends them to the slab kernels: other orders of the same sums.
+NARROW_CASES = [
+    (128, 1, 1, 256, 10, 1, 1, 1, 1, "valid"),    # Layer_Dense(256, 10) on a batch of 128
+    (1000, 1, 1, 37, 16, 1, 1, 1, 1, "valid"),    # 16 channels, K not a multiple of 4
+    (3, 9, 7, 24, 1, 1, 1, 1, 1, "same"),         # a 1x1 convolution onto one channel
+    (1500, 1, 1, 64, 5, 1, 1, 1, 1, "valid"),     # 1500 rows: wgrad by the slab kernels
+    (2, 6, 6, 8, 17, 1, 1, 1, 1, "valid"),        # 17 channels: the slab kernels
+]
+
+
+@pytest.mark.parametrize("case", NARROW_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_products_with_few_output_channels(case, tune):
+    from tests import abi
+    S, H, W, C, D, fH, fW, sH, sW, pad = case
+    x, w, b, dy = _case(case, 31)
+    got = {}
+    for mode in (-1, 0):
+        tune(narrow=mode)
+        y = abi.fprop(x, w, b, (sH, sW), pad)
+        abi.close(y, O.conv_fprop(x, w, b, (sH, sW), pad, dtype=np.float64))
+        abi.close(abi.fprop(x, w, None, (sH, sW), pad), O.conv_fprop(x, w, None, (sH, sW), pad, dtype=np.float64))
+        dx = abi.dgrad(dy, w, x.shape, (sH, sW), pad)
+        abi.close(dx, O.conv_dgrad(dy, w, (H, W), (sH, sW), pad, dtype=np.float64))
+        dw, db = abi.wgrad(x, dy, w.shape, (sH, sW), pad)
+        abi.close(dw, O.conv_wgrad(x, dy, (fH, fW), (sH, sW), pad, dtype=np.float64), rms_scaled=True)
+        abi.close(db, O.conv_dbias(dy, dtype=np.float64), rms_scaled=True)
+        dw2, _ = abi.wgrad(x, dy, w.shape, (sH, sW), pad, want_dbias=False)
+        assert np.array_equal(dw, dw2)
+        got[mode] = (y, dx, dw, db)
+    for a, c in zip(got[-1], got[0]):
+        abi.close(a, c, rtol=1e-4, atol=1e-5, rms_scaled=True)
+
+
 # Strided dgrad whose last rows / columns are reached by no output pixel: the classes' pixel grids stop
 # at the last reachable index and one small launch zeroes the strips.  The gather_clip switch at 0
 # multiplies the full grids (every tap of those pixels falls outside dy: zeros); same bits either way.
