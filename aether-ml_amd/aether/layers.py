@@ -707,6 +707,25 @@ class Loss_CategoricalCrossEntropy(Loss):
         y_pred._cache = {"argmax": host[rows:].view(np.int32)}
         return host[:rows]
 
+    def head_launch(self, logits, y_true, softmax, fused):
+        """A training step's classifier head in one launch (Model.train_step): `softmax`'s output, this
+        loss with the row argmax, and the gradient `fused` (the softmax / cross-entropy object) would work
+        out in backward, which then finds it done.  The same operations in the same order as the three
+        separate launches."""
+        logits = as_device(logits, _F32)
+        rows, K = logits.shape
+        labels = _device_labels(y_true)
+        ls = self.label_smoothing if self.label_smoothing > 0 else 0.0
+        probs = DeviceTensor(logits.shape, _F32)
+        buf = DeviceTensor(2 * rows, _F32)
+        dlogits = DeviceTensor(logits.shape, _F32)
+        _ck(_L().aeth_softmax_cce_train_f32(logits.ptr, labels.ptr, ls, probs.ptr, buf.ptr, buf.ptr + 4 * rows,
+                                            dlogits.ptr, rows, K))
+        softmax.output = probs
+        fused.dinputs = dlogits
+        fused._done_for = probs
+        return buf, rows, probs
+
     def backward(self, dvalues, y_true):
         dvalues = as_device(dvalues, _F32)
         rows, K = dvalues.shape
@@ -728,6 +747,9 @@ class Activation_Softmax_Loss_CategoricalCrossEntropy():
         return self.loss.calculate(self.output, y_true, training=training)
 
     def backward(self, dvalues, y_true, training=True):
+        if getattr(self, "_done_for", None) is dvalues and dvalues is not None:
+            self._done_for = None                        # the head kernel of this step has written dinputs
+            return
         dvalues = as_device(dvalues, _F32)
         rows, K = dvalues.shape
         labels = _device_labels(y_true)

@@ -13,6 +13,7 @@ reference's CuPy pickles use (``cupy._core.core.array``) is mapped to
 anything else from it.
 """
 import io
+import os
 import pickle
 import warnings
 
@@ -226,8 +227,7 @@ class Model:
             L._label_buffer[0] = rec["labels"]
             L._recording[0] = True
             try:
-                output = self.forward(rec["x"], training=True)
-                rec["pending"] = self.loss.launch(output, batch_y, training=True)
+                output, rec["pending"] = self._forward_and_loss(rec["x"], batch_y)
                 rec["output"] = output
                 self.backward(output, batch_y)
                 self.optimizer.record_update(self.trainable_layers)
@@ -272,12 +272,14 @@ class Model:
             result = self._recorded_step(batch_X, batch_y)
             if result is not None:
                 return result
-        output = self.forward(batch_X, training=True)
         # The loss kernel is queued here and read after backward and the update have been
         # queued too, so the device never idles while the host prepares the backward pass.
         # With an active regulariser its sums must see the weights before the update, so
         # the loss is then read first, as the reference does.
-        pending = self.loss.launch(output, batch_y, training=True) if self.loss.can_defer() else None
+        if self.loss.can_defer():
+            output, pending = self._forward_and_loss(batch_X, batch_y)
+        else:
+            output, pending = self.forward(batch_X, training=True), None
         if pending is None:
             data_loss, regularization_loss = self.loss.calculate(output, batch_y, include_regularization=True,
                                                                  training=True)
@@ -291,6 +293,25 @@ class Model:
         predictions = self.output_layer_activation.predictions(output)
         accuracy = self.accuracy.calculate(predictions, batch_y)
         return data_loss + regularization_loss, data_loss, regularization_loss, accuracy
+
+    def _forward_and_loss(self, X, y):
+        """The forward pass of a training step with the loss kernel queued behind it.  A SoftMax
+        output under the fused softmax / cross-entropy object goes out as one launch with the loss,
+        the predictions and the gradient of the logits (`AETHER_FUSE_HEAD=0` keeps them apart)."""
+        head = self.layers[-1]
+        if (self.softmax_classifier_output is None or not isinstance(head, SoftMax) or len(self.layers) < 2
+                or not hasattr(self.loss, "head_launch") or os.environ.get("AETHER_FUSE_HEAD", "1") == "0"):
+            output = self.forward(X, training=True)
+            return output, self.loss.launch(output, y, training=True)
+        self.input_layer.forward(X, True)
+        for layer in self.layers[:-1]:
+            layer.forward(layer.prev.output, True)
+        logits = head.prev.output
+        if len(getattr(logits, "shape", ())) != 2:
+            head.forward(logits, True)
+            return head.output, self.loss.launch(head.output, y, training=True)
+        pending = self.loss.head_launch(logits, y, head, self.softmax_classifier_output)
+        return head.output, pending
 
     def forward(self, X, training):
         """Every layer reads its predecessor's `.output` (CNN_model_cupy.py:153-163)."""

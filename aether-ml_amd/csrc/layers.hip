@@ -642,6 +642,46 @@ __global__ void softmax_cce_bwd_kernel(const float* __restrict__ probs, const in
     dlogits[i] = (probs[i] - t) / (float)rows;
 }
 
+// softmax, the loss with the row argmax and the gradient of the logits in one pass over a row: the three kernels above
+// one after the other, with the same operations in the same order (a training step's classifier head)
+__global__ void softmax_cce_train_kernel(const float* __restrict__ logits, const int32_t* __restrict__ labels, float ls,
+                                         float* __restrict__ probs, float* __restrict__ loss, int32_t* __restrict__ pred,
+                                         float* __restrict__ dlogits, int rows, int K) {
+    int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= rows) return;
+    const float* in = logits + (size_t)r * K;
+    float* out = probs + (size_t)r * K;
+    float* dl = dlogits + (size_t)r * K;
+    float mx = in[0];
+    for (int k = 1; k < K; ++k) mx = fmaxf(mx, in[k]);
+    float sum = 0.f;
+    for (int k = 0; k < K; ++k) {
+        float e = expf(in[k] - mx);
+        out[k] = e;
+        sum += e;
+    }
+    const int y = labels[r];
+    const float t_off = ls / (float)K;
+    const float t_on = (1.0f - ls) + t_off;
+    float acc = 0.f;
+    float best = 0.f;
+    int bi = 0;
+    for (int k = 0; k < K; ++k) {
+        const float v = out[k] / sum;
+        out[k] = v;
+        if (k == 0 || v > best) {
+            best = v;
+            bi = k;
+        }
+        const float pc = fminf(fmaxf(v, 1e-7f), 1.0f - 1e-7f);
+        const float t = (k == y) ? t_on : t_off;
+        acc += t * logf(pc);
+        dl[k] = (v - t) / (float)rows;
+    }
+    loss[r] = -acc;
+    pred[r] = bi;
+}
+
 static int pool_dims(const char* fn, int S, int H, int W, int C, int fH, int fW, int sH, int sW, PoolParams* p) {
     if (S <= 0 || H <= 0 || W <= 0 || C <= 0 || fH <= 0 || fW <= 0 || sH <= 0 || sW <= 0)
         return fail(AETH_E_INVALID, "%s: non-positive dimension", fn);
@@ -1142,6 +1182,17 @@ int aeth_softmax_cce_bwd_f32(const float* probs, const int32_t* labels, float la
     AETH_CHECK_ARG((int64_t)rows * K < ((int64_t)1 << 31));
     hipLaunchKernelGGL(softmax_cce_bwd_kernel, dim3(cdiv((int64_t)rows * K, 256)), dim3(256), 0, ctx().stream, probs,
                        labels, label_smoothing, dlogits, rows, K);
+    AETH_LAUNCH_CHECK();
+    return AETH_OK;
+}
+
+int aeth_softmax_cce_train_f32(const float* logits, const int32_t* labels, float label_smoothing, float* probs,
+                               float* sample_loss, int32_t* pred, float* dlogits, int rows, int K) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(logits && labels && probs && sample_loss && pred && dlogits && rows > 0 && K > 0);
+    AETH_CHECK_ARG((int64_t)rows * K < ((int64_t)1 << 31));
+    hipLaunchKernelGGL(softmax_cce_train_kernel, dim3(cdiv(rows, 64)), dim3(64), 0, ctx().stream, logits, labels,
+                       label_smoothing, probs, sample_loss, pred, dlogits, rows, K);
     AETH_LAUNCH_CHECK();
     return AETH_OK;
 }

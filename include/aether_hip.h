@@ -227,6 +227,10 @@ int aeth_cce_fwd_f32(const float* probs, const int32_t* labels, float label_smoo
  * dlogits = (probs - smooth(onehot)) / rows. */
 int aeth_softmax_cce_bwd_f32(const float* probs, const int32_t* labels, float label_smoothing,
                              float* dlogits, int rows, int K);
+/* The classifier head of a training step in one launch: SoftMax.forward :542-547, the loss and predictions of
+ * aeth_cce_fwd_f32 and the gradient of aeth_softmax_cce_bwd_f32, with their operations in their order (same bits). */
+int aeth_softmax_cce_train_f32(const float* logits, const int32_t* labels, float label_smoothing, float* probs,
+                               float* sample_loss, int32_t* pred, float* dlogits, int rows, int K);
 /* Optimizer_Adam.update_parameters for one tensor :702-734; t = iterations (0-based). */
 int aeth_adam_f32(float* theta, const float* grad, float* m, float* v, int64_t n,
                   float lr, float beta1, float beta2, float eps, int t);

@@ -295,6 +295,36 @@ def test_recorded_steps_equal_eager_steps():
     assert eager.train_step(Xs[0], ys[0]) == rec.train_step(Xs[0], ys[0])
 
 
+def test_classifier_head_in_one_launch_equals_the_three_launches(monkeypatch):
+    """A training step queues softmax, loss + predictions and the gradient of the logits as one launch
+    (AETHER_FUSE_HEAD=0: the three launches of the layers).  Same operations in the same order: the
+    steps must agree exactly, eager and recorded, and the layer attributes must be those of the step."""
+    import aether
+
+    def run(fuse, record):
+        monkeypatch.setenv("AETHER_FUSE_HEAD", fuse)
+        np.random.seed(3)
+        m = build_model(aether, label_smoothing=0.05, hw=16)
+        m.loss.new_pass()
+        m.accuracy.new_pass()
+        m.record_steps(record)
+        rng = np.random.RandomState(5)
+        out = []
+        for step in range(5):
+            X, y = rng.rand(32, 16, 16, 3).astype(np.float32), rng.randint(0, 10, 32)
+            out.append(m.train_step(X, y))
+        return out, np.asarray(m.layers[-1].output), np.asarray(m.layers[-1].dinputs), \
+            [np.asarray(l.weights) for l in m.trainable_layers]
+
+    ref = run("0", False)
+    for fuse, record in (("1", False), ("1", True)):
+        got = run(fuse, record)
+        assert got[0] == ref[0]
+        assert np.array_equal(got[1], ref[1]) and np.array_equal(got[2], ref[2])
+        for a, b in zip(got[3], ref[3]):
+            assert np.array_equal(a, b)
+
+
 def test_recorded_steps_survive_a_workspace_that_grows():
     """A recorded step has the address of the library's scratch workspace in its kernel
     arguments.  Eager work that needs a larger workspace after the recording was made
