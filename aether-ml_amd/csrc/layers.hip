@@ -682,6 +682,48 @@ __global__ void softmax_cce_train_kernel(const float* __restrict__ logits, const
     pred[r] = bi;
 }
 
+// The same for at most 16 classes with 16 lanes per row: the exponentials and logarithms of a row are worked out side by
+// side, the sums are added by the row's first lane in the order of the one-thread form (same bits).
+__global__ void softmax_cce_train16_kernel(const float* __restrict__ logits, const int32_t* __restrict__ labels, float ls,
+                                           float* __restrict__ probs, float* __restrict__ loss, int32_t* __restrict__ pred,
+                                           float* __restrict__ dlogits, int rows, int K) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    const int r = min(t >> 4, rows - 1), k = t & 15;     // (rows past the end repeat the last one: every lane takes part in the exchanges)
+    const bool mine = k < K;
+    const int base = (threadIdx.x & 63) & ~15;           // first lane of the row inside the wave
+    const float in = mine ? logits[(size_t)r * K + k] : 0.0f;
+    float mx = __shfl(in, base, 64);
+    for (int j = 1; j < K; ++j) mx = fmaxf(mx, __shfl(in, base + j, 64));
+    const float e = expf(in - mx);
+    float sum = 0.f;
+    for (int j = 0; j < K; ++j) sum += __shfl(e, base + j, 64);
+    const float v = e / sum;
+    const int y = labels[r];
+    const float t_off = ls / (float)K;
+    const float t_on = (1.0f - ls) + t_off;
+    const float tk = (k == y) ? t_on : t_off;
+    const float term = tk * logf(fminf(fmaxf(v, 1e-7f), 1.0f - 1e-7f));
+    float acc = 0.f, best = 0.f;
+    int bi = 0;
+    for (int j = 0; j < K; ++j) {
+        const float vj = __shfl(v, base + j, 64);
+        if (j == 0 || vj > best) {
+            best = vj;
+            bi = j;
+        }
+        acc += __shfl(term, base + j, 64);
+    }
+    if ((t >> 4) >= rows) return;
+    if (mine) {
+        probs[(size_t)r * K + k] = v;
+        dlogits[(size_t)r * K + k] = (v - tk) / (float)rows;
+    }
+    if (k == 0) {
+        loss[r] = -acc;
+        pred[r] = bi;
+    }
+}
+
 static int pool_dims(const char* fn, int S, int H, int W, int C, int fH, int fW, int sH, int sW, PoolParams* p) {
     if (S <= 0 || H <= 0 || W <= 0 || C <= 0 || fH <= 0 || fW <= 0 || sH <= 0 || sW <= 0)
         return fail(AETH_E_INVALID, "%s: non-positive dimension", fn);
@@ -1191,8 +1233,12 @@ int aeth_softmax_cce_train_f32(const float* logits, const int32_t* labels, float
     AETH_REQUIRE_INIT();
     AETH_CHECK_ARG(logits && labels && probs && sample_loss && pred && dlogits && rows > 0 && K > 0);
     AETH_CHECK_ARG((int64_t)rows * K < ((int64_t)1 << 31));
-    hipLaunchKernelGGL(softmax_cce_train_kernel, dim3(cdiv(rows, 64)), dim3(64), 0, ctx().stream, logits, labels,
-                       label_smoothing, probs, sample_loss, pred, dlogits, rows, K);
+    if (K <= 16 && (int64_t)rows * 16 < ((int64_t)1 << 31))
+        hipLaunchKernelGGL(softmax_cce_train16_kernel, dim3(cdiv((int64_t)rows * 16, 256)), dim3(256), 0, ctx().stream, logits,
+                           labels, label_smoothing, probs, sample_loss, pred, dlogits, rows, K);
+    else
+        hipLaunchKernelGGL(softmax_cce_train_kernel, dim3(cdiv(rows, 64)), dim3(64), 0, ctx().stream, logits, labels,
+                           label_smoothing, probs, sample_loss, pred, dlogits, rows, K);
     AETH_LAUNCH_CHECK();
     return AETH_OK;
 }
