@@ -754,6 +754,10 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma_bf16(const Wgr
 //   the four 64-byte quarters of the banks.  The loads are inline assembly so that the compiler
 //   does not order the LDS reads of a slab behind the loads of later slabs; the wave waits for
 //   its own loads of the slab with a partial vmcnt, the barrier covers the other waves'.
+//   dbias (column sums of dy) is one more MFMA on the dy operand, ones as the other operand,
+//   in the waves of the k tile 0: adding the columns with ordinary LDS reads made those
+//   workgroups end last (stride-2 layer 28x28x128 -> 256: 0.166 ms, 0.146 without dbias; the
+//   same with it now).
 // ------------------------------------------------------------------------------
 constexpr int kWwBR = 32;
 
@@ -866,8 +870,8 @@ static __global__ __launch_bounds__(128 * KW, KW == 4 ? 1 : (NB == 4 ? 2 : 3)) v
         a_eo[kb] = (((col >> 3) ^ sw) << 3) + (col & 4);
     }
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-        const int col = nw * 32 * NB + nb * 32 + 16 * (G & 1) + 4 * (j16 & 3);
+    for (int nb = 0; nb < NB; ++nb) {                    // the wave's block nb is n block (nb + kw) % NB of its half: see dbias
+        const int col = nw * 32 * NB + ((nb + kw) % NB) * 32 + 16 * (G & 1) + 4 * (j16 & 3);
         y_eo[nb] = (((col >> 3) ^ sw) << 3) + (col & 4);
     }
     auto tr = [&](const uint16_t* base) {
@@ -884,46 +888,56 @@ static __global__ __launch_bounds__(128 * KW, KW == 4 ? 1 : (NB == 4 ? 2 : 3)) v
             for (int v = 0; v < 16; ++v) acc[kb][nb][v] = 0.f;
     const bool active = kt0 + kw * 64 < p.K;             // wave-uniform
 
-    float dbsum = 0.f;                                   // thread t < BN sums column t of every dy slab
-    auto add_columns = [&](const uint16_t* ly) {
-        if (tid < BN) {
-#pragma unroll 8
-            for (int row = 0; row < BR; ++row) {
-                const int e = (((tid >> 3) ^ ((row & 3) << 2)) << 3) + (tid & 7);
-                dbsum += __uint_as_float((unsigned)ly[row * BN + e] << 16);
-            }
+    // dbias: the column sums of dy are one more product, a block of ones times the dy operand that the wave
+    // holds anyway (every row of the result is the sum; exact products, float32 sums).  Wave kw of the k tile 0
+    // takes the n blocks kw, kw + KW, ...: one MFMA more per eight, no reads of its own.  Those are the wave's
+    // blocks 0, KW, ... (its blocks are numbered from kw on), so no register is chosen at run time.
+    constexpr int DBN = (NB + KW - 1) / KW;
+    f16v acc_db[DBN];
+#pragma unroll
+    for (int j = 0; j < DBN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc_db[j][v] = 0.f;
+    const bool wave_db = do_db && kw < NB;
+    auto multiply_db = [&](const s8v* bv) {
+        const s8v ones = (s8v)(short)0x3F80;
+#pragma unroll
+        for (int j = 0; j < DBN; ++j) {
+            acc_db[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ones),
+                                                                __builtin_bit_cast(bf16x8, bv[j * KW]), acc_db[j], 0, 0, 0);
         }
     };
 
-    auto compute = [&](const uint16_t* la, const uint16_t* ly) {
-        if (do_db) add_columns(ly);
-        if (active) {
+    // operands of one 16-row step of a slab: 2 blocks of 32 k columns, NB blocks of 32 n columns
+    auto load_ops = [&](const uint16_t* la, const uint16_t* ly, int st, s8v* av, s8v* bv) {
+        const int r0 = st * 16 + t_row;
 #pragma unroll
-            for (int st = 0; st < BR / 16; ++st) {
-                const int r0 = st * 16 + t_row;
-                s8v av[2], bv[NB];
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb) {
-                    const s4v lo = tr(la + r0 * BK + a_eo[kb]);
-                    const s4v hi = tr(la + (r0 + 4) * BK + a_eo[kb]);
-                    av[kb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                }
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb) {
-                    const s4v lo = tr(ly + r0 * BN + y_eo[nb]);
-                    const s4v hi = tr(ly + (r0 + 4) * BN + y_eo[nb]);
-                    bv[nb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                }
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb) {
-                    acc[0][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av[0]),
-                                                                         __builtin_bit_cast(bf16x8, bv[nb]), acc[0][nb], 0, 0, 0);
-                    // (k rows past K were loaded as zeros: their products vanish without a branch between the MFMAs)
-                    acc[1][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av[1]),
-                                                                             __builtin_bit_cast(bf16x8, bv[nb]), acc[1][nb], 0, 0, 0);
-                }
-            }
+        for (int kb = 0; kb < 2; ++kb) {
+            const s4v lo = tr(la + r0 * BK + a_eo[kb]);
+            const s4v hi = tr(la + (r0 + 4) * BK + a_eo[kb]);
+            av[kb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         }
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const s4v lo = tr(ly + r0 * BN + y_eo[nb]);
+            const s4v hi = tr(ly + (r0 + 4) * BN + y_eo[nb]);
+            bv[nb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+    };
+    auto multiply = [&](const s8v* av, const s8v* bv) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            acc[0][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av[0]),
+                                                                 __builtin_bit_cast(bf16x8, bv[nb]), acc[0][nb], 0, 0, 0);
+            // (k rows past K were loaded as zeros: their products vanish without a branch between the MFMAs)
+            acc[1][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av[1]),
+                                                                 __builtin_bit_cast(bf16x8, bv[nb]), acc[1][nb], 0, 0, 0);
+        }
+    };
+    auto wait_behind = [&](int slabs_behind) {           // this wave's loads have landed, all but those of the newest slabs
+        if (RING >= 4 && slabs_behind >= 2) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * LOADS) : "memory");
+        else if (slabs_behind >= 1) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(LOADS) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     };
 
     // slab k of the split lives in buffer k % RING; its loads go out RING - 1 slabs earlier
@@ -933,16 +947,24 @@ static __global__ __launch_bounds__(128 * KW, KW == 4 ? 1 : (NB == 4 ? 2 : 3)) v
         if (k < nslab) issue(m_begin + k * BR, lds_a[k], lds_y[k]);
     int cur = 0;
     for (int k = 0; k < nslab; ++k) {
-        // this wave's loads of slab k have landed: everything but the loads of the slabs behind it (at most RING - 2)
-        const int behind = nslab - 1 - k;
-        if (RING >= 4 && behind >= 2) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * LOADS) : "memory");
-        else if (behind >= 1) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(LOADS) : "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();                                 // ... and so have the other waves'; slab k - 1 has been read by all
+        wait_behind(min(nslab - 1 - k, RING - 2));       // slab k has landed
+        __syncthreads();                                 // ... and so have the other waves' loads; slab k - 1 has been read by all
         int nxt = cur + RING - 1;
         if (nxt >= RING) nxt -= RING;
-        if (k + RING - 1 < nslab) issue(m_begin + (k + RING - 1) * BR, lds_a[nxt], lds_y[nxt]);
-        compute(lds_a[cur], lds_y[cur]);
+        // the two waves of a SIMD (nw = 0 and 1) take turns: one works out the addresses of its loads while
+        // the other multiplies
+        const bool more = k + RING - 1 < nslab;
+        if (more && nw == 0) issue(m_begin + (k + RING - 1) * BR, lds_a[nxt], lds_y[nxt]);
+        if (active || wave_db) {                         // (a wave past K that sums columns multiplies zeros)
+#pragma unroll
+            for (int st = 0; st < BR / 16; ++st) {
+                s8v av[2], bv[NB];
+                load_ops(lds_a[cur], lds_y[cur], st, av, bv);
+                multiply(av, bv);
+                if (wave_db) multiply_db(bv);
+            }
+        }
+        if (more && nw != 0) issue(m_begin + (k + RING - 1) * BR, lds_a[nxt], lds_y[nxt]);
         cur = cur + 1 == RING ? 0 : cur + 1;
     }
 
@@ -952,14 +974,20 @@ static __global__ __launch_bounds__(128 * KW, KW == 4 ? 1 : (NB == 4 ? 2 : 3)) v
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-            const int n = n0 + nw * 32 * NB + nb * 32 + l32;
+            const int n = n0 + nw * 32 * NB + ((nb + kw) % NB) * 32 + l32;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int k = kt0 + kw * 64 + kb * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
                 if (k < p.K && n < p.D) outp[(size_t)k * p.D + n] = acc[kb][nb][v];
             }
         }
-    if (do_db && tid < BN && n0 + tid < p.D) outp[(size_t)p.K * p.D + n0 + tid] = dbsum;
+    if (wave_db && lane < 32) {                          // row 0 of the sums: element 0 of the lanes 0..31
+#pragma unroll
+        for (int j = 0; j < DBN; ++j) {
+            const int n = n0 + nw * 32 * NB + (j * KW + kw) * 32 + lane;
+            if (n < p.D) outp[(size_t)p.K * p.D + n] = acc_db[j][0];
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------
