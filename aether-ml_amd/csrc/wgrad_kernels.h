@@ -827,6 +827,23 @@ static __global__ __launch_bounds__(128 * KW, KW == 4 ? 1 : (NB == 4 ? 2 : 3)) v
     const u32x4 rsrc_x = raw_rsrc(p.x, p.x_bytes);
     const u32x4 rsrc_y = raw_rsrc(p.dy, p.dy_bytes);
 
+    // The slabs are issued in order, so the image position of the pixel a load fetches moves by 32 rows of m from
+    // one call to the next: adds and two carries instead of two divisions per load (integer multiplies run at a
+    // quarter of the rate; with the waves of a SIMD taking turns this is worth about 1 %).
+    int xs_r[XLOADS], xs_c[XLOADS], xs_off[XLOADS];      // row, column (tap (0,0), no padding) and element offset of that pixel
+#pragma unroll
+    for (int i = 0; i < XLOADS; ++i) {
+        const int m = m_begin + (wave * XLOADS + i) * XROWS + x_row;
+        unsigned s, rem, ho, wo;
+        p.div_howo.divmod((unsigned)m, s, rem);
+        p.div_wo.divmod(rem, ho, wo);
+        xs_r[i] = (int)ho * p.sH;
+        xs_c[i] = (int)wo * p.sW;
+        xs_off[i] = (((int)s * p.H + xs_r[i]) * p.W + xs_c[i]) * p.C;
+    }
+    const int wrap_c = p.Wo * p.sW, wrap_r = p.Ho * p.sH;
+    const int inc0 = p.inc0 >> 2, inc1 = p.inc1 >> 2, inc2 = p.inc2 >> 2;   // the host counts them in bytes of float32
+
     auto issue = [&](int mb, uint16_t* la, uint16_t* ly) {
         const unsigned la_base = lds_address(la), ly_base = lds_address(ly);
 #pragma unroll
@@ -834,15 +851,17 @@ static __global__ __launch_bounds__(128 * KW, KW == 4 ? 1 : (NB == 4 ? 2 : 3)) v
             const int ld = wave * XLOADS + i;            // wave-level load number inside the slab
             const int q = XCLS == 1 ? 0 : (i & (XCLS - 1));          // (ld * XROWS) & 3 == XROWS * (i & (XCLS - 1)): XLOADS is even
             const int m = mb + ld * XROWS + x_row;
-            unsigned s, rem, ho, wo;
-            p.div_howo.divmod((unsigned)m, s, rem);
-            p.div_wo.divmod(rem, ho, wo);
-            const int r0 = (int)ho * p.sH, c0 = (int)wo * p.sW;
-            const int pix = (((int)s * p.H + r0) * p.W + c0) * p.C;
-            const unsigned bad = (unsigned)!((m < m_end) & a_kok[q] & ((unsigned)(r0 + a_fx[q]) < (unsigned)p.H) &
-                                             ((unsigned)(c0 + a_fy[q]) < (unsigned)p.W));
-            const unsigned voff = ((unsigned)(pix + a_tap_off[q]) * 2u) | (bad << 31);
+            const unsigned bad = (unsigned)!((m < m_end) & a_kok[q] & ((unsigned)(xs_r[i] + a_fx[q]) < (unsigned)p.H) &
+                                             ((unsigned)(xs_c[i] + a_fy[q]) < (unsigned)p.W));
+            const unsigned voff = ((unsigned)(xs_off[i] + a_tap_off[q]) * 2u) | (bad << 31);
             lds_direct_load16(rsrc_x, la_base + (unsigned)ld * 1024u, voff);
+            xs_c[i] += p.step_c;                         // m += BR
+            const bool c1 = xs_c[i] >= wrap_c;
+            xs_c[i] -= c1 ? wrap_c : 0;
+            xs_r[i] += c1 ? p.step_r + p.sH : p.step_r;
+            const bool c2 = xs_r[i] >= wrap_r;
+            xs_r[i] -= c2 ? wrap_r : 0;
+            xs_off[i] += (c1 ? inc0 + inc1 : inc0) + (c2 ? inc2 : 0);
         }
 #pragma unroll
         for (int i = 0; i < YLOADS; ++i) {
