@@ -1025,7 +1025,7 @@ static __global__ __launch_bounds__(128 * KW, KW == 4 ? 1 : (NB == 4 ? 2 : 3)) v
 // consecutive m of one k (or n) column per lane, while both tiles lie m-major in LDS:
 // `ds_read_b64_tr_b16` transposes on the way (see wgrad_gemm_dma_bf16); chunk q of a 128-byte row
 // is stored at q ^ (((row >> 1) & 1) << 2), row = slot number or dy row.
-// The loading wave also adds up the dy columns for dbias.  Partial results go to
+// dbias is one more MFMA (ones times the dy operand) in two of the waves.  Partial results go to
 // out + z * (K * D + D) like those of the other wgrad kernels.
 // ------------------------------------------------------------------------------
 struct WgradHaloParams {
@@ -1155,11 +1155,14 @@ static __global__ __launch_bounds__(64 * (kWhMaxTaps + 1), 1) void wgrad_halo_bf
             const int slot = (int)r * p.Wp + (int)wo + shift;
             offa[st][h] = slot * 64 + ((((col0 >> 3) ^ (((slot >> 1) & 1) << 2)) << 3) + (col0 & 4));
         }
-    int offb[2];                                                           // into a dy buffer, step 0 (n block 0; ^ 32: block 1)
+    // into a dy buffer, step 0: the wave's n block 0 (^ 32: its block 1).  Odd waves number the two blocks the other
+    // way round, so that the block a wave sums for dbias (below) is its block 0 whatever the wave.
+    const int nflip = wave & 1;
+    int offb[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
         const int row = tr_row + 4 * h;
-        offb[h] = row * 64 + ((((col0 >> 3) ^ (((row >> 1) & 1) << 2)) << 3) + (col0 & 4));
+        offb[h] = (row * 64 + ((((col0 >> 3) ^ (((row >> 1) & 1) << 2)) << 3) + (col0 & 4))) ^ (32 * nflip);
     }
     f16v acc[2][2];
 #pragma unroll
@@ -1172,25 +1175,22 @@ static __global__ __launch_bounds__(64 * (kWhMaxTaps + 1), 1) void wgrad_halo_bf
     auto tr = [&](const uint16_t* q) __attribute__((always_inline)) {
         return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr_t)q);
     };
-    // dbias: wave t adds up the dy rows of the 8-row groups t, t + T, ... of every slab; a lane takes one
-    // chunk position (8 columns) of row lrow of those groups
-    const int lrow = lane >> 3;
-    float db[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // dbias: the column sums of dy are one more product, ones times the dy operand a wave holds anyway (every row
+    // of the result is the sum).  Two waves take one n block each, on SIMDs that carry two multiplying waves where
+    // another carries three (waves 2 and 3 of a 3x3 filter's nine); a lone wave takes both blocks.
+    const int db_first = T >= 4 ? 2 : 0;
+    const bool db_one = p.want_dbias && (wave == db_first || (T >= 2 && wave == db_first + 1));
+    const bool db_two = p.want_dbias && T == 1;
+    f16v acc_db;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc_db[v] = 0.f;
+    // (the lone wave: ones in the rows 0..15 for block 0 and in the rows 16..31 for block 1, one set of accumulators)
+    const s8v ones0 = (s8v)(short)(db_two && l32 >= 16 ? 0 : 0x3F80);
+    const s8v ones1 = (s8v)(short)(l32 >= 16 ? 0x3F80 : 0);
     asm volatile("s_barrier" ::: "memory");
     for (int t = 0; t < nsl; ++t) {
         const uint16_t* hb = halo[t & 1];
         const uint16_t* yb = dyb[t & 1];
-        if (p.want_dbias) {
-            for (int j = wave; 8 * j < p.slab_m; j += T) {
-                const f4 v = reinterpret_cast<const f4*>(yb)[(8 * j + lrow) * 8 + (lane & 7)];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const unsigned u = __float_as_uint(v[e]);
-                    db[2 * e] += __uint_as_float(u << 16);
-                    db[2 * e + 1] += __uint_as_float(u & 0xffff0000u);
-                }
-            }
-        }
         // the operands of step st + 1 are read while the four MFMAs of step st run
         s8v a[2][2], b[2][2];
         auto read_step = [&](int st, s8v (&ra)[2], s8v (&rb)[2]) __attribute__((always_inline)) {
@@ -1215,30 +1215,27 @@ static __global__ __launch_bounds__(64 * (kWhMaxTaps + 1), 1) void wgrad_halo_bf
                         acc[kb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[st & 1][kb]),
                                                                               __builtin_bit_cast(bf16x8, b[st & 1][nb]),
                                                                               acc[kb][nb], 0, 0, 0);
+                if (db_one || db_two)
+                    acc_db = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ones0),
+                                                                     __builtin_bit_cast(bf16x8, b[st & 1][0]), acc_db, 0, 0, 0);
+                if (db_two)
+                    acc_db = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ones1),
+                                                                     __builtin_bit_cast(bf16x8, b[st & 1][1]), acc_db, 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
         asm volatile("s_barrier" ::: "memory");
     }
-    if (p.want_dbias) {
-        // everyone is past the last barrier of the loop: the first halo buffer is free.  Row lrow of wave
-        // t holds its sums by logical chunk: the position with bit 2 flipped for rows whose bit 1 is set.
-        float* red = reinterpret_cast<float*>(&halo[0][0]);
-        const int lc = (lane & 7) ^ (((lrow >> 1) & 1) << 2);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) red[(wave * 8 + lrow) * 64 + 8 * lc + e] = db[e];
-        __syncthreads();
-        if (wave == 0 && lane < p.D) {
-            float sum = 0.f;
-            for (int r = 0; r < 8 * T; ++r) sum += red[r * 64 + lane];
-            outp[(size_t)K * p.D + lane] = sum;
-        }
+    if ((db_one || db_two) && lane < 32) {               // row 0 of the sums: element 0 of the lanes 0..31
+        const int n = 32 * nflip + lane;                 // the wave's block 0
+        if (n < p.D) outp[(size_t)K * p.D + n] = acc_db[0];
+        if (db_two && 32 + lane < p.D) outp[(size_t)K * p.D + 32 + lane] = acc_db[8];       // row 16
     }
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) {
-            const int n = 32 * nb + l32;
+            const int n = 32 * (nb ^ nflip) + l32;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int k = wave * 64 + 32 * kb + 8 * (v >> 2) + 4 * lh + (v & 3);
