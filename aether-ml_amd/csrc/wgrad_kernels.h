@@ -581,7 +581,6 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma_bf16(const Wgr
     __shared__ uint16_t lds_a1[BR * kWgBK];
     __shared__ uint16_t lds_y0[BR * kWgBN];
     __shared__ uint16_t lds_y1[BR * kWgBN];
-    __shared__ float lds_db[4 * 64];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -661,8 +660,10 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma_bf16(const Wgr
     const int y_col = 16 * (G & 1) + 4 * (j16 & 3);                  // first n element (n tile 0; +32: tile 1)
     // element offsets (in bf16) inside a slab row, swizzle applied; row & 3 == j16 >> 2, (row >> 1) & 1 == j16 >> 3
     const int a_eo = (((a_col >> 3) ^ ((j16 >> 2) << 1)) << 3) + (a_col & 4);
-    const int y_eo0 = (((y_col >> 3) ^ ((j16 >> 3) << 2)) << 3) + (y_col & 4);
-    const int y_eo1 = ((((y_col + 32) >> 3) ^ ((j16 >> 3) << 2)) << 3) + (y_col & 4);
+    // (odd waves number the two n blocks the other way round: the block a wave sums for dbias is then its block 0)
+    const int nflip = wave & 1;
+    const int y_eo0 = ((((y_col + 32 * nflip) >> 3) ^ ((j16 >> 3) << 2)) << 3) + (y_col & 4);
+    const int y_eo1 = ((((y_col + 32 - 32 * nflip) >> 3) ^ ((j16 >> 3) << 2)) << 3) + (y_col & 4);
     auto tr = [&](const uint16_t* base) {
         return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr_t)base);
     };
@@ -674,23 +675,21 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma_bf16(const Wgr
         for (int v = 0; v < 16; ++v) acc[jn][v] = 0.f;
     const bool active = kt0 + wave * 32 < p.K;           // wave-uniform
 
-    float dbsum = 0.f;
-    const int db_col = tid & 63, db_rg = tid >> 6;       // 4 row groups of 16 rows
-    auto add_columns = [&](const uint16_t* ly) {
+    // dbias: the column sums of dy are one more product, ones times the dy operand the wave holds anyway (every
+    // row of the result is the sum); waves 0 and 1 of the k tile 0 take one n block each.  (Adding the columns
+    // with 16 two-byte LDS reads per thread and slab made the workgroups of that tile end last.)
+    const bool wave_db = do_db && wave < 2;
+    f16v acc_db;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int row = db_rg * 16 + r;
-            const int e = (((db_col >> 3) ^ (((row >> 1) & 1) << 2)) << 3) + (db_col & 7);
-            dbsum += __uint_as_float((unsigned)ly[row * kWgBN + e] << 16);
-        }
-    };
+    for (int v = 0; v < 16; ++v) acc_db[v] = 0.f;
+    typedef short s8v __attribute__((ext_vector_type(8)));
+    const s8v ones = (s8v)(short)0x3F80;
 
     auto slab = [&](int mb, const uint16_t* la, const uint16_t* ly, uint16_t* na, uint16_t* ny, bool has_next) {
         __builtin_amdgcn_s_waitcnt(0);                   // this wave's loads of the slab have landed
         __syncthreads();
         if (has_next) issue(mb + BR, na, ny);
-        if (do_db) add_columns(ly);
-        if (active) {
+        if (active || wave_db) {                         // (a wave past K that sums columns multiplies zeros)
 #pragma unroll
             for (int st = 0; st < BR / 16; ++st) {
                 const int r0 = st * 16 + t_row;
@@ -700,7 +699,6 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma_bf16(const Wgr
                 s4v b01 = tr(ly + (r0 + 4) * kWgBN + y_eo0);
                 s4v b10 = tr(ly + r0 * kWgBN + y_eo1);
                 s4v b11 = tr(ly + (r0 + 4) * kWgBN + y_eo1);
-                typedef short s8v __attribute__((ext_vector_type(8)));
                 const s8v av = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
                 const s8v bv0 = __builtin_shufflevector(b00, b01, 0, 1, 2, 3, 4, 5, 6, 7);
                 const s8v bv1 = __builtin_shufflevector(b10, b11, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -708,6 +706,9 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma_bf16(const Wgr
                                                                  __builtin_bit_cast(bf16x8, bv0), acc[0], 0, 0, 0);
                 acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av),
                                                                  __builtin_bit_cast(bf16x8, bv1), acc[1], 0, 0, 0);
+                if (wave_db)
+                    acc_db = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ones),
+                                                                     __builtin_bit_cast(bf16x8, bv0), acc_db, 0, 0, 0);
             }
         }
     };
@@ -722,18 +723,16 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma_bf16(const Wgr
     float* outp = p.out + (size_t)split * split_stride;
 #pragma unroll
     for (int jn = 0; jn < 2; ++jn) {
-        const int n = n0 + 32 * jn + l32;
+        const int n = n0 + 32 * (jn ^ nflip) + l32;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int k = kt0 + wave * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
             if (k < p.K && n < p.D) outp[(size_t)k * p.D + n] = acc[jn][v];
         }
     }
-    if (do_db) {
-        lds_db[db_rg * 64 + db_col] = dbsum;
-        __syncthreads();
-        if (tid < 64 && n0 + tid < p.D)
-            outp[(size_t)p.K * p.D + n0 + tid] = (lds_db[tid] + lds_db[64 + tid]) + (lds_db[128 + tid] + lds_db[192 + tid]);
+    if (wave_db && lane < 32) {                          // row 0 of the sums: element 0 of the lanes 0..31
+        const int n = n0 + 32 * nflip + lane;
+        if (n < p.D) outp[(size_t)p.K * p.D + n] = acc_db[0];
     }
 }
 
