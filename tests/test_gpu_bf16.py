@@ -28,6 +28,9 @@ CASES = [
     (5, 28, 28, 1, 32, 3, 3, 1, 1, "same"),       # direct kernels on bf16 inputs
     (3, 12, 12, 2, 16, 5, 5, 2, 2, "same"),       # 5x5 on 2 channels: not built, gather kernels
     (2, 11, 13, 3, 64, 5, 5, 1, 1, "same"),
+    (3, 10, 10, 16, 48, 1, 1, 1, 1, "valid"),     # K = 16: wgrad waves past K still sum their dbias columns
+    (2, 9, 9, 32, 64, 1, 1, 1, 1, "valid"),       # K = 32
+    (2, 9, 9, 8, 24, 1, 1, 1, 1, "valid"),
 ]
 
 
@@ -256,6 +259,9 @@ WGRAD_HALO_CASES = [
     (24, 56, 56, 64, 64, 3, 3, 1, 1, "same"),     # 672 slabs on 224 workgroups of 3
     (2, 14, 14, 64, 64, 3, 3, 1, 1, "same"),      # 8 rows of 14 would make a slab, but 8 does not divide 14: other kernel
     (2, 16, 16, 128, 64, 3, 3, 1, 1, "same"),     # 128 input channels: other kernel
+    (2, 16, 16, 64, 64, 1, 1, 1, 1, "valid"),     # one tap: the lone multiplying wave sums both column blocks for dbias
+    (2, 16, 16, 64, 40, 1, 1, 1, 1, "valid"),     # ... the second block partly filled
+    (2, 8, 33, 64, 24, 1, 2, 1, 1, "valid"),      # two taps, 24 columns: the second block's sums are never stored
 ]
 
 
