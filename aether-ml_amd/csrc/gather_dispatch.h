@@ -131,7 +131,11 @@ static bool plan_halo(GatherParams& gp, bool dma, int* mtiles, int* stages, int 
     if (taps < min_taps || taps > 32 || gp.N <= 32 || gp.Cs <= 0 || gp.K != taps * gp.Cs) return false;
     if (tuning().gather_halo == 0) return false;
     const int hw = gp.Hg * gp.Wg;
-    const int wp = gp.Wg + gp.Tw - 1, hp = gp.Hg + gp.Th - 1;
+    // row pitch and image pitch of the padded tensor keep the parity of the pixel grid's (one idle slot per row or
+    // image for even filter sizes): the kernel places a slot's chunks by the number of the pixel it serves
+    int wp = gp.Wg + gp.Tw - 1, hp = gp.Hg + gp.Th - 1;
+    if ((wp - gp.Wg) & 1) ++wp;
+    if ((gp.Wg & 1) && ((hp - gp.Hg) & 1)) ++hp;
     if ((int64_t)gp.S * hp * wp >= ((int64_t)1 << 30)) return false;
     auto slot0 = [&](int64_t m) {
         const int64_t s = m / hw, rem = m % hw;
@@ -183,7 +187,9 @@ static bool plan_halo_res(GatherParams& gp, bool dma, int cus, int* mtiles) {
     const bool force = tuning().gather_res > 0;
     if (gp.Wg <= 0 || kResBM % gp.Wg != 0) return false;
     const int hw = gp.Hg * gp.Wg;
-    const int wp = gp.Wg + gp.Tw - 1, hp = gp.Hg + gp.Th - 1;
+    int wp = gp.Wg + gp.Tw - 1;                                          // row pitch of the halo: the parity of the pixel rows'
+    if ((wp - gp.Wg) & 1) ++wp;                                          // (chunks are placed by pixel number, see the kernel)
+    const int hp = gp.Hg + gp.Th - 1;
     const int rows = kResBM / gp.Wg;                                     // image rows per tile
     if ((int64_t)(rows + gp.Th - 1) * wp > kResSlots) return false;      // the tile's rows and the halo below them
     const int per_img = cdiv(hw, kResBM);
@@ -294,7 +300,12 @@ static bool plan_class_pairs(const std::vector<GatherSetup>& sets, GatherClasses
         htw = std::max(htw, gs.gp.rw0 - rw_min + gs.gp.Tw);
     }
     const int hw = g0.Hg * g0.Wg;
-    const int wp = g0.Wg + htw - 1, hp = g0.Hg + hth - 1;
+    // The padded tensor's row pitch and image pitch keep the parity of the pixel grid's (one idle slot per row or
+    // image where needed): a slot's number and the number of the pixel it serves under a tap then differ by an
+    // even amount, which is what lets the kernel place chunks by pixel number (no bank conflicts at row ends).
+    int wp = g0.Wg + htw - 1, hp = g0.Hg + hth - 1;
+    if ((wp - g0.Wg) & 1) ++wp;
+    if ((g0.Wg & 1) && ((hp - g0.Hg) & 1)) ++hp;
     if ((int64_t)g0.S * hp * wp >= ((int64_t)1 << 30)) return false;
     auto slot0 = [&](int64_t m) {
         const int64_t s = m / hw, rem = m % hw;

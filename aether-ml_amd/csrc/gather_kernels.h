@@ -641,8 +641,8 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
 //     that does not fit (56x56: 500), tiles are cut per image and an image's last tile
 //     is partly empty: taken when that costs at most 10 % of the rows; else tiles run
 //     over all of M if every span fits; else gather_gemm_dma runs.
-//   * slot s keeps logical 16-byte chunk c at position c ^ ((s >> 1) & 7), like the
-//     slab rows of gather_gemm_dma: 16 consecutive pixels cover the 64 banks once;
+//   * a slot keeps logical 16-byte chunk c at position c ^ key, key from the number of the pixel it serves
+//     (see the slot table below): 16 consecutive pixels cover the 64 banks once under every tap, row ends included;
 //   * channel blocks beyond the first reload the halo (Cs = 64 j: j passes over the taps).
 // ------------------------------------------------------------------------------
 // STAGES ring buffers of 8 KB and the rest of 80 KB (two workgroups per CU) for the halo:
@@ -717,29 +717,40 @@ static __device__ __forceinline__ void halo_tile_bf16(const GatherParams& p, con
     // slot -> byte offset of the pixel's channel 0 (bit 31: padding or past the span), one slot per
     // thread, through LDS to the lanes that fetch it.  The table sits in the last ring buffer, which
     // the filter loads reach after the first barrier of the loop.
+    // Where a slot keeps its 16-byte chunks: chunk c at position c ^ key, key = bits 1..3 of the NUMBER OF THE PIXEL
+    // the slot would be under tap (0, 0), v = (s Hg + row) Wg + column.  The 16 lanes of an operand read serve 16
+    // consecutive pixels, and under any tap their slots have consecutive v, also across a row end, where the slot
+    // numbers jump: parity (the slot's half of the banks; v and the slot number differ by an even amount, see the
+    // host's choice of the pitches) and key are those of 16 consecutive numbers, all different.  (Keyed by the slot
+    // number, rows of 14 pixels gave every read a pair of lanes 16 slots apart: 29 % of the LDS cycles were conflicts.)
     int* tab = reinterpret_cast<int*>(ring_last);
+    int* tabkey = tab + kHaloSlots;
+    static_assert(2 * kHaloSlots * sizeof(int) <= sizeof(ring2), "slot tables fit a ring buffer");
     for (int sl = tid; sl < kHaloSlots; sl += kThreads) {
         unsigned rg, cc, s_, rr;
         p.div_halo_wp.divmod((unsigned)(lfirst + sl), rg, cc);
         p.div_halo_hp.divmod(rg, s_, rr);
         const int srow = (int)rr + p.rh0, scol = (int)cc + p.rw0;
-        const bool ok = sl < span && (unsigned)srow < (unsigned)p.Hs && (unsigned)scol < (unsigned)p.Ws && (int)s_ < p.S;
+        const bool ok = sl < span && (unsigned)srow < (unsigned)p.Hs && (unsigned)scol < (unsigned)p.Ws && (int)s_ < p.S &&
+                        (int)rr < p.Hg + p.Th - 1 && (int)cc < p.Wg + p.Tw - 1;                  // (not the idle slots of the pitch)
         const unsigned off = (unsigned)((((int)s_ * p.Hs + srow) * p.Ws + scol) * p.Cs) * 2u;
         tab[sl] = (int)(ok ? off : 0x80000000u);
+        tabkey[sl] = ((((int)s_ * p.Hg + (int)rr) * p.Wg + (int)cc) >> 1) & 7;
     }
     __syncthreads();
     unsigned hoff[HL];
 #pragma unroll
     for (int k = 0; k < HL; ++k) {
         const int sl = (wave * HL + k) * 8 + (lane >> 3);
-        hoff[k] = (unsigned)tab[sl] + (unsigned)((((lane & 7) ^ (sl >> 1)) & 7) * 16);
+        hoff[k] = (unsigned)tab[sl] + (unsigned)((((lane & 7) ^ tabkey[sl]) & 7) * 16);
     }
-    // slot of tap (0,0) for the pixels this lane multiplies (rows past the end: slot 0, never stored)
-    int pslot[TM];
+    // slot of tap (0,0) for the pixels this lane multiplies (rows past the end: slot 0, never stored), and their numbers
+    int pslot[TM], pnum[TM];
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int m = m0 + wm0 + 32 * i + l32;
         pslot[i] = m < m_end ? slot0(m) - lfirst : 0;
+        pnum[i] = m < m_end ? m : m0;
     }
     // filter slab loads: as in gather_gemm_dma (rows of 8 chunks, chunk c of row r at c ^ ((r >> 1) & 7))
     const int k4e = (lane & 7) ^ (lane >> 4);
@@ -803,12 +814,12 @@ static __device__ __forceinline__ void halo_tile_bf16(const GatherParams& p, con
             asm volatile("s_barrier" ::: "memory");
         }
         load_filter(pf_next(), nb);
-        const int shift = th * Wp + tw;
+        const int shift = th * Wp + tw, tapv = th * p.Wg + tw;
         int x0[TM];
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             const int sl = pslot[i] + shift;
-            x0[i] = sl * 8 + ((lh ^ (sl >> 1)) & 7);
+            x0[i] = sl * 8 + ((lh ^ ((pnum[i] + tapv) >> 1)) & 7);
         }
         // all operand reads of the step go out at once (64 registers): with a read-ahead of one
         // k group the MFMAs of every group waited for LDS, whose queue under 8 waves of 16-byte
@@ -921,28 +932,39 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_pairs_bf16(con
 
     const int lfirst = slot0(m0);
     const int span = slot0(min(m0 + BM, m_end) - 1) + (p0.halo_th - 1) * Wp + p0.halo_tw - lfirst;   // <= kHaloSlots, checked by the host
+    // Where a slot keeps its 16-byte chunks: chunk c at position c ^ key, key = bits 1..3 of the NUMBER OF THE PIXEL
+    // the slot would be under tap (0, 0), v = (s Hg + row) Wg + column.  The 16 lanes of an operand read serve 16
+    // consecutive pixels, and under any tap their slots have consecutive v, also across a row end, where the slot
+    // numbers jump: parity (the slot's half of the banks; v and the slot number differ by an even amount, see the
+    // host) and key are those of 16 consecutive numbers, all different.  (Keyed by the slot number, rows of 14
+    // pixels gave every read a pair of lanes 16 slots apart: 29 % of the LDS cycles were conflicts.)
     int* tab = reinterpret_cast<int*>(&ring[STAGES - 1][0]);             // the filter loads reach it after the first barrier of the loop
+    int* tabkey = tab + kHaloSlots;
+    static_assert(2 * kHaloSlots * sizeof(int) <= sizeof(ring[0]), "slot tables fit a ring buffer");
     for (int sl = tid; sl < kHaloSlots; sl += kThreads) {
         unsigned rg, cc, s_, rr;
         p0.div_halo_wp.divmod((unsigned)(lfirst + sl), rg, cc);
         p0.div_halo_hp.divmod(rg, s_, rr);
         const int srow = (int)rr + p0.rh0, scol = (int)cc + p0.rw0;
-        const bool ok = sl < span && (unsigned)srow < (unsigned)p0.Hs && (unsigned)scol < (unsigned)p0.Ws && (int)s_ < p0.S;
+        const bool ok = sl < span && (unsigned)srow < (unsigned)p0.Hs && (unsigned)scol < (unsigned)p0.Ws && (int)s_ < p0.S &&
+                        (int)rr < p0.Hg + p0.halo_th - 1 && (int)cc < p0.Wg + p0.halo_tw - 1;    // (not the idle slots of the pitch)
         const unsigned off = (unsigned)((((int)s_ * p0.Hs + srow) * p0.Ws + scol) * p0.Cs) * 2u;
         tab[sl] = (int)(ok ? off : 0x80000000u);
+        tabkey[sl] = ((((int)s_ * p0.Hg + (int)rr) * p0.Wg + (int)cc) >> 1) & 7;
     }
     __syncthreads();
     unsigned hoff[HL];
 #pragma unroll
     for (int k = 0; k < HL; ++k) {
         const int sl = (wave * HL + k) * 8 + (lane >> 3);
-        hoff[k] = (unsigned)tab[sl] + (unsigned)((((lane & 7) ^ (sl >> 1)) & 7) * 16);
+        hoff[k] = (unsigned)tab[sl] + (unsigned)((((lane & 7) ^ tabkey[sl]) & 7) * 16);
     }
-    int pslot[TM];
+    int pslot[TM], pnum[TM];
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int m = m0 + wm0 + 32 * i + l32;
         pslot[i] = m < m_end ? slot0(m) - lfirst : 0;
+        pnum[i] = m < m_end ? m : m0;                    // (a row past the end reads slot 0, whose key is that of pixel m0)
     }
     // filter slab loads: rows of 8 chunks, chunk c of row r at c ^ ((r >> 1) & 7); the filter itself, rows n of bt_ld elements
     const int k4e = (lane & 7) ^ (lane >> 4);
@@ -1000,7 +1022,7 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_pairs_bf16(con
 
     const int sw7 = (l32 >> 1) & 7;
     int u = 0;
-    auto step = [&](int shift, f16v (&a)[TM][TN], bool new_block, int cb) __attribute__((always_inline)) {
+    auto step = [&](int shift, int tapv, f16v (&a)[TM][TN], bool new_block, int cb) __attribute__((always_inline)) {
         // loads complete in the order of issue (no stores are pending here): all but the younger filter slabs (two loads each)
         __builtin_amdgcn_s_waitcnt((2 * (STAGES - 2)) | (7 << 4) | (15 << 8));
         asm volatile("s_barrier" ::: "memory");
@@ -1017,7 +1039,7 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_pairs_bf16(con
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             const int sl = pslot[i] + shift;
-            x0[i] = sl * 8 + ((lh ^ (sl >> 1)) & 7);
+            x0[i] = sl * 8 + ((lh ^ ((pnum[i] + tapv) >> 1)) & 7);
         }
         f4 fa[4][TM], fb[4][TN];
 #pragma unroll
@@ -1039,17 +1061,17 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_pairs_bf16(con
     for (int cb = 0; cb < ncb; ++cb) {
         bool first = cb > 0;
         {
-            const int shift0 = pa.tap_dh * Wp + pa.tap_dw;
+            const int shift0 = pa.tap_dh * Wp + pa.tap_dw, v0 = pa.tap_dh * p0.Wg + pa.tap_dw;
             for (int th = 0; th < pa.Th; ++th)
                 for (int tw = 0; tw < pa.Tw; ++tw) {
-                    step(shift0 + th * Wp + tw, acc[0], first, cb);
+                    step(shift0 + th * Wp + tw, v0 + th * p0.Wg + tw, acc[0], first, cb);
                     first = false;
                 }
         }
         {
-            const int shift0 = pb.tap_dh * Wp + pb.tap_dw;
+            const int shift0 = pb.tap_dh * Wp + pb.tap_dw, v0 = pb.tap_dh * p0.Wg + pb.tap_dw;
             for (int th = 0; th < pb.Th; ++th)
-                for (int tw = 0; tw < pb.Tw; ++tw) step(shift0 + th * Wp + tw, acc[1], false, cb);
+                for (int tw = 0; tw < pb.Tw; ++tw) step(shift0 + th * Wp + tw, v0 + th * p0.Wg + tw, acc[1], false, cb);
         }
     }
     (void)nsteps;
@@ -1177,8 +1199,12 @@ static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(co
             const int sl = i * 8 + lslot;
             unsigned r, c;
             p.div_halo_wp.divmod((unsigned)sl, r, c);
-            rel[i] = ((int)r * p.Ws + (int)c) * 128 + (((lane & 7) ^ (sl >> 1)) & 7) * 16;
-            const unsigned bad = (unsigned)((int)c + p.rw0) >= (unsigned)p.Ws ? 1u : 0u;
+            // chunk q of the slot sits at q ^ key, key from the number of the pixel the slot is under tap (0, 0), counted
+            // from the tile's first pixel: the 16 lanes of an operand read serve 16 consecutive pixels, whose slots under
+            // any tap have consecutive such numbers also where the slot numbers jump at a row end (see halo_tile_bf16)
+            const int key = (((int)r * p.Wg + (int)c) >> 1) & 7;
+            rel[i] = ((int)r * p.Ws + (int)c) * 128 + (((lane & 7) ^ key) & 7) * 16;
+            const unsigned bad = ((unsigned)((int)c + p.rw0) >= (unsigned)p.Ws || (int)c >= p.Wg + p.Tw - 1) ? 1u : 0u;
             if (i < 32) colbad_lo |= bad << i;
             else colbad_hi |= bad << (i - 32);
         }
@@ -1248,7 +1274,7 @@ static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(co
         f4 fa[2][4], fb[2][4][TN];
         auto read_tap = [&](int tap, f4 (&ra)[4], f4 (&rb)[4][TN]) __attribute__((always_inline)) {
             const int sl = pslot + th * Wp + tw;
-            const int x0 = sl * 8 + ((lh ^ (sl >> 1)) & 7);
+            const int x0 = sl * 8 + ((lh ^ ((wave * 32 + l32 + th * p.Wg + tw) >> 1)) & 7);
             const f4* lb = filt + tap * (BN * KC);
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
