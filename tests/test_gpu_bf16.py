@@ -112,6 +112,9 @@ HALO_CASES = [
     (2, 31, 31, 64, 64, 3, 3, 2, 2, "valid"),     # stride 2: the dgrad class of 2x2 taps on a 16x16 grid
     (2, 16, 16, 64, 64, 3, 5, 1, 1, "same"),      # 3x5 filter, pad 1 on both axes: columns lose their border
     (1, 16, 16, 64, 64, 5, 5, 1, 1, "same"),      # 25 taps: span too long for the buffer, the slab kernel runs
+    (2, 15, 15, 64, 64, 2, 2, 1, 1, "valid"),     # even filter on an odd grid (dgrad): the halo's row and image pitches get an idle slot
+    (2, 13, 13, 64, 64, 4, 4, 1, 1, "same"),      # 4x4 on 13x13
+    (3, 14, 14, 128, 64, 3, 3, 1, 1, "same"),     # rows of 14: every 16-lane read group crosses a row end
 ]
 
 
@@ -329,6 +332,8 @@ MERGE_CASES = [
     (4, 16, 16, 96, 128, 3, 3, 2, 1, "same"),     # two classes (one pair) and 96 channels of dx
     (3, 12, 18, 72, 64, 5, 5, 2, 2, "same"),      # 9, 6, 6 and 4 taps on 72 channels of dx: windows of 3 x 3 in the common halo
     (2, 24, 24, 128, 128, 4, 4, 2, 2, "valid"),   # 4 taps in every class
+    (2, 18, 14, 64, 64, 3, 3, 2, 2, "valid"),     # class grids of 9 x 7 pixels, windows of 2 x 2: odd widths, both pitches padded
+    (3, 10, 22, 128, 64, 4, 4, 2, 2, "valid"),    # class grids of 5 x 11
 ]
 
 
