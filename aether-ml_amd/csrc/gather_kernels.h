@@ -1570,7 +1570,10 @@ __device__ __forceinline__ void direct_load_filter(const DirectParams& p, float*
 
 // FH, FW, C are compile-time so that the taps unroll and their loads go out together; the
 // filter takes as much LDS as it has floats (dynamic), so that a CU holds 8 workgroups.
-template <typename T, int FH, int FW, int C>
+// CPT = output channels per lane, 4, 8 or 16: the pixel's position, its FH*FW*C source values and their bounds tests are
+// worked out per lane, so with 4 channels a lane spends more instructions on them than on its 4 FH FW C multiply-adds;
+// the host picks CPT from the filter size.  The sums run over k in the same order whatever CPT: same bits.
+template <typename T, int FH, int FW, int C, int CPT = 4>
 static __global__ __launch_bounds__(kThreads) void direct_fprop_smallc(const DirectParams p) {
     extern __shared__ __attribute__((aligned(16))) float wl[];
     direct_load_filter<T>(p, wl);
@@ -1582,8 +1585,12 @@ static __global__ __launch_bounds__(kThreads) void direct_fprop_smallc(const Dir
     unsigned s_, rem, ho, wo;
     p.div_hw.divmod((unsigned)m, s_, rem);
     p.div_w.divmod(rem, ho, wo);
-    f4 acc = p.bias != nullptr ? *reinterpret_cast<const f4*>(p.bias + 4 * q) : f4{0.f, 0.f, 0.f, 0.f};
-    const float* wq = wl + 4 * q;
+    constexpr int NV = CPT / 4;
+    f4 acc[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+        acc[v] = p.bias != nullptr ? *reinterpret_cast<const f4*>(p.bias + CPT * q + 4 * v) : f4{0.f, 0.f, 0.f, 0.f};
+    const float* wq = wl + CPT * q;
     float xv[FH * FW * C];
 #pragma unroll
     for (int fx = 0; fx < FH; ++fx)
@@ -1598,11 +1605,15 @@ static __global__ __launch_bounds__(kThreads) void direct_fprop_smallc(const Dir
         }
 #pragma unroll
     for (int k = 0; k < FH * FW * C; ++k) {
-        const f4 wv = *reinterpret_cast<const f4*>(wq + k * p.D);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[e] = fmaf(xv[k], wv[e], acc[e]);
+        for (int v = 0; v < NV; ++v) {
+            const f4 wv = *reinterpret_cast<const f4*>(wq + k * p.D + 4 * v);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[v][e] = fmaf(xv[k], wv[e], acc[v][e]);
+        }
     }
-    *reinterpret_cast<f4*>(p.out + (size_t)m * p.D + 4 * q) = acc;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) *reinterpret_cast<f4*>(p.out + (size_t)m * p.D + CPT * q + 4 * v) = acc[v];
 }
 
 template <typename T, int FH, int FW, int C>

@@ -228,6 +228,29 @@ def test_fprop_with_the_filter_resident_in_lds(case, tune):
     assert np.array_equal(got, abi.fprop(x, w, b, stride, pad))
 
 
+# The direct kernels' fprop gives a lane 8 output channels (16 for 5x5 filters on 2 or 3 channels), 4 with direct = 2:
+# the same sums in the same order.
+DIRECT_CASES = [
+    (5, 28, 28, 1, 32, 3, 3, 1, 1, "same"),
+    (3, 12, 12, 2, 16, 3, 3, 2, 2, "same"),      # 16 output channels: two lanes per pixel
+    (2, 11, 13, 3, 64, 5, 5, 1, 1, "same"),      # 75 values per channel: 16 per lane
+    (2, 9, 9, 3, 256, 3, 3, 1, 1, "valid"),
+    (3, 10, 10, 1, 32, 5, 5, 3, 2, "valid"),
+    (40, 16, 16, 3, 32, 3, 3, 1, 1, "same"),
+]
+
+
+@pytest.mark.parametrize("case", DIRECT_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_direct_fprop_with_more_channels_per_lane(case, tune):
+    from tests import abi
+    x, w, b, dy = _case(case, 31)
+    stride, pad = (case[7], case[8]), case[9]
+    got = abi.fprop(x, w, b, stride, pad)
+    abi.close(got, O.conv_fprop(x, w, b, stride, pad, dtype=np.float64))
+    tune(direct=2)
+    assert np.array_equal(got, abi.fprop(x, w, b, stride, pad))
+
+
 # fp32 gathers whose slabs lie inside one tap load with addresses made on the scalar unit: lane offsets
 # that are constants of the tile, counted from a base the padding below the tensor, the tap in the scalar
 # offset, rows outside the image told by one ballot per slab.  the gather_sa switch at 0 is the form with vector
