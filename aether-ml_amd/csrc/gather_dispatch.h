@@ -500,14 +500,17 @@ static bool launch_direct(DirectParams& dp, bool dgrad, hipStream_t st) {
     const bool few = dgrad || tuning().direct == 2;
     const bool wide = !few && dp.D % 16 == 0 && dp.fH * dp.fW * dp.C >= 48;
     const bool wide8 = !few && !wide && dp.D % 8 == 0;
-    const int lanes = wide ? chunks / 4 : wide8 ? chunks / 2 : chunks;            // per pixel: a power of two
+    // dgrad: two groups of 4 output channels per lane where that leaves a lane per input channel (tuning: direct = 2 keeps one)
+    const bool dgrad2 = dgrad && chunks >= 8 && tuning().direct != 2;
+    const int lanes = wide ? chunks / 4 : (wide8 || dgrad2) ? chunks / 2 : chunks;   // per pixel: a power of two
     dp.q_shift = 0;
     while ((1 << dp.q_shift) < lanes) ++dp.q_shift;
     const dim3 grid((unsigned)cdiv((int64_t)dp.M * lanes, kThreads));
     const size_t lds = (size_t)dp.fH * dp.fW * dp.C * dp.D * sizeof(float);
 #define AETH_DIRECT_CASE(FH_, FW_, C_)                                                                              \
     if (dp.fH == FH_ && dp.fW == FW_ && dp.C == C_) {                                                               \
-        if (dgrad) hipLaunchKernelGGL((direct_dgrad_smallc<T, FH_, FW_, C_>), grid, dim3(kThreads), lds, st, dp);   \
+        if (dgrad2) hipLaunchKernelGGL((direct_dgrad_smallc<T, FH_, FW_, C_, 2>), grid, dim3(kThreads), lds, st, dp); \
+        else if (dgrad) hipLaunchKernelGGL((direct_dgrad_smallc<T, FH_, FW_, C_>), grid, dim3(kThreads), lds, st, dp); \
         else if (wide) hipLaunchKernelGGL((direct_fprop_smallc<T, FH_, FW_, C_, 16>), grid, dim3(kThreads), lds, st, dp); \
         else if (wide8) hipLaunchKernelGGL((direct_fprop_smallc<T, FH_, FW_, C_, 8>), grid, dim3(kThreads), lds, st, dp); \
         else hipLaunchKernelGGL((direct_fprop_smallc<T, FH_, FW_, C_>), grid, dim3(kThreads), lds, st, dp);         \

@@ -1616,7 +1616,9 @@ static __global__ __launch_bounds__(kThreads) void direct_fprop_smallc(const Dir
     for (int v = 0; v < NV; ++v) *reinterpret_cast<f4*>(p.out + (size_t)m * p.D + CPT * q + 4 * v) = acc[v];
 }
 
-template <typename T, int FH, int FW, int C>
+// NG = groups of 4 output channels per lane, 1 or 2.  With 2 a lane does the work of two neighbouring lanes of the
+// one-group form and adds their sums as the first xor-shuffle of that form would: same bits, half the address work.
+template <typename T, int FH, int FW, int C, int NG = 1>
 static __global__ __launch_bounds__(kThreads) void direct_dgrad_smallc(const DirectParams p) {
     extern __shared__ __attribute__((aligned(16))) float wl[];
     direct_load_filter<T>(p, wl);
@@ -1627,11 +1629,13 @@ static __global__ __launch_bounds__(kThreads) void direct_dgrad_smallc(const Dir
     unsigned s_, rem, i, j;
     p.div_hw.divmod((unsigned)min(m, p.M - 1), s_, rem);
     p.div_w.divmod(rem, i, j);
-    float acc[C];
+    float acc[NG][C];
 #pragma unroll
-    for (int c = 0; c < C; ++c) acc[c] = 0.f;
-    const float* wq = wl + 4 * q;
-    f4 gv[FH * FW];
+    for (int h = 0; h < NG; ++h)
+#pragma unroll
+        for (int c = 0; c < C; ++c) acc[h][c] = 0.f;
+    const float* wq = wl + 4 * NG * q;
+    f4 gv[FH * FW][NG];
     bool oks[FH * FW];
 #pragma unroll
     for (int fx = 0; fx < FH; ++fx)
@@ -1640,36 +1644,45 @@ static __global__ __launch_bounds__(kThreads) void direct_dgrad_smallc(const Dir
             const int t = (int)i + p.pH - fx, u = (int)j + p.pW - fy;        // = ho * sH, wo * sW
             const int ho = t / p.sH, wo = u / p.sW;
             const bool ok = t >= 0 && u >= 0 && ho * p.sH == t && wo * p.sW == u && ho < p.Ho && wo < p.Wo;
-            const T* pd = dy + (size_t)(((int)s_ * p.Ho + (ok ? ho : 0)) * p.Wo + (ok ? wo : 0)) * p.D + 4 * q;
+            const T* pd = dy + (size_t)(((int)s_ * p.Ho + (ok ? ho : 0)) * p.Wo + (ok ? wo : 0)) * p.D + 4 * NG * q;
             oks[fx * FW + fy] = ok;
-            if constexpr (sizeof(T) == 4) {
-                gv[fx * FW + fy] = *reinterpret_cast<const f4*>(pd);
-            } else {
-                const uint2 v = *reinterpret_cast<const uint2*>(pd);
-                gv[fx * FW + fy] = f4{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u),
-                                      __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u)};
+#pragma unroll
+            for (int h = 0; h < NG; ++h) {
+                if constexpr (sizeof(T) == 4) {
+                    gv[fx * FW + fy][h] = *reinterpret_cast<const f4*>(pd + 4 * h);
+                } else {
+                    const uint2 v = *reinterpret_cast<const uint2*>(pd + 4 * h);
+                    gv[fx * FW + fy][h] = f4{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u),
+                                             __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u)};
+                }
             }
         }
 #pragma unroll
     for (int tap = 0; tap < FH * FW; ++tap) {
 #pragma unroll
         for (int c = 0; c < C; ++c) {
-            const f4 wv = *reinterpret_cast<const f4*>(wq + (tap * C + c) * p.D);
-            float d = 0.f;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) d = fmaf(gv[tap][e], wv[e], d);
-            acc[c] += oks[tap] ? d : 0.f;
+            for (int h = 0; h < NG; ++h) {
+                const f4 wv = *reinterpret_cast<const f4*>(wq + (tap * C + c) * p.D + 4 * h);
+                float d = 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) d = fmaf(gv[tap][h][e], wv[e], d);
+                acc[h][c] += oks[tap] ? d : 0.f;
+            }
         }
     }
+    float sum[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) sum[c] = NG == 2 ? acc[0][c] + acc[NG - 1][c] : acc[0][c];
     // add up the lanes of the pixel; every lane ends with the full sums and lane q < C stores channel q
     for (int sh = 1; sh < (1 << p.q_shift); sh <<= 1) {
 #pragma unroll
-        for (int c = 0; c < C; ++c) acc[c] += __shfl_xor(acc[c], sh);
+        for (int c = 0; c < C; ++c) sum[c] += __shfl_xor(sum[c], sh);
     }
     if (m < p.M) {
 #pragma unroll
         for (int c = 0; c < C; ++c)
-            if (q == c) p.out[(size_t)m * C + c] = acc[c];
+            if (q == c) p.out[(size_t)m * C + c] = sum[c];
     }
 }
 

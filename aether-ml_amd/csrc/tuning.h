@@ -27,7 +27,7 @@ struct Tuning {
     int gather_wide = -1;    // bf16 8-wave tiles: 0 never, 1 also for few tiles
     int gather_res = -1;     // gather_halo_res_bf16: 0 off, 1 also for few tiles
     int dense_res = -1;      // dense_res_f32: 0 off, 1 also for few tiles
-    int direct = -1;         // 0: no direct kernels for 1 to 3 input channels; 2: their fprop with 4 output channels per lane
+    int direct = -1;         // 0: no direct kernels for 1 to 3 input channels; 2: 4 output channels per lane in them
     int wgrad_halo = -1;     // wgrad_halo_f32 / _bf16: 0 off, 1 also for few slabs
     int wgrad_wide = -1;     // bf16 wgrad on wide wave tiles: 0 never, 1 wherever D > 64 (2: but never 256 k rows, 3: always)
     int wgrad_cw = -1;       // fp32 wgrad tile form: 4 (128-wide) or 6 (192-wide)

@@ -228,8 +228,8 @@ def test_fprop_with_the_filter_resident_in_lds(case, tune):
     assert np.array_equal(got, abi.fprop(x, w, b, stride, pad))
 
 
-# The direct kernels' fprop gives a lane 8 output channels (16 for 5x5 filters on 2 or 3 channels), 4 with direct = 2:
-# the same sums in the same order.
+# The direct kernels' fprop gives a lane 8 output channels (16 for 5x5 filters on 2 or 3 channels) and their dgrad 8 from
+# 32 output channels on; 4 with direct = 2: the same sums in the same order.
 DIRECT_CASES = [
     (5, 28, 28, 1, 32, 3, 3, 1, 1, "same"),
     (3, 12, 12, 2, 16, 3, 3, 2, 2, "same"),      # 16 output channels: two lanes per pixel
@@ -241,14 +241,17 @@ DIRECT_CASES = [
 
 
 @pytest.mark.parametrize("case", DIRECT_CASES, ids=lambda c: "x".join(str(v) for v in c))
-def test_direct_fprop_with_more_channels_per_lane(case, tune):
+def test_direct_kernels_with_more_channels_per_lane(case, tune):
     from tests import abi
     x, w, b, dy = _case(case, 31)
     stride, pad = (case[7], case[8]), case[9]
     got = abi.fprop(x, w, b, stride, pad)
     abi.close(got, O.conv_fprop(x, w, b, stride, pad, dtype=np.float64))
+    dx = abi.dgrad(dy, w, x.shape, stride, pad)         # two groups of 4 output channels per lane from 32 channels on
+    abi.close(dx, O.conv_dgrad(dy, w, x.shape[1:3], stride, pad, dtype=np.float64))
     tune(direct=2)
     assert np.array_equal(got, abi.fprop(x, w, b, stride, pad))
+    assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
 
 
 # fp32 gathers whose slabs lie inside one tap load with addresses made on the scalar unit: lane offsets
