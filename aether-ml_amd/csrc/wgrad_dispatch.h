@@ -198,10 +198,15 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     splits = cdiv(slabs, slabs_per);
     p.m_per_split = slabs_per * slab_rows;
     const int64_t kd = (int64_t)p.K * D;
-    void* ws;
-    rc = workspace((int64_t)splits * (kd + D) * sizeof(float), &ws);
-    if (rc) return rc;
-    p.out = (float*)ws;
+    // one split (few rows: a dense layer on a small batch): the kernel writes dw and dbias themselves, no reduction launch
+    const bool single = splits == 1;
+    void* ws = nullptr;
+    if (!single) {
+        rc = workspace((int64_t)splits * (kd + D) * sizeof(float), &ws);
+        if (rc) return rc;
+    }
+    p.out = single ? dw : (float*)ws;
+    p.db_out = single ? dbias : nullptr;
     p.kt = kt; p.nt = nt;
     dim3 grid(kt * nt * splits);
     if (wide_k) hipLaunchKernelGGL((wgrad_gemm_dma_bf16w<4, 4>), grid, dim3(512), 0, c.stream, p);
@@ -216,6 +221,7 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     else if (vy) hipLaunchKernelGGL((wgrad_gemm<T, 1, CE>), grid, dim3(kThreads), 0, c.stream, p);
     else hipLaunchKernelGGL((wgrad_gemm<T, 1, 1>), grid, dim3(kThreads), 0, c.stream, p);
     AETH_LAUNCH_CHECK();
+    if (single) return AETH_OK;
     const int n = (int)(kd + (dbias ? D : 0));
     const bool r4 = kd % 4 == 0 && D % 4 == 0 && (reinterpret_cast<uintptr_t>(dw) & 15) == 0 &&
                     (dbias == nullptr || (reinterpret_cast<uintptr_t>(dbias) & 15) == 0);

@@ -18,6 +18,7 @@ struct WgradParams {
     const void* x;       // [S,H,W,C] of T
     const void* dy;      // [S,Ho,Wo,D] = [M,D] of T
     float* out;          // [splits][K*D + D]
+    float* db_out;       // one split only: dbias itself (out is then dw itself and no reduction follows); else null
     int want_dbias;
     int S, H, W, C, Ho, Wo, D;
     int M, K;
@@ -230,7 +231,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_gemm(const WgradParams p) {
             float s = 0.f;
 #pragma unroll
             for (int r = 0; r < Y_RPP; ++r) s += lds_db[r * 64 + tid];
-            if (n0 + tid < p.D) outp[(size_t)p.K * p.D + n0 + tid] = s;
+            if (n0 + tid < p.D) (p.db_out ? p.db_out : outp + (size_t)p.K * p.D)[n0 + tid] = s;
         }
     }
 }
@@ -518,7 +519,7 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
         lds_y0[db_rg * 64 + db_col] = dbsum;
         __syncthreads();
         if (tid < 64 && n0 + tid < p.D)
-            outp[(size_t)p.K * p.D + n0 + tid] = (lds_y0[tid] + lds_y0[64 + tid]) + (lds_y0[128 + tid] + lds_y0[192 + tid]);
+            (p.db_out ? p.db_out : outp + (size_t)p.K * p.D)[n0 + tid] = (lds_y0[tid] + lds_y0[64 + tid]) + (lds_y0[128 + tid] + lds_y0[192 + tid]);
     }
 }
 
@@ -732,7 +733,7 @@ static __global__ __launch_bounds__(kThreads) void wgrad_gemm_dma_bf16(const Wgr
     }
     if (wave_db && lane < 32) {                          // row 0 of the sums: element 0 of the lanes 0..31
         const int n = n0 + 32 * nflip + lane;
-        if (n < p.D) outp[(size_t)p.K * p.D + n] = acc_db[0];
+        if (n < p.D) (p.db_out ? p.db_out : outp + (size_t)p.K * p.D)[n] = acc_db[0];
     }
 }
 
@@ -1003,7 +1004,7 @@ static __global__ __launch_bounds__(128 * KW, KW == 4 ? 1 : (NB == 4 ? 2 : 3)) v
 #pragma unroll
         for (int j = 0; j < DBN; ++j) {
             const int n = n0 + nw * 32 * NB + (j * KW + kw) * 32 + lane;
-            if (n < p.D) outp[(size_t)p.K * p.D + n] = acc_db[j][0];
+            if (n < p.D) (p.db_out ? p.db_out : outp + (size_t)p.K * p.D)[n] = acc_db[j][0];
         }
     }
 }
