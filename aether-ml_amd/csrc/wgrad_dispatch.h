@@ -142,7 +142,12 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     }
     // operand width of the fp32 LDS-direct kernel: 192-wide k tiles where they pad fewer rows than 128-wide ones
     p.cw = !va ? 1 : (p.K <= 64 ? 2 : 4);
-    if (dma && p.cw == 4 && cdiv(p.K, 192) * 192 < cdiv(p.K, kWgBK) * kWgBK) p.cw = 6;
+    if (dma && p.cw == 4) {
+        // (equal padding and a last 128-wide tile at most a quarter full, K = 288: 27.5 us on 192-wide tiles against 29.2;
+        // equal padding with whole 128-wide tiles, K = 384, 768, 1152: 128-wide is 3 to 6 % faster)
+        const int pad192 = cdiv(p.K, 192) * 192, pad128 = cdiv(p.K, kWgBK) * kWgBK, last128 = p.K % kWgBK;
+        if (pad192 < pad128 || (pad192 == pad128 && last128 != 0 && last128 <= kWgBK / 4)) p.cw = 6;
+    }
     if (dma && va && p.K > 64 && (tuning().wgrad_cw == 4 || tuning().wgrad_cw == 6)) p.cw = tuning().wgrad_cw;
     // slab height of the 192-wide kernel: 16 rows (three workgroups per CU) where a workgroup walks at
     // least 64 of them (56x56x64: 0.481 ms against 0.487 with 32 rows; 8x8x64 -> 128, batch 128, 8 slabs of
