@@ -204,7 +204,8 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     p.m_per_split = slabs_per * slab_rows;
     const int64_t kd = (int64_t)p.K * D;
     // one split (few rows: a dense layer on a small batch): the kernel writes dw and dbias themselves, no reduction launch
-    const bool single = splits == 1;
+    // (dw aligned for the 16-byte stores of the fp32 kernel, as the workspace is)
+    const bool single = splits == 1 && (reinterpret_cast<uintptr_t>(dw) & 15) == 0;
     void* ws = nullptr;
     if (!single) {
         rc = workspace((int64_t)splits * (kd + D) * sizeof(float), &ws);
