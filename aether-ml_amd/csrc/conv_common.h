@@ -269,7 +269,7 @@ __device__ __forceinline__ void store_tile_lines(const GatherParams& p, float* o
                 const int n = nw0 + 32 * j + l32;
                 const unsigned off = (base + (unsigned)n * 4u) | ((unsigned)!(n < p.N) << 31);   // bit 31 from either part: outside the descriptor
                 const float value = acc[i][j][v];        // (a bit cast of the vector element itself reads element 0)
-                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(value), rsrc, (int)off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(value), rsrc, (int)off, 0, 2);
             }
         }
     }
@@ -304,7 +304,7 @@ __device__ __forceinline__ void store_tile_lines2(const GatherParams& p, float* 
             const unsigned base = (unsigned)__builtin_amdgcn_ds_bpermute(4 * pix + 16 * lh, rowbytes);
             const float a = acc[i][0][v], b = acc[i][1][v];    // (a bit cast of the vector element itself reads element 0)
             const u2 value = {__float_as_uint(a), __float_as_uint(b)};
-            __builtin_amdgcn_raw_buffer_store_b64(value, rsrc, (int)((base + (col & 0x7fffffffu)) | (col & 0x80000000u)), 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b64(value, rsrc, (int)((base + (col & 0x7fffffffu)) | (col & 0x80000000u)), 0, 2);
         }
     }
 }
@@ -344,10 +344,10 @@ __device__ __forceinline__ void store_tile_runs(const GatherParams& p, float* ou
             for (int j = 0; j < TN; ++j) e[j] = acc[i][j][v];
             if constexpr (TN == 2) {
                 const u2 value = {__float_as_uint(e[0]), __float_as_uint(e[1])};
-                __builtin_amdgcn_raw_buffer_store_b64(value, rsrc, off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b64(value, rsrc, off, 0, 2);
             } else {
                 const u4 value = {__float_as_uint(e[0]), __float_as_uint(e[1]), __float_as_uint(e[2]), __float_as_uint(e[3])};
-                __builtin_amdgcn_raw_buffer_store_b128(value, rsrc, off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(value, rsrc, off, 0, 2);
             }
         }
     }
