@@ -453,8 +453,12 @@ static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
         int mtiles = 0;
         const bool dma = vec && hp.src_bytes != 0 && gs.pp.w_elems * 2 < ((int64_t)1 << 31) && gs.pp.N % 2 == 0;
         if (gs.nsplit == 1 && hp.M > 0 && plan_halo_res(hp, dma, c.prop.multiProcessorCount, &mtiles)) {
-            hipLaunchKernelGGL(gather_halo_res_bf16, dim3((unsigned)std::min(mtiles, c.prop.multiProcessorCount)),
-                               dim3(kResThreads), 0, c.stream, hp, gs.pp, mtiles);
+            const dim3 rgrid((unsigned)std::min(mtiles, c.prop.multiProcessorCount));
+            // tiles stored as runs of 256 contiguous bytes per pixel (tuning: gather_runs = 0 keeps the 16-byte pieces)
+            if (hp.out_bytes != 0 && tuning().gather_runs != 0)
+                hipLaunchKernelGGL(gather_halo_res_bf16<true>, rgrid, dim3(kResThreads), 0, c.stream, hp, gs.pp, mtiles);
+            else
+                hipLaunchKernelGGL(gather_halo_res_bf16<false>, rgrid, dim3(kResThreads), 0, c.stream, hp, gs.pp, mtiles);
             AETH_LAUNCH_CHECK();
             return AETH_OK;
         }

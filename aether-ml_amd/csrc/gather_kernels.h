@@ -1110,6 +1110,10 @@ constexpr int kResThreads = 512;
 constexpr int kResSlots = 352;        // 2 x 352 x 128 B of halo + 72 KB of filter = 160 KB
 constexpr int kResMaxTaps = 9;
 
+// RUNS: the pixels are the MFMAs' first operand and slab row r of the filter holds channel 2 (r % 32) + r / 32, so that a lane
+// owns two neighbouring channels of 16 pixels and 32 lanes write the 256 contiguous bytes of a pixel with one 8-byte store
+// each (store_tile_runs, whole lines, non-temporal) instead of 64 pieces of 16 bytes in 32 lines per instruction; same bits.
+template <bool RUNS>
 static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(const GatherParams p, const PackParams pk,
                                                                                const int mtiles) {
     constexpr int BM = kResBM, BN = 64, TN = 2, KC = 8, NL = kResSlots / 8;
@@ -1148,7 +1152,8 @@ static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(co
                 unsigned t_h, t_w;
                 p.div_tw.divmod((unsigned)tap, t_h, t_w);
                 const int x = pk.xa + pk.xs * (int)t_h, y = pk.ya + pk.ys * (int)t_w;
-                const int n = part * 8 + (lane >> 3);
+                const int row = part * 8 + (lane >> 3);
+                const int n = RUNS ? 2 * (row & 31) + (row >> 5) : row;           // the channel this slab row holds
                 const int k4 = k4e ^ ((part & 1) ? 4 : 0);
                 const unsigned off = (unsigned)((((x * pk.fW + y) * pk.C + n) * pk.D + 8 * k4) * 2) |
                                      ((unsigned)(n >= p.N) << 31);
@@ -1174,9 +1179,11 @@ static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(co
                     const unsigned off = (unsigned)((((x * pk.fW + y) * pk.C + c) * pk.D + n2) * 2) | nbad;
                     const unsigned a = __builtin_amdgcn_raw_buffer_load_b32(rsrc_w, (int)off, 0, 0);
                     const unsigned b = __builtin_amdgcn_raw_buffer_load_b32(rsrc_w, (int)off, pk.D * 2, 0);
-                    const int pos = ((c >> 3) ^ ((n2 >> 1) & 7)) * 16 + (c & 7) * 2;   // n2 and n2 + 1 share the key
-                    *reinterpret_cast<unsigned*>(fbytes + tap * 8192 + n2 * 128 + pos) = (a & 0xffffu) | (b << 16);
-                    *reinterpret_cast<unsigned*>(fbytes + tap * 8192 + (n2 + 1) * 128 + pos) = (a >> 16) | (b & 0xffff0000u);
+                    // the slab rows of channels n2 and n2 + 1: neighbours, or (RUNS) rows n2 / 2 and n2 / 2 + 32; the same key either way
+                    const int r0 = RUNS ? (n2 >> 1) : n2, r1 = RUNS ? (n2 >> 1) + 32 : n2 + 1;
+                    const int pos = ((c >> 3) ^ ((r0 >> 1) & 7)) * 16 + (c & 7) * 2;
+                    *reinterpret_cast<unsigned*>(fbytes + tap * 8192 + r0 * 128 + pos) = (a & 0xffffu) | (b << 16);
+                    *reinterpret_cast<unsigned*>(fbytes + tap * 8192 + r1 * 128 + pos) = (a >> 16) | (b & 0xffff0000u);
                 }
             }
         }
@@ -1248,6 +1255,9 @@ static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(co
     // ---- the multiplying waves ----
     f4 bv[TN][4];
     load_bias<TN>(p, p.bias, bv, 0, lh);
+    float bias_run[TN];                                                    // RUNS: the lane's channels 2 l32 + j
+#pragma unroll
+    for (int j = 0; j < TN; ++j) bias_run[j] = (RUNS && p.bias != nullptr && 2 * l32 + j < p.N) ? p.bias[2 * l32 + j] : 0.f;
     const int sw7 = (l32 >> 1) & 7;
     int pslot;                                                             // slot of tap (0,0) of this lane's row
     {
@@ -1259,6 +1269,10 @@ static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(co
     int done_m0 = 0, done_end = 0;
     bool have_done = false;
     const int store_after = min(wave + 1, T - 1);
+    auto store_done = [&]() __attribute__((always_inline)) {
+        if constexpr (RUNS) store_tile_runs<1, TN>(p, p.out, done, done_m0, 0, l32, lh, done_end);
+        else store_tile<1, TN>(p, p.out, done, done_m0, 0, l32, lh, done_end);
+    };
     __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (0 << 8));                   // this wave's part of the filter
     asm volatile("s_barrier" ::: "memory");
     for (int t = 0; t < ntl; ++t) {
@@ -1268,7 +1282,14 @@ static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(co
         const int m_end = ((int)s_img + 1) * hw;                           // rows past the image: multiplied, never stored
         const f4* h = halo[t & 1];
         f16v acc[1][TN];
-        fill_acc<1, TN>(bv, acc);
+        if constexpr (RUNS) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[0][j][v] = bias_run[j];
+        } else {
+            fill_acc<1, TN>(bv, acc);
+        }
         // the operands of tap u + 1 are read while the MFMAs of tap u run (two sets of 48 registers)
         int th = 0, tw = 0;
         f4 fa[2][4], fb[2][4][TN];
@@ -1289,7 +1310,10 @@ static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(co
 #pragma unroll
             for (int g = 0; g < 4; ++g)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) mma_chunk<uint16_t>(rb[g][j], ra[g], acc[0][j]);
+                for (int j = 0; j < TN; ++j) {
+                    if constexpr (RUNS) mma_chunk<uint16_t>(ra[g], rb[g][j], acc[0][j]);
+                    else mma_chunk<uint16_t>(rb[g][j], ra[g], acc[0][j]);
+                }
             __builtin_amdgcn_sched_barrier(0);
         };
         // All seven waves finish a tile together; if they also stored together, each would wait
@@ -1300,11 +1324,11 @@ static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(co
         for (int tap = 0; tap < T; tap += 2) {
             if (tap + 1 < T) read_tap(tap + 1, fa[1], fb[1]);
             multiply(fa[0], fb[0]);
-            if (tap == store_after && have_done) store_tile<1, TN>(p, p.out, done, done_m0, 0, l32, lh, done_end);
+            if (tap == store_after && have_done) store_done();
             if (tap + 1 < T) {
                 if (tap + 2 < T) read_tap(tap + 2, fa[0], fb[0]);
                 multiply(fa[1], fb[1]);
-                if (tap + 1 == store_after && have_done) store_tile<1, TN>(p, p.out, done, done_m0, 0, l32, lh, done_end);
+                if (tap + 1 == store_after && have_done) store_done();
             }
         }
         have_done = true;
@@ -1314,7 +1338,7 @@ static __global__ __launch_bounds__(kResThreads, 1) void gather_halo_res_bf16(co
         done_end = m_end;
         asm volatile("s_barrier" ::: "memory");
     }
-    if (have_done) store_tile<1, TN>(p, p.out, done, done_m0, 0, l32, lh, done_end);
+    if (have_done) store_done();
 }
 
 // Packs the filter w[fH][fW][C][D] into bt[Npad][Kpad] (k contiguous) for one

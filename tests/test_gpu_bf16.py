@@ -209,6 +209,9 @@ def test_bf16_fprop_dgrad_with_the_filter_resident_in_lds(case, tune):
     abi.close(abi.fprop_bf16(x, w, None, stride, pad), O.conv_fprop(xr, wr, None, stride, pad, dtype=np.float64))
     dx = abi.dgrad_bf16(dy, w, x.shape, stride, pad)
     abi.close(dx, O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
+    tune(gather_runs=0)                           # tiles stored as 16-byte pieces (the filter as the MFMAs' first operand): same bits
+    assert np.array_equal(got, abi.fprop_bf16(x, w, b, stride, pad))
+    assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
     # the same sums of the same products in another order of taps and tiles
     tune(gather_res=0)
     abi.close(abi.fprop_bf16(x, w, b, stride, pad), got, rtol=1e-5, atol=1e-5)
