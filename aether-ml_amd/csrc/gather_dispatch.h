@@ -217,8 +217,13 @@ static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t
         int mtiles = 0, stages = 0;
         if (plan_halo(hp, dma, &mtiles, &stages)) {
             dim3 grid((unsigned)(mtiles * cdiv(gp.N, 64)));
-            if (stages == 4) hipLaunchKernelGGL(gather_halo_bf16<4>, grid, dim3(kThreads), 0, st, hp);
-            else hipLaunchKernelGGL(gather_halo_bf16<3>, grid, dim3(kThreads), 0, st, hp);
+            // a dense or strided output that the descriptor covers: tiles go out as runs of 256 contiguous bytes per pixel
+            // (tuning: gather_runs = 0 keeps the 16-byte pieces; same bits)
+            const bool lines = hp.out_bytes != 0 && tuning().gather_runs != 0;
+            if (stages == 4 && lines) hipLaunchKernelGGL((gather_halo_bf16<4, true>), grid, dim3(kThreads), 0, st, hp);
+            else if (stages == 4) hipLaunchKernelGGL((gather_halo_bf16<4, false>), grid, dim3(kThreads), 0, st, hp);
+            else if (lines) hipLaunchKernelGGL((gather_halo_bf16<3, true>), grid, dim3(kThreads), 0, st, hp);
+            else hipLaunchKernelGGL((gather_halo_bf16<3, false>), grid, dim3(kThreads), 0, st, hp);
             return;
         }
     }
@@ -741,8 +746,8 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
                     }
                 }
                 const dim3 grid((unsigned)((int64_t)mtiles * nclass * cdiv(C, 64)));
-                // no bias and a dx that the descriptor covers: tiles go out as whole lines (0.197 against 0.213 ms on the stride-2 layer)
-                const bool lines = sets[0].gp.bias == nullptr && sets[0].gp.out_bytes != 0;
+                // a dx that the descriptor covers: tiles go out as whole lines (0.197 against 0.213 ms on the stride-2 layer)
+                const bool lines = sets[0].gp.out_bytes != 0 && tuning().gather_runs != 0;
                 if (stages == 4 && lines) hipLaunchKernelGGL((gather_halo_classes_bf16<4, true>), grid, dim3(kThreads), 0, ctx().stream, gc);
                 else if (stages == 4) hipLaunchKernelGGL((gather_halo_classes_bf16<4, false>), grid, dim3(kThreads), 0, ctx().stream, gc);
                 else if (lines) hipLaunchKernelGGL((gather_halo_classes_bf16<3, true>), grid, dim3(kThreads), 0, ctx().stream, gc);

@@ -758,7 +758,11 @@ static __device__ __forceinline__ void halo_tile_bf16(const GatherParams& p, con
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const int k4 = k4e ^ (((wave * 2 + i) & 1) ? 4 : 0);
-        b_off[i] = (unsigned)(((n0 + (wave * 2 + i) * 8 + (lane >> 3)) * p.bt_ld + 8 * k4) * 2);
+        // LINES: slab row r holds channel n0 + 2 (r % 32) + r / 32: a lane of the multiplying waves then owns two
+        // neighbouring channels, one in each of its 32-column blocks (store_tile_runs)
+        const int r = (wave * 2 + i) * 8 + (lane >> 3);
+        const int n = LINES ? n0 + 2 * (r & 31) + (r >> 5) : n0 + r;
+        b_off[i] = (unsigned)((n * p.bt_ld + 8 * k4) * 2);
     }
     const u32x4 rsrc_a = raw_rsrc(p.src, p.src_bytes);
     const u32x4 rsrc_b = raw_rsrc(p.bt, p.bt_bytes);
@@ -798,7 +802,20 @@ static __device__ __forceinline__ void halo_tile_bf16(const GatherParams& p, con
     if constexpr (STAGES == 4) load_filter(pf_next(), ring2);
 
     f16v acc[TM][TN];
-    fill_acc<TM, TN>(bv, acc);
+    if constexpr (LINES) {
+        // a lane's accumulators of block j all belong to channel n0 + 2 l32 + j
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int n = n0 + 2 * l32 + j;
+            const float bj = (p.bias != nullptr && n < p.N) ? p.bias[n] : 0.0f;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = bj;
+        }
+    } else {
+        fill_acc<TM, TN>(bv, acc);
+    }
 
     const int sw7 = (l32 >> 1) & 7;
     int th = 0, tw = 0, cb = 0;                          // the step being multiplied
@@ -859,13 +876,13 @@ static __device__ __forceinline__ void halo_tile_bf16(const GatherParams& p, con
             if (u + 2 < nsteps) step(u + 2, ring2, ring1);
         }
     }
-    if (LINES) store_tile_lines<TM, TN>(p, p.out, acc, m0 + wm0, n0, l32, lh, m_end);
+    if (LINES) store_tile_runs<TM, TN>(p, p.out, acc, m0 + wm0, n0, l32, lh, m_end);
     else store_tile<TM, TN>(p, p.out, acc, m0 + wm0, n0, l32, lh, m_end);
 }
 
-template <int STAGES>
+template <int STAGES, bool LINES = false>
 static __global__ __launch_bounds__(kThreads, 2) void gather_halo_bf16(const GatherParams p) {
-    halo_tile_bf16<STAGES>(p, xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x));
+    halo_tile_bf16<STAGES, LINES>(p, xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x));
 }
 
 // The stride classes of one dgrad (2 or 4 problems over the same dy, each writing its own pixels of dx) as one

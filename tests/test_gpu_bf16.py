@@ -125,10 +125,14 @@ def test_bf16_fprop_dgrad_without_split_k(case, tune):
     x, w, b, dy = _case(case, 5)
     stride, pad = (case[7], case[8]), case[9]
     xr, wr, dyr = O.round_to_bf16(x), O.round_to_bf16(w), O.round_to_bf16(dy)
-    abi.close(abi.fprop_bf16(x, w, b, stride, pad), O.conv_fprop(xr, wr, b, stride, pad, dtype=np.float64))
+    got = abi.fprop_bf16(x, w, b, stride, pad)
+    abi.close(got, O.conv_fprop(xr, wr, b, stride, pad, dtype=np.float64))
     abi.close(abi.fprop_bf16(x, w, None, stride, pad), O.conv_fprop(xr, wr, None, stride, pad, dtype=np.float64))
-    abi.close(abi.dgrad_bf16(dy, w, x.shape, stride, pad),
-              O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
+    dx = abi.dgrad_bf16(dy, w, x.shape, stride, pad)
+    abi.close(dx, O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
+    tune(gather_runs=0)                           # tiles stored as 16-byte pieces instead of runs of contiguous channels: same bits
+    assert np.array_equal(got, abi.fprop_bf16(x, w, b, stride, pad))
+    assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
 
 
 def _random_halo_cases(n, seed):
