@@ -44,9 +44,24 @@ static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
         const int taps = gp.Cs > 0 ? gp.K / gp.Cs : 0;
         const int64_t bias = ((int64_t)std::max(-gp.rh0, 0) * gp.Ws + std::max(-gp.rw0, 0)) * gp.Cs * (int64_t)sizeof(T);
         if (ut && taps <= 32 && (int64_t)gp.src_bytes + bias < ((int64_t)1 << 31) && tuning().gather_sa != 0) {
+            // 64-column wave tiles store runs of 256 contiguous bytes per pixel (tuning: gather_runs = 0 keeps the 16-byte pieces)
+            bool runs = false;
+            if constexpr (WN == 64) runs = gp.out_bytes != 0 && gp.split_slabs == 0 && tuning().gather_runs != 0;
             if constexpr (KC == 8) {
                 if (gp.bt_kn) {
+                    if constexpr (WN == 64) {
+                        if (runs) {
+                            hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, true, true, true>), grid, dim3(kThreads), 0, st, gp);
+                            return;
+                        }
+                    }
                     hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, true, false, true>), grid, dim3(kThreads), 0, st, gp);
+                    return;
+                }
+            }
+            if constexpr (WN == 64) {
+                if (runs) {
+                    hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, true, true>), grid, dim3(kThreads), 0, st, gp);
                     return;
                 }
             }

@@ -198,11 +198,12 @@ __global__ __launch_bounds__(kThreads, 3) void gather_gemm(const GatherParams p)
 // from four rows instead of one 16-byte read.  No packing launch.
 template <typename T, int BM, int BN, int WM, int WN, bool UT, int KC, bool NLOOP, bool SA = false, bool RUNS = false, bool BKN = false>
 __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(const GatherParams p) {
-    static_assert(!BKN || (sizeof(T) == 4 && KC == 8 && !NLOOP && !RUNS && (BN == 64 || BN == 32)), "filter in place: fp32 slab tiles");
+    static_assert(!BKN || (sizeof(T) == 4 && KC == 8 && !NLOOP && (BN == 64 || BN == 32)), "filter in place: fp32 slab tiles");
     // 4 waves, or 8 for the widest bf16 tiles (256 x 128 and 256 x 256: one workgroup per CU)
     constexpr int NW = (BM / WM) * (BN / WN);
     static_assert(NW == 4 || (NW == 8 && !NLOOP && !SA), "4 or 8 waves per workgroup");
-    static_assert(!RUNS || (NW == 8 && sizeof(T) == 2 && (WN == 64 || WN == 128)), "runs: the 8-wave bf16 tiles");
+    static_assert(!RUNS || ((WN == 64 || WN == 128) && ((NW == 8 && sizeof(T) == 2) || (SA && sizeof(T) == 4))),
+                  "runs: the 8-wave bf16 tiles and the fp32 tiles with 64-column wave tiles");
     static_assert(!SA || (UT && !NLOOP && (BM == 128 || BM == 64) && sizeof(T) == 4), "scalar addressing: fp32 uniform-tap tiles of 64 or 128 rows");
     static_assert(KC == 8 || KC == 4, "slab rows of 8 or 4 chunks");
     constexpr int CE = Elem<T>::CE;
@@ -436,7 +437,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
             const float* lbf = reinterpret_cast<const float*>(lb) + (8 * g + 4 * lh) * BN;
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                const int n = wn0 + 32 * j + l32;
+                const int n = RUNS ? wn0 + TN * l32 + j : wn0 + 32 * j + l32;   // (runs: a lane's blocks hold neighbouring channels)
 #pragma unroll
                 for (int t = 0; t < 4; ++t) fb[slot][j][t] = lbf[t * BN + (n ^ ((BN == 64 && (t & 1)) ? 32 : 0))];
             }
@@ -477,8 +478,10 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
 #pragma unroll
-                        for (int j = 0; j < TN; ++j)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[g & 1][j][t], fa[g & 1][i][t], acc[i][j], 0, 0, 0);
+                        for (int j = 0; j < TN; ++j) {
+                            if constexpr (RUNS) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[g & 1][i][t], fb[g & 1][j][t], acc[i][j], 0, 0, 0);
+                            else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[g & 1][j][t], fa[g & 1][i][t], acc[i][j], 0, 0, 0);
+                        }
                     __builtin_amdgcn_sched_barrier(0);
                 }
             } else {
