@@ -278,7 +278,7 @@ __device__ __forceinline__ void store_tile_lines(const GatherParams& p, float* o
 // The same for a wave tile of two 32-column blocks whose columns are interleaved: column l of block j is channel
 // nw0 + 2 l + j (the kernel fetches the filter rows in that order), so a lane holds two neighbouring channels of a pixel
 // and 32 lanes write 256 contiguous bytes with 8-byte stores: half the store instructions of store_tile_lines.
-template <int TM>
+template <int TM, bool NT>
 __device__ __forceinline__ void store_tile_lines2(const GatherParams& p, float* out, const f16v (&acc)[TM][2], int mw0,
                                                   int nw0, int l32, int lh, int m_end) {
     typedef unsigned u2 __attribute__((ext_vector_type(2)));
@@ -304,7 +304,9 @@ __device__ __forceinline__ void store_tile_lines2(const GatherParams& p, float* 
             const unsigned base = (unsigned)__builtin_amdgcn_ds_bpermute(4 * pix + 16 * lh, rowbytes);
             const float a = acc[i][0][v], b = acc[i][1][v];    // (a bit cast of the vector element itself reads element 0)
             const u2 value = {__float_as_uint(a), __float_as_uint(b)};
-            __builtin_amdgcn_raw_buffer_store_b64(value, rsrc, (int)((base + (col & 0x7fffffffu)) | (col & 0x80000000u)), 0, 2);
+            // (2: the non-temporal hint, for whole lines that stream to memory)
+            if constexpr (NT) __builtin_amdgcn_raw_buffer_store_b64(value, rsrc, (int)((base + (col & 0x7fffffffu)) | (col & 0x80000000u)), 0, 2);
+            else __builtin_amdgcn_raw_buffer_store_b64(value, rsrc, (int)((base + (col & 0x7fffffffu)) | (col & 0x80000000u)), 0, 0);
         }
     }
 }

@@ -23,6 +23,15 @@ static bool plan_dense_res(const GatherParams& gp, bool dma, int cus, int* mtile
     return true;
 }
 
+// Tiles stored as runs of contiguous channels carry the non-temporal hint: right for an output that streams to memory,
+// wrong for one that the next kernel would have found in L2 (the layers of a small network: training step of the three-block
+// CNN 0.389 ms with them, 0.384 with the 16-byte pieces).  From 64 MB of output on; tuning: gather_runs = 1 always, 0 never.
+static inline bool run_stores(const GatherParams& gp) {
+    const int v = tuning().gather_runs;
+    if (v == 0 || gp.out_bytes == 0) return false;
+    return v > 0 || gp.out_bytes >= (64u << 20);
+}
+
 template <typename T, int BM, int BN, int WM, int WN, int KC>
 static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
     constexpr int kThreads = 64 * (BM / WM) * (BN / WN);     // of this tile shape (shadows the 256 of the others)
@@ -46,10 +55,10 @@ static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
         if (ut && taps <= 32 && (int64_t)gp.src_bytes + bias < ((int64_t)1 << 31) && tuning().gather_sa != 0) {
             // 64-column wave tiles store runs of 256 contiguous bytes per pixel (tuning: gather_runs = 0 keeps the 16-byte pieces)
             bool runs = false;
-            if constexpr (WN == 64) runs = gp.out_bytes != 0 && gp.split_slabs == 0 && tuning().gather_runs != 0;
+            if constexpr (WN == 64 || WN == 32) runs = gp.split_slabs == 0 && run_stores(gp);
             if constexpr (KC == 8) {
                 if (gp.bt_kn) {
-                    if constexpr (WN == 64) {
+                    if constexpr (WN == 64 || WN == 32) {
                         if (runs) {
                             hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, true, true, true>), grid, dim3(kThreads), 0, st, gp);
                             return;
@@ -59,7 +68,7 @@ static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
                     return;
                 }
             }
-            if constexpr (WN == 64) {
+            if constexpr (WN == 64 || WN == 32) {
                 if (runs) {
                     hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, true, true>), grid, dim3(kThreads), 0, st, gp);
                     return;
@@ -78,7 +87,7 @@ static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
     }
     if constexpr (kThreads == 512 && sizeof(T) == 2) {
         // the 8-wave bf16 tiles store runs of contiguous channels (tuning: gather_runs = 0 keeps the 16-byte pieces per pixel)
-        if (gp.out_bytes != 0 && gp.split_slabs == 0 && tuning().gather_runs != 0) {
+        if (gp.split_slabs == 0 && run_stores(gp)) {
             if (ut) hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, false, true>), grid, dim3(kThreads), 0, st, gp);
             else hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, false, KC, false, false, true>), grid, dim3(kThreads), 0, st, gp);
             return;
@@ -234,7 +243,7 @@ static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t
             dim3 grid((unsigned)(mtiles * cdiv(gp.N, 64)));
             // a dense or strided output that the descriptor covers: tiles go out as runs of 256 contiguous bytes per pixel
             // (tuning: gather_runs = 0 keeps the 16-byte pieces; same bits)
-            const bool lines = hp.out_bytes != 0 && tuning().gather_runs != 0;
+            const bool lines = run_stores(hp);
             if (stages == 4 && lines) hipLaunchKernelGGL((gather_halo_bf16<4, true>), grid, dim3(kThreads), 0, st, hp);
             else if (stages == 4) hipLaunchKernelGGL((gather_halo_bf16<4, false>), grid, dim3(kThreads), 0, st, hp);
             else if (lines) hipLaunchKernelGGL((gather_halo_bf16<3, true>), grid, dim3(kThreads), 0, st, hp);
@@ -266,7 +275,7 @@ static void launch_gather(const GatherParams& gp, bool vec, int cus, hipStream_t
         int mtiles = 0;
         if (plan_dense_res(gp, dma, cus, &mtiles)) {
             const dim3 grid((unsigned)std::min(mtiles, cus));
-            const bool runs = tuning().gather_runs != 0 && gp.N % 2 == 0;
+            const bool runs = run_stores(gp) && gp.N % 2 == 0;
             if (gp.Kpad == 64 && runs) hipLaunchKernelGGL((dense_res_f32<2, true>), grid, dim3(kD1Threads), 0, st, gp, mtiles);
             else if (gp.Kpad == 64) hipLaunchKernelGGL((dense_res_f32<2, false>), grid, dim3(kD1Threads), 0, st, gp, mtiles);
             else if (runs) hipLaunchKernelGGL((dense_res_f32<1, true>), grid, dim3(kD1Threads), 0, st, gp, mtiles);
@@ -475,7 +484,7 @@ static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
         if (gs.nsplit == 1 && hp.M > 0 && plan_halo_res(hp, dma, c.prop.multiProcessorCount, &mtiles)) {
             const dim3 rgrid((unsigned)std::min(mtiles, c.prop.multiProcessorCount));
             // tiles stored as runs of 256 contiguous bytes per pixel (tuning: gather_runs = 0 keeps the 16-byte pieces)
-            if (hp.out_bytes != 0 && tuning().gather_runs != 0)
+            if (run_stores(hp))
                 hipLaunchKernelGGL(gather_halo_res_bf16<true>, rgrid, dim3(kResThreads), 0, c.stream, hp, gs.pp, mtiles);
             else
                 hipLaunchKernelGGL(gather_halo_res_bf16<false>, rgrid, dim3(kResThreads), 0, c.stream, hp, gs.pp, mtiles);
@@ -754,15 +763,18 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
                     int64_t pmt = 0, longest = 0;
                     if (direct && plan_class_pairs(sets, pc, kHaloBM, kHaloSlotsMax, &pmt, &longest)) {
                         const dim3 pgrid((unsigned)(pmt * (nclass / 2) * cdiv(C, 64)));
-                        if (longest <= halo_slots(4)) hipLaunchKernelGGL(gather_halo_pairs_bf16<4>, pgrid, dim3(kThreads), 0, ctx().stream, pc);
-                        else hipLaunchKernelGGL(gather_halo_pairs_bf16<3>, pgrid, dim3(kThreads), 0, ctx().stream, pc);
+                        const bool nt = run_stores(pc.cls[0]);   // (the kernel stores whole lines either way; the hint only for outputs that stream)
+                        if (longest <= halo_slots(4) && nt) hipLaunchKernelGGL((gather_halo_pairs_bf16<4, true>), pgrid, dim3(kThreads), 0, ctx().stream, pc);
+                        else if (longest <= halo_slots(4)) hipLaunchKernelGGL((gather_halo_pairs_bf16<4, false>), pgrid, dim3(kThreads), 0, ctx().stream, pc);
+                        else if (nt) hipLaunchKernelGGL((gather_halo_pairs_bf16<3, true>), pgrid, dim3(kThreads), 0, ctx().stream, pc);
+                        else hipLaunchKernelGGL((gather_halo_pairs_bf16<3, false>), pgrid, dim3(kThreads), 0, ctx().stream, pc);
                         AETH_LAUNCH_CHECK();
                         return AETH_OK;
                     }
                 }
                 const dim3 grid((unsigned)((int64_t)mtiles * nclass * cdiv(C, 64)));
                 // a dx that the descriptor covers: tiles go out as whole lines (0.197 against 0.213 ms on the stride-2 layer)
-                const bool lines = sets[0].gp.out_bytes != 0 && tuning().gather_runs != 0;
+                const bool lines = run_stores(sets[0].gp);
                 if (stages == 4 && lines) hipLaunchKernelGGL((gather_halo_classes_bf16<4, true>), grid, dim3(kThreads), 0, ctx().stream, gc);
                 else if (stages == 4) hipLaunchKernelGGL((gather_halo_classes_bf16<4, false>), grid, dim3(kThreads), 0, ctx().stream, gc);
                 else if (lines) hipLaunchKernelGGL((gather_halo_classes_bf16<3, true>), grid, dim3(kThreads), 0, ctx().stream, gc);

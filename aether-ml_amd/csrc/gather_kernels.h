@@ -202,8 +202,8 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
     // 4 waves, or 8 for the widest bf16 tiles (256 x 128 and 256 x 256: one workgroup per CU)
     constexpr int NW = (BM / WM) * (BN / WN);
     static_assert(NW == 4 || (NW == 8 && !NLOOP && !SA), "4 or 8 waves per workgroup");
-    static_assert(!RUNS || ((WN == 64 || WN == 128) && ((NW == 8 && sizeof(T) == 2) || (SA && sizeof(T) == 4))),
-                  "runs: the 8-wave bf16 tiles and the fp32 tiles with 64-column wave tiles");
+    static_assert(!RUNS || ((NW == 8 && sizeof(T) == 2 && (WN == 64 || WN == 128)) || (SA && sizeof(T) == 4 && (WN == 64 || WN == 32))),
+                  "runs: the 8-wave bf16 tiles and the fp32 tiles with scalar addressing");
     static_assert(!SA || (UT && !NLOOP && (BM == 128 || BM == 64) && sizeof(T) == 4), "scalar addressing: fp32 uniform-tap tiles of 64 or 128 rows");
     static_assert(KC == 8 || KC == 4, "slab rows of 8 or 4 chunks");
     constexpr int CE = Elem<T>::CE;
@@ -620,7 +620,8 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
         if (s + 1 < nslabs) slab(lds_a1, lds_b1, lds_a0, lds_b0, (s + 2) * BK, s + 2 < nslabs);
     }
 
-    if constexpr (RUNS) store_tile_runs<TM, TN>(p, p.out + (size_t)split * p.M * p.N, acc, m0 + wm0, n0 + wn0, l32, lh, p.M);
+    if constexpr (RUNS && TN == 1) store_tile_lines<TM, TN>(p, p.out + (size_t)split * p.M * p.N, acc, m0 + wm0, n0 + wn0, l32, lh, p.M);
+    else if constexpr (RUNS) store_tile_runs<TM, TN>(p, p.out + (size_t)split * p.M * p.N, acc, m0 + wm0, n0 + wn0, l32, lh, p.M);
     else store_tile<TM, TN>(p, p.out + (size_t)split * p.M * p.N, acc, m0 + wm0, n0 + wn0, l32, lh);
 }
 
@@ -914,7 +915,7 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_classes_bf16(c
 // workgroup of the CU fills the gap) comes half as often.  The pixels are the MFMAs' first operand and the tiles go
 // out in 4-byte stores of whole lines (store_tile_lines).  All classes read the filter in place (one descriptor).
 // ------------------------------------------------------------------------------
-template <int STAGES>
+template <int STAGES, bool NT>
 static __global__ __launch_bounds__(kThreads, 2) void gather_halo_pairs_bf16(const GatherClasses q) {
     constexpr int BM = kHaloBM, BN = 64, TM = 2, TN = 2, KC = 8, BK = 64, CPP = 2;
     constexpr int kHaloSlots = halo_slots(STAGES);
@@ -1095,8 +1096,8 @@ static __global__ __launch_bounds__(kThreads, 2) void gather_halo_pairs_bf16(con
         }
     }
     (void)nsteps;
-    store_tile_lines2<TM>(pa, pa.out, acc[0], m0 + wm0, n0, l32, lh, m_end);
-    store_tile_lines2<TM>(pb, pb.out, acc[1], m0 + wm0, n0, l32, lh, m_end);
+    store_tile_lines2<TM, NT>(pa, pa.out, acc[0], m0 + wm0, n0, l32, lh, m_end);
+    store_tile_lines2<TM, NT>(pb, pb.out, acc[1], m0 + wm0, n0, l32, lh, m_end);
 }
 
 struct PackParams {

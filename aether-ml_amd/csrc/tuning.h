@@ -23,7 +23,7 @@ struct Tuning {
     int gather_pairs = -1;   // 0: the merged launch keeps one class per workgroup
     int gather_bkn = -1;     // 0: fp32 fprop always packs its filter
     int narrow = -1;         // 0: products with at most 16 output channels go to the slab kernels too
-    int gather_runs = -1;    // 0: the 8-wave bf16 tiles store 16-byte pieces per pixel
+    int gather_runs = -1;    // tiles stored as runs of contiguous channels (non-temporal): 0 never, 1 always (default: from 64 MB of output on)
     int gather_wide = -1;    // bf16 8-wave tiles: 0 never, 1 also for few tiles
     int gather_res = -1;     // gather_halo_res_bf16: 0 off, 1 also for few tiles
     int dense_res = -1;      // dense_res_f32: 0 off, 1 also for few tiles

@@ -121,7 +121,7 @@ HALO_CASES = [
 @pytest.mark.parametrize("case", HALO_CASES, ids=lambda c: "x".join(str(v) for v in c))
 def test_bf16_fprop_dgrad_without_split_k(case, tune):
     from tests import abi
-    tune(gather_split=0)
+    tune(gather_split=0, gather_runs=1)           # (run stores are taken from 64 MB of output on)
     x, w, b, dy = _case(case, 5)
     stride, pad = (case[7], case[8]), case[9]
     xr, wr, dyr = O.round_to_bf16(x), O.round_to_bf16(w), O.round_to_bf16(dy)
@@ -203,7 +203,7 @@ RES_CASES = [
 @pytest.mark.parametrize("case", RES_CASES, ids=lambda c: "x".join(str(v) for v in c))
 def test_bf16_fprop_dgrad_with_the_filter_resident_in_lds(case, tune):
     from tests import abi
-    tune(gather_split=0)
+    tune(gather_split=0, gather_runs=1)
     tune(gather_res=1)
     x, w, b, dy = _case(case, 11)
     stride, pad = (case[7], case[8]), case[9]
@@ -238,7 +238,7 @@ WIDE_CASES = [
 def test_bf16_fprop_dgrad_with_wide_tiles_on_eight_waves(case, tune):
     from tests import abi
     tune(gather_split=0, gather_merge=0)          # (one launch per dgrad class: the merged launch has kernels of its own)
-    tune(gather_wide=1)
+    tune(gather_wide=1, gather_runs=1)
     x, w, b, dy = _case(case, 13)
     stride, pad = (case[7], case[8]), case[9]
     xr, wr, dyr = O.round_to_bf16(x), O.round_to_bf16(w), O.round_to_bf16(dy)
@@ -349,14 +349,19 @@ def test_bf16_dgrad_with_all_stride_classes_in_one_launch(case, tune):
     from tests import abi
     x, w, b, dy = _case(case, 29)
     stride, pad = (case[7], case[8]), case[9]
-    tune(gather_split=0, gather_pairs=0)
+    tune(gather_split=0, gather_pairs=0, gather_runs=1)   # one class per workgroup, tiles stored as runs of contiguous channels
     dyr, wr = O.round_to_bf16(dy), O.round_to_bf16(w)
     dx = abi.dgrad_bf16(dy, w, x.shape, stride, pad)
     abi.close(dx, O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
+    tune(gather_runs=0)                           # ... as 16-byte pieces
+    assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
     tune(gather_merge=0)
     assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
-    # two classes per workgroup from one halo (what the library takes where all classes read the filter in place)
-    tune(gather_merge=-1, gather_pairs=-1)
+    # two classes per workgroup from one halo (what the library takes where all classes read the filter in place),
+    # with and without the non-temporal hint on its stores
+    tune(gather_merge=-1, gather_pairs=-1, gather_runs=1)
+    assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
+    tune(gather_runs=-1)
     assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
 
 

@@ -215,7 +215,7 @@ DENSE_RES_CASES = [
 @pytest.mark.parametrize("case", DENSE_RES_CASES, ids=lambda c: "x".join(str(v) for v in c))
 def test_fprop_with_the_filter_resident_in_lds(case, tune):
     from tests import abi
-    tune(dense_res=1)
+    tune(dense_res=1, gather_runs=1)              # (run stores are taken from 64 MB of output on)
     x, w, b, dy = _case(case, 12)
     stride, pad = (case[7], case[8]), case[9]
     got = abi.fprop(x, w, b, stride, pad)
@@ -283,6 +283,14 @@ def test_fprop_dgrad_with_scalar_addressed_loads(case, bm, tune):
     dx = abi.dgrad(dy, w, x.shape, stride, pad)
     abi.close(dx, O.conv_dgrad(dy, w, x.shape[1:3], stride, pad, dtype=np.float64))
     tune(gather_sa=0)
+    assert np.array_equal(y, abi.fprop(x, w, b, stride, pad))
+    assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
+    # tiles stored as runs of contiguous channels (what outputs of 64 MB and more get): the pixels as the MFMAs' first
+    # operand, the filter's columns read interleaved
+    tune(gather_sa=-1, gather_runs=1)
+    assert np.array_equal(y, abi.fprop(x, w, b, stride, pad))
+    assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
+    tune(gather_bkn=0, gather_direct_b=0)          # ... with the filter packed
     assert np.array_equal(y, abi.fprop(x, w, b, stride, pad))
     assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
 
