@@ -85,8 +85,8 @@ static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
             return;
         }
     }
-    if constexpr (kThreads == 512 && sizeof(T) == 2) {
-        // the 8-wave bf16 tiles store runs of contiguous channels (tuning: gather_runs = 0 keeps the 16-byte pieces per pixel)
+    if constexpr (sizeof(T) == 2) {
+        // the bf16 tiles store runs of contiguous channels (tuning: gather_runs = 0 keeps the 16-byte pieces per pixel)
         if (gp.split_slabs == 0 && run_stores(gp)) {
             if (ut) hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, false, true>), grid, dim3(kThreads), 0, st, gp);
             else hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, false, KC, false, false, true>), grid, dim3(kThreads), 0, st, gp);

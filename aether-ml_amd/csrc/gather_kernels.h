@@ -202,8 +202,9 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
     // 4 waves, or 8 for the widest bf16 tiles (256 x 128 and 256 x 256: one workgroup per CU)
     constexpr int NW = (BM / WM) * (BN / WN);
     static_assert(NW == 4 || (NW == 8 && !NLOOP && !SA), "4 or 8 waves per workgroup");
-    static_assert(!RUNS || ((NW == 8 && sizeof(T) == 2 && (WN == 64 || WN == 128)) || (SA && sizeof(T) == 4 && (WN == 64 || WN == 32))),
-                  "runs: the 8-wave bf16 tiles and the fp32 tiles with scalar addressing");
+    static_assert(!RUNS || !NLOOP, "runs: not in the n-loop mode");
+    static_assert(!RUNS || ((sizeof(T) == 2 && (WN == 32 || WN == 64 || WN == 128)) || (SA && sizeof(T) == 4 && (WN == 64 || WN == 32))),
+                  "runs: the bf16 tiles and the fp32 tiles with scalar addressing");
     static_assert(!SA || (UT && !NLOOP && (BM == 128 || BM == 64) && sizeof(T) == 4), "scalar addressing: fp32 uniform-tap tiles of 64 or 128 rows");
     static_assert(KC == 8 || KC == 4, "slab rows of 8 or 4 chunks");
     constexpr int CE = Elem<T>::CE;
