@@ -311,6 +311,9 @@ __device__ __forceinline__ void store_tile_lines2(const GatherParams& p, float* 
     }
 }
 
+// (These whole-line stores carry the non-temporal hint, cache policy 2: the output streams to memory.  Worth 5 to 15 % of a
+// launch that writes hundreds of MB; on the 16-byte pieces of store_tile the hint costs 50 %, and an output that the next
+// kernel reads out of L2 is better off without it: the host takes these forms for large outputs only.)
 // The general form: a wave tile of TN 32-column blocks with interleaved columns (column l of block j is channel
 // nw0 + TN l + j; TN = 2 or 4): a lane holds TN neighbouring channels of a pixel and 32 lanes write 32 TN contiguous
 // floats per pixel with one 8- or 16-byte store each.  N is a multiple of 4 (p.out_bytes != 0).
