@@ -317,7 +317,8 @@ __device__ __forceinline__ void store_tile_lines2(const GatherParams& p, float* 
 // The general form: a wave tile of TN 32-column blocks with interleaved columns (column l of block j is channel
 // nw0 + TN l + j; TN = 2 or 4): a lane holds TN neighbouring channels of a pixel and 32 lanes write 32 TN contiguous
 // floats per pixel with one 8- or 16-byte store each.  N is a multiple of 4 (p.out_bytes != 0).
-template <int TM, int TN>
+// PLAIN: the caller guarantees p.dense_out and a tile that lies inside m_end.
+template <int TM, int TN, bool PLAIN = false>
 __device__ __forceinline__ void store_tile_runs(const GatherParams& p, float* out, const f16v (&acc)[TM][TN], int mw0,
                                                 int nw0, int l32, int lh, int m_end) {
     static_assert(TN == 2 || TN == 4, "8- or 16-byte stores");
@@ -327,32 +328,60 @@ __device__ __forceinline__ void store_tile_runs(const GatherParams& p, float* ou
         __builtin_amdgcn_make_buffer_rsrc(out, 0, (int)p.out_bytes, 0x00020000);
     const int n = nw0 + TN * l32;
     const unsigned col = (unsigned)n * 4u, colbad = (unsigned)!(n < p.N) << 31;   // N is a multiple of TN here: all channels or none
+    // Rows stored at out + m N with the whole tile inside m_end (mw0 is wave-uniform): one vector offset per tile, the
+    // pixel's row as the scalar offset of an 8-byte store (one addition per 16-byte store), no lane exchange.  (Measured
+    // as a run-time choice in every kernel that stores runs: 4 % for dense_res_f32, whose stores sit between MFMA groups,
+    // nothing or a loss of 0.3 % where the stores end a workgroup.)
+    if constexpr (PLAIN) {
+        const unsigned rowb = (unsigned)p.N * 4u;
+        const int voff = (int)(((unsigned)(mw0 + 4 * lh) * rowb + col) | colbad);
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int m = mw0 + 32 * i + l32;
-        const bool mok = m < m_end;
-        unsigned row = (unsigned)m;
-        if (!p.dense_out) {
-            unsigned s, rem, ii, jj;
-            p.div_hw.divmod(mok ? (unsigned)m : 0u, s, rem);
-            p.div_w.divmod(rem, ii, jj);
-            row = ((unsigned)s * p.Hof + p.oh0 + ii * p.ohs) * p.Wof + p.ow0 + jj * p.ows;
-        }
-        const int rowbytes = (int)((row * (unsigned)p.N * 4u) | ((unsigned)!mok << 31));   // < 2^31: checked by the host
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int pix = 8 * (v >> 2) + (v & 3);
-            const unsigned base = (unsigned)__builtin_amdgcn_ds_bpermute(4 * pix + 16 * lh, rowbytes);
-            const int off = (int)((base + col) | colbad);
-            float e[TN];                                 // (a bit cast of the vector element itself reads element 0)
+            for (int v = 0; v < 16; ++v) {
+                const int soff = (int)((unsigned)(32 * i + 8 * (v >> 2) + (v & 3)) * rowb);
+                float e[TN];
 #pragma unroll
-            for (int j = 0; j < TN; ++j) e[j] = acc[i][j][v];
-            if constexpr (TN == 2) {
-                const u2 value = {__float_as_uint(e[0]), __float_as_uint(e[1])};
-                __builtin_amdgcn_raw_buffer_store_b64(value, rsrc, off, 0, 2);
-            } else {
-                const u4 value = {__float_as_uint(e[0]), __float_as_uint(e[1]), __float_as_uint(e[2]), __float_as_uint(e[3])};
-                __builtin_amdgcn_raw_buffer_store_b128(value, rsrc, off, 0, 2);
+                for (int j = 0; j < TN; ++j) e[j] = acc[i][j][v];
+                if constexpr (TN == 2) {
+                    const u2 value = {__float_as_uint(e[0]), __float_as_uint(e[1])};
+                    __builtin_amdgcn_raw_buffer_store_b64(value, rsrc, voff, soff, 2);
+                } else {
+                    // (a 16-byte store with its scalar offset in a register is the form behind which the compiler leaves
+                    // no wait state before the next write of the data registers, see store_tile, and here the next store's
+                    // data is assembled in the same registers right behind it: the row goes into the vector offset)
+                    const u4 value = {__float_as_uint(e[0]), __float_as_uint(e[1]), __float_as_uint(e[2]), __float_as_uint(e[3])};
+                    __builtin_amdgcn_raw_buffer_store_b128(value, rsrc, voff + soff, 0, 2);
+                }
+            }
+    } else {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int m = mw0 + 32 * i + l32;
+            const bool mok = m < m_end;
+            unsigned row = (unsigned)m;
+            if (!p.dense_out) {
+                unsigned s, rem, ii, jj;
+                p.div_hw.divmod(mok ? (unsigned)m : 0u, s, rem);
+                p.div_w.divmod(rem, ii, jj);
+                row = ((unsigned)s * p.Hof + p.oh0 + ii * p.ohs) * p.Wof + p.ow0 + jj * p.ows;
+            }
+            const int rowbytes = (int)((row * (unsigned)p.N * 4u) | ((unsigned)!mok << 31));   // < 2^31: checked by the host
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int pix = 8 * (v >> 2) + (v & 3);
+                const unsigned base = (unsigned)__builtin_amdgcn_ds_bpermute(4 * pix + 16 * lh, rowbytes);
+                const int off = (int)((base + col) | colbad);
+                float e[TN];                             // (a bit cast of the vector element itself reads element 0)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) e[j] = acc[i][j][v];
+                if constexpr (TN == 2) {
+                    const u2 value = {__float_as_uint(e[0]), __float_as_uint(e[1])};
+                    __builtin_amdgcn_raw_buffer_store_b64(value, rsrc, off, 0, 2);
+                } else {
+                    const u4 value = {__float_as_uint(e[0]), __float_as_uint(e[1]), __float_as_uint(e[2]), __float_as_uint(e[3])};
+                    __builtin_amdgcn_raw_buffer_store_b128(value, rsrc, off, 0, 2);
+                }
             }
         }
     }

@@ -1429,20 +1429,20 @@ static __global__ __launch_bounds__(kD1Threads, 1) void dense_res_f32(const Gath
     }
     // A rows of a tile: 16 pieces per slab; rows past M lie outside the descriptor and read as zeros
     const u32x4 rsrc_a = raw_rsrc(p.src, p.src_bytes);
-    unsigned rela[2 * (BM / 8)];
+    unsigned rela[2][2];                                 // [slab][piece parity]: the lane's part of a piece's offset
 #pragma unroll
-    for (int i = 0; i < 2 * (BM / 8); ++i) {
-        const int sl = i / (BM / 8), part = i % (BM / 8);
-        const int k4 = k4e ^ ((part & 1) ? 4 : 0);
-        rela[i] = (unsigned)(((part * 8 + prow) * p.Cs + 32 * sl + 4 * k4) * 4);
-    }
+    for (int sl = 0; sl < 2; ++sl)
+#pragma unroll
+        for (int o = 0; o < 2; ++o) rela[sl][o] = (unsigned)((prow * p.Cs + 32 * sl + 4 * (k4e ^ (o ? 4 : 0))) * 4);
+    const unsigned piece_bytes = (unsigned)(8 * p.Cs * 4);
     auto fetch = [&](int tile, int buf) __attribute__((always_inline)) {
         const unsigned base = (unsigned)tile * (unsigned)(BM * p.Cs * 4);
 #pragma unroll
         for (int i = 0; i < 2 * (BM / 8); ++i) {
             if (i < nslab * (BM / 8)) {
                 const int sl = i / (BM / 8), part = i % (BM / 8);
-                lds_direct_load16(rsrc_a, lds_address(&abuf[buf][sl][0]) + (unsigned)part * 1024u, base + rela[i]);
+                lds_direct_load16(rsrc_a, lds_address(&abuf[buf][sl][0]) + (unsigned)part * 1024u,
+                                  base + (unsigned)part * piece_bytes + rela[sl][part & 1]);
             }
         }
     };
@@ -1450,38 +1450,22 @@ static __global__ __launch_bounds__(kD1Threads, 1) void dense_res_f32(const Gath
     __builtin_amdgcn_s_waitcnt(0);
     asm volatile("s_barrier" ::: "memory");
 
+    // the bias as the C operand of a tile's first MFMAs: no copies into the accumulators at the start of a tile,
+    // where the 8 waves have just met
+    f16v bvec[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int n = RUNS ? wn0 + 2 * l32 + j : wn0 + 32 * j + 8 * (v >> 2) + 4 * lh + (v & 3);
+            bvec[j][v] = reinterpret_cast<const float*>(bias_lds)[n];
+        }
+
     const int sw7 = (l32 >> 1) & 7;
     f16v acc[TM][TN], done[TM][TN];
-    int done_m0 = 0;
-    bool have_done = false;
-    auto store_done = [&]() __attribute__((always_inline)) {
-        if constexpr (RUNS) store_tile_runs<TM, TN>(p, p.out, done, done_m0 + wm0, wn0, l32, lh, p.M);
-        else store_tile<TM, TN, true>(p, p.out, done, done_m0 + wm0, wn0, l32, lh);
-    };
     for (int t = 0; t < ntl; ++t) {
         if (wave == 0 && t + 1 < ntl) fetch(tile0 + t + 1, (t + 1) & 1);
         if (active) {
-            if constexpr (RUNS) {
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    const float bj = reinterpret_cast<const float*>(bias_lds)[wn0 + 2 * l32 + j];
-#pragma unroll
-                    for (int i = 0; i < TM; ++i)
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) acc[i][j][v] = bj;
-                }
-            } else {
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const f4 b = bias_lds[(wn0 + 32 * j + 8 * q + 4 * lh) >> 2];
-#pragma unroll
-                    for (int i = 0; i < TM; ++i)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = b[e];
-                }
-            }
             // k groups u = 4 slab + g of 8 k each; the operands of group u + 1 are read during the MFMAs of group u
             f4 fa[2][TM], fb[2][TN];
             auto read_frags = [&](int u, int slot) __attribute__((always_inline)) {
@@ -1504,26 +1488,40 @@ static __global__ __launch_bounds__(kD1Threads, 1) void dense_res_f32(const Gath
                     for (int i = 0; i < TM; ++i)
 #pragma unroll
                         for (int j = 0; j < TN; ++j) {
-                            if constexpr (RUNS) mma_chunk<float>(fa[u & 1][i], fb[u & 1][j], acc[i][j]);
-                            else mma_chunk<float>(fb[u & 1][j], fa[u & 1][i], acc[i][j]);
+                            const f4& a = RUNS ? fa[u & 1][i] : fb[u & 1][j];
+                            const f4& b = RUNS ? fb[u & 1][j] : fa[u & 1][i];
+                            if (u == 0) {
+                                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[0], b[0], bvec[j], 0, 0, 0);
+#pragma unroll
+                                for (int e = 1; e < 4; ++e)
+                                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], acc[i][j], 0, 0, 0);
+                            } else {
+                                mma_chunk<float>(a, b, acc[i][j]);
+                            }
                         }
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 // the finished tile leaves after k group `wave` (a few 16-byte pieces after every group
                 // were slower: 0.298 ms against 0.266 on 56x56, 64 -> 256)
-                if (have_done && u == min(wave, 4 * nslab - 1)) store_done();
+                if (t > 0 && u == min(wave, 4 * nslab - 1)) {
+                    const int m0 = (tile0 + t - 1) * BM + wm0;       // (not the workgroup's last tile: it lies inside M)
+                    if constexpr (RUNS) store_tile_runs<TM, TN, true>(p, p.out, done, m0, wn0, l32, lh, p.M);
+                    else store_tile<TM, TN, true>(p, p.out, done, m0, wn0, l32, lh);
+                }
             }
-            have_done = true;
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j) done[i][j] = acc[i][j];
-            done_m0 = (tile0 + t) * BM;
         }
         if (wave == 0) __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));   // the next tile's rows (and its own old stores)
         asm volatile("s_barrier" ::: "memory");
     }
-    if (active && have_done) store_done();
+    if (active && ntl > 0) {
+        const int m0 = (tile0 + ntl - 1) * BM + wm0;
+        if constexpr (RUNS) store_tile_runs<TM, TN>(p, p.out, done, m0, wn0, l32, lh, p.M);
+        else store_tile<TM, TN, true>(p, p.out, done, m0, wn0, l32, lh);
+    }
 }
 
 // dx[s][i][j][:] = 0 for i >= h0 or j >= w0: the trailing rows and columns of a strided dgrad that
