@@ -442,10 +442,11 @@ __device__ __forceinline__ unsigned select_by_mask(unsigned a, unsigned b, unsig
 
 // out[i] = sum_s part[s*stride + i] for i < n, in a fixed order: 4 split lanes per
 // output (splits s, s+4, ...), then the 4 lanes in order.  i < n_dw goes to dw,
-// the rest to dbias.
+// the rest to dbias.  tr > 0: the partials hold the transpose, rows of tr floats: element
+// i = r tr + c of a partial is dw[c (n_dw / tr) + r].
 static __global__ __launch_bounds__(kThreads) void reduce_splits(const float* __restrict__ part, float* __restrict__ dw,
                                                          float* __restrict__ dbias, int n_dw, int n, int stride,
-                                                         int splits) {
+                                                         int splits, int tr = 0) {
     __shared__ float red[4][64];
     const int col = threadIdx.x & 63;
     const int sl = threadIdx.x >> 6;
@@ -468,7 +469,7 @@ static __global__ __launch_bounds__(kThreads) void reduce_splits(const float* __
     __syncthreads();
     if (sl == 0 && i < n) {
         float t = (red[0][col] + red[1][col]) + (red[2][col] + red[3][col]);
-        if (i < n_dw) dw[i] = t;
+        if (i < n_dw) dw[tr > 0 ? (i % tr) * (n_dw / tr) + i / tr : i] = t;
         else if (dbias != nullptr) dbias[i - n_dw] = t;
     }
 }
@@ -476,9 +477,10 @@ static __global__ __launch_bounds__(kThreads) void reduce_splits(const float* __
 // The same sum for 16-byte aligned partials (stride and n_dw multiples of 4): a thread
 // owns 4 consecutive outputs, 16 split lanes per output add splits j, j+16, ... with
 // four loads in flight, and the lanes are added in lane order.
+// (tr as above, a multiple of 4: the 4 outputs of a thread then go to 4 rows of dw)
 static __global__ __launch_bounds__(kThreads) void reduce_splits4(const float* __restrict__ part, float* __restrict__ dw,
                                                           float* __restrict__ dbias, int n_dw, int n, int stride,
-                                                          int splits) {
+                                                          int splits, int tr = 0) {
     __shared__ f4 red[16][16];
     const int cg = threadIdx.x & 15;                     // group of 4 outputs
     const int sl = threadIdx.x >> 4;                     // split lane
@@ -503,8 +505,15 @@ static __global__ __launch_bounds__(kThreads) void reduce_splits4(const float* _
         f4 t = red[0][cg];
 #pragma unroll
         for (int j = 1; j < 16; ++j) t += red[j][cg];
-        if (i < n_dw) *reinterpret_cast<f4*>(dw + i) = t;
-        else if (dbias != nullptr) *reinterpret_cast<f4*>(dbias + (i - n_dw)) = t;
+        if (i < n_dw && tr > 0) {
+            const int r = i / tr, c = i - r * tr, ld = n_dw / tr;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dw[(c + e) * ld + r] = t[e];
+        } else if (i < n_dw) {
+            *reinterpret_cast<f4*>(dw + i) = t;
+        } else if (dbias != nullptr) {
+            *reinterpret_cast<f4*>(dbias + (i - n_dw)) = t;
+        }
     }
 }
 

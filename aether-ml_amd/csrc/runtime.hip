@@ -51,6 +51,7 @@ bool tuning_set(const char* name, int value) {
         {"gather_pairs", &Tuning::gather_pairs},
         {"gather_runs", &Tuning::gather_runs},   {"narrow", &Tuning::narrow},   {"gather_bkn", &Tuning::gather_bkn},
         {"wgrad_br", &Tuning::wgrad_br},         {"wgrad_rounds", &Tuning::wgrad_rounds},
+        {"wgrad_swap", &Tuning::wgrad_swap},
     };
     for (const Field& f : fields)
         if (strcmp(f.name, name) == 0) {

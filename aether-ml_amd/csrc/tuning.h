@@ -32,6 +32,7 @@ struct Tuning {
     int wgrad_wide = -1;     // bf16 wgrad on wide wave tiles: 0 never, 1 wherever D > 64 (2: but never 256 k rows, 3: always)
     int wgrad_cw = -1;       // fp32 wgrad tile form: 4 (128-wide) or 6 (192-wide)
     int wgrad_br = -1;       // slab height of the 192-wide form: 32 or 16
+    int wgrad_swap = -1;     // fp32 1x1 wgrad on few input channels with the operands swapped: 0 never, 1 wherever it applies
     int wgrad_rounds = -1;   // rounds of resident workgroups the splits are sized for: 1 to 4
 };
 

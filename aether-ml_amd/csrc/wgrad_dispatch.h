@@ -69,7 +69,8 @@ static int plan_wgrad_halo_f32(WgradHaloParams& p, int C, int sH, int sW, int cu
 
 template <typename T>
 int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* dbias,
-                    int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW) {
+                    int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW,
+                    bool swapped = false) {      // swapped: x and dy (C and D) arrive exchanged, see below
     int Ho, Wo;
     int rc = check_conv_dims(fn, S, H, W, C, D, fH, fW, sH, sW, pH, pW, &Ho, &Wo);
     if (rc) return rc;
@@ -86,8 +87,24 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
         }
     }
     Context& c = ctx();
+    if constexpr (sizeof(T) == 4) {
+        // A 1x1 filter on at most 64 input channels, many more output channels and many rows (64 -> 256 on 56x56
+        // images): as dw[64][D] the product has one half-width k tile, D / 64 n tiles that all re-read x, and two
+        // MFMAs per pair of operand reads.  Its transpose dy^T . x has D / 128 full-width k tiles over one n tile:
+        // the same kernel with the operands swapped, four MFMAs per pair of reads, dy read once and x twice
+        // (0.256 ms against 0.290 on that shape); the reduction writes the transpose back.
+        const int64_t M = (int64_t)S * H * W;
+        const bool shape = fH == 1 && fW == 1 && sH == 1 && sW == 1 && pH == 0 && pW == 0 && C > 32 && C <= 64 &&
+                           C % 4 == 0 && D >= 128 && D % 4 == 0 && (int64_t)C * D < ((int64_t)1 << 27) &&
+                           M * D * 4 < ((int64_t)1 << 31);
+        const bool swap = shape && (tuning().wgrad_swap > 0 ||
+                                    (tuning().wgrad_swap < 0 && M >= (int64_t)256 * 3 * c.prop.multiProcessorCount));
+        if (swap && !swapped) return conv_wgrad_impl<T>(fn, dy, x, dw, dbias, S, H, W, D, C, 1, 1, 1, 1, 0, 0, true);
+    }
     WgradParams p;
     p.x = x; p.dy = dy;
+    p.swap = swapped ? 1 : 0;
+    p.db_len = swapped ? C : D;
     p.S = S; p.H = H; p.W = W; p.C = C; p.Ho = Ho; p.Wo = Wo; p.D = D;
     p.M = S * Ho * Wo; p.K = fH * fW * C;
     p.fW = fW; p.sH = sH; p.sW = sW; p.pH = pH; p.pW = pW;
@@ -110,7 +127,7 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
         hp.want_dbias = dbias != nullptr;
         int splits = 0;
         if constexpr (sizeof(T) == 2) splits = dma16 ? plan_wgrad_halo(hp, C, sH, sW, c.prop.multiProcessorCount) : 0;
-        else splits = (dma && va) ? plan_wgrad_halo_f32(hp, C, sH, sW, c.prop.multiProcessorCount) : 0;
+        else splits = (dma && va && !swapped) ? plan_wgrad_halo_f32(hp, C, sH, sW, c.prop.multiProcessorCount) : 0;
         if (splits > 0) {
             const int64_t kd = (int64_t)p.K * D;
             void* ws;
@@ -149,6 +166,7 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
         if (pad192 < pad128 || (pad192 == pad128 && last128 != 0 && last128 <= kWgBK / 4)) p.cw = 6;
     }
     if (dma && va && p.K > 64 && (tuning().wgrad_cw == 4 || tuning().wgrad_cw == 6)) p.cw = tuning().wgrad_cw;
+    if (swapped) p.cw = 4;                             // (the form that adds up the columns of its x slabs)
     // slab height of the 192-wide kernel: 16 rows (three workgroups per CU) where a workgroup walks at
     // least 64 of them (56x56x64: 0.481 ms against 0.487 with 32 rows; 8x8x64 -> 128, batch 128, 8 slabs of
     // 32 per workgroup: 27.2 us with 32 rows, 28.3 with 16); tuning: wgrad_br overrides
@@ -205,10 +223,10 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     const int64_t kd = (int64_t)p.K * D;
     // one split (few rows: a dense layer on a small batch): the kernel writes dw and dbias themselves, no reduction launch
     // (dw aligned for the 16-byte stores of the fp32 kernel, as the workspace is)
-    const bool single = splits == 1 && (reinterpret_cast<uintptr_t>(dw) & 15) == 0;
+    const bool single = splits == 1 && (reinterpret_cast<uintptr_t>(dw) & 15) == 0 && !swapped;   // (the reduction writes the transpose back)
     void* ws = nullptr;
     if (!single) {
-        rc = workspace((int64_t)splits * (kd + D) * sizeof(float), &ws);
+        rc = workspace((int64_t)splits * (kd + p.db_len) * sizeof(float), &ws);
         if (rc) return rc;
     }
     p.out = single ? dw : (float*)ws;
@@ -228,15 +246,16 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     else hipLaunchKernelGGL((wgrad_gemm<T, 1, 1>), grid, dim3(kThreads), 0, c.stream, p);
     AETH_LAUNCH_CHECK();
     if (single) return AETH_OK;
-    const int n = (int)(kd + (dbias ? D : 0));
-    const bool r4 = kd % 4 == 0 && D % 4 == 0 && (reinterpret_cast<uintptr_t>(dw) & 15) == 0 &&
+    const int n = (int)(kd + (dbias ? p.db_len : 0));
+    const bool r4 = kd % 4 == 0 && D % 4 == 0 && p.db_len % 4 == 0 && (reinterpret_cast<uintptr_t>(dw) & 15) == 0 &&
                     (dbias == nullptr || (reinterpret_cast<uintptr_t>(dbias) & 15) == 0);
+    const int tr = swapped ? D : 0;                      // the partials hold dw^T in rows of D (the caller's C) floats
     if (r4)
         hipLaunchKernelGGL(reduce_splits4, dim3(cdiv(n, 64)), dim3(kThreads), 0, c.stream, (const float*)ws, dw, dbias,
-                           (int)kd, n, (int)(kd + D), splits);
+                           (int)kd, n, (int)(kd + p.db_len), splits, tr);
     else
         hipLaunchKernelGGL(reduce_splits, dim3(cdiv(n, 64)), dim3(kThreads), 0, c.stream, (const float*)ws, dw, dbias,
-                           (int)kd, n, (int)(kd + D), splits);
+                           (int)kd, n, (int)(kd + p.db_len), splits, tr);
     AETH_LAUNCH_CHECK();
     return AETH_OK;
 }

@@ -26,6 +26,10 @@ struct WgradParams {
     int m_per_split;     // multiple of 32
     int kt, nt;          // output tiles along k and n
     int cw;              // fp32 LDS-direct kernel: floats of k per lane of an operand read (4, 2 or 1)
+    // swap (fp32 LDS-direct kernel, 1x1 filters): the caller handed over dy as `x` and x as `dy`, the result is the
+    // transpose of dw, and dbias is the column sums of the `x` operand: every k tile adds up its own columns.
+    int swap;
+    int db_len;          // floats of dbias behind the K*D floats of a split's partial block (D, or K when swapped)
     unsigned x_bytes, dy_bytes;   // extents for the buffer descriptors (LDS-direct kernel)
     // moving 32 rows of m ahead: 32 = qs*Ho*Wo + qh*Wo + qw.  step_c = qw*sW, step_r = qh*sH;
     // byte offset += inc0 (+ inc1 when the column wraps) (+ inc2 when the row wraps)
@@ -298,7 +302,8 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
     const int m_begin = split * p.m_per_split;
     int m_end = m_begin + p.m_per_split;
     if (m_end > p.M) m_end = p.M;
-    const bool do_db = p.want_dbias && (ktile == 0);
+    const bool do_db = p.want_dbias && (ktile == 0) && !p.swap;
+    const bool do_dba = CW == 4 && p.want_dbias && p.swap;     // (the 128-wide form is the one the host swaps operands for)
 
     // ---- x: a wave loads 8 slab rows with XL loads; lane l of load j is load lane 64 j + l ----
     //      of those rows: row (64 j + l) / CPR, chunk (64 j + l) % CPR
@@ -408,6 +413,15 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
 #pragma unroll
         for (int j = 0; j < RW; ++j) dbsum += ly[(db_rg * RW + j) * kWgBN + (db_col ^ ((j & 1) << 5))];
     };
+    // swapped operands: the column sums of the x slab (rows stored plainly, RS floats each); a thread owns 4
+    // neighbouring columns of 4 rows
+    f4 dbsum_a = {0.f, 0.f, 0.f, 0.f};
+    auto add_columns_a = [&](const float* la) {
+        if constexpr (CW == 4) {
+#pragma unroll
+            for (int j = 0; j < BR / 8; ++j) dbsum_a += *reinterpret_cast<const f4*>(la + ((tid >> 5) * (BR / 8) + j) * RS + 4 * (tid & 31));
+        }
+    };
 
     f16v acc[CW];
 #pragma unroll
@@ -459,6 +473,7 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
             __builtin_amdgcn_sched_barrier(0);
         }
         if (do_db) add_columns(ly);
+        if (do_dba) add_columns_a(la);
     };
 
     if (m_begin < m_end) {
@@ -478,7 +493,7 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
     constexpr int QP = (BR * RS * 4 >= CW * 4096) ? CW : CW / 2;
     static_assert(BR * RS * 4 >= QP * 4096 && CW % QP == 0, "accumulator exchange buffer");
     f4* xch = reinterpret_cast<f4*>(nt == 0 ? lds_a0 : lds_a1);
-    const size_t split_stride = (size_t)p.K * p.D + p.D;
+    const size_t split_stride = (size_t)p.K * p.D + p.db_len;
     float* outp = p.out + (size_t)split * split_stride;
     // one split's partial block is far below 2^31 bytes (K * D < 2^29 is checked by the host)
     const __amdgpu_buffer_rsrc_t rsrc_o =
@@ -520,6 +535,19 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
         __syncthreads();
         if (tid < 64 && n0 + tid < p.D)
             (p.db_out ? p.db_out : outp + (size_t)p.K * p.D)[n0 + tid] = (lds_y0[tid] + lds_y0[64 + tid]) + (lds_y0[128 + tid] + lds_y0[192 + tid]);
+    }
+    if constexpr (CW == 4) {
+        if (do_dba) {                                    // 8 row groups x 128 columns, added in order
+            __syncthreads();
+            *reinterpret_cast<f4*>(lds_a0 + (tid >> 5) * 128 + 4 * (tid & 31)) = dbsum_a;
+            __syncthreads();
+            if (tid < 128 && kt0 + tid < p.K) {
+                float s = lds_a0[tid];
+#pragma unroll
+                for (int g = 1; g < 8; ++g) s += lds_a0[g * 128 + tid];
+                (p.db_out ? p.db_out : outp + (size_t)p.K * p.D)[kt0 + tid] = s;
+            }
+        }
     }
 }
 

@@ -442,3 +442,37 @@ def test_wgrad_with_the_whole_result_in_registers(case, tune):
     assert np.abs(dw - want).max() <= 2.0 * np.abs(ref32 - want).max() + 1e-6
     dw2, none = abi.wgrad(x, dy, w.shape, stride, pad, want_dbias=False)
     assert none is None and np.array_equal(dw, dw2)       # deterministic
+
+
+# 1x1 filters on 33 to 64 input channels and at least 128 output channels: the library multiplies dy^T . x (full-width
+# k tiles over dy's columns, one n tile over x's) and the split reduction writes the transpose back.
+WGRAD_SWAP_CASES = [
+    (2, 56, 56, 64, 256, 1, 1, 1, 1, "valid"),    # the 64 -> 256 layer
+    (3, 9, 11, 64, 128, 1, 1, 1, 1, "valid"),     # 297 rows: a last slab with 9 rows
+    (2, 14, 14, 48, 192, 1, 1, 1, 1, "valid"),    # 48 input channels, a second k tile half full
+    (1, 33, 31, 36, 132, 1, 1, 1, 1, "valid"),    # 36 and 132 channels: edge tiles in both directions
+    (5, 1, 1, 64, 320, 1, 1, 1, 1, "valid"),      # 5 rows (a dense layer's shape), three k tiles
+    (2, 28, 28, 64, 256, 1, 1, 1, 1, "same"),     # "same" on a 1x1 filter pads nothing
+]
+
+
+@pytest.mark.parametrize("case", WGRAD_SWAP_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_wgrad_of_1x1_filters_with_swapped_operands(case, tune):
+    from tests import abi
+    x, w, b, dy = _case(case, 15)
+    stride, pad = (case[7], case[8]), case[9]
+    want = O.conv_wgrad(x, dy, w.shape[:2], stride, pad, dtype=np.float64)
+    want_db = O.conv_dbias(dy, dtype=np.float64)
+    ref32 = O.conv_wgrad(x, dy, w.shape[:2], stride, pad, dtype=np.float32)
+    results = {}
+    for swap in (1, 0):
+        tune(wgrad_swap=swap)
+        dw, db = abi.wgrad(x, dy, w.shape, stride, pad)
+        abi.close(dw, want, rms_scaled=True)
+        abi.close(db, want_db, rms_scaled=True)
+        assert np.abs(dw - want).max() <= 2.0 * np.abs(ref32 - want).max() + 1e-6
+        dw2, none = abi.wgrad(x, dy, w.shape, stride, pad, want_dbias=False)
+        assert none is None and np.array_equal(dw, dw2)   # deterministic, with and without dbias
+        results[swap] = dw
+    # two orders of summation over the same products
+    assert np.allclose(results[0], results[1], rtol=1e-4, atol=1e-4 * max(1.0, float(np.abs(want).max())))
