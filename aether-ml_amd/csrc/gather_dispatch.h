@@ -121,10 +121,13 @@ static inline int gather_bn(int N) { return N <= 32 ? 32 : 64; }
 // Tile height.  The LDS-direct kernel keeps two slabs per operand in LDS, so a
 // 128-row tile (48 KB) lets three workgroups share a CU where a 256-row tile
 // (80 KB) allows one or two; measured on the 56x56x64 shape, 128 rows is 11 %
-// faster.  64-row tiles (32 KB, five per CU) run at the same rate and leave a
-// smaller last round, so fp32 takes 128 rows only from about 8 rounds of tiles on
-// (6272 tiles, 56x56x64: 0.483 ms either way; 1568 tiles, 56x56x256 batch 64: 0.503 ms
-// with 128 rows, 0.488 with 64).  The register-staged kernel prefers 256 rows.
+// faster.  64-row tiles (32 KB, five per CU) leave a smaller last round and
+// win on few tiles, 128-row tiles (wave tiles of 32 x 64: three operand reads per
+// two MFMAs instead of two per one) on many: fp32 takes 128 rows from 10 tiles per
+// CU on (128 against 64 rows on 56x56x64 -> 64 and 28x28x128 -> 128, 3x3: +10 % at
+// 784 tiles, +4 % at 1568, +1 % at 2352, -1 % at 3136, -2 % at 4704, -3 % at 5488;
+// 28x28x128 -> 256 stride 2, 2704 tiles: -3.8 %).  The register-staged kernel
+// prefers 256 rows.
 static inline int gather_bm(int M, int N, int cus, bool dma, int elem_bytes = 4) {
     const int bn = gather_bn(N);
     {                                                       // tuning override: 256, 128 or 64
@@ -139,7 +142,7 @@ static inline int gather_bm(int M, int N, int cus, bool dma, int elem_bytes = 4)
         int bm = cands[i];
         if (bn == 32 && bm == 64) break;
         const int64_t tiles = (int64_t)cdiv(M, bm) * ntiles;
-        if (dma && elem_bytes == 4 && bm == 128 && bn == 64 && tiles < 24 * (int64_t)cus) continue;
+        if (dma && elem_bytes == 4 && bm == 128 && bn == 64 && tiles < 10 * (int64_t)cus) continue;
         if (tiles >= want) return bm;
     }
     return bn == 32 ? 128 : 64;
