@@ -203,6 +203,33 @@ __global__ void bn_apply(const float* __restrict__ x, const float* __restrict__ 
     }
 }
 
+// the same on groups of 4 channels (C % 4 == 0, 16-byte aligned tensors)
+__global__ __launch_bounds__(kEwThreads) void bn_apply4(const ew_f4* __restrict__ x, const ew_f4* __restrict__ gamma,
+                                                       const ew_f4* __restrict__ beta, const ew_f4* __restrict__ mean,
+                                                       const ew_f4* __restrict__ invstd, ew_f4* __restrict__ y,
+                                                       unsigned n4, int C4) {
+    const unsigned stride = gridDim.x * blockDim.x;
+    for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+        const unsigned c4 = i % (unsigned)C4;
+        y[i] = gamma[c4] * ((x[i] - mean[c4]) * invstd[c4]) + beta[c4];
+    }
+}
+
+__global__ __launch_bounds__(kEwThreads) void bn_apply_infer4(const ew_f4* __restrict__ x, const ew_f4* __restrict__ gamma,
+                                                             const ew_f4* __restrict__ beta, const ew_f4* __restrict__ rm,
+                                                             const ew_f4* __restrict__ rv, ew_f4* __restrict__ y,
+                                                             unsigned n4, int C4, float eps) {
+    const unsigned stride = gridDim.x * blockDim.x;
+    for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+        const unsigned c4 = i % (unsigned)C4;
+        const ew_f4 v = rv[c4], d = x[i] - rm[c4];
+        ew_f4 q;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) q[e] = d[e] / sqrtf(v[e] + eps);
+        y[i] = gamma[c4] * q + beta[c4];
+    }
+}
+
 __global__ void bn_apply_infer(const float* __restrict__ x, const float* __restrict__ gamma,
                                const float* __restrict__ beta, const float* __restrict__ rm,
                                const float* __restrict__ rv, float* __restrict__ y, int64_t n, int C, float eps) {
@@ -504,6 +531,51 @@ __global__ void maxpool_fwd_kernel(const float* __restrict__ x, float* __restric
     }
 }
 
+// 4 neighbouring channels per thread (C % 4 == 0, 16-byte aligned tensors, 4-byte aligned idx): 16-byte loads, the same
+// comparisons in the same order per channel.  p.div_c divides by C / 4, p.div_w by Wo, p.div_h by Ho here.
+__global__ void maxpool_fwd_kernel4(const ew_f4* __restrict__ x, ew_f4* __restrict__ y, uint32_t* __restrict__ idx,
+                                    PoolParams p, unsigned n4) {
+    const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n4) return;
+    const unsigned C4 = (unsigned)p.C >> 2;
+    unsigned t, u, c, wo, ho, s;
+    p.div_c.divmod(i, t, c);
+    p.div_w.divmod(t, u, wo);
+    p.div_h.divmod(u, s, ho);
+    const ew_f4* base = x + ((s * p.H + ho * p.sH) * p.W + wo * p.sW) * C4 + c;
+    ew_f4 best = base[0];
+    uint32_t bi = 0;
+    for (int fh = 0; fh < p.fH; ++fh)
+        for (int fw = 0; fw < p.fW; ++fw) {
+            const ew_f4 v = base[(fh * p.W + fw) * C4];
+            const uint32_t k = (uint32_t)(fh * p.fW + fw);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (v[e] > best[e]) {    // strict: the first maximum keeps its place
+                    best[e] = v[e];
+                    bi = (bi & ~(0xffu << (8 * e))) | (k << (8 * e));
+                }
+        }
+    y[i] = best;
+    idx[i] = bi;
+}
+
+__global__ void avgpool_fwd_kernel4(const ew_f4* __restrict__ x, ew_f4* __restrict__ y, PoolParams p, unsigned n4) {
+    const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n4) return;
+    const unsigned C4 = (unsigned)p.C >> 2;
+    const float inv = 1.0f / (float)(p.fH * p.fW);
+    unsigned t, u, c, wo, ho, s;
+    p.div_c.divmod(i, t, c);
+    p.div_w.divmod(t, u, wo);
+    p.div_h.divmod(u, s, ho);
+    const ew_f4* base = x + ((s * p.H + ho * p.sH) * p.W + wo * p.sW) * C4 + c;
+    ew_f4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int fh = 0; fh < p.fH; ++fh)
+        for (int fw = 0; fw < p.fW; ++fw) acc += base[(fh * p.W + fw) * C4];
+    y[i] = acc * inv;
+}
+
 // gather form of the scatter-add: every input element sums, in (h,w) order, the
 // windows that contain it and whose argmax points at it
 __global__ void maxpool_bwd_kernel(const float* __restrict__ dy, const uint8_t* __restrict__ idx,
@@ -532,6 +604,66 @@ __global__ void maxpool_bwd_kernel(const float* __restrict__ dy, const uint8_t* 
             }
         dx[i] = acc;
     }
+}
+
+// The same for 4 neighbouring channels per thread (C % 4 == 0, 16-byte aligned tensors): 16-byte loads and stores,
+// 4-byte index loads; every element takes the sums of the scalar form in the same order.  p.div_c divides by C / 4.
+__global__ void maxpool_bwd_kernel4(const ew_f4* __restrict__ dy, const uint32_t* __restrict__ idx,
+                                    ew_f4* __restrict__ dx, PoolParams p, unsigned n4) {
+    const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n4) return;
+    const unsigned C4 = (unsigned)p.C >> 2;
+    unsigned t, u, c, col, row, s;
+    p.div_c.divmod(i, t, c);
+    p.div_w.divmod(t, u, col);
+    p.div_h.divmod(u, s, row);
+    int h_lo = (int)row - p.fH + 1;
+    h_lo = h_lo <= 0 ? 0 : (int)p.div_sh.div((unsigned)(h_lo + p.sH - 1));
+    int h_hi = (int)p.div_sh.div(row);
+    if (h_hi > p.Ho - 1) h_hi = p.Ho - 1;
+    int w_lo = (int)col - p.fW + 1;
+    w_lo = w_lo <= 0 ? 0 : (int)p.div_sw.div((unsigned)(w_lo + p.sW - 1));
+    int w_hi = (int)p.div_sw.div(col);
+    if (w_hi > p.Wo - 1) w_hi = p.Wo - 1;
+    ew_f4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int h = h_lo; h <= h_hi; ++h)
+        for (int w = w_lo; w <= w_hi; ++w) {
+            const unsigned o = ((s * p.Ho + h) * p.Wo + w) * C4 + c;
+            const unsigned want = (unsigned)(((int)row - h * p.sH) * p.fW + ((int)col - w * p.sW));
+            const uint32_t k = idx[o];
+            const ew_f4 g = dy[o];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (((k >> (8 * e)) & 0xffu) == want) acc[e] += g[e];
+        }
+    dx[i] = acc;
+}
+
+__global__ void avgpool_bwd_kernel4(const ew_f4* __restrict__ dy, ew_f4* __restrict__ dx, PoolParams p, unsigned n4) {
+    const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n4) return;
+    const unsigned C4 = (unsigned)p.C >> 2;
+    const float div = (float)(p.fH * p.fW);
+    unsigned t, u, c, col, row, s;
+    p.div_c.divmod(i, t, c);
+    p.div_w.divmod(t, u, col);
+    p.div_h.divmod(u, s, row);
+    int h_lo = (int)row - p.fH + 1;
+    h_lo = h_lo <= 0 ? 0 : (int)p.div_sh.div((unsigned)(h_lo + p.sH - 1));
+    int h_hi = (int)p.div_sh.div(row);
+    if (h_hi > p.Ho - 1) h_hi = p.Ho - 1;
+    int w_lo = (int)col - p.fW + 1;
+    w_lo = w_lo <= 0 ? 0 : (int)p.div_sw.div((unsigned)(w_lo + p.sW - 1));
+    int w_hi = (int)p.div_sw.div(col);
+    if (w_hi > p.Wo - 1) w_hi = p.Wo - 1;
+    ew_f4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int h = h_lo; h <= h_hi; ++h)
+        for (int w = w_lo; w <= w_hi; ++w) {
+            const ew_f4 g = dy[((s * p.Ho + h) * p.Wo + w) * C4 + c];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] += g[e] / div;
+        }
+    dx[i] = acc;
 }
 
 __global__ void avgpool_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, PoolParams p, int64_t n) {
@@ -935,6 +1067,13 @@ int aeth_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta,
                        running_mean, running_var, save_mean, save_invstd);
     AETH_LAUNCH_CHECK();
     int64_t n = (int64_t)rows * C;
+    if (col_vec4(C, x, y) && col_vec4(C, gamma, beta) && col_vec4(C, save_mean, save_invstd)) {
+        const unsigned n4 = (unsigned)(n / 4);
+        hipLaunchKernelGGL(bn_apply4, dim3(ew_blocks(n4)), dim3(kEwThreads), 0, st, (const ew_f4*)x, (const ew_f4*)gamma,
+                           (const ew_f4*)beta, (const ew_f4*)save_mean, (const ew_f4*)save_invstd, (ew_f4*)y, n4, C / 4);
+        AETH_LAUNCH_CHECK();
+        return AETH_OK;
+    }
     EW_LAUNCH(bn_apply, n, x, gamma, beta, save_mean, save_invstd, y, n, C);
     return AETH_OK;
 }
@@ -1051,6 +1190,14 @@ int aeth_bn_fwd_infer_f32(const float* x, const float* gamma, const float* beta,
     AETH_CHECK_ARG(x && gamma && beta && running_mean && running_var && y);
     AETH_CHECK_ARG(rows > 0 && C > 0 && (int64_t)rows * C < ((int64_t)1 << 31));
     int64_t n = (int64_t)rows * C;
+    if (col_vec4(C, x, y) && col_vec4(C, gamma, beta) && col_vec4(C, running_mean, running_var)) {
+        const unsigned n4 = (unsigned)(n / 4);
+        hipLaunchKernelGGL(bn_apply_infer4, dim3(ew_blocks(n4)), dim3(kEwThreads), 0, ctx().stream, (const ew_f4*)x,
+                           (const ew_f4*)gamma, (const ew_f4*)beta, (const ew_f4*)running_mean, (const ew_f4*)running_var,
+                           (ew_f4*)y, n4, C / 4, eps);
+        AETH_LAUNCH_CHECK();
+        return AETH_OK;
+    }
     EW_LAUNCH(bn_apply_infer, n, x, gamma, beta, running_mean, running_var, y, n, C, eps);
     return AETH_OK;
 }
@@ -1144,6 +1291,14 @@ int aeth_maxpool_fwd_f32(const float* x, float* y, uint8_t* idx, int S, int H, i
     int rc = pool_dims(__func__, S, H, W, C, fH, fW, sH, sW, &p);
     if (rc) return rc;
     int64_t n = (int64_t)S * p.Ho * p.Wo * C;
+    if (C % 4 == 0 && n > 0 && aligned16(x) && aligned16(y) && (reinterpret_cast<uintptr_t>(idx) & 3) == 0) {
+        p.div_c = FastDiv(C / 4); p.div_w = FastDiv(p.Wo); p.div_h = FastDiv(p.Ho);
+        const unsigned n4 = (unsigned)(n / 4);
+        hipLaunchKernelGGL(maxpool_fwd_kernel4, dim3(cdiv(n4, kEwThreads)), dim3(kEwThreads), 0, ctx().stream,
+                           (const ew_f4*)x, (ew_f4*)y, (uint32_t*)idx, p, n4);
+        AETH_LAUNCH_CHECK();
+        return AETH_OK;
+    }
     EW_LAUNCH(maxpool_fwd_kernel, n, x, y, idx, p, n);
     return AETH_OK;
 }
@@ -1156,6 +1311,14 @@ int aeth_maxpool_bwd_f32(const float* dy, const uint8_t* idx, float* dx, int S, 
     int rc = pool_dims(__func__, S, H, W, C, fH, fW, sH, sW, &p);
     if (rc) return rc;
     int64_t n = (int64_t)S * H * W * C;
+    if (C % 4 == 0 && aligned16(dy) && aligned16(dx) && (reinterpret_cast<uintptr_t>(idx) & 3) == 0) {
+        p.div_c = FastDiv(C / 4);
+        const unsigned n4 = (unsigned)(n / 4);
+        hipLaunchKernelGGL(maxpool_bwd_kernel4, dim3(cdiv(n4, kEwThreads)), dim3(kEwThreads), 0, ctx().stream,
+                           (const ew_f4*)dy, (const uint32_t*)idx, (ew_f4*)dx, p, n4);
+        AETH_LAUNCH_CHECK();
+        return AETH_OK;
+    }
     EW_LAUNCH(maxpool_bwd_kernel, n, dy, idx, dx, p, n);
     return AETH_OK;
 }
@@ -1167,6 +1330,14 @@ int aeth_avgpool_fwd_f32(const float* x, float* y, int S, int H, int W, int C, i
     int rc = pool_dims(__func__, S, H, W, C, fH, fW, sH, sW, &p);
     if (rc) return rc;
     int64_t n = (int64_t)S * p.Ho * p.Wo * C;
+    if (C % 4 == 0 && n > 0 && aligned16(x) && aligned16(y)) {
+        p.div_c = FastDiv(C / 4); p.div_w = FastDiv(p.Wo); p.div_h = FastDiv(p.Ho);
+        const unsigned n4 = (unsigned)(n / 4);
+        hipLaunchKernelGGL(avgpool_fwd_kernel4, dim3(cdiv(n4, kEwThreads)), dim3(kEwThreads), 0, ctx().stream,
+                           (const ew_f4*)x, (ew_f4*)y, p, n4);
+        AETH_LAUNCH_CHECK();
+        return AETH_OK;
+    }
     EW_LAUNCH(avgpool_fwd_kernel, n, x, y, p, n);
     return AETH_OK;
 }
@@ -1178,6 +1349,14 @@ int aeth_avgpool_bwd_f32(const float* dy, float* dx, int S, int H, int W, int C,
     int rc = pool_dims(__func__, S, H, W, C, fH, fW, sH, sW, &p);
     if (rc) return rc;
     int64_t n = (int64_t)S * H * W * C;
+    if (C % 4 == 0 && aligned16(dy) && aligned16(dx)) {
+        p.div_c = FastDiv(C / 4);
+        const unsigned n4 = (unsigned)(n / 4);
+        hipLaunchKernelGGL(avgpool_bwd_kernel4, dim3(cdiv(n4, kEwThreads)), dim3(kEwThreads), 0, ctx().stream,
+                           (const ew_f4*)dy, (ew_f4*)dx, p, n4);
+        AETH_LAUNCH_CHECK();
+        return AETH_OK;
+    }
     EW_LAUNCH(avgpool_bwd_kernel, n, dy, dx, p, n);
     return AETH_OK;
 }

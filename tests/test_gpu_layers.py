@@ -126,7 +126,8 @@ def test_maxpool_notebook_example_and_ties():
 
 @pytest.mark.parametrize("shape,f,s", [((4, 16, 16, 32), (2, 2), (2, 2)), ((2, 7, 6, 3), (2, 2), (2, 2)),
                                        ((2, 9, 9, 5), (3, 3), (2, 2)), ((2, 8, 8, 4), (2, 2), (1, 1)),
-                                       ((3, 10, 7, 6), (3, 2), (1, 2))])
+                                       ((3, 10, 7, 6), (3, 2), (1, 2)), ((2, 9, 10, 8), (3, 3), (2, 2)),
+                                       ((2, 11, 7, 12), (3, 2), (1, 1))])
 def test_maxpool_bit_exact(shape, f, s):
     import aether
     r = np.random.RandomState(4)
@@ -161,6 +162,15 @@ def test_avgpool_and_pooling_errors():
     dy = r.randn(*pool.output.shape).astype(np.float32)
     pool.backward(dy)
     _close(pool.dinputs, O.avgpool_backward(dy, x.shape, (3, 3), (2, 1)))
+    # channel counts that are multiples of 4 take 16-byte loads and stores: same sums
+    for shape, f, s in (((2, 9, 8, 8), (3, 3), (2, 1)), ((3, 8, 6, 12), (2, 2), (2, 2)), ((2, 7, 7, 4), (2, 3), (1, 1))):
+        x = r.randn(*shape).astype(np.float32)
+        pool = aether.Pooling(f, s, pooling_type="average")
+        pool.forward(x, True)
+        _close(pool.output, O.avgpool_forward(x, f, s))
+        dy = r.randn(*pool.output.shape).astype(np.float32)
+        pool.backward(dy)
+        _close(pool.dinputs, O.avgpool_backward(dy, x.shape, f, s))
     with pytest.raises(ValueError):
         aether.Pooling().forward(np.zeros((2, 4, 4), np.float32), True)
     with pytest.raises(ValueError):
