@@ -251,6 +251,59 @@ def bf16_layer(steps, warmup):
             "layer_over_abi": round(fed / calls, 3)}
 
 
+def layer_kernels(steps, warmup):
+    """The supporting kernels on the headline tensor, NHWC [256,56,56,64] fp32 (205.5 MB): ms per call and
+    algorithmic bytes / time.  A call that is several launches (batch norm: partial sums, their reduction,
+    the apply pass) is timed as a whole and priced with the bytes its passes must move."""
+    import ctypes as C
+    from aether import _lib
+    from aether.tensor import DeviceTensor
+    L = _lib.lib()
+    S, H, W, Ch = 256, 56, 56, 64
+    n = S * H * W * Ch
+    rows = S * H * W
+    rng = np.random.default_rng(0)
+    x = DeviceTensor.from_numpy(rng.standard_normal((S, H, W, Ch), dtype=np.float32))
+    dy = DeviceTensor.from_numpy(rng.standard_normal((S, H, W, Ch), dtype=np.float32))
+    y, y2, y3 = (DeviceTensor((S, H, W, Ch)) for _ in range(3))
+    gamma = DeviceTensor.from_numpy(np.ones(Ch, np.float32))
+    rv = DeviceTensor.from_numpy(np.ones(Ch, np.float32))
+    beta, rm, sm, si, dgamma, dbeta = (DeviceTensor.zeros(Ch) for _ in range(6))
+    pooled = DeviceTensor((S, H // 2, W // 2, Ch))
+    dpooled = DeviceTensor.from_numpy(rng.standard_normal((S, H // 2, W // 2, Ch), dtype=np.float32))
+    idx = DeviceTensor((n // 16,))                          # one byte per pooled element
+    f, i64 = C.c_float, C.c_int64
+    fp = 4 * n                                              # bytes of one full-size tensor
+    calls = [
+        ("relu_fwd", 2 * fp, lambda: L.aeth_relu_fwd_f32(x.ptr, y.ptr, f(0.0), i64(n))),
+        ("relu_bwd", 3 * fp, lambda: L.aeth_relu_bwd_f32(x.ptr, dy.ptr, y.ptr, f(0.0), i64(n))),
+        ("bn_fwd_train (3 launches)", 3 * fp, lambda: L.aeth_bn_fwd_train_f32(
+            x.ptr, gamma.ptr, beta.ptr, rm.ptr, rv.ptr, sm.ptr, si.ptr, y.ptr, rows, Ch, f(1e-5), f(0.9))),
+        ("bn_bwd (3 launches)", 5 * fp, lambda: L.aeth_bn_bwd_f32(
+            x.ptr, dy.ptr, gamma.ptr, sm.ptr, si.ptr, y.ptr, dgamma.ptr, dbeta.ptr, rows, Ch)),
+        ("maxpool_fwd 2x2/2", fp + fp // 4 + n // 4, lambda: L.aeth_maxpool_fwd_f32(
+            x.ptr, pooled.ptr, idx.ptr, S, H, W, Ch, 2, 2, 2, 2)),
+        ("maxpool_bwd 2x2/2", fp + fp // 4 + n // 4, lambda: L.aeth_maxpool_bwd_f32(
+            dpooled.ptr, idx.ptr, y.ptr, S, H, W, Ch, 2, 2, 2, 2)),
+        ("avgpool_fwd 2x2/2", fp + fp // 4, lambda: L.aeth_avgpool_fwd_f32(x.ptr, pooled.ptr, S, H, W, Ch, 2, 2, 2, 2)),
+        ("avgpool_bwd 2x2/2", fp + fp // 4, lambda: L.aeth_avgpool_bwd_f32(dpooled.ptr, y.ptr, S, H, W, Ch, 2, 2, 2, 2)),
+        ("bn_relu_maxpool2_fwd (3 launches)", 4 * fp + fp // 4 + n // 4, lambda: L.aeth_bn_relu_maxpool2_fwd_f32(
+            x.ptr, gamma.ptr, beta.ptr, rm.ptr, rv.ptr, sm.ptr, si.ptr, y.ptr, y2.ptr, pooled.ptr, idx.ptr,
+            S, H, W, Ch, f(1e-5), f(0.9), f(0.0), None)),
+        ("maxpool2_relu_bn_bwd (3 launches)", 7 * fp + fp // 4 + n // 4, lambda: L.aeth_maxpool2_relu_bn_bwd_f32(
+            dpooled.ptr, idx.ptr, y.ptr, x.ptr, gamma.ptr, sm.ptr, si.ptr, y2.ptr, y3.ptr, y.ptr, dgamma.ptr,
+            dbeta.ptr, S, H, W, Ch, f(0.0), None)),
+        ("cast_f32_to_bf16", fp + fp // 2, lambda: L.aeth_cast_f32_to_bf16(x.ptr, y.ptr, i64(n))),
+        ("fill_f32", fp, lambda: L.aeth_fill_f32(y.ptr, f(0.0), i64(n))),
+        ("memcpy_d2d", 2 * fp, lambda: L.aeth_memcpy_d2d(y.ptr, x.ptr, i64(fp))),
+    ]
+    out = {}
+    for name, nbytes, call in calls:
+        ms = _time(lambda: _lib.check(call()), steps, warmup)
+        out[name] = {"ms": round(ms, 4), "algorithmic_MB": round(nbytes / 1e6, 1), "TB_per_s": round(nbytes / ms / 1e9, 2)}
+    return out
+
+
 def run(steps, warmup):
     return {"conv_shapes": conv_table(max(20, steps), 2), "bf16_through_the_layer": bf16_layer(max(20, steps), 3),
             "train_step_cnn3": train_step(max(steps, 20), warmup)}
@@ -260,6 +313,8 @@ if __name__ == "__main__":
     import json
     if "--bf16-layer" in sys.argv:
         print(json.dumps(bf16_layer(20, 3), indent=1))
+    elif "--layers" in sys.argv:
+        print(json.dumps(layer_kernels(20, 5), indent=1))
     elif "--train-only" in sys.argv:
         print(json.dumps(train_step(50, 10), indent=1))
     elif "--shape" in sys.argv:
