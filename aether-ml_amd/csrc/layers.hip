@@ -480,14 +480,14 @@ __global__ void adam_multi_dev_kernel(const AdamTable tb, float b1, float b2, fl
     }
 }
 
-// single block: out[0] = sum |x| or sum x^2, summed in a fixed tree
+// single block: out[0] = sum |x| (mode 0), sum x^2 (1) or sum x (2), summed in a fixed tree
 __global__ __launch_bounds__(1024) void reduce_kernel(const float* __restrict__ x, int64_t n, int mode,
                                                       float* __restrict__ out) {
     __shared__ float red[1024];
     float s = 0.f;
     for (int64_t i = threadIdx.x; i < n; i += 1024) {
         float v = x[i];
-        s += mode == 0 ? fabsf(v) : v * v;
+        s += mode == 0 ? fabsf(v) : (mode == 1 ? v * v : v);
     }
     red[threadIdx.x] = s;
     __syncthreads();
@@ -496,6 +496,27 @@ __global__ __launch_bounds__(1024) void reduce_kernel(const float* __restrict__ 
         __syncthreads();
     }
     if (threadIdx.x == 0) out[0] = red[0];
+}
+
+// the same sums over `chunk` consecutive elements per block, one partial each: the first stage for long inputs
+// (the chunk size follows from n alone, so the order of the additions does too)
+__global__ __launch_bounds__(256) void reduce_chunks_kernel(const float* __restrict__ x, int64_t n, int64_t chunk, int mode,
+                                                            float* __restrict__ part) {
+    __shared__ float red[256];
+    const int64_t lo = (int64_t)blockIdx.x * chunk;
+    const int64_t hi = lo + chunk < n ? lo + chunk : n;
+    float s = 0.f;
+    for (int64_t i = lo + threadIdx.x; i < hi; i += 256) {
+        float v = x[i];
+        s += mode == 0 ? fabsf(v) : v * v;
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) part[blockIdx.x] = red[0];
 }
 
 // ---- pooling ---------------------------------------------------------------------------
@@ -1516,6 +1537,21 @@ int aeth_reduce_f32(const float* x, int64_t n, int mode, float* out) {
     AETH_REQUIRE_INIT();
     AETH_CHECK_ARG(n >= 0 && (mode == 0 || mode == 1) && out);
     AETH_CHECK_ARG(n == 0 || x);
+    // one block up to 16 Ki elements; beyond that chunks of at least 4096 on at most 1024 blocks, then their partials
+    // (a single block over the 786 432 weights of a 3072 x 256 layer: 81 us)
+    if (n > 16384) {
+        int64_t chunk = 4096;
+        while (cdiv(n, chunk) > 1024) chunk *= 2;
+        const int blocks = (int)cdiv(n, chunk);
+        void* ws;
+        int rc = workspace((int64_t)blocks * sizeof(float), &ws);
+        if (rc) return rc;
+        hipLaunchKernelGGL(reduce_chunks_kernel, dim3(blocks), dim3(256), 0, ctx().stream, x, n, chunk, mode, (float*)ws);
+        AETH_LAUNCH_CHECK();
+        hipLaunchKernelGGL(reduce_kernel, dim3(1), dim3(1024), 0, ctx().stream, (const float*)ws, (int64_t)blocks, 2, out);
+        AETH_LAUNCH_CHECK();
+        return AETH_OK;
+    }
     hipLaunchKernelGGL(reduce_kernel, dim3(1), dim3(1024), 0, ctx().stream, x, n, mode, out);
     AETH_LAUNCH_CHECK();
     return AETH_OK;

@@ -279,6 +279,25 @@ def test_flatten_softmax_loss():
         _close(comb.dinputs, O.softmax_cce_backward(p64, y, ls))
 
 
+@pytest.mark.parametrize("n", [1, 1000, 16384, 16385, 100001, 786432, 5000003])
+def test_sums_for_the_regularisers(n):
+    """aeth_reduce_f32 (sum |x| and sum x^2 behind Loss.regularization_loss, CNN_classes_cupy.py:593-609): one block
+    for short inputs, chunks and a second stage for long ones; the same bits on every call."""
+    import ctypes as C
+    import aether
+    from aether import _lib
+    L = _lib.lib()
+    x = np.random.RandomState(n % 1000).randn(n).astype(np.float32)
+    xd = aether.DeviceTensor.from_numpy(x)
+    out = aether.DeviceTensor.zeros(1)
+    for mode, want in ((0, np.abs(x.astype(np.float64)).sum()), (1, (x.astype(np.float64) ** 2).sum())):
+        _lib.check(L.aeth_reduce_f32(xd.ptr, C.c_int64(n), mode, out.ptr))
+        got = float(out.get()[0])
+        assert abs(got - want) <= 2e-6 * want + 1e-30, (n, mode, got, want)
+        _lib.check(L.aeth_reduce_f32(xd.ptr, C.c_int64(n), mode, out.ptr))
+        assert float(out.get()[0]) == got
+
+
 def test_regularization_loss_and_adam():
     import aether
     np.random.seed(9)
