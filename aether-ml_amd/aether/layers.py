@@ -626,13 +626,15 @@ class Loss:
     # ``calculate`` in two halves for Model.train_step: ``launch`` queues the loss kernel,
     # ``finish`` reads its result.  With backward and the optimizer queued in between, the
     # host never waits in the middle of a step.  Only for losses that offer
-    # ``forward_launch`` and when no regulariser is active (its sums must see the weights
-    # before the update).
+    # ``forward_launch``.  A regulariser's sums go the same way (``regularization_launch``
+    # before the update is queued, so that they see the weights the reference's see;
+    # ``regularization_finish`` after it).
     def can_defer(self):
-        if not hasattr(self, "forward_launch"):
-            return False
-        return not any(l.weight_regularizer_l1 > 0 or l.weight_regularizer_l2 > 0 or l.bias_regularizer_l1 > 0
-                       or l.bias_regularizer_l2 > 0 for l in self.trainable_layers)
+        return hasattr(self, "forward_launch")
+
+    def has_regularizer(self):
+        return any(l.weight_regularizer_l1 > 0 or l.weight_regularizer_l2 > 0 or l.bias_regularizer_l1 > 0
+                   or l.bias_regularizer_l2 > 0 for l in self.trainable_layers)
 
     def launch(self, output, y, *, training=True):
         return self.forward_launch(output, y, training)
@@ -665,23 +667,37 @@ class Loss:
         self.accumulated_sum = 0
         self.accumulated_count = 0
 
-    def _device_sum(self, t, mode):
-        out = DeviceTensor(1, _F32)
-        _ck(_L().aeth_reduce_f32(t.ptr, t.size, mode, out.ptr))
-        return float(out.get()[0])
-
-    def regularization_loss(self):
-        regularization_loss = 0
+    def regularization_launch(self):
+        """Queues the sums of Loss.regularization_loss (CNN_classes_cupy.py:593-609), sum |x| (mode 0) or
+        sum x^2 (1) per active coefficient in the reference's order, into one device buffer."""
+        terms = []
         for layer in self.trainable_layers:
             if layer.weight_regularizer_l1 > 0:
-                regularization_loss += layer.weight_regularizer_l1 * self._device_sum(layer.weights, 0)
+                terms.append((layer.weight_regularizer_l1, layer.weights, 0))
             if layer.weight_regularizer_l2 > 0:
-                regularization_loss += layer.weight_regularizer_l2 * self._device_sum(layer.weights, 1)
+                terms.append((layer.weight_regularizer_l2, layer.weights, 1))
             if layer.bias_regularizer_l1 > 0:
-                regularization_loss += layer.bias_regularizer_l1 * self._device_sum(layer.biases, 0)
+                terms.append((layer.bias_regularizer_l1, layer.biases, 0))
             if layer.bias_regularizer_l2 > 0:
-                regularization_loss += layer.bias_regularizer_l2 * self._device_sum(layer.biases, 1)
+                terms.append((layer.bias_regularizer_l2, layer.biases, 1))
+        if not terms:
+            return None
+        sums = DeviceTensor(len(terms), _F32)
+        for i, (_, t, mode) in enumerate(terms):
+            _ck(_L().aeth_reduce_f32(t.ptr, t.size, mode, sums.ptr + 4 * i))
+        return [coef for coef, _, _ in terms], sums
+
+    def regularization_finish(self, pending):
+        """One read-back for all the sums; the weighted total is added up on the host in the reference's order."""
+        regularization_loss = 0
+        if pending is not None:
+            coefs, sums = pending
+            for coef, value in zip(coefs, sums.get()):
+                regularization_loss += coef * float(value)
         return regularization_loss
+
+    def regularization_loss(self):
+        return self.regularization_finish(self.regularization_launch())
 
 
 class Loss_CategoricalCrossEntropy(Loss):

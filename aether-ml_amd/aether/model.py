@@ -193,7 +193,7 @@ class Model:
         from .layers import Layer_Dropout, Layer_Dropout_Spatial, Optimizer_Adam
         if self.softmax_classifier_output is None or not isinstance(self.optimizer, Optimizer_Adam):
             return False
-        if not self.loss.can_defer():
+        if not self.loss.can_defer() or self.loss.has_regularizer():
             return False
         if any(isinstance(layer, (Layer_Dropout, Layer_Dropout_Spatial)) for layer in self.layers):
             return False                                 # their masks are drawn and uploaded by the host every step
@@ -274,10 +274,12 @@ class Model:
                 return result
         # The loss kernel is queued here and read after backward and the update have been
         # queued too, so the device never idles while the host prepares the backward pass.
-        # With an active regulariser its sums must see the weights before the update, so
-        # the loss is then read first, as the reference does.
+        # A regulariser's sums are queued here as well: they see the weights before the update,
+        # as the reference's do (it works the loss out before backward, :113-115).
+        reg_pending = None
         if self.loss.can_defer():
             output, pending = self._forward_and_loss(batch_X, batch_y)
+            reg_pending = self.loss.regularization_launch()
         else:
             output, pending = self.forward(batch_X, training=True), None
         if pending is None:
@@ -289,7 +291,8 @@ class Model:
             self.optimizer.update_parameters(layer)
         self.optimizer.post_update_parameters()
         if pending is not None:
-            data_loss, regularization_loss = self.loss.finish(pending, include_regularization=True)
+            data_loss = self.loss.finish(pending)
+            regularization_loss = self.loss.regularization_finish(reg_pending)
         predictions = self.output_layer_activation.predictions(output)
         accuracy = self.accuracy.calculate(predictions, batch_y)
         return data_loss + regularization_loss, data_loss, regularization_loss, accuracy
