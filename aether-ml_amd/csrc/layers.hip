@@ -300,10 +300,25 @@ __global__ void bn_bwd_apply(const float* __restrict__ x, const float* __restric
 }
 
 // ---- elementwise ---------------------------------------------------------------------
+// (16-byte loads and stores over the aligned part when both pointers allow it, single floats for the rest)
 __global__ void relu_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, float alpha, int64_t n) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (; i < n; i += stride) {
+    int64_t done = 0;
+    if (((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0) {
+        const int64_t n4 = n >> 2;
+        const ew_f4* __restrict__ x4 = reinterpret_cast<const ew_f4*>(x);
+        ew_f4* __restrict__ y4 = reinterpret_cast<ew_f4*>(y);
+        for (int64_t j = i; j < n4; j += stride) {
+            const ew_f4 v = x4[j];
+            ew_f4 r;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r[e] = v[e] > 0.f ? v[e] : alpha * v[e];
+            y4[j] = r;
+        }
+        done = n4 << 2;
+    }
+    for (i += done; i < n; i += stride) {
         float v = x[i];
         y[i] = v > 0.f ? v : alpha * v;
     }
