@@ -167,14 +167,15 @@ class Model:
         normally, the second is recorded as a HIP graph, later ones replay it: one host
         call per step.  Same kernels, same order, same results; the step number and the
         learning rate live on the device.  Falls back to normal steps for models the
-        recording cannot express (dropout masks drawn on the host, active regularisers,
-        anything but Adam with the fused softmax / cross-entropy output)."""
+        recording cannot express (dropout masks drawn on the host, anything but Adam with
+        the fused softmax / cross-entropy output).  Regularisers are recorded: their sums
+        and their gradient terms are kernels like the rest."""
         self._record = bool(enabled)
         if not enabled:
             self._drop_recordings()
         elif not self._can_record():
-            warnings.warn("record_steps: this model cannot be recorded (dropout masks from the host, an active "
-                          "regulariser, or no Adam / fused softmax cross-entropy); steps run eagerly",
+            warnings.warn("record_steps: this model cannot be recorded (dropout masks from the host, "
+                          "or no Adam / fused softmax cross-entropy); steps run eagerly",
                           RuntimeWarning, stacklevel=2)
 
     @property
@@ -193,7 +194,7 @@ class Model:
         from .layers import Layer_Dropout, Layer_Dropout_Spatial, Optimizer_Adam
         if self.softmax_classifier_output is None or not isinstance(self.optimizer, Optimizer_Adam):
             return False
-        if not self.loss.can_defer() or self.loss.has_regularizer():
+        if not self.loss.can_defer():
             return False
         if any(isinstance(layer, (Layer_Dropout, Layer_Dropout_Spatial)) for layer in self.layers):
             return False                                 # their masks are drawn and uploaded by the host every step
@@ -228,6 +229,7 @@ class Model:
             L._recording[0] = True
             try:
                 output, rec["pending"] = self._forward_and_loss(rec["x"], batch_y)
+                rec["reg_pending"] = self.loss.regularization_launch()      # (before the update, as in train_step)
                 rec["output"] = output
                 self.backward(output, batch_y)
                 self.optimizer.record_update(self.trainable_layers)
@@ -258,7 +260,8 @@ class Model:
         if self.layers[-1].__dict__.get("output") is not rec["output"]:
             for obj, name, val in rec["bindings"]:
                 setattr(obj, name, val)
-        data_loss, regularization_loss = self.loss.finish(rec["pending"], include_regularization=True)
+        data_loss = self.loss.finish(rec["pending"])
+        regularization_loss = self.loss.regularization_finish(rec.get("reg_pending"))
         loss = data_loss + regularization_loss
         predictions = self.output_layer_activation.predictions(rec["output"])
         accuracy = self.accuracy.calculate(predictions, batch_y)

@@ -147,3 +147,35 @@ def test_mlp_recipe_train_loop_prints_the_reference_lines(capsys):
     for la, lb in zip(a.trainable_layers, b.trainable_layers):
         for pa, pb in zip(la.get_parameters(), lb.get_parameters()):
             assert np.array_equal(np.asarray(pa), np.asarray(pb))
+
+
+def test_mlp_recipe_recorded_steps_equal_eager_steps():
+    """The recipe has no dropout, so `record_steps` may replay it: the regulariser's sums and gradient terms are kernels of
+    the recording.  Same kernels in the same order: losses (data and regularisation), learning rate and parameters
+    must agree exactly with the steps launched from Python, replay after replay."""
+    import aether
+
+    def make():
+        np.random.seed(8)
+        m = mlp_model(aether)
+        _scaled(m, aether)
+        m.loss.new_pass()
+        m.accuracy.new_pass()
+        return m
+
+    rng = np.random.RandomState(12)
+    Xs = [rng.rand(128, 3072).astype(np.float32) for _ in range(2)]
+    ys = [rng.randint(0, 10, 128) for _ in range(2)]
+    eager, rec = make(), make()
+    rec.record_steps(True)
+    assert rec.recording_active
+    for step in range(6):
+        a = eager.train_step(Xs[step % 2], ys[step % 2])
+        b = rec.train_step(Xs[step % 2], ys[step % 2])
+        assert a == b, "step %d: eager %r, recorded %r" % (step, a, b)
+        assert a[2] > 1e-3                                   # the regularisation loss is part of the comparison
+        assert eager.optimizer.current_learning_rate == rec.optimizer.current_learning_rate
+        for la, lb in zip(eager.trainable_layers, rec.trainable_layers):
+            assert np.array_equal(np.asarray(la.weights), np.asarray(lb.weights)), "weights differ after step %d" % step
+            assert np.array_equal(np.asarray(la.biases), np.asarray(lb.biases)), "biases differ after step %d" % step
+    assert len([r for r in rec._recordings.values() if r.get("graph")]) == 1
