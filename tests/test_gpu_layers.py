@@ -401,3 +401,20 @@ def test_fused_block_entry_points_reject_what_they_do_not_cover():
     assert L.aeth_bn_relu_maxpool2_fwd_f32(*args2, 4, 4, 4, 8, 1e-5, 0.9, 0.0, p16.ptr) == 0
     assert np.all(np.isfinite(pool.get())) and np.array_equal(p16.get(), O.bf16_bits(pool.get()))
 
+
+
+@pytest.mark.parametrize("nbytes", [4, 65536, 262144 - 4, 262144, 262144 + 4, 1572864, 2097152, 2097152 + 4, 5000000])
+def test_host_copies_through_the_staging_slots(nbytes):
+    """aeth_memcpy_h2d sends up to 2 MB through pinned slots of 256 KB, piece by piece, and returns at once; the
+    source may be overwritten right after the call.  Sizes around a slot, around all 8 slots, and beyond."""
+    import aether
+    r = np.random.RandomState(nbytes % 977)
+    n = nbytes // 4
+    src = r.randint(0, 1 << 30, n).astype(np.int32)
+    want = src.copy()
+    t = aether.DeviceTensor((n,), dtype=np.int32)
+    t.set(src)
+    src[:] = -1                                    # the call has taken its copy
+    again = aether.DeviceTensor.from_numpy(want)   # a second copy queued behind the first: slots are reused in order
+    assert np.array_equal(t.get(), want)
+    assert np.array_equal(again.get(), want)
