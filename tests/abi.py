@@ -1,5 +1,8 @@
 """Thin helpers the GPU parity tests use to call the C ABI directly (through
 ctypes) on NumPy inputs and get NumPy outputs back."""
+import json
+import os
+
 import numpy as np
 
 from aether import _lib
@@ -97,3 +100,35 @@ def wgrad_bf16(x, dy, w_shape, strides, padding):
     db = DeviceTensor.full(w_shape[3], np.nan)
     _lib.check(_lib.lib().aeth_conv_wgrad_bf16(xd.ptr, dyd.ptr, dw.ptr, db.ptr, *dims))
     return dw.get(), db.get()
+
+
+# ---- the benchmark's input recipe and the parity figures quoted beside its timings ----
+def baseline_inputs(kind, x_shape, num_filters, filter_size=(3, 3), strides=(1, 1), padding="same"):
+    """Inputs of one benchmark configuration, drawn the way the benchmark draws them: the legacy global RNG
+    seeded with 0, then in this order the input (`kind`: "rand" = U[0,1), "randn" = N(0,1), "relu_randn" =
+    N(0,1) clipped at 0), the layer (its constructor draws the He-normal filter, CNN_classes_cupy.py:61-66; zero
+    bias) and the upstream gradient N(0,1).  Returns x, w, b, dy as float32 host arrays."""
+    import aether
+    np.random.seed(0)
+    if kind == "rand":
+        x = np.random.rand(*x_shape).astype(np.float32)
+    else:
+        x = np.random.randn(*x_shape).astype(np.float32)
+        if kind == "relu_randn":
+            x = np.maximum(x, 0)
+    layer = aether.Conv_Layer(x_shape[1:], num_filters=num_filters, filter_size=filter_size, strides=strides,
+                              padding=padding)
+    w, b = layer.filter_weights.get(), layer.biases.get()
+    _, yshape = conv_dims(x.shape, w.shape, strides, padding)
+    dy = np.random.randn(*yshape).astype(np.float32)
+    return x, w, b, dy
+
+
+def report(config, direction, worst, note=""):
+    """Appends one measured max err/tol to the file $AETHER_PARITY_REPORT names (JSON lines), if it names one:
+    the source of the parity table that stands beside the benchmark's timings."""
+    path = os.environ.get("AETHER_PARITY_REPORT")
+    if path:
+        with open(path, "a") as f:
+            f.write(json.dumps({"config": config, "direction": direction, "max_err_over_tol": worst,
+                                "note": note}) + "\n")

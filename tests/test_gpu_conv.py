@@ -124,6 +124,41 @@ def test_wgrad_parity(case):
     assert none is None and np.array_equal(dw, dw2)       # deterministic
 
 
+# The benchmark's first configurations at their exact workload: shape, input distribution and draw order.
+BASELINE_SMALL = [
+    ("cfg1 [128,32,32,3] U[0,1) -> 32", "rand", (128, 32, 32, 3), 32),
+    ("cfg2a [128,16,16,32] relu(N(0,1)) -> 64", "relu_randn", (128, 16, 16, 32), 64),
+    ("cfg2b [128,8,8,64] relu(N(0,1)) -> 128", "relu_randn", (128, 8, 8, 64), 128),
+]
+
+
+@pytest.mark.parametrize("cfg", BASELINE_SMALL, ids=lambda c: c[0].split()[0])
+def test_baseline_configs_at_their_exact_workload(cfg):
+    """3x3, stride 1, "same": every output element of fprop and dgrad within 1e-5 + 1e-4*|oracle|; wgrad and dbias
+    under the same bar with the absolute term scaled by max(1, rms) (tests/abi.py says why), and no further from
+    the float64 value than twice the reference arithmetic run in float32."""
+    from tests import abi
+    name, kind, x_shape, D = cfg
+    x, w, b, dy = abi.baseline_inputs(kind, x_shape, D)
+    assert not b.any() and w.shape == (3, 3, x_shape[3], D)
+    if kind != "randn":
+        assert x.min() >= 0
+    st, pad = (1, 1), "same"
+    abi.report(name, "fprop", abi.close(abi.fprop(x, w, b, st, pad), O.conv_fprop(x, w, b, st, pad, dtype=np.float64)))
+    abi.report(name, "dgrad", abi.close(abi.dgrad(dy, w, x.shape, st, pad),
+                                        O.conv_dgrad(dy, w, x.shape[1:3], st, pad, dtype=np.float64)))
+    dw, db = abi.wgrad(x, dy, w.shape, st, pad)
+    want = O.conv_wgrad(x, dy, (3, 3), st, pad, dtype=np.float64)
+    rms = float(np.sqrt(np.mean(want * want)))
+    abi.report(name, "wgrad", abi.close(dw, want, rms_scaled=True), "atol * max(1, rms), rms = %.3g" % rms)
+    abi.report(name, "dbias", abi.close(db, O.conv_dbias(dy, dtype=np.float64), rms_scaled=True))
+    ref32 = O.conv_wgrad(x, dy, (3, 3), st, pad, dtype=np.float32)
+    assert np.abs(dw - want).max() <= 2.0 * np.abs(ref32 - want).max() + 1e-6
+    abi.report(name, "wgrad vs float32 reference arithmetic",
+               float(np.abs(dw - want).max() / max(np.abs(ref32 - want).max(), 1e-30)),
+               "max |gpu - f64| / max |f32 einsum - f64|")
+
+
 def test_bad_arguments_are_errors_not_crashes():
     from aether import _lib
     from aether.tensor import DeviceTensor

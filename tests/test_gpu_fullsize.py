@@ -33,12 +33,24 @@ def whole_tensor_close(got, oracle_of_rows, S, chunk=8, threads=8):
     with ThreadPoolExecutor(max_workers=threads) as pool:
         return max(pool.map(check, spans))
 
+def whole_batch_wgrad(x, dy, filter_size, stride, pad, chunk=8, threads=8):
+    """The oracle's float64 wgrad of the whole batch: the sum of its wgrads of the chunks (wgrad is additive over
+    samples; float64 addition of 32 to 128 partial results does not touch the digits compared)."""
+    spans = [(lo, min(lo + chunk, x.shape[0])) for lo in range(0, x.shape[0], chunk)]
+    with ThreadPoolExecutor(max_workers=threads) as pool:
+        parts = pool.map(lambda s: O.conv_wgrad(x[s[0]:s[1]], dy[s[0]:s[1]], filter_size, stride, pad,
+                                                dtype=np.float64), spans)
+        return sum(parts)
+
+
 FULL = [
     # name, S, H, W, C, D, fH, fW, stride, padding
     ("resnet3x3", 256, 56, 56, 64, 64, 3, 3, 1, "same"),
     ("resnet1x1", 256, 56, 56, 64, 256, 1, 1, 1, "valid"),
     ("wide_s2", 1024, 28, 28, 128, 256, 3, 3, 2, "valid"),
 ]
+LABEL = {"resnet3x3": "cfg4 [256,56,56,64] N(0,1) -> 64, 3x3", "resnet1x1": "cfg4' [256,56,56,64] N(0,1) -> 256, 1x1 valid",
+         "wide_s2": "cfg5 [1024,28,28,128] N(0,1) -> 256, 3x3 stride 2 valid"}
 
 
 @pytest.mark.parametrize("cfg", FULL, ids=lambda c: c[0])
@@ -48,12 +60,10 @@ def test_full_size_conv(cfg, tune):
     from tests import abi
     name, S, H, W, C, D, fH, fW, st, pad = cfg
     stride = (st, st)
-    rng = np.random.default_rng(0)
-    x = rng.standard_normal((S, H, W, C), dtype=np.float32)
-    w = (rng.standard_normal((fH, fW, C, D), dtype=np.float32) * np.float32(np.sqrt(2.0 / (fH * fW * C))))
-    b = rng.standard_normal(D, dtype=np.float32)
+    # the benchmark's draw: seed 0, input, layer constructor, upstream gradient; then a bias that is not zero
+    x, w, _, dy = abi.baseline_inputs("randn", (S, H, W, C), D, (fH, fW), stride, pad)
+    b = np.random.randn(D).astype(np.float32)
     dims, yshape = abi.conv_dims(x.shape, w.shape, stride, pad)
-    dy = rng.standard_normal(yshape, dtype=np.float32)
     L = _lib.lib()
     xd, wd, bd, dyd = (DeviceTensor.from_numpy(a) for a in (x, w, b, dy))
     y = DeviceTensor.full(yshape, np.nan)
@@ -67,8 +77,10 @@ def test_full_size_conv(cfg, tune):
     assert np.all(np.isfinite(y_h)) and np.all(np.isfinite(dx_h))
 
     # every element against the oracle
-    whole_tensor_close(y_h, lambda lo, hi: O.conv_fprop(x[lo:hi], w, b, stride, pad, dtype=np.float64), S)
-    whole_tensor_close(dx_h, lambda lo, hi: O.conv_dgrad(dy[lo:hi], w, (H, W), stride, pad, dtype=np.float64), S)
+    abi.report(LABEL[name], "fprop", whole_tensor_close(
+        y_h, lambda lo, hi: O.conv_fprop(x[lo:hi], w, b, stride, pad, dtype=np.float64), S))
+    abi.report(LABEL[name], "dgrad", whole_tensor_close(
+        dx_h, lambda lo, hi: O.conv_dgrad(dy[lo:hi], w, (H, W), stride, pad, dtype=np.float64), S))
     # and bit for bit against the library's other kernels for these shapes
     tune(**OTHER_KERNELS)
     y2 = DeviceTensor.full(yshape, np.nan)
@@ -91,7 +103,11 @@ def test_full_size_conv(cfg, tune):
     scale = float(np.sqrt(np.sum(y_h.astype(np.float64) ** 2)) * np.sqrt(np.sum(dy.astype(np.float64) ** 2)))
     assert abs(lhs - rhs_x) <= 1e-6 * scale, (lhs, rhs_x)
     assert abs(lhs - rhs_w) <= 1e-6 * scale, (lhs, rhs_w)
-    abi.close(db_h, np.sum(dy.astype(np.float64), axis=(0, 1, 2)), rms_scaled=True)
+    abi.report(LABEL[name], "dbias", abi.close(db_h, np.sum(dy.astype(np.float64), axis=(0, 1, 2)), rms_scaled=True))
+    # every element of wgrad against the oracle's float64 sum over the whole batch
+    want = whole_batch_wgrad(x, dy, (fH, fW), stride, pad)
+    abi.report(LABEL[name], "wgrad", abi.close(dw_h, want, rms_scaled=True),
+               "atol * max(1, rms), rms = %.3g" % float(np.sqrt(np.mean(want * want))))
 
     # wgrad of a gradient supported on one sample == the oracle's wgrad of that sample
     for s in (0, S - 1):

@@ -11,6 +11,7 @@ import numpy as np
 import pytest
 
 from oracle import oracle as O
+from tests import step_checks as SC
 from tests.test_gpu_model import host_params, outside_share, rel_l2
 
 pytestmark = pytest.mark.gpu
@@ -96,6 +97,7 @@ def test_mlp_recipe_steps_match_oracle():
     model.loss.new_pass()
     model.accuracy.new_pass()
     for step in range(3):
+        before = SC.snapshot(model)
         ref = net.step(X, y)
         loss, data_loss, reg_loss, acc = model.train_step(X, y)
         assert ref["reg_loss"] > 1e-3
@@ -112,11 +114,9 @@ def test_mlp_recipe_steps_match_oracle():
                 assert rel_l2(layer.dweights.get(), gw.reshape(layer.dweights.shape)) <= 2e-4, i
                 assert outside_share(layer.dweights.get(), gw.reshape(layer.dweights.shape)) <= 1e-3, i
                 assert rel_l2(layer.dbiases.get(), gb.reshape(layer.dbiases.shape)) <= 2e-4, i
-        lr_allow = 2e-3 * (step + 1)
-        for i, layer in enumerate(model.trainable_layers):
-            got = [np.asarray(a) for a in layer.get_parameters()]
-            for j, want in enumerate(net.p[i]):
-                assert np.all(np.abs(got[j].reshape(want.shape) - want) <= lr_allow + 1e-3 * np.abs(want)), (step, i, j)
+        SC.check_update_from_own_state(model, before, ref["lr"], step)
+        if step == 0:
+            SC.check_update_against_oracle(model, before, net.p, ref["grads"], ref["lr"])
     probs_eval, _, _ = net.forward(X)
     assert rel_l2(model.predict(X, batch_size=50), probs_eval) <= 5e-3
 
