@@ -103,11 +103,12 @@ class Conv_Layer:
         set_parameters change the version).  While a step is being recorded the cast always
         runs, so that it is part of the recording."""
         w = self.filter_weights
-        key = (w.ptr, w._version)
-        if _recording[0] or getattr(self, "_w16_key", None) != key:
+        # keyed on the tensor object, not its address: the allocator hands a freed block's address out again
+        fresh = getattr(self, "_w16_src", None) is w and getattr(self, "_w16_version", None) == w._version
+        if _recording[0] or not fresh:
             out = DeviceTensor(w.shape, np.uint16)
             _ck(_L().aeth_cast_f32_to_bf16(w.ptr, out.ptr, w.size))
-            self._w16, self._w16_key = out, key
+            self._w16, self._w16_src, self._w16_version = out, w, w._version
         return self._w16
 
     def forward(self, inputs, training):

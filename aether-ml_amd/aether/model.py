@@ -339,6 +339,25 @@ class Model:
         for layer in reversed(walk):
             layer.backward(layer.next.dinputs)
 
+    def backward_debug(self, X, y):
+        """One training forward and backward pass that prints every layer's output shape, then every
+        layer's gradient shapes (CNN_model_cupy.py:195-229); the reference's scripts call it on one
+        sample before training.  No loss is computed and no parameter changes."""
+        print("Forward pass:")
+        self.input_layer.forward(X, True)
+        for i, layer in enumerate(self.layers):
+            layer.forward(layer.prev.output, True)
+            print(f"Layer {i} ({layer.__class__.__name__}) output: {tuple(layer.output.shape)}")
+        print("\nBackward pass:")
+        self.backward(self.layers[-1].output, y)
+        fused = self.softmax_classifier_output is not None
+        walk = self.layers[:-1] if fused else self.layers
+        for i, layer in enumerate(reversed(walk)):
+            print(f"Layer {-i - (2 if fused else 1)} ({layer.__class__.__name__}) dinputs: {tuple(layer.dinputs.shape)}")
+            for name in ("dweights", "dbiases"):
+                if hasattr(layer, name):
+                    print(f"             {name}: {tuple(getattr(layer, name).shape)}")
+
     def evaluate(self, X_val, y_val, *, batch_size=None):
         self.loss.new_pass()
         self.accuracy.new_pass()
@@ -395,6 +414,20 @@ class Accuracy:
 
     def calculate_accumulated(self):
         return self.accumulated_sum / self.accumulated_count
+
+
+class Accuracy_Regression(Accuracy):
+    """A prediction counts as correct within std(y) / 250 of the target (CNN_model_cupy.py:367-378)."""
+
+    def __init__(self):
+        self.precision = None
+
+    def init(self, y, reinit=False):
+        if self.precision is None or reinit:
+            self.precision = np.std(np.asarray(y)) / 250
+
+    def compare(self, predictions, y):
+        return np.absolute(np.asarray(predictions) - np.asarray(y)) < self.precision
 
 
 class Accuracy_Categorical(Accuracy):

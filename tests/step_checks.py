@@ -37,6 +37,11 @@ def snapshot(model):
     that do not exist yet (no step taken) count as zeros, as the reference creates them."""
     snap = []
     for layer in model.trainable_layers:
+        if layer.weights is None:
+            # a batch norm before its first forward pass: it will create gamma = 1, beta = 0 over the channels
+            # it then sees (CNN_classes_cupy.py:453-460); the checks fill the shapes in from the gradients
+            snap.append(None)
+            continue
         w, b = np.asarray(layer.weights, dtype=np.float64), np.asarray(layer.biases, dtype=np.float64)
         if hasattr(layer, "weight_cache"):
             mw, vw = np.asarray(layer.weight_momentums, np.float64), np.asarray(layer.weight_cache, np.float64)
@@ -45,6 +50,14 @@ def snapshot(model):
             mw, vw, mb, vb = np.zeros_like(w), np.zeros_like(w), np.zeros_like(b), np.zeros_like(b)
         snap.append(((w, mw, vw), (b, mb, vb)))
     return snap
+
+
+def _lazy(entry, layer):
+    """A snapshot entry; for a layer that had no parameters yet, the values its first forward pass gives them."""
+    if entry is not None:
+        return entry
+    w, b = np.ones(np.asarray(layer.weights).shape), np.zeros(np.asarray(layer.biases).shape)
+    return ((w, np.zeros_like(w), np.zeros_like(w)), (b, np.zeros_like(b), np.zeros_like(b)))
 
 
 def update_errors(theta0, g, m0, v0, theta1, m1, v1, lr, iterations, eps=1e-7, beta1=0.9, beta2=0.999):
@@ -63,7 +76,8 @@ def update_errors(theta0, g, m0, v0, theta1, m1, v1, lr, iterations, eps=1e-7, b
 
 def check_update_from_own_state(model, before, lr, iterations, eps=1e-7):
     """`before` = snapshot(model) taken before the step; the layers now hold the step's gradients and results."""
-    for i, (layer, (sw, sb)) in enumerate(zip(model.trainable_layers, before)):
+    for i, (layer, entry) in enumerate(zip(model.trainable_layers, before)):
+        sw, sb = _lazy(entry, layer)
         for name, (t0, m0, v0), g, t1, m1, v1 in (
                 ("weights", sw, layer.dweights, layer.weights, layer.weight_momentums, layer.weight_cache),
                 ("biases", sb, layer.dbiases, layer.biases, layer.bias_momentums, layer.bias_cache)):
@@ -90,7 +104,8 @@ def check_update_against_oracle(model, before, oracle_params, oracle_grads, lr, 
     """First step only: `before` = snapshot(model) before it, `oracle_params` / `oracle_grads` the oracle
     network's parameters after and gradients of the same step.  Returns what was measured per tensor."""
     seen = []
-    for i, (layer, (sw, sb)) in enumerate(zip(model.trainable_layers, before)):
+    for i, (layer, entry) in enumerate(zip(model.trainable_layers, before)):
+        sw, sb = _lazy(entry, layer)
         for j, (name, (t0, _, _), t1) in enumerate((("weights", sw, layer.weights), ("biases", sb, layer.biases))):
             g = np.asarray(oracle_grads[i][j], np.float64)
             if np.linalg.norm(g) <= 1e-12:

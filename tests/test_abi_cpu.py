@@ -111,6 +111,30 @@ def test_two_dimensional_targets_must_be_one_hot():
         _sparse_labels(np.array([[1.0, 1.0, 0.0]]))
 
 
+def test_accuracy_classes_follow_the_reference():
+    """Accuracy_Regression (CNN_model_cupy.py:367-378): correct within std(y)/250, a precision kept until
+    `reinit`; Accuracy_Categorical (:380-387): one-hot targets are reduced to indices.  Host-only classes."""
+    import numpy as np
+    import aether
+    assert set(aether.__all__) >= {"Accuracy", "Accuracy_Regression", "Accuracy_Categorical", "Layer_Input", "Model"}
+    y = np.array([[0.0], [250.0], [500.0]])
+    acc = aether.Accuracy_Regression()
+    acc.init(y)
+    assert acc.precision == np.std(y) / 250
+    acc.new_pass()
+    hits = acc.calculate(y + np.array([[0.5], [-0.9], [0.1]]), y)      # precision = 0.8165
+    assert hits == 2 / 3
+    acc.calculate(y, y)
+    assert acc.calculate_accumulated() == 5 / 6
+    acc.init(y * 2)
+    assert acc.precision == np.std(y) / 250                 # kept
+    acc.init(y * 2, reinit=True)
+    assert acc.precision == np.std(y * 2) / 250
+    cat = aether.Accuracy_Categorical()
+    cat.new_pass()
+    assert cat.calculate(np.array([2, 0, 1]), np.eye(3)[[2, 1, 1]]) == 2 / 3
+
+
 def test_debug_switches_are_known_by_name(lib):
     """aeth_debug_set may be called before aeth_init: known names are accepted, -1 and NULL reset,
     an unknown name is refused with a message that names it."""

@@ -101,6 +101,31 @@ def test_conv_layer_bf16_precision_switch():
     _loose(layer.dbiases.get(), O.conv_dbias(dy, dtype=np.float64))
 
 
+def test_bf16_filter_follows_parameters_set_twice_in_a_row():
+    """The layer keeps a bfloat16 copy of its filter.  Two set_parameters calls without a forward pass between
+    them can put the second filter at the address the first one had (the allocator hands a freed block out
+    again): the copy must follow the tensor, not the address."""
+    import aether
+    np.random.seed(6)
+    layer = aether.Conv_Layer((10, 10, 16), num_filters=32)
+    layer.precision = "bf16"
+    x = np.random.randn(3, 10, 10, 16).astype(np.float32)
+    layer.forward(x, False)
+    b = np.zeros(32, np.float32)
+    p1 = np.random.randn(3, 3, 16, 32).astype(np.float32)
+    p2 = np.random.randn(3, 3, 16, 32).astype(np.float32)
+    for rounds in range(3):                                  # the first filter's block is free from the second round on
+        layer.set_parameters(p1, b)
+        layer.set_parameters(p2, b)
+        got = layer.forward(x, False).get()
+        fresh = aether.Conv_Layer((10, 10, 16), num_filters=32)
+        fresh.precision = "bf16"
+        fresh.set_parameters(p2, b)
+        assert np.array_equal(got, fresh.forward(x, False).get()), rounds
+        layer.set_parameters(p1, b)
+        assert not np.array_equal(got, layer.forward(x, False).get())
+
+
 # Unit-stride gathers over whole 64-channel blocks on images of about a multiple of 256 pixels
 # take the kernel that keeps the source pixels of a tile in LDS for all taps.  Small inputs
 # would split K instead; the tuning switch turns that off so that they reach the same code.

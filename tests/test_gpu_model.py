@@ -390,3 +390,30 @@ def test_recording_refuses_calls_that_wait_for_the_device():
         assert np.all(t.get() == 2)
     _lib.check(lib.aeth_graph_destroy(g))
     assert lib.aeth_graph_end(C.byref(g)) == _lib.AETH_E_STATE
+
+
+def test_backward_debug_prints_the_reference_lines(capsys):
+    """Model.backward_debug (CNN_model_cupy.py:195-229), as the reference's scripts call it on one sample
+    (CNN/architectures/CNN_test2.py:75): every layer's output shape, then every layer's gradient shapes walking back."""
+    import aether
+    np.random.seed(11)
+    X = np.random.rand(1, 16, 16, 3).astype(np.float32)
+    y = np.random.randint(0, 10, 1)
+    model = build_model(aether, hw=16)
+    before = [np.asarray(p) for layer in model.trainable_layers if type(layer).__name__ != "Batch_Norm"
+              for p in layer.get_parameters()]
+    model.backward_debug(X, y)
+    out = capsys.readouterr().out.splitlines()
+    assert out[0] == "Forward pass:"
+    assert out[1] == "Layer 0 (Conv_Layer) output: (1, 16, 16, 32)"
+    assert out[len(model.layers)] == "Layer %d (SoftMax) output: (1, 10)" % (len(model.layers) - 1)
+    i = out.index("Backward pass:")
+    assert out[i - 1] == ""
+    assert out[i + 1] == "Layer -2 (Layer_Dense) dinputs: (1, 256)"
+    assert out[i + 2] == "             dweights: (256, 10)"
+    assert out[i + 3] == "             dbiases: (1, 10)"
+    assert out[-3] == "Layer -%d (Conv_Layer) dinputs: (1, 16, 16, 3)" % len(model.layers)
+    assert out[-2] == "             dweights: (3, 3, 3, 32)" and out[-1] == "             dbiases: (32,)"
+    after = [np.asarray(p) for layer in model.trainable_layers if type(layer).__name__ != "Batch_Norm"
+             for p in layer.get_parameters()]
+    assert all(np.array_equal(a, b) for a, b in zip(before, after))
