@@ -64,6 +64,9 @@ SIGNATURES = {
     "aeth_cce_fwd_f32": [_p, _p, _f, _p, _p, _i, _i],
     "aeth_softmax_cce_bwd_f32": [_p, _p, _f, _p, _i, _i],
     "aeth_softmax_cce_train_f32": [_p, _p, _f, _p, _p, _p, _p, _i, _i],
+    "aeth_cce_fwd_dense_f32": [_p, _p, _f, _p, _p, _i, _i],
+    "aeth_softmax_cce_bwd_dense_f32": [_p, _p, _f, _p, _i, _i],
+    "aeth_softmax_cce_train_dense_f32": [_p, _p, _f, _p, _p, _p, _p, _i, _i],
     "aeth_adam_f32": [_p, _p, _p, _p, _i64, _f, _f, _f, _f, _i],
     "aeth_adam_multi_f32": [_i, _p, _p, _p, _p, _p, _f, _f, _f, _f, _i],
     "aeth_adam_state_step": [_p, _d, _d, _d, _d],

@@ -12,10 +12,7 @@ Departures from the reference, each deliberate:
     "same" (the reference slices ``[:, 0:-0]`` to an empty array, :149-151);
   * ``Conv_Layer.set_parameters`` refreshes the ``weights`` alias (:159-161 does not);
   * ``Pooling(padding="same")`` raises ValueError (the reference reads ``H_out``
-    before assigning it, :226-228);
-  * 2-D ``y_true`` must be one-hot rows (they are reduced to class indices for the
-    loss kernels).  The reference multiplies a 2-D ``y_true`` in as given (:622-626,
-    :672-676), so soft or pre-smoothed targets work there; here they raise ValueError.
+    before assigning it, :226-228).
 """
 import os
 
@@ -36,6 +33,7 @@ def _ck(rc):
 
 
 _recording = [False]        # a training step is being recorded (Model sets it around the capture)
+_recorded_masks = []        # while recording: (dropout layer, the device buffer its recorded kernels read the mask from)
 
 
 def _wants_bf16(layer):
@@ -302,17 +300,24 @@ class Layer_Dropout:
         self.rate = 1 - rate
         self.fixed_mask = None
 
+    def host_mask(self, shape):
+        """This step's mask on the host: Bernoulli(keep) / keep from the legacy global RNG (:375-376), or `fixed_mask`."""
+        if self.fixed_mask is not None:
+            return np.ascontiguousarray(np.broadcast_to(np.asarray(self.fixed_mask, dtype=_F32), shape))
+        return (np.random.binomial(1, self.rate, size=shape) / self.rate).astype(_F32)
+
     def forward(self, inputs, training):
         inputs = as_device(inputs, _F32)
         self.inputs = inputs
         if not training:
             self.output = inputs.copy()
             return self.output
-        if self.fixed_mask is not None:
-            mask = np.asarray(self.fixed_mask, dtype=_F32)
+        if _recording[0]:
+            # the recorded kernels read the mask from this buffer; Model fills it before every replay
+            self.binary_mask = DeviceTensor(inputs.shape, _F32)
+            _recorded_masks.append((self, self.binary_mask))
         else:
-            mask = (np.random.binomial(1, self.rate, size=inputs.shape) / self.rate).astype(_F32)
-        self.binary_mask = DeviceTensor.from_numpy(np.broadcast_to(mask, inputs.shape), _F32)
+            self.binary_mask = DeviceTensor.from_numpy(self.host_mask(inputs.shape), _F32)
         self.output = DeviceTensor(inputs.shape, _F32)
         _ck(_L().aeth_mul_mask_f32(inputs.ptr, self.binary_mask.ptr, self.output.ptr, inputs.size, inputs.size))
         return self.output
@@ -329,6 +334,12 @@ class Layer_Dropout_Spatial:
         self.keep_prob = 1 - rate
         self.fixed_mask = None
 
+    def host_mask(self, shape):
+        """One draw per channel, shared by the whole batch (:397-398), or `fixed_mask`."""
+        if self.fixed_mask is not None:
+            return np.asarray(self.fixed_mask, dtype=_F32).reshape(shape)
+        return (np.random.binomial(1, self.keep_prob, size=shape) / self.keep_prob).astype(_F32)
+
     def forward(self, inputs, training):
         inputs = as_device(inputs, _F32)
         self.inputs = inputs
@@ -336,11 +347,11 @@ class Layer_Dropout_Spatial:
             self.output = inputs.copy()
             return self.output
         C = inputs.shape[-1]
-        if self.fixed_mask is not None:
-            mask = np.asarray(self.fixed_mask, dtype=_F32).reshape(1, 1, 1, C)
+        if _recording[0]:
+            self.channel_mask = DeviceTensor((1, 1, 1, C), _F32)    # filled by Model before every replay
+            _recorded_masks.append((self, self.channel_mask))
         else:
-            mask = (np.random.binomial(1, self.keep_prob, size=(1, 1, 1, C)) / self.keep_prob).astype(_F32)
-        self.channel_mask = DeviceTensor.from_numpy(mask, _F32)
+            self.channel_mask = DeviceTensor.from_numpy(self.host_mask((1, 1, 1, C)), _F32)
         self.output = DeviceTensor(inputs.shape, _F32)
         _ck(_L().aeth_mul_mask_f32(inputs.ptr, self.channel_mask.ptr, self.output.ptr, inputs.size, C))
         return self.output
@@ -588,36 +599,39 @@ class SoftMax:
 # ----------------------------------------------------------------------------------
 # Loss  (CNN_classes_cupy.py:565-680)
 # ----------------------------------------------------------------------------------
-def _sparse_labels(y_true):
-    """int32 class indices; one-hot rows are reduced with argmax.  Rows that are not
-    one-hot (soft or already smoothed targets) are refused rather than silently
-    replaced by their argmax."""
+def _targets(y_true):
+    """What the loss kernels take for `y_true`: ("index", int32 class indices) for a vector of labels or for
+    one-hot rows, ("dense", float32 [S, K]) for any other 2-D array: soft or already smoothed targets, which the
+    reference multiplies in as given (:622-626, :672-676)."""
     y = np.asarray(y_true)
     if y.ndim == 2:
         idx = np.argmax(y, axis=1)
         onehot = np.zeros(y.shape, dtype=y.dtype)
         onehot[np.arange(y.shape[0]), idx] = 1
-        if not np.array_equal(y, onehot):
-            raise ValueError("2-D y_true must hold one-hot rows: soft or pre-smoothed targets are not supported "
-                             "(use class indices and the loss's label_smoothing)")
-        y = idx
-    return np.ascontiguousarray(y, dtype=np.int32)
+        if np.array_equal(y, onehot):
+            return "index", np.ascontiguousarray(idx, dtype=np.int32)
+        return "dense", np.ascontiguousarray(y, dtype=_F32)
+    return "index", np.ascontiguousarray(y, dtype=np.int32)
 
 
-_label_cache = [None, None]     # (bytes of the last label batch, its device copy)
-_label_buffer = [None]          # while a step is being recorded: the buffer its kernels read labels from
+_label_cache = [None, None]     # (kind and bytes of the last target batch, its device copy)
+_label_buffer = [None]          # while a step is being recorded: (kind, the buffer its kernels read the targets from)
 
 
-def _device_labels(y_true):
-    """Labels on the device; the forward and backward pass of one step share the upload."""
+def _device_targets(y_true):
+    """(kind, targets on the device); the forward and backward pass of one step share the upload."""
     if _label_buffer[0] is not None:
         return _label_buffer[0]
-    y = _sparse_labels(y_true)
-    key = y.tobytes()
+    kind, y = _targets(y_true)
+    key = (kind, y.shape, y.tobytes())
     if _label_cache[0] != key:
         _label_cache[0] = key
-        _label_cache[1] = DeviceTensor.from_numpy(y, np.int32)
-    return _label_cache[1]
+        _label_cache[1] = DeviceTensor.from_numpy(y, y.dtype)
+    return kind, _label_cache[1]
+
+
+def _for_targets(kind, index_fn, dense_fn):
+    return getattr(_L(), index_fn if kind == "index" else dense_fn)
 
 
 class Loss:
@@ -711,11 +725,12 @@ class Loss_CategoricalCrossEntropy(Loss):
     def forward_launch(self, y_pred, y_true, training=True):
         y_pred = as_device(y_pred, _F32)
         rows, K = y_pred.shape
-        labels = _device_labels(y_true)
+        kind, labels = _device_targets(y_true)
         ls = self.label_smoothing if (self.label_smoothing > 0 and training) else 0.0
         # per-sample loss and row argmax side by side: one read-back for both
         buf = DeviceTensor(2 * rows, _F32)
-        _ck(_L().aeth_cce_fwd_f32(y_pred.ptr, labels.ptr, ls, buf.ptr, buf.ptr + 4 * rows, rows, K))
+        fn = _for_targets(kind, "aeth_cce_fwd_f32", "aeth_cce_fwd_dense_f32")
+        _ck(fn(y_pred.ptr, labels.ptr, ls, buf.ptr, buf.ptr + 4 * rows, rows, K))
         return buf, rows, y_pred
 
     def forward_finish(self, pending):
@@ -731,13 +746,13 @@ class Loss_CategoricalCrossEntropy(Loss):
         separate launches."""
         logits = as_device(logits, _F32)
         rows, K = logits.shape
-        labels = _device_labels(y_true)
+        kind, labels = _device_targets(y_true)
         ls = self.label_smoothing if self.label_smoothing > 0 else 0.0
         probs = DeviceTensor(logits.shape, _F32)
         buf = DeviceTensor(2 * rows, _F32)
         dlogits = DeviceTensor(logits.shape, _F32)
-        _ck(_L().aeth_softmax_cce_train_f32(logits.ptr, labels.ptr, ls, probs.ptr, buf.ptr, buf.ptr + 4 * rows,
-                                            dlogits.ptr, rows, K))
+        fn = _for_targets(kind, "aeth_softmax_cce_train_f32", "aeth_softmax_cce_train_dense_f32")
+        _ck(fn(logits.ptr, labels.ptr, ls, probs.ptr, buf.ptr, buf.ptr + 4 * rows, dlogits.ptr, rows, K))
         softmax.output = probs
         fused.dinputs = dlogits
         fused._done_for = probs
@@ -746,9 +761,10 @@ class Loss_CategoricalCrossEntropy(Loss):
     def backward(self, dvalues, y_true):
         dvalues = as_device(dvalues, _F32)
         rows, K = dvalues.shape
-        labels = _device_labels(y_true)
+        kind, labels = _device_targets(y_true)
         self.dinputs = DeviceTensor(dvalues.shape, _F32)
-        _ck(_L().aeth_softmax_cce_bwd_f32(dvalues.ptr, labels.ptr, self.label_smoothing, self.dinputs.ptr, rows, K))
+        fn = _for_targets(kind, "aeth_softmax_cce_bwd_f32", "aeth_softmax_cce_bwd_dense_f32")
+        _ck(fn(dvalues.ptr, labels.ptr, self.label_smoothing, self.dinputs.ptr, rows, K))
 
 
 class Activation_Softmax_Loss_CategoricalCrossEntropy():
@@ -769,10 +785,11 @@ class Activation_Softmax_Loss_CategoricalCrossEntropy():
             return
         dvalues = as_device(dvalues, _F32)
         rows, K = dvalues.shape
-        labels = _device_labels(y_true)
+        kind, labels = _device_targets(y_true)
         ls = self.label_smoothing if (self.label_smoothing > 0 and training) else 0.0
         self.dinputs = DeviceTensor(dvalues.shape, _F32)
-        _ck(_L().aeth_softmax_cce_bwd_f32(dvalues.ptr, labels.ptr, ls, self.dinputs.ptr, rows, K))
+        fn = _for_targets(kind, "aeth_softmax_cce_bwd_f32", "aeth_softmax_cce_bwd_dense_f32")
+        _ck(fn(dvalues.ptr, labels.ptr, ls, self.dinputs.ptr, rows, K))
 
 
 # ----------------------------------------------------------------------------------

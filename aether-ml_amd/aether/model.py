@@ -166,17 +166,18 @@ class Model:
         Python (no counterpart in the reference).  The first step of a batch shape runs
         normally, the second is recorded as a HIP graph, later ones replay it: one host
         call per step.  Same kernels, same order, same results; the step number and the
-        learning rate live on the device.  Falls back to normal steps for models the
-        recording cannot express (dropout masks drawn on the host, anything but Adam with
-        the fused softmax / cross-entropy output).  Regularisers are recorded: their sums
-        and their gradient terms are kernels like the rest."""
+        learning rate live on the device.  Dropout masks are still drawn on the host, in
+        the layers' order from the reference's random stream, and copied into the buffers
+        the recorded kernels read before every replay.  Regularisers are recorded: their
+        sums and their gradient terms are kernels like the rest.  Falls back to normal
+        steps for models the recording cannot express (anything but Adam with the fused
+        softmax / cross-entropy output)."""
         self._record = bool(enabled)
         if not enabled:
             self._drop_recordings()
         elif not self._can_record():
-            warnings.warn("record_steps: this model cannot be recorded (dropout masks from the host, "
-                          "or no Adam / fused softmax cross-entropy); steps run eagerly",
-                          RuntimeWarning, stacklevel=2)
+            warnings.warn("record_steps: this model cannot be recorded (no Adam / fused softmax cross-entropy); "
+                          "steps run eagerly", RuntimeWarning, stacklevel=2)
 
     @property
     def recording_active(self):
@@ -191,21 +192,17 @@ class Model:
         self._recordings = {}
 
     def _can_record(self):
-        from .layers import Layer_Dropout, Layer_Dropout_Spatial, Optimizer_Adam
+        from .layers import Optimizer_Adam
         if self.softmax_classifier_output is None or not isinstance(self.optimizer, Optimizer_Adam):
             return False
-        if not self.loss.can_defer():
-            return False
-        if any(isinstance(layer, (Layer_Dropout, Layer_Dropout_Spatial)) for layer in self.layers):
-            return False                                 # their masks are drawn and uploaded by the host every step
-        return True
+        return self.loss.can_defer()
 
     def _recorded_step(self, batch_X, batch_y):
         import ctypes as C
         from . import _lib, layers as L
         from .tensor import DeviceTensor
-        labels = L._sparse_labels(batch_y)
-        key = (tuple(batch_X.shape), labels.shape[0])
+        kind, labels = L._targets(batch_y)
+        key = (tuple(batch_X.shape), kind, labels.shape)
         recs = self.__dict__.setdefault("_recordings", {})
         rec = recs.get(key)
         if rec is None or not all(hasattr(l, "weight_cache") for l in self.trainable_layers):
@@ -222,11 +219,12 @@ class Model:
             recs[key] = rec = {"graph": None}
         if rec["graph"] is None:
             rec["x"] = DeviceTensor(batch_X.shape, np.float32)
-            rec["labels"] = DeviceTensor(labels.shape, np.int32)
+            rec["labels"] = DeviceTensor(labels.shape, labels.dtype)
             self.optimizer.device_state()
             _lib.check(lib.aeth_graph_begin())
-            L._label_buffer[0] = rec["labels"]
+            L._label_buffer[0] = (kind, rec["labels"])
             L._recording[0] = True
+            del L._recorded_masks[:]
             try:
                 output, rec["pending"] = self._forward_and_loss(rec["x"], batch_y)
                 rec["reg_pending"] = self.loss.regularization_launch()      # (before the update, as in train_step)
@@ -236,6 +234,8 @@ class Model:
             finally:
                 L._label_buffer[0] = None
                 L._recording[0] = False
+                rec["masks"] = list(L._recorded_masks)      # in the order the forward pass met the dropout layers
+                del L._recorded_masks[:]
                 handle = C.c_void_p()
                 rc = lib.aeth_graph_end(C.byref(handle))
             _lib.check(rc)
@@ -255,6 +255,8 @@ class Model:
         else:
             rec["x"].set(np.asarray(batch_X, dtype=np.float32))
         rec["labels"].set(labels)
+        for layer, buffer in rec["masks"]:                  # this step's dropout masks, drawn in the layers' order
+            buffer.set(layer.host_mask(buffer.shape))
         _lib.check(lib.aeth_graph_launch(rec["graph"]))
         self.optimizer.replayed()
         if self.layers[-1].__dict__.get("output") is not rec["output"]:

@@ -775,14 +775,31 @@ __global__ void softmax_bwd_kernel(const float* __restrict__ probs, const float*
     for (int k = 0; k < K; ++k) dx[(size_t)r * K + k] = p[k] * (g[k] - dot);
 }
 
-__global__ void cce_fwd_kernel(const float* __restrict__ probs, const int32_t* __restrict__ labels, float ls,
+// The target row of a sample: class indices (the one-hot row of labels[r]) or a dense row of K floats given by
+// the caller (soft or already smoothed targets, CNN_classes_cupy.py:622-626 uses a 2-D y_true as it is).  Label
+// smoothing is the reference's t (1 - ls) + ls / K (:626-628) in both forms; for a one-hot row the dense form
+// gives the very floats of the index form.
+struct IndexTargets {
+    const int32_t* __restrict__ labels;
+    __device__ __forceinline__ float at(int r, int k, float ls, float t_off) const {
+        return (k == labels[r]) ? (1.0f - ls) + t_off : t_off;
+    }
+};
+struct DenseTargets {
+    const float* __restrict__ t;
+    int K;
+    __device__ __forceinline__ float at(int r, int k, float ls, float t_off) const {
+        return t[(size_t)r * K + k] * (1.0f - ls) + t_off;
+    }
+};
+
+template <typename Targets>
+__global__ void cce_fwd_kernel(const float* __restrict__ probs, const Targets tg, float ls,
                                float* __restrict__ loss, int32_t* __restrict__ pred, int rows, int K) {
     int r = blockIdx.x * blockDim.x + threadIdx.x;
     if (r >= rows) return;
     const float* p = probs + (size_t)r * K;
-    const int y = labels[r];
     const float t_off = ls / (float)K;
-    const float t_on = (1.0f - ls) + t_off;
     float acc = 0.f;
     float best = p[0];
     int bi = 0;
@@ -793,26 +810,26 @@ __global__ void cce_fwd_kernel(const float* __restrict__ probs, const int32_t* _
             bi = k;
         }
         float pc = fminf(fmaxf(v, 1e-7f), 1.0f - 1e-7f);
-        float t = (k == y) ? t_on : t_off;
-        acc += t * logf(pc);
+        acc += tg.at(r, k, ls, t_off) * logf(pc);
     }
     loss[r] = -acc;
     pred[r] = bi;
 }
 
-__global__ void softmax_cce_bwd_kernel(const float* __restrict__ probs, const int32_t* __restrict__ labels, float ls,
+template <typename Targets>
+__global__ void softmax_cce_bwd_kernel(const float* __restrict__ probs, const Targets tg, float ls,
                                        float* __restrict__ dlogits, int rows, int K) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= rows * K) return;
     int r = i / K, k = i - r * K;
     const float t_off = ls / (float)K;
-    float t = (k == labels[r]) ? (1.0f - ls) + t_off : t_off;
-    dlogits[i] = (probs[i] - t) / (float)rows;
+    dlogits[i] = (probs[i] - tg.at(r, k, ls, t_off)) / (float)rows;
 }
 
 // softmax, the loss with the row argmax and the gradient of the logits in one pass over a row: the three kernels above
 // one after the other, with the same operations in the same order (a training step's classifier head)
-__global__ void softmax_cce_train_kernel(const float* __restrict__ logits, const int32_t* __restrict__ labels, float ls,
+template <typename Targets>
+__global__ void softmax_cce_train_kernel(const float* __restrict__ logits, const Targets tg, float ls,
                                          float* __restrict__ probs, float* __restrict__ loss, int32_t* __restrict__ pred,
                                          float* __restrict__ dlogits, int rows, int K) {
     int r = blockIdx.x * blockDim.x + threadIdx.x;
@@ -828,9 +845,7 @@ __global__ void softmax_cce_train_kernel(const float* __restrict__ logits, const
         out[k] = e;
         sum += e;
     }
-    const int y = labels[r];
     const float t_off = ls / (float)K;
-    const float t_on = (1.0f - ls) + t_off;
     float acc = 0.f;
     float best = 0.f;
     int bi = 0;
@@ -842,7 +857,7 @@ __global__ void softmax_cce_train_kernel(const float* __restrict__ logits, const
             bi = k;
         }
         const float pc = fminf(fmaxf(v, 1e-7f), 1.0f - 1e-7f);
-        const float t = (k == y) ? t_on : t_off;
+        const float t = tg.at(r, k, ls, t_off);
         acc += t * logf(pc);
         dl[k] = (v - t) / (float)rows;
     }
@@ -852,7 +867,8 @@ __global__ void softmax_cce_train_kernel(const float* __restrict__ logits, const
 
 // The same for at most 16 classes with 16 lanes per row: the exponentials and logarithms of a row are worked out side by
 // side, the sums are added by the row's first lane in the order of the one-thread form (same bits).
-__global__ void softmax_cce_train16_kernel(const float* __restrict__ logits, const int32_t* __restrict__ labels, float ls,
+template <typename Targets>
+__global__ void softmax_cce_train16_kernel(const float* __restrict__ logits, const Targets tg, float ls,
                                            float* __restrict__ probs, float* __restrict__ loss, int32_t* __restrict__ pred,
                                            float* __restrict__ dlogits, int rows, int K) {
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
@@ -866,10 +882,8 @@ __global__ void softmax_cce_train16_kernel(const float* __restrict__ logits, con
     float sum = 0.f;
     for (int j = 0; j < K; ++j) sum += __shfl(e, base + j, 64);
     const float v = e / sum;
-    const int y = labels[r];
     const float t_off = ls / (float)K;
-    const float t_on = (1.0f - ls) + t_off;
-    const float tk = (k == y) ? t_on : t_off;
+    const float tk = mine ? tg.at(r, k, ls, t_off) : t_off;
     const float term = tk * logf(fminf(fmaxf(v, 1e-7f), 1.0f - 1e-7f));
     float acc = 0.f, best = 0.f;
     int bi = 0;
@@ -1422,40 +1436,80 @@ int aeth_softmax_bwd_f32(const float* probs, const float* dy, float* dx, int row
     return AETH_OK;
 }
 
-int aeth_cce_fwd_f32(const float* probs, const int32_t* labels, float label_smoothing, float* sample_loss,
-                     int32_t* pred, int rows, int K) {
+extern "C++" {
+template <typename Targets>
+static int cce_fwd_impl(const char* fn, const float* probs, const Targets tg, const void* targets, float label_smoothing,
+                        float* sample_loss, int32_t* pred, int rows, int K) {
     AETH_REQUIRE_INIT();
-    AETH_CHECK_ARG(probs && labels && sample_loss && pred && rows > 0 && K > 0);
-    hipLaunchKernelGGL(cce_fwd_kernel, dim3(cdiv(rows, 64)), dim3(64), 0, ctx().stream, probs, labels,
+    if (!(probs && targets && sample_loss && pred && rows > 0 && K > 0)) return fail(AETH_E_INVALID, "%s: argument check failed", fn);
+    hipLaunchKernelGGL(cce_fwd_kernel<Targets>, dim3(cdiv(rows, 64)), dim3(64), 0, ctx().stream, probs, tg,
                        label_smoothing, sample_loss, pred, rows, K);
     AETH_LAUNCH_CHECK();
     return AETH_OK;
 }
 
-int aeth_softmax_cce_bwd_f32(const float* probs, const int32_t* labels, float label_smoothing, float* dlogits,
-                             int rows, int K) {
+template <typename Targets>
+static int softmax_cce_bwd_impl(const char* fn, const float* probs, const Targets tg, const void* targets,
+                                float label_smoothing, float* dlogits, int rows, int K) {
     AETH_REQUIRE_INIT();
-    AETH_CHECK_ARG(probs && labels && dlogits && rows > 0 && K > 0);
-    AETH_CHECK_ARG((int64_t)rows * K < ((int64_t)1 << 31));
-    hipLaunchKernelGGL(softmax_cce_bwd_kernel, dim3(cdiv((int64_t)rows * K, 256)), dim3(256), 0, ctx().stream, probs,
-                       labels, label_smoothing, dlogits, rows, K);
+    if (!(probs && targets && dlogits && rows > 0 && K > 0 && (int64_t)rows * K < ((int64_t)1 << 31)))
+        return fail(AETH_E_INVALID, "%s: argument check failed", fn);
+    hipLaunchKernelGGL(softmax_cce_bwd_kernel<Targets>, dim3(cdiv((int64_t)rows * K, 256)), dim3(256), 0, ctx().stream,
+                       probs, tg, label_smoothing, dlogits, rows, K);
     AETH_LAUNCH_CHECK();
     return AETH_OK;
 }
 
-int aeth_softmax_cce_train_f32(const float* logits, const int32_t* labels, float label_smoothing, float* probs,
-                               float* sample_loss, int32_t* pred, float* dlogits, int rows, int K) {
+template <typename Targets>
+static int softmax_cce_train_impl(const char* fn, const float* logits, const Targets tg, const void* targets,
+                                  float label_smoothing, float* probs, float* sample_loss, int32_t* pred, float* dlogits,
+                                  int rows, int K) {
     AETH_REQUIRE_INIT();
-    AETH_CHECK_ARG(logits && labels && probs && sample_loss && pred && dlogits && rows > 0 && K > 0);
-    AETH_CHECK_ARG((int64_t)rows * K < ((int64_t)1 << 31));
+    if (!(logits && targets && probs && sample_loss && pred && dlogits && rows > 0 && K > 0 &&
+          (int64_t)rows * K < ((int64_t)1 << 31)))
+        return fail(AETH_E_INVALID, "%s: argument check failed", fn);
     if (K <= 16 && (int64_t)rows * 16 < ((int64_t)1 << 31))
-        hipLaunchKernelGGL(softmax_cce_train16_kernel, dim3(cdiv((int64_t)rows * 16, 256)), dim3(256), 0, ctx().stream, logits,
-                           labels, label_smoothing, probs, sample_loss, pred, dlogits, rows, K);
+        hipLaunchKernelGGL(softmax_cce_train16_kernel<Targets>, dim3(cdiv((int64_t)rows * 16, 256)), dim3(256), 0,
+                           ctx().stream, logits, tg, label_smoothing, probs, sample_loss, pred, dlogits, rows, K);
     else
-        hipLaunchKernelGGL(softmax_cce_train_kernel, dim3(cdiv(rows, 64)), dim3(64), 0, ctx().stream, logits, labels,
+        hipLaunchKernelGGL(softmax_cce_train_kernel<Targets>, dim3(cdiv(rows, 64)), dim3(64), 0, ctx().stream, logits, tg,
                            label_smoothing, probs, sample_loss, pred, dlogits, rows, K);
     AETH_LAUNCH_CHECK();
     return AETH_OK;
+}
+
+}  // extern "C++"
+
+int aeth_cce_fwd_f32(const float* probs, const int32_t* labels, float label_smoothing, float* sample_loss,
+                     int32_t* pred, int rows, int K) {
+    return cce_fwd_impl(__func__, probs, IndexTargets{labels}, labels, label_smoothing, sample_loss, pred, rows, K);
+}
+
+int aeth_cce_fwd_dense_f32(const float* probs, const float* targets, float label_smoothing, float* sample_loss,
+                           int32_t* pred, int rows, int K) {
+    return cce_fwd_impl(__func__, probs, DenseTargets{targets, K}, targets, label_smoothing, sample_loss, pred, rows, K);
+}
+
+int aeth_softmax_cce_bwd_f32(const float* probs, const int32_t* labels, float label_smoothing, float* dlogits,
+                             int rows, int K) {
+    return softmax_cce_bwd_impl(__func__, probs, IndexTargets{labels}, labels, label_smoothing, dlogits, rows, K);
+}
+
+int aeth_softmax_cce_bwd_dense_f32(const float* probs, const float* targets, float label_smoothing, float* dlogits,
+                                   int rows, int K) {
+    return softmax_cce_bwd_impl(__func__, probs, DenseTargets{targets, K}, targets, label_smoothing, dlogits, rows, K);
+}
+
+int aeth_softmax_cce_train_f32(const float* logits, const int32_t* labels, float label_smoothing, float* probs,
+                               float* sample_loss, int32_t* pred, float* dlogits, int rows, int K) {
+    return softmax_cce_train_impl(__func__, logits, IndexTargets{labels}, labels, label_smoothing, probs, sample_loss, pred,
+                                  dlogits, rows, K);
+}
+
+int aeth_softmax_cce_train_dense_f32(const float* logits, const float* targets, float label_smoothing, float* probs,
+                                     float* sample_loss, int32_t* pred, float* dlogits, int rows, int K) {
+    return softmax_cce_train_impl(__func__, logits, DenseTargets{targets, K}, targets, label_smoothing, probs, sample_loss,
+                                  pred, dlogits, rows, K);
 }
 
 int aeth_adam_f32(float* theta, const float* grad, float* m, float* v, int64_t n, float lr, float beta1, float beta2,

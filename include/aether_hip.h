@@ -232,6 +232,16 @@ int aeth_softmax_cce_bwd_f32(const float* probs, const int32_t* labels, float la
  * aeth_cce_fwd_f32 and the gradient of aeth_softmax_cce_bwd_f32, with their operations in their order (same bits). */
 int aeth_softmax_cce_train_f32(const float* logits, const int32_t* labels, float label_smoothing, float* probs,
                                float* sample_loss, int32_t* pred, float* dlogits, int rows, int K);
+/* The three calls above for a 2-D y_true that is not one-hot: soft or already smoothed targets, which the
+ * reference multiplies in as given (:622-626, :672-676).  targets[rows][K] takes the place of the labels;
+ * label smoothing is applied to it as to the one-hot rows, t (1 - ls) + ls / K (:626-628).  For one-hot rows
+ * the results are bit-identical to the index forms. */
+int aeth_cce_fwd_dense_f32(const float* probs, const float* targets, float label_smoothing,
+                           float* sample_loss, int32_t* pred, int rows, int K);
+int aeth_softmax_cce_bwd_dense_f32(const float* probs, const float* targets, float label_smoothing,
+                                   float* dlogits, int rows, int K);
+int aeth_softmax_cce_train_dense_f32(const float* logits, const float* targets, float label_smoothing, float* probs,
+                                     float* sample_loss, int32_t* pred, float* dlogits, int rows, int K);
 /* Optimizer_Adam.update_parameters for one tensor :702-734; t = iterations (0-based). */
 int aeth_adam_f32(float* theta, const float* grad, float* m, float* v, int64_t n,
                   float lr, float beta1, float beta2, float eps, int t);

@@ -96,19 +96,22 @@ def test_product_package_does_not_import_the_oracle():
                 assert "oracle" not in text, os.path.join(dirpath, f)
 
 
-def test_two_dimensional_targets_must_be_one_hot():
-    """Host logic of the loss: one-hot rows become class indices, anything softer is refused
-    (the loss kernels take indices; the reference would use the rows as given)."""
+def test_targets_are_indices_or_dense_rows():
+    """Host logic of the loss: labels and one-hot rows become class indices; any other 2-D array (soft or
+    already smoothed targets, which the reference uses as given, CNN_classes_cupy.py:622-626) goes to the
+    kernels as dense float32 rows."""
     import numpy as np
-    import pytest
-    from aether.layers import _sparse_labels
+    from aether.layers import _targets
     y = np.array([2, 0, 1])
-    assert _sparse_labels(y).dtype == np.int32 and list(_sparse_labels(y)) == [2, 0, 1]
-    assert list(_sparse_labels(np.eye(3)[y])) == [2, 0, 1]
-    with pytest.raises(ValueError):
-        _sparse_labels(np.eye(3)[y] * 0.9 + 0.1 / 3)
-    with pytest.raises(ValueError):
-        _sparse_labels(np.array([[1.0, 1.0, 0.0]]))
+    kind, t = _targets(y)
+    assert kind == "index" and t.dtype == np.int32 and list(t) == [2, 0, 1]
+    kind, t = _targets(np.eye(3)[y])
+    assert kind == "index" and list(t) == [2, 0, 1]
+    soft = np.eye(3)[y] * 0.9 + 0.1 / 3
+    kind, t = _targets(soft)
+    assert kind == "dense" and t.dtype == np.float32 and t.shape == (3, 3) and np.allclose(t, soft)
+    kind, t = _targets(np.array([[1.0, 1.0, 0.0]]))
+    assert kind == "dense"
 
 
 def test_accuracy_classes_follow_the_reference():

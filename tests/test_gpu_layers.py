@@ -279,6 +279,55 @@ def test_flatten_softmax_loss():
         _close(comb.dinputs, O.softmax_cce_backward(p64, y, ls))
 
 
+@pytest.mark.parametrize("K", [10, 16, 37])
+def test_soft_targets(K):
+    """2-D targets that are not one-hot (CNN_classes_cupy.py:622-626, :672-676 use them as given): the loss, both
+    backward forms and the one-launch head take dense rows; one-hot rows handed in as dense rows give the very
+    bits of the index form."""
+    import aether
+    from aether import _lib
+    from aether.tensor import DeviceTensor
+    r = np.random.RandomState(18)
+    S = 77
+    logits = (r.randn(S, K) * 3).astype(np.float32)
+    t = (r.rand(S, K) ** 3).astype(np.float32)
+    t /= t.sum(axis=1, keepdims=True)
+    p64 = O.softmax(logits.astype(np.float64))
+    sm = aether.SoftMax()
+    sm.forward(logits, True)
+    for ls in (0.0, 0.05):
+        loss = aether.Loss_CategoricalCrossEntropy(label_smoothing=ls)
+        loss.new_pass()
+        loss.remember_trainable_layers([])
+        per_sample = loss.forward(sm.output, t, training=True)
+        _close(per_sample, O.cce_forward(p64, t.astype(np.float64), ls, training=True))
+        _close(loss.forward(sm.output, t, training=False), O.cce_forward(p64, t.astype(np.float64), ls, training=False))
+        assert np.array_equal(sm.predictions(sm.output), np.argmax(p64, axis=1))
+        want = O.softmax_cce_backward(p64, t.astype(np.float64), ls)
+        comb = aether.Activation_Softmax_Loss_CategoricalCrossEntropy(ls)
+        comb.backward(sm.output, t, training=True)
+        _close(comb.dinputs, want)
+        loss.backward(sm.output, t)
+        _close(loss.dinputs, want)
+        # the head of a training step in one launch
+        head, fused = aether.SoftMax(), aether.Activation_Softmax_Loss_CategoricalCrossEntropy(ls)
+        pending = loss.head_launch(DeviceTensor.from_numpy(logits), t, head, fused)
+        _close(loss.forward_finish(pending), O.cce_forward(p64, t.astype(np.float64), ls, training=True))
+        assert np.array_equal(head.output.get(), sm.output.get())
+        assert np.array_equal(fused.dinputs.get(), comb.dinputs.get())
+    # one-hot rows through the dense entry points == the index entry points, bit for bit
+    L = _lib.lib()
+    y = r.randint(0, K, S).astype(np.int32)
+    lg, yd, td = DeviceTensor.from_numpy(logits), DeviceTensor.from_numpy(y, np.int32), DeviceTensor.from_numpy(np.eye(K, dtype=np.float32)[y])
+    outs = []
+    for fn, tg in ((L.aeth_softmax_cce_train_f32, yd), (L.aeth_softmax_cce_train_dense_f32, td)):
+        probs, buf, dl = DeviceTensor.full((S, K), np.nan), DeviceTensor.full(2 * S, np.nan), DeviceTensor.full((S, K), np.nan)
+        _lib.check(fn(lg.ptr, tg.ptr, 0.1, probs.ptr, buf.ptr, buf.ptr + 4 * S, dl.ptr, S, K))
+        outs.append((probs.get(), buf.get(), dl.get()))
+    assert all(np.array_equal(a, b) for a, b in zip(*outs))
+    assert L.aeth_cce_fwd_dense_f32(lg.ptr, None, 0.0, lg.ptr, lg.ptr, S, K) == _lib.AETH_E_INVALID
+
+
 @pytest.mark.parametrize("n", [1, 1000, 16384, 16385, 100001, 786432, 5000003])
 def test_sums_for_the_regularisers(n):
     """aeth_reduce_f32 (sum |x| and sum x^2 behind Loss.regularization_loss, CNN_classes_cupy.py:593-609): one block

@@ -179,3 +179,49 @@ def test_mlp_recipe_recorded_steps_equal_eager_steps():
             assert np.array_equal(np.asarray(la.weights), np.asarray(lb.weights)), "weights differ after step %d" % step
             assert np.array_equal(np.asarray(la.biases), np.asarray(lb.biases)), "biases differ after step %d" % step
     assert len([r for r in rec._recordings.values() if r.get("graph")]) == 1
+
+
+def test_mlp_recipe_with_soft_targets_recorded_and_eager():
+    """Model.train_step with a 2-D y_true of class probabilities (mixed labels): the loss and the gradients of the first
+    step against the oracle, the accuracy from the rows' argmax (CNN_model_cupy.py:384-386), and recorded steps
+    bit-identical to eager ones (the recording reads the dense targets from a buffer fed before every replay)."""
+    import aether
+    from tests import abi
+
+    def make():
+        np.random.seed(8)
+        m = mlp_model(aether)
+        _scaled(m, aether)
+        m.loss.new_pass()
+        m.accuracy.new_pass()
+        return m
+
+    rng = np.random.RandomState(15)
+    X = rng.rand(128, 3072).astype(np.float32)
+    ys = []
+    for _ in range(2):
+        a, b = np.eye(10)[rng.randint(0, 10, 128)], np.eye(10)[rng.randint(0, 10, 128)]
+        lam = rng.rand(128, 1)
+        ys.append((lam * a + (1 - lam) * b).astype(np.float32))
+    eager, rec = make(), make()
+    net = OracleMlp(host_params(eager))
+    rec.record_steps(True)
+    for step in range(5):
+        y = ys[step % 2]
+        before = SC.snapshot(eager)
+        a = eager.train_step(X, y)
+        b = rec.train_step(X, y)
+        assert a == b, "step %d: eager %r, recorded %r" % (step, a, b)
+        if step == 0:
+            probs, ins, pre = net.forward(X)
+            want = float(np.mean(O.cce_forward(probs, y.astype(np.float64), 0.0)))
+            assert abs(a[1] - want) <= 1e-5 + 1e-4 * want
+            assert a[3] == float(np.mean(np.argmax(probs, axis=1) == np.argmax(y, axis=1)))
+            d = O.softmax_cce_backward(probs, y.astype(np.float64), 0.0)
+            dw, db, _ = O.dense_backward(ins[-1], net.p[-1][0], net.p[-1][1], d, wl2=WIDTHS[-1][2], bl2=WIDTHS[-1][2],
+                                         dtype=np.float64)
+            abi.close(eager.trainable_layers[-1].dweights.get(), dw, rms_scaled=True)
+        SC.check_update_from_own_state(eager, before, eager.optimizer.current_learning_rate, step)
+        for la, lb in zip(eager.trainable_layers, rec.trainable_layers):
+            assert np.array_equal(np.asarray(la.weights), np.asarray(lb.weights)), step
+    assert len([r for r in rec._recordings.values() if r.get("graph")]) == 1

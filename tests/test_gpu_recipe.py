@@ -54,7 +54,10 @@ def draw_masks(rng, S):
             "dense": (rng.binomial(1, 1 - 0.075, size=(S, 256)) / (1 - 0.075)).astype(np.float32)}
 
 
-def test_cifar1_recipe_steps_match_oracle():
+@pytest.mark.parametrize("recorded", [False, True], ids=["eager", "recorded"])
+def test_cifar1_recipe_steps_match_oracle(recorded):
+    """`recorded`: the same steps through Model.record_steps(True): step 0 runs eagerly, step 1 is recorded as a HIP
+    graph and launched, steps 2 and 3 replay it with that step's masks copied into the buffers the graph reads."""
     import aether
     from tests import abi
     np.random.seed(0)
@@ -71,12 +74,13 @@ def test_cifar1_recipe_steps_match_oracle():
     params = host_params(model)
     net = O.OracleCNN(params, label_smoothing=0.01, lr=1e-3, decay=5e-5, dtype=np.float64, dense1_l2=(2e-5, 2e-5))
 
-    model.record_steps(True)                                # this model cannot be recorded: the request must say so
-    assert model.recording_active is False
+    if recorded:
+        model.record_steps(True)
+        assert model.recording_active is True
     model.loss.new_pass()
     model.accuracy.new_pass()
     rng = np.random.RandomState(9)
-    for step in range(3):
+    for step in range(4):
         masks = draw_masks(rng, S)
         spatial[0].fixed_mask, spatial[1].fixed_mask, dense_drop.fixed_mask = \
             masks["spatial1"], masks["spatial2"], masks["dense"]
@@ -122,12 +126,51 @@ def test_cifar1_recipe_steps_match_oracle():
         for i, layer in enumerate(model.trainable_layers):
             got = [np.asarray(a) for a in layer.get_parameters()]
             for j, want in enumerate(net.p[i]):
-                if j >= 2:                                  # BN running statistics
+                if j >= 2 and step < 3:                     # BN running statistics (float32 and float64 parameters drift apart from step to step)
                     g = got[j].reshape(want.shape)
                     assert np.all(np.abs(g - want) <= 1e-5 + 1e-3 * np.abs(want)), (step, i, j)
-    assert model.optimizer.iterations == 3
+    assert model.optimizer.iterations == 4
+    assert len([r for r in getattr(model, "_recordings", {}).values() if r.get("graph")]) == (1 if recorded else 0)
 
     # evaluation: dropout layers pass their input through, no smoothing
     probs_eval, _ = net.forward(X, training=False)
     pred = model.predict(X, batch_size=64)
     assert rel_l2(pred, probs_eval) <= 5e-3
+
+
+def test_cifar1_recipe_recorded_steps_draw_the_same_masks_as_eager_steps():
+    """Without `fixed_mask` the layers draw their masks from the legacy global RNG, as the reference does.  A
+    recorded step draws them on the host in the layers' order before the replay: the same random stream as the
+    eager step, so losses and parameters agree bit for bit, replay after replay, and the masks differ from
+    step to step."""
+    import aether
+    rng = np.random.RandomState(21)
+    Xs = [rng.rand(128, 32, 32, 3).astype(np.float32) for _ in range(2)]
+    ys = [rng.randint(0, 10, 128) for _ in range(2)]
+
+    def run(record):
+        np.random.seed(13)
+        model = cifar1_model(aether)
+        d1 = [l for l in model.layers if isinstance(l, aether.Layer_Dense)][0]
+        d1.set_parameters(np.asarray(d1.weights) * 200, np.full((1, 256), 0.5, np.float32))
+        model.record_steps(record)
+        model.loss.new_pass()
+        model.accuracy.new_pass()
+        np.random.seed(14)
+        out, masks = [], []
+        drop = [l for l in model.layers if isinstance(l, aether.Layer_Dropout)][0]
+        for step in range(6):
+            out.append(model.train_step(Xs[step % 2], ys[step % 2]))
+            masks.append(drop.binary_mask.get())
+        params = [np.asarray(p) for layer in model.trainable_layers for p in layer.get_parameters()]
+        return out, masks, params, model
+
+    eager, masks_e, params_e, _ = run(False)
+    rec, masks_r, params_r, model = run(True)
+    assert model.recording_active
+    assert len([r for r in model._recordings.values() if r.get("graph")]) == 1
+    assert eager == rec, (eager, rec)
+    assert all(np.array_equal(a, b) for a, b in zip(masks_e, masks_r))
+    assert not np.array_equal(masks_r[3], masks_r[4])        # a fresh draw every replay
+    assert 0.85 < float((masks_r[4] > 0).mean()) < 0.98      # keep probability 0.925
+    assert all(np.array_equal(a, b) for a, b in zip(params_e, params_r))

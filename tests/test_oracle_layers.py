@@ -131,6 +131,26 @@ def test_softmax_cce_vs_torch():
     assert np.isclose(O.cce_forward(hard, np.array([1]), 0.0)[0], -np.log(1e-7))
 
 
+def test_soft_targets_vs_torch():
+    """A 2-D y_true is used as given (CNN_classes_cupy.py:622-626, :672-676): rows that are probabilities, not
+    one-hot.  torch's cross_entropy takes class probabilities as target and smooths them the same way."""
+    r = np.random.RandomState(12)
+    logits = r.randn(16, 10) * 1.5                          # (no probability below the reference's clip at 1e-7)
+    assert O.softmax(logits).min() > 1e-6
+    t = r.rand(16, 10) ** 3
+    t /= t.sum(axis=1, keepdims=True)
+    for ls in (0.0, 0.05):
+        p = O.softmax(logits)
+        lt = torch.from_numpy(logits).clone().requires_grad_(True)
+        want = F.cross_entropy(lt, torch.from_numpy(t), label_smoothing=ls, reduction="none")
+        np.testing.assert_allclose(O.cce_forward(p, t, ls, training=True), want.detach().numpy(), rtol=1e-6, atol=1e-7)
+        want.mean().backward()
+        np.testing.assert_allclose(O.softmax_cce_backward(p, t, ls), lt.grad.numpy(), rtol=1e-9, atol=1e-12)
+    # a dropped smoothing term or targets replaced by their argmax would not pass
+    assert not np.allclose(O.cce_forward(p, t, 0.05), O.cce_forward(p, t, 0.0), rtol=1e-3)
+    assert not np.allclose(O.cce_forward(p, t, 0.0), O.cce_forward(p, np.argmax(t, axis=1), 0.0), rtol=1e-2)
+
+
 # ---- Adam ----------------------------------------------------------------------------
 def test_adam_vs_torch_and_closed_form():
     r = np.random.RandomState(3)
