@@ -52,9 +52,11 @@ SIGNATURES = {
     "aeth_relu_fwd_twin_f32": [_p, _p, _p, _f, _i64],
     "aeth_bn_bwd_twin_f32": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i],
     "aeth_maxpool_fwd_f32": [_p, _p, _p] + [_i] * 8,
-    "aeth_bn_relu_maxpool2_fwd_f32": [_p] * 11 + [_i] * 4 + [_f, _f, _f, _p],
+    "aeth_bn_relu_maxpool2_fwd_f32": [_p] * 11 + [_i] * 4 + [_f, _f, _f],
+    "aeth_bn_relu_maxpool2_fwd_twin_f32": [_p] * 12 + [_i] * 4 + [_f, _f, _f],
     "aeth_maxpool2_relu_bwd_f32": [_p] * 5 + [_i] * 4 + [_f],
-    "aeth_maxpool2_relu_bn_bwd_f32": [_p] * 12 + [_i] * 4 + [_f, _p],
+    "aeth_maxpool2_relu_bn_bwd_f32": [_p] * 12 + [_i] * 4 + [_f],
+    "aeth_maxpool2_relu_bn_bwd_twin_f32": [_p] * 13 + [_i] * 4 + [_f],
     "aeth_maxpool_bwd_f32": [_p, _p, _p] + [_i] * 8,
     "aeth_avgpool_fwd_f32": [_p, _p] + [_i] * 8,
     "aeth_avgpool_bwd_f32": [_p, _p] + [_i] * 8,

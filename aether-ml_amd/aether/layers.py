@@ -212,11 +212,13 @@ class Pooling:
                 bn.dinputs = DeviceTensor(self.inputs.shape, _F32)
                 bn.dweights = DeviceTensor(C, _F32)
                 bn.dbiases = DeviceTensor(C, _F32)
-                dx16 = _twin(bn.dinputs).ptr if _wants_bf16(getattr(bn, "prev", None)) else None
-                _ck(_L().aeth_maxpool2_relu_bn_bwd_f32(
-                    dvalues.ptr, self.max_indicies.ptr, relu.inputs.ptr, bn.inputs.ptr, bn.gamma.ptr,
-                    bn.batch_mean.ptr, bn.batch_invstd.ptr, self.dinputs.ptr, relu.dinputs.ptr, bn.dinputs.ptr,
-                    bn.dweights.ptr, bn.dbiases.ptr, S, H_in, W_in, C, _relu_alpha(relu), dx16))
+                head = (dvalues.ptr, self.max_indicies.ptr, relu.inputs.ptr, bn.inputs.ptr, bn.gamma.ptr,
+                        bn.batch_mean.ptr, bn.batch_invstd.ptr, self.dinputs.ptr, relu.dinputs.ptr, bn.dinputs.ptr)
+                tail = (bn.dweights.ptr, bn.dbiases.ptr, S, H_in, W_in, C, _relu_alpha(relu))
+                if _wants_bf16(getattr(bn, "prev", None)):
+                    _ck(_L().aeth_maxpool2_relu_bn_bwd_twin_f32(*head, _twin(bn.dinputs).ptr, *tail))
+                else:
+                    _ck(_L().aeth_maxpool2_relu_bn_bwd_f32(*head, *tail))
                 bn._bwd_prefilled_for = relu.dinputs
             else:
                 _ck(_L().aeth_maxpool2_relu_bwd_f32(dvalues.ptr, self.max_indicies.ptr, relu.inputs.ptr,
@@ -519,11 +521,13 @@ class Batch_Norm:
         pool.inputs = act.output
         pool.output = DeviceTensor((S, H // 2, W // 2, C), _F32)
         pool.max_indicies = DeviceTensor((S, H // 2, W // 2, C), np.uint8)
-        out16 = _twin(pool.output).ptr if _wants_bf16(getattr(pool, "next", None)) else None
-        _ck(_L().aeth_bn_relu_maxpool2_fwd_f32(
-            inputs.ptr, self.gamma.ptr, self.beta.ptr, self.running_mean.ptr, self.running_var.ptr,
-            self.batch_mean.ptr, self.batch_invstd.ptr, self.output.ptr, act.output.ptr, pool.output.ptr,
-            pool.max_indicies.ptr, S, H, W, C, self.epsilon, self.momentum, _relu_alpha(act), out16))
+        head = (inputs.ptr, self.gamma.ptr, self.beta.ptr, self.running_mean.ptr, self.running_var.ptr,
+                self.batch_mean.ptr, self.batch_invstd.ptr, self.output.ptr, act.output.ptr, pool.output.ptr)
+        tail = (pool.max_indicies.ptr, S, H, W, C, self.epsilon, self.momentum, _relu_alpha(act))
+        if _wants_bf16(getattr(pool, "next", None)):
+            _ck(_L().aeth_bn_relu_maxpool2_fwd_twin_f32(*head, _twin(pool.output).ptr, *tail))
+        else:
+            _ck(_L().aeth_bn_relu_maxpool2_fwd_f32(*head, *tail))
         act._prefilled_for = self.output
         pool._prefilled_for = act.output
         pool._fused_relu = act

@@ -1141,10 +1141,10 @@ static int pool2_params(int S, int H, int W, int C, Pool2Params* p, unsigned* n)
 
 static inline bool aligned16(const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; }
 
-int aeth_bn_relu_maxpool2_fwd_f32(const float* x, const float* gamma, const float* beta, float* running_mean,
-                                  float* running_var, float* save_mean, float* save_invstd, float* bn_out,
-                                  float* relu_out, float* pool_out, uint8_t* idx, int S, int H, int W, int C,
-                                  float eps, float momentum, float alpha, uint16_t* pool_out_bf16) {
+static int bn_relu_maxpool2_fwd_impl(const float* x, const float* gamma, const float* beta,
+                                     float* running_mean, float* running_var, float* save_mean, float* save_invstd,
+                                     float* bn_out, float* relu_out, float* pool_out, uint8_t* idx, int S, int H, int W,
+                                     int C, float eps, float momentum, float alpha, uint16_t* pool_out_bf16) {
     AETH_REQUIRE_INIT();
     AETH_CHECK_ARG(x && gamma && beta && running_mean && running_var && save_mean && save_invstd);
     AETH_CHECK_ARG(bn_out && relu_out && pool_out && idx);
@@ -1181,6 +1181,23 @@ int aeth_bn_relu_maxpool2_fwd_f32(const float* x, const float* gamma, const floa
     return AETH_OK;
 }
 
+int aeth_bn_relu_maxpool2_fwd_f32(const float* x, const float* gamma, const float* beta, float* running_mean,
+                                  float* running_var, float* save_mean, float* save_invstd, float* bn_out,
+                                  float* relu_out, float* pool_out, uint8_t* idx, int S, int H, int W, int C,
+                                  float eps, float momentum, float alpha) {
+    return bn_relu_maxpool2_fwd_impl(x, gamma, beta, running_mean, running_var, save_mean, save_invstd, bn_out, relu_out,
+                                     pool_out, idx, S, H, W, C, eps, momentum, alpha, nullptr);
+}
+
+int aeth_bn_relu_maxpool2_fwd_twin_f32(const float* x, const float* gamma, const float* beta, float* running_mean,
+                                       float* running_var, float* save_mean, float* save_invstd, float* bn_out,
+                                       float* relu_out, float* pool_out, uint16_t* pool_out_bf16, uint8_t* idx, int S,
+                                       int H, int W, int C, float eps, float momentum, float alpha) {
+    AETH_CHECK_ARG(pool_out_bf16 != nullptr);
+    return bn_relu_maxpool2_fwd_impl(x, gamma, beta, running_mean, running_var, save_mean, save_invstd, bn_out, relu_out,
+                                     pool_out, idx, S, H, W, C, eps, momentum, alpha, pool_out_bf16);
+}
+
 int aeth_maxpool2_relu_bwd_f32(const float* dy, const uint8_t* idx, const float* relu_in, float* pool_dx,
                                float* relu_dx, int S, int H, int W, int C, float alpha) {
     AETH_REQUIRE_INIT();
@@ -1197,10 +1214,10 @@ int aeth_maxpool2_relu_bwd_f32(const float* dy, const uint8_t* idx, const float*
     return AETH_OK;
 }
 
-int aeth_maxpool2_relu_bn_bwd_f32(const float* dy, const uint8_t* idx, const float* relu_in, const float* x,
-                                  const float* gamma, const float* save_mean, const float* save_invstd,
-                                  float* pool_dx, float* relu_dx, float* bn_dx, float* dgamma, float* dbeta,
-                                  int S, int H, int W, int C, float alpha, uint16_t* bn_dx_bf16) {
+static int maxpool2_relu_bn_bwd_impl(const float* dy, const uint8_t* idx, const float* relu_in, const float* x,
+                                     const float* gamma, const float* save_mean, const float* save_invstd,
+                                     float* pool_dx, float* relu_dx, float* bn_dx, float* dgamma, float* dbeta,
+                                     int S, int H, int W, int C, float alpha, uint16_t* bn_dx_bf16) {
     AETH_REQUIRE_INIT();
     AETH_CHECK_ARG(dy && idx && relu_in && x && gamma && save_mean && save_invstd);
     AETH_CHECK_ARG(pool_dx && relu_dx && bn_dx && dgamma && dbeta);
@@ -1232,6 +1249,23 @@ int aeth_maxpool2_relu_bn_bwd_f32(const float* dy, const uint8_t* idx, const flo
                        (const ew_f4*)relu_dx, (const ew_f4*)save_mean, coef, (ew_f4*)bn_dx, (ew_u2*)bn_dx_bf16, n4, C / 4);
     AETH_LAUNCH_CHECK();
     return AETH_OK;
+}
+
+int aeth_maxpool2_relu_bn_bwd_f32(const float* dy, const uint8_t* idx, const float* relu_in, const float* x,
+                                  const float* gamma, const float* save_mean, const float* save_invstd,
+                                  float* pool_dx, float* relu_dx, float* bn_dx, float* dgamma, float* dbeta,
+                                  int S, int H, int W, int C, float alpha) {
+    return maxpool2_relu_bn_bwd_impl(dy, idx, relu_in, x, gamma, save_mean, save_invstd, pool_dx, relu_dx, bn_dx, dgamma,
+                                     dbeta, S, H, W, C, alpha, nullptr);
+}
+
+int aeth_maxpool2_relu_bn_bwd_twin_f32(const float* dy, const uint8_t* idx, const float* relu_in, const float* x,
+                                       const float* gamma, const float* save_mean, const float* save_invstd,
+                                       float* pool_dx, float* relu_dx, float* bn_dx, uint16_t* bn_dx_bf16,
+                                       float* dgamma, float* dbeta, int S, int H, int W, int C, float alpha) {
+    AETH_CHECK_ARG(bn_dx_bf16 != nullptr);
+    return maxpool2_relu_bn_bwd_impl(dy, idx, relu_in, x, gamma, save_mean, save_invstd, pool_dx, relu_dx, bn_dx, dgamma,
+                                     dbeta, S, H, W, C, alpha, bn_dx_bf16);
 }
 
 int aeth_bn_fwd_infer_f32(const float* x, const float* gamma, const float* beta, const float* running_mean,

@@ -309,20 +309,8 @@ struct Stage {
     bool busy[kStageSlots] = {};
     int next = 0;
     bool ready = false;
+    bool failed = false;     // the slots could not be allocated once: copies go the pageable way, no second attempt
 } g_stage;
-
-bool stage_init() {
-    if (g_stage.ready) return true;
-    for (int i = 0; i < kStageSlots; ++i) {
-        if (hipHostMalloc((void**)&g_stage.host[i], (size_t)kStageBytes, hipHostMallocDefault) != hipSuccess ||
-            hipEventCreateWithFlags(&g_stage.done[i], hipEventDisableTiming) != hipSuccess) {
-            (void)hipGetLastError();
-            return false;
-        }
-    }
-    g_stage.ready = true;
-    return true;
-}
 
 void stage_release() {
     for (int i = 0; i < kStageSlots; ++i) {
@@ -330,6 +318,22 @@ void stage_release() {
         if (g_stage.host[i]) (void)hipHostFree(g_stage.host[i]);
     }
     g_stage = Stage();
+}
+
+bool stage_init() {
+    if (g_stage.ready) return true;
+    if (g_stage.failed) return false;
+    for (int i = 0; i < kStageSlots; ++i) {
+        if (hipHostMalloc((void**)&g_stage.host[i], (size_t)kStageBytes, hipHostMallocDefault) != hipSuccess ||
+            hipEventCreateWithFlags(&g_stage.done[i], hipEventDisableTiming) != hipSuccess) {
+            (void)hipGetLastError();
+            stage_release();                 // what was allocated so far
+            g_stage.failed = true;
+            return false;
+        }
+    }
+    g_stage.ready = true;
+    return true;
 }
 
 // a free slot (waits for the copy that last used it)

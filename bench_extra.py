@@ -289,10 +289,10 @@ def layer_kernels(steps, warmup):
         ("avgpool_bwd 2x2/2", fp + fp // 4, lambda: L.aeth_avgpool_bwd_f32(dpooled.ptr, y.ptr, S, H, W, Ch, 2, 2, 2, 2)),
         ("bn_relu_maxpool2_fwd (3 launches)", 4 * fp + fp // 4 + n // 4, lambda: L.aeth_bn_relu_maxpool2_fwd_f32(
             x.ptr, gamma.ptr, beta.ptr, rm.ptr, rv.ptr, sm.ptr, si.ptr, y.ptr, y2.ptr, pooled.ptr, idx.ptr,
-            S, H, W, Ch, f(1e-5), f(0.9), f(0.0), None)),
+            S, H, W, Ch, f(1e-5), f(0.9), f(0.0))),
         ("maxpool2_relu_bn_bwd (3 launches)", 7 * fp + fp // 4 + n // 4, lambda: L.aeth_maxpool2_relu_bn_bwd_f32(
             dpooled.ptr, idx.ptr, y.ptr, x.ptr, gamma.ptr, sm.ptr, si.ptr, y2.ptr, y3.ptr, y.ptr, dgamma.ptr,
-            dbeta.ptr, S, H, W, Ch, f(0.0), None)),
+            dbeta.ptr, S, H, W, Ch, f(0.0))),
         ("cast_f32_to_bf16", fp + fp // 2, lambda: L.aeth_cast_f32_to_bf16(x.ptr, y.ptr, i64(n))),
         ("fill_f32", fp, lambda: L.aeth_fill_f32(y.ptr, f(0.0), i64(n))),
         ("memcpy_d2d", 2 * fp, lambda: L.aeth_memcpy_d2d(y.ptr, x.ptr, i64(fp))),

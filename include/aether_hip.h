@@ -192,8 +192,7 @@ int aeth_bn_relu_maxpool2_fwd_f32(const float* x, const float* gamma, const floa
                                   float* running_mean, float* running_var,
                                   float* save_mean, float* save_invstd,
                                   float* bn_out, float* relu_out, float* pool_out, uint8_t* idx,
-                                  int S, int H, int W, int C, float eps, float momentum, float alpha,
-                                  uint16_t* pool_out_bf16 /* may be NULL */);
+                                  int S, int H, int W, int C, float eps, float momentum, float alpha);
 int aeth_maxpool2_relu_bwd_f32(const float* dy, const uint8_t* idx, const float* relu_in,
                                float* pool_dx, float* relu_dx,
                                int S, int H, int W, int C, float alpha);
@@ -205,8 +204,22 @@ int aeth_maxpool2_relu_bn_bwd_f32(const float* dy, const uint8_t* idx, const flo
                                   const float* save_mean, const float* save_invstd,
                                   float* pool_dx, float* relu_dx, float* bn_dx,
                                   float* dgamma, float* dbeta,
-                                  int S, int H, int W, int C, float alpha,
-                                  uint16_t* bn_dx_bf16 /* may be NULL */);
+                                  int S, int H, int W, int C, float alpha);
+/* The two fused calls above with a bfloat16 copy (round to nearest even) of pool_out / bn_dx written beside the
+ * float32 tensor, for a bf16 convolution that takes it as input / upstream gradient (as aeth_relu_fwd_twin_f32
+ * and aeth_bn_bwd_twin_f32 do for the separate layers).  No counterpart in the reference. */
+int aeth_bn_relu_maxpool2_fwd_twin_f32(const float* x, const float* gamma, const float* beta,
+                                       float* running_mean, float* running_var,
+                                       float* save_mean, float* save_invstd,
+                                       float* bn_out, float* relu_out, float* pool_out, uint16_t* pool_out_bf16,
+                                       uint8_t* idx,
+                                       int S, int H, int W, int C, float eps, float momentum, float alpha);
+int aeth_maxpool2_relu_bn_bwd_twin_f32(const float* dy, const uint8_t* idx, const float* relu_in,
+                                       const float* x, const float* gamma,
+                                       const float* save_mean, const float* save_invstd,
+                                       float* pool_dx, float* relu_dx, float* bn_dx, uint16_t* bn_dx_bf16,
+                                       float* dgamma, float* dbeta,
+                                       int S, int H, int W, int C, float alpha);
 /* Pooling "average" :267-268 and the scatter kernel :163-202. */
 int aeth_avgpool_fwd_f32(const float* x, float* y,
                          int S, int H, int W, int C, int fH, int fW, int sH, int sW);

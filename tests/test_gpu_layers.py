@@ -432,11 +432,11 @@ def test_fused_block_entry_points_reject_what_they_do_not_cover():
     c = DeviceTensor.zeros(8)
     i8 = DeviceTensor((4 * 2 * 2 * 8,), np.uint8)
     args = (t.ptr, c.ptr, c.ptr, c.ptr, c.ptr, c.ptr, c.ptr, t.ptr, t.ptr, t.ptr, i8.ptr)
-    assert L.aeth_bn_relu_maxpool2_fwd_f32(*args, 4, 3, 4, 8, 1e-5, 0.9, 0.0, None) == _lib.AETH_E_INVALID     # odd H
-    assert L.aeth_bn_relu_maxpool2_fwd_f32(*args, 4, 4, 4, 6, 1e-5, 0.9, 0.0, None) == _lib.AETH_E_INVALID     # C % 4
+    assert L.aeth_bn_relu_maxpool2_fwd_f32(*args, 4, 3, 4, 8, 1e-5, 0.9, 0.0) == _lib.AETH_E_INVALID     # odd H
+    assert L.aeth_bn_relu_maxpool2_fwd_f32(*args, 4, 4, 4, 6, 1e-5, 0.9, 0.0) == _lib.AETH_E_INVALID     # C % 4
     assert L.aeth_maxpool2_relu_bwd_f32(t.ptr, i8.ptr, t.ptr, t.ptr, t.ptr, 4, 4, 5, 8, 0.0) == _lib.AETH_E_INVALID
     assert L.aeth_maxpool2_relu_bwd_f32(None, i8.ptr, t.ptr, t.ptr, t.ptr, 4, 4, 4, 8, 0.0) == _lib.AETH_E_INVALID
-    assert L.aeth_bn_relu_maxpool2_fwd_f32(*args, 4, 4, 4, 8, 1e-5, 0.9, 0.0, None) == 0
+    assert L.aeth_bn_relu_maxpool2_fwd_f32(*args, 4, 4, 4, 8, 1e-5, 0.9, 0.0) == 0
     # with the optional bfloat16 copy of the pooling output: the cast of what was written
     from oracle import oracle as O
     r = np.random.RandomState(0)
@@ -446,9 +446,11 @@ def test_fused_block_entry_points_reject_what_they_do_not_cover():
     g, rv = DeviceTensor.full(8, 1.0), DeviceTensor.full(8, 1.0)
     rm, sm, si = DeviceTensor.zeros(8), DeviceTensor.zeros(8), DeviceTensor.zeros(8)
     bn_out, relu_out = DeviceTensor(t.size), DeviceTensor(t.size)
-    args2 = (t.ptr, g.ptr, c.ptr, rm.ptr, rv.ptr, sm.ptr, si.ptr, bn_out.ptr, relu_out.ptr, pool.ptr, i8.ptr)
-    assert L.aeth_bn_relu_maxpool2_fwd_f32(*args2, 4, 4, 4, 8, 1e-5, 0.9, 0.0, p16.ptr) == 0
+    args2 = (t.ptr, g.ptr, c.ptr, rm.ptr, rv.ptr, sm.ptr, si.ptr, bn_out.ptr, relu_out.ptr, pool.ptr, p16.ptr, i8.ptr)
+    assert L.aeth_bn_relu_maxpool2_fwd_twin_f32(*args2, 4, 4, 4, 8, 1e-5, 0.9, 0.0) == 0
     assert np.all(np.isfinite(pool.get())) and np.array_equal(p16.get(), O.bf16_bits(pool.get()))
+    args3 = args2[:10] + (None,) + args2[11:]
+    assert L.aeth_bn_relu_maxpool2_fwd_twin_f32(*args3, 4, 4, 4, 8, 1e-5, 0.9, 0.0) == _lib.AETH_E_INVALID   # the copy is the point
 
 
 
