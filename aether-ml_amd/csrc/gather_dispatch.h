@@ -3,6 +3,7 @@
 #pragma once
 #include "gather_kernels.h"
 #include "narrow_kernels.h"
+#include "sample_runs.h"
 #include "tuning.h"
 
 namespace aeth {
@@ -571,6 +572,18 @@ int conv_fprop_impl(const char* fn, const T* x, const T* w, const float* bias, f
     int Ho, Wo;
     int rc = check_conv_dims(fn, S, H, W, C, D, fH, fW, sH, sW, pH, pW, &Ho, &Wo);
     if (rc) return rc;
+    {   // a batch whose input or output reaches 2^31 bytes goes out in runs of whole samples (sample_runs.h)
+        const int64_t xs = (int64_t)H * W * C, ys = (int64_t)Ho * Wo * D;
+        const SampleRuns runs = plan_sample_runs(S, xs * (int64_t)sizeof(T), ys * 4);
+        if (runs.runs > 1) {
+            for (int s0 = 0; s0 < S; s0 += runs.per) {
+                rc = conv_fprop_impl<T>(fn, x + s0 * xs, w, bias, y + s0 * ys, std::min(runs.per, S - s0), H, W, C, D, fH, fW,
+                                        sH, sW, pH, pW, fixed_scratch, fixed_capacity);
+                if (rc) return rc;
+            }
+            return AETH_OK;
+        }
+    }
     if constexpr (sizeof(T) == 4) {
         const int64_t M = (int64_t)S * H * W;
         if (narrow_shape(D, fH, fW, sH, sW, pH, pW) && M > 0 && M * 64 < ((int64_t)1 << 31) && C <= 16384) {
@@ -637,6 +650,18 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
     int Ho, Wo;
     int rc = check_conv_dims(fn, S, H, W, C, D, fH, fW, sH, sW, pH, pW, &Ho, &Wo);
     if (rc) return rc;
+    {   // runs of whole samples for a dy or dx of 2^31 bytes and more (sample_runs.h)
+        const int64_t xs = (int64_t)H * W * C, ys = (int64_t)Ho * Wo * D;
+        const SampleRuns runs = plan_sample_runs(S, ys * (int64_t)sizeof(T), xs * 4);
+        if (runs.runs > 1) {
+            for (int s0 = 0; s0 < S; s0 += runs.per) {
+                rc = conv_dgrad_impl<T>(fn, dy + s0 * ys, w, dx + s0 * xs, std::min(runs.per, S - s0), H, W, C, D, fH, fW, sH,
+                                        sW, pH, pW);
+                if (rc) return rc;
+            }
+            return AETH_OK;
+        }
+    }
     constexpr int BK = Elem<T>::BK;
     const int nclass = sH * sW;
     if (nclass > 64) return fail(AETH_E_INVALID, "%s: stride too large", fn);

@@ -2,6 +2,7 @@
 #pragma once
 #include "wgrad_kernels.h"
 #include "narrow_kernels.h"
+#include "sample_runs.h"
 #include "tuning.h"
 
 namespace aeth {
@@ -74,6 +75,36 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     int Ho, Wo;
     int rc = check_conv_dims(fn, S, H, W, C, D, fH, fW, sH, sW, pH, pW, &Ho, &Wo);
     if (rc) return rc;
+    if (!swapped) {
+        // An x or dy of 2^31 bytes and more: the samples go in runs (sample_runs.h), every run's dw and dbias into a
+        // row of a temporary [runs][K D + D], and the rows are added in run order like the partial sums of one launch.
+        const int64_t xs = (int64_t)H * W * C, ys = (int64_t)Ho * Wo * D;
+        const SampleRuns runs = plan_sample_runs(S, xs * (int64_t)sizeof(T), ys * (int64_t)sizeof(T));
+        if (runs.runs > 1) {
+            const int64_t kd = (int64_t)fH * fW * C * D;
+            const int64_t stride = round_up(kd, 4) + round_up(D, 4);            // rows and their dbias parts 16-byte aligned
+            void* tmp = nullptr;
+            rc = aeth_malloc(&tmp, runs.runs * stride * (int64_t)sizeof(float));
+            if (rc) return rc;
+            float* rows = static_cast<float*>(tmp);
+            int r = 0;
+            for (int s0 = 0; s0 < S && rc == AETH_OK; s0 += runs.per, ++r)
+                rc = conv_wgrad_impl<T>(fn, x + s0 * xs, dy + s0 * ys, rows + r * stride,
+                                        dbias ? rows + r * stride + round_up(kd, 4) : nullptr, std::min(runs.per, S - s0), H, W,
+                                        C, D, fH, fW, sH, sW, pH, pW);
+            if (rc == AETH_OK) {
+                // two reductions over the rows: dw, then dbias (the plain kernel: any alignment of dw and dbias)
+                hipLaunchKernelGGL(reduce_splits, dim3(cdiv(kd, 64)), dim3(kThreads), 0, ctx().stream, (const float*)rows, dw,
+                                   (float*)nullptr, (int)kd, (int)kd, (int)stride, r);
+                if (dbias)
+                    hipLaunchKernelGGL(reduce_splits, dim3(cdiv(D, 64)), dim3(kThreads), 0, ctx().stream,
+                                       (const float*)(rows + round_up(kd, 4)), dbias, (float*)nullptr, D, D, (int)stride, r);
+                if (hipGetLastError() != hipSuccess) rc = fail(AETH_E_HIP, "%s: kernel launch failed", fn);
+            }
+            const int rc_free = aeth_free(tmp);             // (stream order: the block is reused only by later launches)
+            return rc ? rc : rc_free;
+        }
+    }
     if constexpr (sizeof(T) == 4) {
         // at most 16 output channels and few rows: one thread per element of dw walks the rows
         const int64_t M = (int64_t)S * H * W;

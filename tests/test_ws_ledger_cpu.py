@@ -18,3 +18,15 @@ def test_workspace_ledger_rules(tmp_path):
     names = [line.split()[1] for line in r.stdout.splitlines() if line.startswith("ok ")]
     assert names == ["reuse", "grow_frees_old", "no_growth_while_recording", "live_recordings_keep_their_workspace",
                      "retired_freed_with_last_recording", "alloc_failure", "reset"]
+
+
+def test_sample_runs_cover_the_batch_below_the_descriptor_limit(tmp_path):
+    """aether-ml_amd/csrc/sample_runs.h: how a batch whose tensors reach 2^31 bytes is cut into runs of whole samples
+    (tests/cpu/sample_runs_check.cpp walks the runs of several shapes and checks cover, order and extent)."""
+    exe = str(tmp_path / "sample_runs_check")
+    src = os.path.join(ROOT, "tests", "cpu", "sample_runs_check.cpp")
+    inc = os.path.join(ROOT, "aether-ml_amd", "csrc")
+    subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-Werror", "-I", inc, src, "-o", exe], check=True)
+    r = subprocess.run([exe], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert len([line for line in r.stdout.splitlines() if line.startswith("ok ")]) == 11
