@@ -17,7 +17,11 @@
  *     [fH,fW,C,D] (the reference's filter_weights layout), dense weights
  *     [n_in,n_out] row-major, all float32 unless the name says bf16 (uint16_t
  *     holding the upper 16 bits of a float32, rounded to nearest even).
- *   - element counts fit int32; byte counts are int64.
+ *   - element counts fit int32; byte counts are int64.  A convolution whose
+ *     batch-sized tensors reach 2^31 bytes (up to the 2^31 elements, 8 GiB of
+ *     float32) is run in several launches over runs of whole samples; results
+ *     are the same bits as for the samples handed in separately (wgrad: the
+ *     runs' sums are added in run order).
  *   - one process-wide context bound to one GPU with one stream; calls are
  *     asynchronous on that stream, aeth_sync() and the d2h copy are the sync
  *     points.  Not re-entrant: one caller thread at a time.
