@@ -51,16 +51,43 @@ def time_loop(fn, steps, warmup):
 COUNTERS = os.path.join(ROOT, "profiles", "conv_f32_resnet3x3_256x56x56x64.counters.json")
 
 
+def sources_digest():
+    """SHA-256 over the kernel sources (aether-ml_amd/csrc, in name order): what a counter summary is stamped
+    with, so that a later run can tell whether the kernels it times are the ones the counters saw."""
+    import hashlib
+    h = hashlib.sha256()
+    d = os.path.join(ROOT, "aether-ml_amd", "csrc")
+    for name in sorted(os.listdir(d)):
+        if name.endswith((".h", ".hip")):
+            h.update(name.encode())
+            with open(os.path.join(d, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def counter_traffic(kernel):
-    """HBM/fabric bytes per launch of `kernel`, from the summary that the last FETCH_SIZE /
-    WRITE_SIZE counter runs of this benchmark left under profiles/ (bench_counters.py writes
-    it, scaled by what the same counters read for a plain copy of known size); None when
-    the file or the kernel is missing."""
+    """(bytes, source): HBM/fabric bytes per launch of `kernel` from the summary that the last FETCH_SIZE /
+    WRITE_SIZE counter runs of this benchmark left under profiles/ (bench_counters.py writes it, scaled by what
+    the same counters read for a plain copy of known size), and where that figure comes from: the file, when it
+    was measured, the digest of the kernel sources it was measured on and whether that is the digest of the
+    sources of this run.  The figure is NOT measured in this run (counters need the profiler); a summary taken on
+    other sources is reported as stale, with a warning.  (None, None) when the file or the kernel is missing."""
     try:
         with open(COUNTERS) as f:
-            return float(json.load(f)["kernels"][kernel]["traffic_bytes"])
+            doc = json.load(f)
+        traffic = float(doc["kernels"][kernel]["traffic_bytes"])
     except (OSError, KeyError, ValueError, TypeError):
-        return None
+        return None, None
+    stamp = doc.get("measured", {})
+    now = sources_digest()
+    source = {"file": os.path.relpath(COUNTERS, ROOT), "measured_on": stamp.get("date"),
+              "sources_digest": stamp.get("sources_digest"), "this_run_sources_digest": now,
+              "same_sources": stamp.get("sources_digest") == now,
+              "how": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this benchmark, summarised by bench_counters.py"}
+    if not source["same_sources"]:
+        print("bench.py: roofline.traffic comes from counters measured on other kernel sources (%s, now %s): "
+              "re-run the counter passes (bench_counters.py)" % (source["sources_digest"], now), file=sys.stderr)
+    return traffic, source
 
 
 def cpu_baseline(S_small, H, W, C, D):
@@ -193,12 +220,17 @@ def main():
         in_step[name] = {"ms": ms, "tflops": fl / (ms * 1e-3) / 1e12,
                          "frac_fp32_mfma_peak": fl / (ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS}
 
-    # The dominant kernel: gather_gemm_dma runs twice per step (fprop and dgrad: two thirds of
-    # the step).  `achieved` = algorithmic flops per launch / its average duration inside the
-    # timed steps; a direction's interval also holds its 5 us filter-packing launch.
-    kernel = "gather_gemm_dma"
+    # The dominant kernel is the one with the largest share of the step: gather_gemm_dma runs twice per step (fprop
+    # and dgrad, both reading the filter in place: no packing launch), wgrad_halo_f32 once (its interval also holds
+    # the reduction of its split sums, a few us).  `achieved` = algorithmic flops per launch / the kernel's average
+    # duration inside the timed steps.  The slowest direction is reported beside it.
     gather_ms = 0.5 * (in_step["fprop"]["ms"] + in_step["dgrad"]["ms"])
-    achieved = fl / (gather_ms * 1e-3) / 1e12
+    share = {"gather_gemm_dma": 2 * gather_ms, "wgrad_halo_f32": in_step["wgrad"]["ms"]}
+    kernel = max(share, key=share.get)
+    kernel_ms = gather_ms if kernel == "gather_gemm_dma" else in_step["wgrad"]["ms"]
+    achieved = fl / (kernel_ms * 1e-3) / 1e12
+    slowest = min(in_step, key=lambda k: in_step[k]["tflops"])
+    traffic, traffic_source = counter_traffic(kernel)
     roofline = {
         "bound": "mfma",
         "kernel": kernel,
@@ -206,8 +238,12 @@ def main():
         "peak": FP32_MFMA_PEAK_TFLOPS,
         "unit": "TFLOP/s",
         "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
-        "traffic": counter_traffic(kernel),
-        "launch_ms_in_step": gather_ms,
+        "traffic": traffic,
+        "traffic_source": traffic_source,
+        "launch_ms_in_step": kernel_ms,
+        "share_of_step": share[kernel] / sum(share.values()),
+        "slowest_direction": {"direction": slowest, "tflops": in_step[slowest]["tflops"],
+                              "frac": in_step[slowest]["frac_fp32_mfma_peak"]},
         "algorithmic_flops_per_launch": fl,
         "algorithmic_bytes_per_launch": 4.0 * (2 * S * H * W * C + 9 * C * D + D),
     }

@@ -11,7 +11,8 @@ that bench.py reads for `roofline.traffic`:
 FETCH_SIZE and WRITE_SIZE count KiB per dispatch in units that depend on the chip; the
 copy probe of bench.py (relu_fwd_kernel with alpha = 1 over 64 Mi floats: 256 MiB read and
 256 MiB written per launch) says what one count is worth, and every kernel's counts are
-scaled by that.  Written: profiles/conv_f32_resnet3x3_256x56x56x64.counters.json.
+scaled by that.  Written: profiles/conv_f32_resnet3x3_256x56x56x64.counters.json, stamped with the date and a
+digest of the kernel sources the counters were taken on (bench.py reports a summary from other sources as stale).
 """
 import collections
 import csv
@@ -62,7 +63,11 @@ def main(fetch_csv, write_csv):
         kernels[k] = {"fetch_size_raw": round(fetch[k][0], 1), "write_size_raw": round(write[k][0], 1),
                       "launches": fetch[k][1], "read_bytes": round(rd), "written_bytes": round(wr),
                       "traffic_bytes": round(rd + wr)}
-    out = {"workload": "fp32 conv fprop + wgrad + dgrad, input NHWC [256,56,56,64], 64 filters 3x3 s1 same",
+    import datetime
+    import bench
+    out = {"measured": {"date": datetime.date.today().isoformat(), "sources_digest": bench.sources_digest(),
+                        "note": "SHA-256 (16 hex digits) over aether-ml_amd/csrc/*.h, *.hip as bench.sources_digest() forms it"},
+           "workload": "fp32 conv fprop + wgrad + dgrad, input NHWC [256,56,56,64], 64 filters 3x3 s1 same",
            "command": "rocprofv3 --pmc FETCH_SIZE (then WRITE_SIZE) --output-format csv -- python3 bench.py "
                       "--steps 3 --warmup 1 --no-cpu --no-extra --copy-probe",
            "copy_probe": {"kernel": PROBE, "kib_read_and_written": PROBE_KIB,
