@@ -384,7 +384,17 @@ class Model:
             layer.set_parameters(*parameter_set)
 
     def save_parameters(self, path, cupy_arrays=False):
-        write_parameters([tuple(np.asarray(a) for a in tup) for tup in self.get_parameters()], path, cupy_arrays)
+        """`cupy_arrays`: the stream of the reference's CuPy checkpoints, dtypes included: its dense layers hold
+        float64 parameters (`cp.random.randn`, CNN_classes_cupy.py:320-322; `CNN/saved_models/model5` stores them
+        as f8), so the float32 dense parameters of this build are widened (exactly) on the way out."""
+        from .layers import Layer_Dense
+        params = []
+        for layer in self.trainable_layers:
+            tup = tuple(np.asarray(a) for a in layer.get_parameters())
+            if cupy_arrays and isinstance(layer, Layer_Dense):
+                tup = tuple(a.astype(np.float64) for a in tup)
+            params.append(tup)
+        write_parameters(params, path, cupy_arrays)
 
     def load_parameters(self, path):
         with open(path, 'rb') as f:

@@ -169,6 +169,13 @@ def test_train_prints_reference_format_and_parameters_round_trip(tmp_path, capsy
     path2 = str(tmp_path / "params_cupy.pkl")
     model.save_parameters(path2, cupy_arrays=True)
     assert b"cupy._core.core" in open(path2, "rb").read()
+    # with the reference's dtypes: float64 dense parameters (CNN_classes_cupy.py:320-322), float32 everything else
+    import io
+    from aether.model import _ArrayOnlyUnpickler
+    stored = _ArrayOnlyUnpickler(io.BytesIO(open(path2, "rb").read())).load()
+    kinds = [type(l).__name__ for l in model.trainable_layers]
+    for kind, tup in zip(kinds, stored):
+        assert all(a.dtype == (np.float64 if kind == "Layer_Dense" else np.float32) for a in tup), kind
     np.random.seed(5)
     third = build_model(aether, hw=16)
     third.forward(X[:4], training=False)
