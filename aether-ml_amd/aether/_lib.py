@@ -41,6 +41,8 @@ SIGNATURES = {
     "aeth_dense_fprop_f32": [_p, _p, _p, _p, _i, _i, _i],
     "aeth_dense_dgrad_f32": [_p, _p, _p, _i, _i, _i],
     "aeth_dense_wgrad_f32": [_p, _p, _p, _p, _i, _i, _i],
+    "aeth_dense_fprop_act_f32": [_p, _p, _p, _p, _p, _f, _i, _i, _i],
+    "aeth_dense_bwd_f32": [_p, _p, _p, _p, _p, _p, _p, _p, _f, _i, _i, _i],
     "aeth_axpy_f32": [_f, _p, _p, _i64],
     "aeth_l1_grad_f32": [_f, _p, _p, _i64],
     "aeth_reduce_f32": [_p, _i64, _i, _p],

@@ -256,9 +256,27 @@ class Layer_Dense:
         M = inputs.shape[0]
         n_in, n_out = self.weights.shape
         self.output = DeviceTensor((M, n_out), _F32)
+        act = self._neighbour("next")
+        if act is not None and not _wants_bf16(getattr(act, "next", None)):
+            # the ReLU / Leaky_ReLU behind this layer in the same call (it then finds its output in place): where K is
+            # split over workgroups, the reduction of the split writes both tensors
+            act.inputs = self.output
+            act.output = DeviceTensor((M, n_out), _F32)
+            _ck(_L().aeth_dense_fprop_act_f32(inputs.ptr, self.weights.ptr, self.biases.ptr, self.output.ptr,
+                                              act.output.ptr, _relu_alpha(act), M, n_in, n_out))
+            act._prefilled_for = self.output
+            return self.output
         _ck(_L().aeth_dense_fprop_f32(inputs.ptr, self.weights.ptr, self.biases.ptr, self.output.ptr,
                                       M, n_in, n_out))
         return self.output
+
+    def _neighbour(self, side):
+        """The ReLU / Leaky_ReLU directly behind ("next") or in front of ("prev") this layer, if the model has linked
+        one there and AETHER_FUSE_DENSE is not 0."""
+        layer = getattr(self, side, None)
+        if isinstance(layer, (ReLU, Leaky_ReLU)) and os.environ.get("AETHER_FUSE_DENSE", "1") != "0":
+            return layer
+        return None
 
     def backward(self, dvalues):
         dvalues = as_device(dvalues, _F32)
@@ -266,8 +284,21 @@ class Layer_Dense:
         n_in, n_out = self.weights.shape
         self.dweights = DeviceTensor(self.weights.shape, _F32)
         self.dbiases = DeviceTensor((1, n_out), _F32)
-        _ck(_L().aeth_dense_wgrad_f32(self.inputs.ptr, dvalues.ptr, self.dweights.ptr, self.dbiases.ptr,
-                                      M, n_in, n_out))
+        self.dinputs = DeviceTensor(self.inputs.shape, _F32)
+        # the three products of the backward pass in one call, with the backward pass of a ReLU / Leaky_ReLU in front of
+        # this layer on the way (that layer then finds its dinputs in place)
+        act = self._neighbour("prev")
+        if act is not None and getattr(act, "output", None) is self.inputs and getattr(act, "inputs", None) is not None \
+                and act.inputs.shape == self.inputs.shape:
+            act.dinputs = DeviceTensor(self.inputs.shape, _F32)
+            act_in, act_dx = act.inputs.ptr, act.dinputs.ptr
+        else:
+            act, act_in, act_dx = None, None, None
+        _ck(_L().aeth_dense_bwd_f32(self.inputs.ptr, dvalues.ptr, self.weights.ptr, self.dweights.ptr, self.dbiases.ptr,
+                                    self.dinputs.ptr, act_in, act_dx, _relu_alpha(act) if act is not None else 0.0,
+                                    M, n_in, n_out))
+        if act is not None:
+            act._bwd_prefilled_for = self.dinputs
         if self.weight_regularizer_l1 > 0:
             _ck(_L().aeth_l1_grad_f32(self.weight_regularizer_l1, self.weights.ptr, self.dweights.ptr,
                                       self.weights.size))
@@ -280,8 +311,6 @@ class Layer_Dense:
         if self.bias_regularizer_l2 > 0:
             _ck(_L().aeth_axpy_f32(2 * self.bias_regularizer_l2, self.biases.ptr, self.dbiases.ptr,
                                    self.biases.size))
-        self.dinputs = DeviceTensor(self.inputs.shape, _F32)
-        _ck(_L().aeth_dense_dgrad_f32(dvalues.ptr, self.weights.ptr, self.dinputs.ptr, M, n_in, n_out))
 
     def get_parameters(self):
         return self.weights, self.biases

@@ -478,9 +478,12 @@ static __global__ __launch_bounds__(kThreads) void reduce_splits(const float* __
 // owns 4 consecutive outputs, 16 split lanes per output add splits j, j+16, ... with
 // four loads in flight, and the lanes are added in lane order.
 // (tr as above, a multiple of 4: the 4 outputs of a thread then go to 4 rows of dw)
+// act_out != nullptr (tr == 0): the sums also go through a ReLU / leaky ReLU, act_out[i] = t > 0 ? t : alpha t, the
+// layer behind a dense product whose K was split (what relu_fwd_kernel would write from dw in a launch of its own).
 static __global__ __launch_bounds__(kThreads) void reduce_splits4(const float* __restrict__ part, float* __restrict__ dw,
                                                           float* __restrict__ dbias, int n_dw, int n, int stride,
-                                                          int splits, int tr = 0) {
+                                                          int splits, int tr = 0, float* __restrict__ act_out = nullptr,
+                                                          float alpha = 0.f) {
     __shared__ f4 red[16][16];
     const int cg = threadIdx.x & 15;                     // group of 4 outputs
     const int sl = threadIdx.x >> 4;                     // split lane
@@ -511,6 +514,12 @@ static __global__ __launch_bounds__(kThreads) void reduce_splits4(const float* _
             for (int e = 0; e < 4; ++e) dw[(c + e) * ld + r] = t[e];
         } else if (i < n_dw) {
             *reinterpret_cast<f4*>(dw + i) = t;
+            if (act_out != nullptr) {
+                f4 a;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) a[e] = t[e] > 0.f ? t[e] : alpha * t[e];
+                *reinterpret_cast<f4*>(act_out + i) = a;
+            }
         } else if (dbias != nullptr) {
             *reinterpret_cast<f4*>(dbias + (i - n_dw)) = t;
         }

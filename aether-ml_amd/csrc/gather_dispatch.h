@@ -308,6 +308,15 @@ struct GatherSetup {
     int64_t bt_bytes;
     int nsplit = 1;          // > 1: split K, partial products behind the packed filter in the workspace
     int64_t part_bytes = 0;
+    struct ActOut* act = nullptr;   // fprop: the activation behind the layer, written by the split reduction where there is one
+};
+
+// The output of the ReLU / leaky ReLU that follows a dense layer, for the split reduction to write on the way
+// (`done` says whether it did: a product that is not split leaves it to the caller's own launch).
+struct ActOut {
+    float* out;
+    float alpha;
+    bool done;
 };
 
 // The kernels that multiply two classes of one dgrad from one halo take 2 or 4 classes that gather_halo_bf16 would take
@@ -508,9 +517,12 @@ static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
         AETH_LAUNCH_CHECK();
         if (gs.nsplit > 1) {
             const int n = gs.gp.M * gs.gp.N;
+            const bool act = gs.act != nullptr && gs.act->out != nullptr && (reinterpret_cast<uintptr_t>(gs.act->out) & 15) == 0;
             hipLaunchKernelGGL(reduce_splits4, dim3(cdiv(n, 64)), dim3(kThreads), 0, c.stream,
-                               (const float*)gs.gp.out, real_out, (float*)nullptr, n, n, n, gs.nsplit);
+                               (const float*)gs.gp.out, real_out, (float*)nullptr, n, n, n, gs.nsplit, 0,
+                               act ? gs.act->out : (float*)nullptr, act ? gs.act->alpha : 0.f);
             AETH_LAUNCH_CHECK();
+            if (act) gs.act->done = true;
         }
     }
     return AETH_OK;
@@ -568,7 +580,7 @@ static bool launch_direct(DirectParams& dp, bool dgrad, hipStream_t st) {
 template <typename T>
 int conv_fprop_impl(const char* fn, const T* x, const T* w, const float* bias, float* y,
                     int S, int H, int W, int C, int D, int fH, int fW, int sH, int sW, int pH, int pW,
-                    char* fixed_scratch = nullptr, int64_t fixed_capacity = 0) {
+                    char* fixed_scratch = nullptr, int64_t fixed_capacity = 0, ActOut* act = nullptr) {
     int Ho, Wo;
     int rc = check_conv_dims(fn, S, H, W, C, D, fH, fW, sH, sW, pH, pW, &Ho, &Wo);
     if (rc) return rc;
@@ -624,6 +636,7 @@ int conv_fprop_impl(const char* fn, const T* x, const T* w, const float* bias, f
     pk.N = D; pk.K = g.K; pk.Npad = (int)round_up(D, 64); pk.Kpad = g.Kpad;
     gs.bt_bytes = (int64_t)pk.Npad * pk.Kpad * sizeof(T);
     g.split_slabs = 0;
+    gs.act = act;
     plan_split<T>(gs, C % Elem<T>::CE == 0, ctx().prop.multiProcessorCount);
     void* ws;
     const int64_t need = round_up(gs.bt_bytes, 256) + gs.part_bytes;

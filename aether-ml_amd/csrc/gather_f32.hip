@@ -56,6 +56,17 @@ int aeth_dense_fprop_f32(const float* x, const float* w, const float* bias, floa
     return conv_fprop_impl<float>(__func__, x, w, bias, y, M, 1, 1, n_in, n_out, 1, 1, 1, 1, 0, 0);
 }
 
+int aeth_dense_fprop_act_f32(const float* x, const float* w, const float* bias, float* y, float* act_y, float alpha, int M,
+                             int n_in, int n_out) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(x != nullptr && w != nullptr && y != nullptr && act_y != nullptr);
+    ActOut act{act_y, alpha, false};
+    int rc = conv_fprop_impl<float>(__func__, x, w, bias, y, M, 1, 1, n_in, n_out, 1, 1, 1, 1, 0, 0, nullptr, 0, &act);
+    if (rc) return rc;
+    if (act.done) return AETH_OK;                       // the reduction of the split K wrote it
+    return aeth_relu_fwd_f32(y, act_y, alpha, (int64_t)M * n_out);
+}
+
 int aeth_dense_dgrad_f32(const float* dy, const float* w, float* dx, int M, int n_in, int n_out) {
     AETH_REQUIRE_INIT();
     AETH_CHECK_ARG(dy != nullptr && w != nullptr && dx != nullptr);

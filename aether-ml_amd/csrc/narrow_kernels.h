@@ -37,10 +37,10 @@ static __global__ __launch_bounds__(kThreads) void narrow_fprop(const NarrowPara
     if (kq == 0 && n < p.N && (t >> 6) < p.M) p.out[(size_t)m * p.N + n] = sum;
 }
 
-// dx[m][k] = sum_n dy[m][n] w[k][n]; thread = (m, k)
-static __global__ __launch_bounds__(kThreads) void narrow_dgrad(const NarrowParams p, const unsigned total) {
-    const unsigned t = blockIdx.x * kThreads + threadIdx.x;
-    if (t >= total) return;
+// dx[m][k] = sum_n dy[m][n] w[k][n]; thread t = (m, k).  act_in != nullptr: the backward pass of the ReLU / leaky ReLU in
+// front of the layer on the way, act_dx[t] = act_in[t] < 0 ? alpha dx : dx (what relu_bwd_kernel would write from dx).
+__device__ __forceinline__ void narrow_dgrad_one(const NarrowParams& p, const unsigned t, const float* __restrict__ act_in,
+                                                 float* __restrict__ act_dx, const float alpha) {
     const unsigned m = t / (unsigned)p.K, k = t - m * (unsigned)p.K;
     const float* dy = p.a + (size_t)m * p.N;
     const float* w = p.b + (size_t)k * p.N;
@@ -48,11 +48,17 @@ static __global__ __launch_bounds__(kThreads) void narrow_dgrad(const NarrowPara
 #pragma unroll 4
     for (int n = 0; n < p.N; ++n) acc = fmaf(dy[n], w[n], acc);
     p.out[t] = acc;
+    if (act_in != nullptr) act_dx[t] = act_in[t] < 0.f ? alpha * acc : acc;
 }
 
-// dw[k][n] = sum_m x[m][k] dy[m][n], dbias[n] = sum_m dy[m][n] (row k == K of the thread grid); thread = (k, n)
-static __global__ __launch_bounds__(kThreads) void narrow_wgrad(const NarrowParams p) {
-    const int t = (int)(blockIdx.x * kThreads + threadIdx.x);
+static __global__ __launch_bounds__(kThreads) void narrow_dgrad(const NarrowParams p, const unsigned total) {
+    const unsigned t = blockIdx.x * kThreads + threadIdx.x;
+    if (t >= total) return;
+    narrow_dgrad_one(p, t, nullptr, nullptr, 0.f);
+}
+
+// dw[k][n] = sum_m x[m][k] dy[m][n], dbias[n] = sum_m dy[m][n] (row k == K of the thread grid); thread t = (k, n)
+__device__ __forceinline__ void narrow_wgrad_one(const NarrowParams& p, const int t) {
     const int k = t >> 4, n = t & 15;
     if (k > p.K || n >= p.N || (k == p.K && p.out2 == nullptr)) return;
     const float* dy = p.b + n;
@@ -67,6 +73,23 @@ static __global__ __launch_bounds__(kThreads) void narrow_wgrad(const NarrowPara
 #pragma unroll 16
     for (int m = 0; m < p.M; ++m) acc = fmaf(x[(size_t)m * p.K], dy[(size_t)m * p.N], acc);
     p.out[(size_t)k * p.N + n] = acc;
+}
+
+static __global__ __launch_bounds__(kThreads) void narrow_wgrad(const NarrowParams p) {
+    narrow_wgrad_one(p, (int)(blockIdx.x * kThreads + threadIdx.x));
+}
+
+// A narrow dense layer's whole backward pass as one launch: the first `wgrad_blocks` workgroups are narrow_wgrad's, the
+// others narrow_dgrad's (neither reads what the other writes), with the activation's backward pass as above.
+static __global__ __launch_bounds__(kThreads) void narrow_bwd(const NarrowParams pw, const NarrowParams pd, const unsigned wgrad_blocks,
+                                                              const unsigned dgrad_total, const float* __restrict__ act_in,
+                                                              float* __restrict__ act_dx, const float alpha) {
+    if (blockIdx.x < wgrad_blocks) {
+        narrow_wgrad_one(pw, (int)(blockIdx.x * kThreads + threadIdx.x));
+        return;
+    }
+    const unsigned t = (blockIdx.x - wgrad_blocks) * kThreads + threadIdx.x;
+    if (t < dgrad_total) narrow_dgrad_one(pd, t, act_in, act_dx, alpha);
 }
 
 // 1x1 filter, unit stride, no padding, at most 16 output channels, few enough rows for one thread per output

@@ -142,6 +142,20 @@ int aeth_dense_dgrad_f32(const float* dy, const float* w, float* dx,
                          int M, int n_in, int n_out);
 int aeth_dense_wgrad_f32(const float* x, const float* dy, float* dw, float* dbias,
                          int M, int n_in, int n_out);
+/* A dense layer together with the ReLU / Leaky_ReLU next to it (:406-428), for callers that
+ * know the neighbour: the same values as the separate calls, fewer launches on small layers.
+ * aeth_dense_fprop_act_f32 also writes act_y = y > 0 ? y : alpha * y (alpha = 0: ReLU), the
+ * activation's output; where K is split over workgroups, the reduction of the split writes
+ * both.  aeth_dense_bwd_f32 is Layer_Dense.backward :333-354 in one call (dw, dbias, dx;
+ * regulariser terms stay with the caller) and, with act_in / act_dx not NULL, the backward
+ * pass of the activation IN FRONT of the layer on the way: act_dx = act_in < 0 ? alpha * dx
+ * : dx (act_in = that activation's input).  A layer of at most 16 outputs on at most 1024
+ * rows goes out as one launch. */
+int aeth_dense_fprop_act_f32(const float* x, const float* w, const float* bias, float* y, float* act_y,
+                             float alpha, int M, int n_in, int n_out);
+int aeth_dense_bwd_f32(const float* x, const float* dy, const float* w, float* dw, float* dbias, float* dx,
+                       const float* act_in /* may be NULL */, float* act_dx /* NULL with act_in */, float alpha,
+                       int M, int n_in, int n_out);
 int aeth_axpy_f32(float alpha, const float* x, float* y, int64_t n);
 int aeth_l1_grad_f32(float lambda, const float* w, float* dw, int64_t n);
 /* out[0] = sum |x| (mode 0) or sum x*x (mode 1): Loss.regularization_loss :593-609 */

@@ -424,6 +424,51 @@ def test_fused_block_equals_the_three_layers(shape, alpha, monkeypatch):
     assert not same or np.array_equal(got["1"][3], got["0"][3])
 
 
+@pytest.mark.parametrize("M,n_in,n_mid,n_out,alpha", [(128, 2048, 256, 10, 0.01), (128, 2048, 256, 10, None), (37, 300, 64, 16, 0.2),
+                                                       (64, 512, 128, 40, None), (5, 24, 8, 3, 0.1), (1100, 96, 32, 10, None)])
+def test_dense_layers_with_the_activation_next_to_them(M, n_in, n_mid, n_out, alpha, monkeypatch):
+    """Layer_Dense -> ReLU / Leaky_ReLU -> Layer_Dense: the first layer's forward call also writes the activation's output
+    (from the reduction of its split K where there is one), the second layer's backward call is one launch for a layer of
+    at most 16 outputs and also does the activation's backward pass.  The same values as layer by layer
+    (AETHER_FUSE_DENSE=0), bit for bit, and the oracle's."""
+    import aether
+    r = np.random.RandomState(19)
+    x = r.randn(M, n_in).astype(np.float32)
+    dy = r.randn(M, n_out).astype(np.float32)
+    w1, b1 = (r.randn(n_in, n_mid) / np.sqrt(n_in)).astype(np.float32), r.randn(1, n_mid).astype(np.float32)
+    w2, b2 = (r.randn(n_mid, n_out) / np.sqrt(n_mid)).astype(np.float32), r.randn(1, n_out).astype(np.float32)
+    got = {}
+    for fuse in ("1", "0"):
+        monkeypatch.setenv("AETHER_FUSE_DENSE", fuse)
+        d1, d2 = aether.Layer_Dense(n_in, n_mid), aether.Layer_Dense(n_mid, n_out, weight_regularizer_l2=1e-3)
+        act = aether.ReLU() if alpha is None else aether.Leaky_ReLU(alpha)
+        d1.set_parameters(w1, b1)
+        d2.set_parameters(w2, b2)
+        d1.next, act.prev, act.next, d2.prev = act, d1, d2, act       # as Model.finalize links them
+        d1.forward(x, True)
+        act.forward(d1.output, True)
+        d2.forward(act.output, True)
+        d2.backward(dy)
+        act.backward(d2.dinputs)
+        d1.backward(act.dinputs)
+        got[fuse] = [t.get() for t in (d1.output, act.output, d2.output, d2.dweights, d2.dbiases, d2.dinputs, act.dinputs,
+                                       d1.dweights, d1.dbiases, d1.dinputs)]
+        assert (getattr(act, "_prefilled_for", None) is None) and (getattr(act, "_bwd_prefilled_for", None) is None)
+    for a, b in zip(got["1"], got["0"]):
+        assert np.array_equal(a, b)
+    a64 = alpha if alpha is not None else 0.0
+    y1 = O.dense_forward(x, w1, b1, dtype=np.float64)
+    h = np.where(y1 > 0, y1, a64 * y1)
+    _close(got["1"][0], y1)
+    _close(got["1"][1], h)
+    dw2, db2, dh = O.dense_backward(h, w2, b2, dy, wl2=1e-3, dtype=np.float64)
+    _close(got["1"][3], dw2, rms_scaled=True)
+    _close(got["1"][4], db2, rms_scaled=True)
+    _close(got["1"][5], dh)
+    # the activation's gradient follows the sign of ITS input as the GPU saw it (float32 y1)
+    _close(got["1"][6], np.where(got["1"][0] < 0, a64 * dh, dh))
+
+
 def test_fused_block_entry_points_reject_what_they_do_not_cover():
     from aether import _lib
     from aether.tensor import DeviceTensor
