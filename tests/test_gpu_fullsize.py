@@ -165,8 +165,14 @@ def test_full_size_conv_bf16(cfg, tune):
     y_h, dx_h, dw_h, db_h = y.get(), dx.get(), dw.get(), db.get()
     assert np.all(np.isfinite(y_h)) and np.all(np.isfinite(dx_h)) and np.all(np.isfinite(dw_h))
 
-    whole_tensor_close(y_h, lambda lo, hi: O.conv_fprop(xr[lo:hi], wr, b, stride, pad, dtype=np.float64), S)
-    whole_tensor_close(dx_h, lambda lo, hi: O.conv_dgrad(dyr[lo:hi], wr, (H, W), stride, pad, dtype=np.float64), S)
+    label = LABEL[name] + ", bf16 inputs"
+    abi.report(label, "fprop", whole_tensor_close(
+        y_h, lambda lo, hi: O.conv_fprop(xr[lo:hi], wr, b, stride, pad, dtype=np.float64), S))
+    abi.report(label, "dgrad", whole_tensor_close(
+        dx_h, lambda lo, hi: O.conv_dgrad(dyr[lo:hi], wr, (H, W), stride, pad, dtype=np.float64), S))
+    want = whole_batch_wgrad(xr, dyr, (fH, fW), stride, pad)
+    abi.report(label, "wgrad", abi.close(dw_h, want, rms_scaled=True),
+               "atol * max(1, rms), rms = %.3g" % float(np.sqrt(np.mean(want * want))))
     tune(**OTHER_KERNELS)
     y2 = DeviceTensor.full(yshape, np.nan)
     _lib.check(L.aeth_conv_fprop_bf16(xd.ptr, wd.ptr, bd.ptr, y2.ptr, *dims))
@@ -184,7 +190,7 @@ def test_full_size_conv_bf16(cfg, tune):
     scale = float(np.sqrt(np.sum(y_h.astype(np.float64) ** 2)) * np.sqrt(np.sum(dyr.astype(np.float64) ** 2)))
     assert abs(lhs - rhs_x) <= 1e-6 * scale, (lhs, rhs_x)
     assert abs(lhs - rhs_w) <= 1e-6 * scale, (lhs, rhs_w)
-    abi.close(db_h, np.sum(dyr.astype(np.float64), axis=(0, 1, 2)), rms_scaled=True)
+    abi.report(label, "dbias", abi.close(db_h, np.sum(dyr.astype(np.float64), axis=(0, 1, 2)), rms_scaled=True))
 
     # one-sample-supported gradient: wgrad of that sample alone
     s = S - 1
