@@ -1,8 +1,8 @@
-"""The binding of INTEGRATION.md, section 2, run end to end: classes shaped like the reference's
+"""The binding a maintainer of the reference would write, run end to end: classes shaped like the reference's
 `Conv_Layer` (CNN_classes_cupy.py:37-161) and `Layer_Dense` (:315-362) that keep their own arrays and call
 libaether_hip.so through nothing but ctypes.  No `aether` class is involved: buffers come from aeth_malloc,
-results are read with aeth_memcpy_d2h, and the call sequence inside forward / backward is the one the document
-shows a maintainer.  Checked against the CPU oracle at the float32 bar."""
+results are read with aeth_memcpy_d2h, and forward / backward make one library call per product in place of
+the reference's pad + as_strided + einsum lines.  Checked against the CPU oracle at the float32 bar."""
 import ctypes as C
 
 import numpy as np
