@@ -24,6 +24,8 @@ SIGNATURES = {
     "aeth_memcpy_h2d": [_p, _p, _i64],
     "aeth_memcpy_d2h": [_p, _p, _i64],
     "aeth_memcpy_d2d": [_p, _p, _i64],
+    "aeth_d2h_begin": [_p, _i64, C.POINTER(_i)],
+    "aeth_d2h_end": [_i, _p, _i64],
     "aeth_fill_f32": [_p, _f, _i64],
     "aeth_sync": [],
     "aeth_event_create": [C.POINTER(_p)],

@@ -148,11 +148,37 @@ class Model:
             print(f' epoch: {epoch}')
             self.loss.new_pass()
             self.accuracy.new_pass()
-            for step, rows in enumerate(spans):
-                loss, data_loss, regularization_loss, accuracy = self.train_step(_rows(X, rows), _rows(y, rows))
+            # Replayed steps (record_steps) are read one step late: the host queues step k + 1 while step k runs
+            # and takes step k's loss and predictions afterwards; sums and printed lines are those of the plain loop.
+            waiting = []                                     # (step, function that reads its scalars)
+
+            def report(step, loss, data_loss, regularization_loss, accuracy, lr):
                 if step % print_every == 0 or step == len(spans) - 1:
-                    print(_progress(f'epoch: {epoch}, ', accuracy, loss, data_loss, regularization_loss,
-                                    self.optimizer.current_learning_rate))
+                    print(_progress(f'epoch: {epoch}, ', accuracy, loss, data_loss, regularization_loss, lr))
+
+            def drain(keep):
+                while len(waiting) > keep:
+                    k, finish = waiting.pop(0)
+                    report(k, *finish())
+
+            try:
+                for step, rows in enumerate(spans):
+                    batch_X, batch_y = _rows(X, rows), _rows(y, rows)
+                    finish = self._recorded_step(batch_X, batch_y, later=True) if self.recording_active else None
+                    if finish is not None:
+                        waiting.append((step, finish))
+                        drain(1)
+                        continue
+                    drain(0)                                 # results enter the sums in the order of the steps
+                    loss, data_loss, regularization_loss, accuracy = self._eager_step(batch_X, batch_y)
+                    report(step, loss, data_loss, regularization_loss, accuracy, self.optimizer.current_learning_rate)
+                drain(0)
+            finally:
+                for _, finish in waiting:                    # (only after an exception: hand the pending copies back)
+                    try:
+                        finish()
+                    except Exception:
+                        pass
         # the summary and the validation pass come once, after the last epoch (:135-151)
         data_loss, regularization_loss = self.loss.calculate_accumulated(include_regularization=True)
         print(_progress(' training, ', self.accuracy.calculate_accumulated(), data_loss + regularization_loss,
@@ -197,7 +223,9 @@ class Model:
             return False
         return self.loss.can_defer()
 
-    def _recorded_step(self, batch_X, batch_y):
+    def _recorded_step(self, batch_X, batch_y, later=False):
+        """One step through a recording.  None: this step has to run normally (first step of a shape).  With
+        `later` and a replay: a function that reads the step's scalars when called, instead of the scalars."""
         import ctypes as C
         from . import _lib, layers as L
         from .tensor import DeviceTensor
@@ -262,12 +290,33 @@ class Model:
         if self.layers[-1].__dict__.get("output") is not rec["output"]:
             for obj, name, val in rec["bindings"]:
                 setattr(obj, name, val)
-        data_loss = self.loss.finish(rec["pending"])
-        regularization_loss = self.loss.regularization_finish(rec.get("reg_pending"))
-        loss = data_loss + regularization_loss
-        predictions = self.output_layer_activation.predictions(rec["output"])
-        accuracy = self.accuracy.calculate(predictions, batch_y)
-        return loss, data_loss, regularization_loss, accuracy
+        if not later:
+            data_loss = self.loss.finish(rec["pending"])
+            regularization_loss = self.loss.regularization_finish(rec.get("reg_pending"))
+            predictions = self.output_layer_activation.predictions(rec["output"])
+            accuracy = self.accuracy.calculate(predictions, batch_y)
+            return data_loss + regularization_loss, data_loss, regularization_loss, accuracy
+        # the step's scalars are copied to the host behind the replay and read when the caller asks for them,
+        # by which time the next replay may be running (Model.train)
+        buf, rows, _ = rec["pending"]
+        loss_later = buf.get_later()
+        reg = rec.get("reg_pending")
+        reg_later = reg[1].get_later() if reg is not None else None
+        lr = self.optimizer.current_learning_rate
+
+        def finish():
+            host = loss_later()
+            sample_losses, predictions = host[:rows], host[rows:].view(np.int32)
+            data_loss = np.mean(sample_losses)
+            self.loss.accumulated_sum += np.sum(sample_losses)
+            self.loss.accumulated_count += len(sample_losses)
+            regularization_loss = 0
+            if reg is not None:
+                for coef, value in zip(reg[0], reg_later()):
+                    regularization_loss += coef * float(value)
+            accuracy = self.accuracy.calculate(predictions, batch_y)
+            return data_loss + regularization_loss, data_loss, regularization_loss, accuracy, lr
+        return finish
 
     def train_step(self, batch_X, batch_y):
         """One iteration of the loop body of ``train`` (CNN_model_cupy.py:107-126):
@@ -277,6 +326,9 @@ class Model:
             result = self._recorded_step(batch_X, batch_y)
             if result is not None:
                 return result
+        return self._eager_step(batch_X, batch_y)
+
+    def _eager_step(self, batch_X, batch_y):
         # The loss kernel is queued here and read after backward and the update have been
         # queued too, so the device never idles while the host prepares the backward pass.
         # A regulariser's sums are queued here as well: they see the weights before the update,

@@ -69,6 +69,19 @@ class DeviceTensor:
     def __len__(self):
         return self.shape[0]
 
+    def __getitem__(self, rows):
+        """A run of consecutive rows (a slice of the first axis with step 1) as a view of the same memory:
+        what batching a data set that lives on the device needs (`X[start:start + batch_size]`)."""
+        if not isinstance(rows, slice) or self.ndim == 0:
+            raise TypeError("DeviceTensor supports slices of its first axis only")
+        start, stop, step = rows.indices(self.shape[0])
+        if step != 1:
+            raise ValueError("DeviceTensor slices must have step 1")
+        n = max(0, stop - start)
+        row_bytes = (self.nbytes // self.shape[0]) if self.shape[0] else 0
+        return DeviceTensor((n,) + self.shape[1:], self.dtype, _ptr=self.ptr + start * row_bytes,
+                            _base=self._base if self._base is not None else self)
+
     # -- host transfer ------------------------------------------------------------------
     def get(self):
         out = np.empty(self.shape, dtype=self.dtype)
@@ -77,6 +90,23 @@ class DeviceTensor:
         return out
 
     numpy = get
+
+    def get_later(self):
+        """Queues the copy to the host behind what is queued so far and returns at once; calling the result
+        waits for that copy alone and gives the array (at most 256 KB; for a loop that reads one step's
+        scalars while the next step already runs).  Every result must be called once."""
+        if self.nbytes == 0 or self.nbytes > 256 * 1024:
+            value = self.get()
+            return lambda: value
+        ticket = C.c_int(-1)
+        _lib.check(_lib.lib().aeth_d2h_begin(self.ptr, self.nbytes, C.byref(ticket)))
+        shape, dtype, nbytes = self.shape, self.dtype, self.nbytes
+
+        def result():
+            out = np.empty(shape, dtype=dtype)
+            _lib.check(_lib.lib().aeth_d2h_end(ticket.value, out.ctypes.data, nbytes))
+            return out
+        return result
 
     def __array__(self, dtype=None, copy=None):
         a = self.get()

@@ -301,12 +301,15 @@ int aeth_free(void* p) {
 // 10 us with the device idle; a batch of 128 32x32x3 images is 1.5 MB, a dropout mask of 128 x 256 floats 128 KB).
 // A slot is reused once the copy it fed has passed (an event per slot).
 namespace {
-constexpr int kStageSlots = 8;
+constexpr int kStageSlots = 16;
+constexpr int kStageHeldMax = 8;                        // slots that pending aeth_d2h_begin copies may hold at a time
 constexpr int64_t kStageBytes = 256 * 1024;
 struct Stage {
     char* host[kStageSlots] = {};
     hipEvent_t done[kStageSlots] = {};
     bool busy[kStageSlots] = {};
+    bool held[kStageSlots] = {};                         // holds the bytes of an aeth_d2h_begin until its aeth_d2h_end
+    int n_held = 0;
     int next = 0;
     bool ready = false;
     bool failed = false;     // the slots could not be allocated once: copies go the pageable way, no second attempt
@@ -336,9 +339,11 @@ bool stage_init() {
     return true;
 }
 
-// a free slot (waits for the copy that last used it)
+// a free slot (waits for the copy that last used it); slots held by pending two-part copies are passed over
+// (at most kStageHeldMax of the kStageSlots are ever held)
 int stage_slot() {
-    const int i = g_stage.next;
+    int i = g_stage.next;
+    while (g_stage.held[i]) i = (i + 1) % kStageSlots;
     g_stage.next = (i + 1) % kStageSlots;
     if (g_stage.busy[i]) {
         (void)hipEventSynchronize(g_stage.done[i]);
@@ -354,7 +359,7 @@ int aeth_memcpy_h2d(void* dst, const void* host_src, int64_t bytes) {
     AETH_CHECK_ARG(bytes >= 0);
     if (bytes == 0) return AETH_OK;
     AETH_CHECK_ARG(dst != nullptr && host_src != nullptr);
-    if (bytes <= kStageSlots * kStageBytes && stage_init()) {
+    if (bytes <= 8 * kStageBytes && stage_init()) {
         // through pinned slots: the caller's buffer is free at once and the copies take their turn on the stream
         for (int64_t done = 0; done < bytes; done += kStageBytes) {
             const int64_t piece = bytes - done < kStageBytes ? bytes - done : kStageBytes;
@@ -388,6 +393,38 @@ int aeth_memcpy_d2h(void* host_dst, const void* src, int64_t bytes) {
     }
     AETH_HIP(hipMemcpyAsync(host_dst, src, (size_t)bytes, hipMemcpyDeviceToHost, ctx().stream));
     AETH_HIP(hipStreamSynchronize(ctx().stream));
+    return AETH_OK;
+}
+
+int aeth_d2h_begin(const void* src, int64_t bytes, int* host_out_ticket) {
+    AETH_REQUIRE_INIT();
+    if (recording_open()) return fail(AETH_E_STATE, "aeth_d2h_begin: a copy to the host cannot be part of a recording");
+    AETH_CHECK_ARG(src != nullptr && host_out_ticket != nullptr);
+    AETH_CHECK_ARG(bytes > 0 && bytes <= kStageBytes);
+    *host_out_ticket = -1;
+    if (!stage_init()) return fail(AETH_E_NOMEM, "aeth_d2h_begin: no pinned staging memory");
+    if (g_stage.n_held >= kStageHeldMax)
+        return fail(AETH_E_STATE, "aeth_d2h_begin: %d copies are pending already (aeth_d2h_end takes them)", kStageHeldMax);
+    const int i = stage_slot();
+    AETH_HIP(hipMemcpyAsync(g_stage.host[i], src, (size_t)bytes, hipMemcpyDeviceToHost, ctx().stream));
+    AETH_HIP(hipEventRecord(g_stage.done[i], ctx().stream));
+    g_stage.busy[i] = true;
+    g_stage.held[i] = true;
+    ++g_stage.n_held;
+    *host_out_ticket = i;
+    return AETH_OK;
+}
+
+int aeth_d2h_end(int ticket, void* host_dst, int64_t bytes) {
+    AETH_REQUIRE_INIT();
+    AETH_CHECK_ARG(ticket >= 0 && ticket < kStageSlots && g_stage.ready && g_stage.held[ticket]);
+    AETH_CHECK_ARG(bytes >= 0 && bytes <= kStageBytes && (host_dst != nullptr || bytes == 0));
+    const hipError_t e = hipEventSynchronize(g_stage.done[ticket]);     // this copy alone, not what was queued after it
+    if (e == hipSuccess && bytes > 0) memcpy(host_dst, g_stage.host[ticket], (size_t)bytes);
+    g_stage.busy[ticket] = false;
+    g_stage.held[ticket] = false;
+    --g_stage.n_held;
+    AETH_HIP(e);
     return AETH_OK;
 }
 

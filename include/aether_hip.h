@@ -68,6 +68,14 @@ int aeth_malloc(void** host_out_ptr, int64_t bytes);
 int aeth_free(void* p);
 int aeth_memcpy_h2d(void* dst, const void* host_src, int64_t bytes);
 int aeth_memcpy_d2h(void* host_dst, const void* src, int64_t bytes);   /* synchronises */
+/* A small device-to-host copy in two halves, for callers that want the bytes later (a training loop that reads
+ * a step's loss while the next step already runs; no counterpart in the reference, whose arrays synchronise on
+ * every read).  aeth_d2h_begin queues the copy of at most 256 KB into pinned memory of the library, behind
+ * what is queued so far, and returns a ticket at once; aeth_d2h_end waits for THAT copy (not for work queued
+ * after it) and hands over the first `bytes` bytes.  At most 8 copies may be pending; every ticket must be
+ * ended (bytes = 0 drops it).  Not possible while recording. */
+int aeth_d2h_begin(const void* src, int64_t bytes, int* host_out_ticket);
+int aeth_d2h_end(int ticket, void* host_dst, int64_t bytes);
 int aeth_memcpy_d2d(void* dst, const void* src, int64_t bytes);
 int aeth_fill_f32(float* dst, float value, int64_t n);
 int aeth_sync(void);

@@ -174,3 +174,51 @@ def test_cifar1_recipe_recorded_steps_draw_the_same_masks_as_eager_steps():
     assert not np.array_equal(masks_r[3], masks_r[4])        # a fresh draw every replay
     assert 0.85 < float((masks_r[4] > 0).mean()) < 0.98      # keep probability 0.925
     assert all(np.array_equal(a, b) for a, b in zip(params_e, params_r))
+
+
+def test_train_reads_replayed_steps_one_step_late_and_prints_the_same_lines(capsys):
+    """Model.train on a recorded model queues step k + 1 before it reads step k's loss and predictions.  The printed
+    lines (every second step and the last of an epoch, the summary, the validation line), the accumulated sums
+    and the parameters are those of the plain loop; the last batch of an epoch is ragged (another shape: it runs
+    normally in the first epoch, is recorded in the second and replayed in the third)."""
+    import aether
+    rng = np.random.RandomState(31)
+    X = rng.rand(150, 32, 32, 3).astype(np.float32)
+    y = rng.randint(0, 10, 150)
+    outs, params = [], []
+    for record in (False, True):
+        np.random.seed(17)
+        model = cifar1_model(aether)
+        model.record_steps(record)
+        np.random.seed(18)                                   # the dropout masks' random stream
+        model.train(X, y, epochs=3, batch_size=32, print_every=2, validation_data=(X[:40], y[:40]))
+        outs.append(capsys.readouterr().out)
+        params.append([np.asarray(p) for layer in model.trainable_layers for p in layer.get_parameters()])
+        if record:
+            assert len([r for r in model._recordings.values() if r.get("graph")]) == 2
+    assert outs[0] == outs[1]
+    assert outs[0].count("epoch: ") == 3 + 3 * 3             # the epoch headers and steps 0, 2, 4 of each
+    assert all(np.array_equal(a, b) for a, b in zip(*params))
+
+
+def test_two_part_copies_to_the_host():
+    """aeth_d2h_begin / aeth_d2h_end: the bytes are those of the moment the copy was queued, whatever is queued
+    behind it; at most 8 may be pending; a ticket is ended once."""
+    import ctypes as C
+    from aether import _lib
+    from aether.tensor import DeviceTensor
+    lib = _lib.lib()
+    t = DeviceTensor.from_numpy(np.arange(1000, dtype=np.float32))
+    later = t.get_later()
+    t.fill(7.0)                                              # queued behind the copy
+    assert np.array_equal(later(), np.arange(1000, dtype=np.float32))
+    assert np.all(t.get() == 7.0)
+    pending = [DeviceTensor.from_numpy(np.full(16, k, np.float32)).get_later() for k in range(8)]
+    ticket = C.c_int(-1)
+    assert lib.aeth_d2h_begin(t.ptr, 64, C.byref(ticket)) == _lib.AETH_E_STATE        # a ninth
+    big = DeviceTensor.zeros(1 << 20)
+    big.set(np.ones(1 << 20, np.float32))                    # a 4 MB upload passes over the held slots
+    assert [int(p()[0]) for p in pending] == list(range(8))
+    assert lib.aeth_d2h_end(0, None, 0) == _lib.AETH_E_INVALID                          # nothing pending there
+    assert np.all(big.get_later()() == 1.0) if big.nbytes <= 256 * 1024 else np.all(big.get() == 1.0)
+    assert lib.aeth_d2h_begin(t.ptr, 1 << 20, C.byref(ticket)) == _lib.AETH_E_INVALID   # more than a slot holds
