@@ -35,6 +35,7 @@ SIGNATURES = {
     "aeth_conv_fprop_f32": [_p, _p, _p, _p] + _conv_dims,
     "aeth_conv_fprop_f32_noalloc": [_p, _p, _p, _p] + _conv_dims,
     "aeth_conv_dgrad_f32": [_p, _p, _p] + _conv_dims,
+    "aeth_conv_bwd_f32": [_p, _p, _p, _p, _p, _p] + _conv_dims,
     "aeth_conv_wgrad_f32": [_p, _p, _p, _p] + _conv_dims,
     "aeth_cast_f32_to_bf16": [_p, _p, _i64],
     "aeth_conv_fprop_bf16": [_p, _p, _p, _p] + _conv_dims,

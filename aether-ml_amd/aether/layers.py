@@ -142,8 +142,9 @@ class Conv_Layer:
             _ck(_L().aeth_conv_wgrad_bf16(self._x_bf16.ptr, dy16.ptr, self.dweights.ptr, self.dbiases.ptr, *dims))
             _ck(_L().aeth_conv_dgrad_bf16(dy16.ptr, w16.ptr, self.dinputs.ptr, *dims))
         else:
-            _ck(_L().aeth_conv_wgrad_f32(self.inputs.ptr, dvalues.ptr, self.dweights.ptr, self.dbiases.ptr, *dims))
-            _ck(_L().aeth_conv_dgrad_f32(dvalues.ptr, self.filter_weights.ptr, self.dinputs.ptr, *dims))
+            # filter / bias gradient and input gradient in one call (one launch for both where neither fills the GPU)
+            _ck(_L().aeth_conv_bwd_f32(self.inputs.ptr, dvalues.ptr, self.filter_weights.ptr, self.dweights.ptr,
+                                       self.dbiases.ptr, self.dinputs.ptr, *dims))
         return self.dinputs
 
     def get_parameters(self):

@@ -14,7 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIBDIR = os.path.join(HERE, "aether", "lib")
 LIB = os.path.join(LIBDIR, "libaether_hip.so")
-SOURCES = ["runtime.hip", "gather_f32.hip", "gather_bf16.hip", "wgrad_f32.hip", "wgrad_bf16.hip", "layers.hip"]
+SOURCES = ["runtime.hip", "gather_f32.hip", "gather_bf16.hip", "wgrad_f32.hip", "wgrad_bf16.hip", "pair_f32.hip", "layers.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",
@@ -52,7 +52,7 @@ def _compile(src, force):
 def build(force=False):
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(LIBDIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=6) as ex:
+    with ThreadPoolExecutor(max_workers=7) as ex:
         objs = list(ex.map(lambda s: _compile(s, force), SOURCES))
     if force or _stale(LIB, objs):
         cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs

@@ -27,6 +27,11 @@ int fail(int code, const char* fmt, ...);
 // replay into is kept until the last recording is destroyed; otherwise the old one is
 // freed after the stream has drained.  Fails with AETH_E_STATE while a step is being recorded.
 int workspace(int64_t bytes, void** out);
+// While a prefix is set, workspace() hands out the bytes BEHIND the first `bytes` of the buffer (and makes the buffer large
+// enough for both): the launch that owns the prefix is held back until a second one has been planned (pair_launch.h).
+// workspace_base() is the start of the current buffer, i.e. of the prefix, after whatever growth the later calls caused.
+void workspace_prefix(int64_t bytes);
+void* workspace_base();
 // Resolves the device address of the fixed scratch array of the entry point that
 // allocates nothing (gather_f32.hip); called by aeth_init with the device current.
 int conv_scratch_init(int device);

@@ -108,6 +108,14 @@ constexpr int kInvalidRow = -16384;
 constexpr int kNloopMaxN = 1024;   // widest output the n-loop mode of the gather kernel takes (its bias sits in LDS)
 constexpr int kXcds = 8;
 
+// A workgroup's place in its launch.  A kernel body that takes it as an argument can also run as one part of a launch
+// that holds two kernels, where the hardware's numbers count the workgroups of both.
+struct BlockId {
+    int x, y;            // what blockIdx.x and blockIdx.y are in a launch of the kernel alone
+    int gx;              // gridDim.x of that launch
+};
+__device__ __forceinline__ BlockId launch_block() { return BlockId{(int)blockIdx.x, (int)blockIdx.y, (int)gridDim.x}; }
+
 // Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has its
 // own L2.  This maps the hardware id to a logical id such that every XCD works on
 // one contiguous range of logical ids: tiles that share operands (the N tiles of
@@ -480,14 +488,14 @@ static __global__ __launch_bounds__(kThreads) void reduce_splits(const float* __
 // (tr as above, a multiple of 4: the 4 outputs of a thread then go to 4 rows of dw)
 // act_out != nullptr (tr == 0): the sums also go through a ReLU / leaky ReLU, act_out[i] = t > 0 ? t : alpha t, the
 // layer behind a dense product whose K was split (what relu_fwd_kernel would write from dw in a launch of its own).
-static __global__ __launch_bounds__(kThreads) void reduce_splits4(const float* __restrict__ part, float* __restrict__ dw,
-                                                          float* __restrict__ dbias, int n_dw, int n, int stride,
-                                                          int splits, int tr = 0, float* __restrict__ act_out = nullptr,
-                                                          float alpha = 0.f) {
+// (the body takes the workgroup's number as an argument: see BlockId)
+static __device__ __forceinline__ void reduce_splits4_body(const unsigned block, const float* __restrict__ part, float* __restrict__ dw,
+                                                           float* __restrict__ dbias, int n_dw, int n, int stride, int splits, int tr,
+                                                           float* __restrict__ act_out, float alpha) {
     __shared__ f4 red[16][16];
     const int cg = threadIdx.x & 15;                     // group of 4 outputs
     const int sl = threadIdx.x >> 4;                     // split lane
-    const int i = (blockIdx.x * 16 + cg) * 4;
+    const int i = (block * 16 + cg) * 4;
     f4 s = {0.f, 0.f, 0.f, 0.f};
     if (i < n) {
         const float* q = part + i;
@@ -524,6 +532,13 @@ static __global__ __launch_bounds__(kThreads) void reduce_splits4(const float* _
             *reinterpret_cast<f4*>(dbias + (i - n_dw)) = t;
         }
     }
+}
+
+static __global__ __launch_bounds__(kThreads) void reduce_splits4(const float* __restrict__ part, float* __restrict__ dw,
+                                                          float* __restrict__ dbias, int n_dw, int n, int stride,
+                                                          int splits, int tr = 0, float* __restrict__ act_out = nullptr,
+                                                          float alpha = 0.f) {
+    reduce_splits4_body(blockIdx.x, part, dw, dbias, n_dw, n, stride, splits, tr, act_out, alpha);
 }
 
 static inline int check_conv_dims(const char* fn, int S, int H, int W, int C, int D, int fH, int fW,

@@ -3,6 +3,7 @@
 #pragma once
 #include "gather_kernels.h"
 #include "narrow_kernels.h"
+#include "pair_launch.h"
 #include "sample_runs.h"
 #include "tuning.h"
 
@@ -31,6 +32,27 @@ static inline bool run_stores(const GatherParams& gp) {
     const int v = tuning().gather_runs;
     if (v == 0 || gp.out_bytes == 0) return false;
     return v > 0 || gp.out_bytes >= (64u << 20);
+}
+
+// A dgrad launch of one of the two slab-kernel forms that small layers get joins the wgrad launch that is being held
+// for it (pair_launch.h) instead of going out on its own.
+// Launches of at most 4 workgroups per CU: a pair has room for 2 per CU (the LDS of the larger body), which a launch that
+// fills the GPU many times over would feel.  (tuning: pair_bwd > 0 is a mask of the dgrad kinds that may join, bit kind - 1)
+static inline bool pair_accepts(int kind) {
+    const PairCtl& pc = pair_ctl();
+    if (!pc.armed || !pc.dgrad_ok || pc.wgrad_kind == kHeldNone || pc.dgrad_kind != kHeldNone) return false;
+    const int v = tuning().pair_bwd;
+    return v < 0 || ((v >> (kind - 1)) & 1) != 0;
+}
+
+static inline bool hold_gather_for_pair(const GatherParams& gp, const dim3& grid, int kind) {
+    PairCtl& pc = pair_ctl();
+    if (!pair_accepts(kind) || (int64_t)grid.x * grid.y > 4 * (int64_t)ctx().prop.multiProcessorCount) return false;
+    pc.dgrad_kind = kind;
+    pc.dgrad_gx = grid.x;
+    pc.dgrad_gy = grid.y;
+    pc.gather = gp;
+    return true;
 }
 
 template <typename T, int BM, int BN, int WM, int WN, int KC>
@@ -74,6 +96,9 @@ static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
                     hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, true, true>), grid, dim3(kThreads), 0, st, gp);
                     return;
                 }
+            }
+            if constexpr (KC == 8 && WM == 32 && WN == 32 && ((BM == 128 && BN == 32) || (BM == 64 && BN == 64))) {
+                if (hold_gather_for_pair(gp, grid, BM == 128 ? kHeldGather128x32 : kHeldGather64x64)) return;
             }
             hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, true>), grid, dim3(kThreads), 0, st, gp);
             return;
@@ -513,8 +538,19 @@ static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
     if (gs.gp.M > 0 && gs.gp.N > 0) {
         float* real_out = gs.gp.out;
         if (gs.nsplit > 1) gs.gp.out = reinterpret_cast<float*>(ws + ws_off + round_up(gs.bt_bytes, 256));
+        const int held_before = pair_ctl().dgrad_kind;
         launch_gather<T>(gs.gp, vec, c.prop.multiProcessorCount, c.stream);
         AETH_LAUNCH_CHECK();
+        if (pair_ctl().dgrad_kind != held_before) {            // the launch is held for a pair: so is the sum of its splits
+            HeldSum& hs = pair_ctl().dgrad_sum;
+            hs = HeldSum();
+            if (gs.nsplit > 1) {
+                hs.on = 1;
+                hs.part = gs.gp.out; hs.out = real_out;
+                hs.n_out = hs.n = hs.stride = gs.gp.M * gs.gp.N; hs.splits = gs.nsplit;
+            }
+            return AETH_OK;
+        }
         if (gs.nsplit > 1) {
             const int n = gs.gp.M * gs.gp.N;
             const bool act = gs.act != nullptr && gs.act->out != nullptr && (reinterpret_cast<uintptr_t>(gs.act->out) & 15) == 0;
@@ -533,6 +569,22 @@ static inline void set_out_divs(GatherParams& g) {
     g.div_w = FastDiv(g.Wg > 0 ? g.Wg : 1);
     g.div_c = FastDiv(g.Cs);
     g.div_tw = FastDiv(g.Tw > 0 ? g.Tw : 1);
+}
+
+// The direct dgrad of a 3x3 filter on 3 input channels (a network's first layer) joins a held wgrad launch the same way.
+template <typename T, int FH, int FW, int C>
+static inline bool hold_direct_for_pair(const DirectParams& dp, const dim3& grid) {
+    if constexpr (sizeof(T) == 4 && FH == 3 && FW == 3 && C == 3) {
+        PairCtl& pc = pair_ctl();
+        if (!pair_accepts(kHeldDirect333)) return false;
+        pc.dgrad_kind = kHeldDirect333;
+        pc.dgrad_gx = grid.x;
+        pc.dgrad_gy = 1;
+        pc.dgrad_sum = HeldSum();
+        held_direct_params() = dp;
+        return true;
+    }
+    return false;
 }
 
 template <typename T>
@@ -558,6 +610,7 @@ static bool launch_direct(DirectParams& dp, bool dgrad, hipStream_t st) {
     const size_t lds = (size_t)dp.fH * dp.fW * dp.C * dp.D * sizeof(float);
 #define AETH_DIRECT_CASE(FH_, FW_, C_)                                                                              \
     if (dp.fH == FH_ && dp.fW == FW_ && dp.C == C_) {                                                               \
+        if (dgrad2 && hold_direct_for_pair<T, FH_, FW_, C_>(dp, grid)) return true;                                   \
         if (dgrad2) hipLaunchKernelGGL((direct_dgrad_smallc<T, FH_, FW_, C_, 2>), grid, dim3(kThreads), lds, st, dp); \
         else if (dgrad) hipLaunchKernelGGL((direct_dgrad_smallc<T, FH_, FW_, C_>), grid, dim3(kThreads), lds, st, dp); \
         else if (wide) hipLaunchKernelGGL((direct_fprop_smallc<T, FH_, FW_, C_, 16>), grid, dim3(kThreads), lds, st, dp); \
@@ -678,6 +731,7 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
     constexpr int BK = Elem<T>::BK;
     const int nclass = sH * sW;
     if (nclass > 64) return fail(AETH_E_INVALID, "%s: stride too large", fn);
+    pair_ctl().dgrad_ok = nclass == 1;       // unit stride: one class, one launch, no strips of zeros
     if constexpr (sizeof(T) == 4) {
         const int64_t M = (int64_t)S * H * W;
         if (narrow_shape(D, fH, fW, sH, sW, pH, pW) && M > 0 && M * C < ((int64_t)1 << 31)) {

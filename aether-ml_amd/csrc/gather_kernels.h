@@ -196,8 +196,11 @@ __global__ __launch_bounds__(kThreads, 3) void gather_gemm(const GatherParams p)
 // x BN floats (1 KB loads of 4 or 8 rows; with 64 columns the odd rows are stored with their halves swapped, so that the two
 // lane halves of a 4-byte operand read, which sit one row apart, use different banks), and an operand read is four 4-byte reads
 // from four rows instead of one 16-byte read.  No packing launch.
+// The body takes the workgroup's place in the launch and its four slab buffers as arguments, so that it can also be one
+// part of a launch that holds two kernels (pair_f32.hip).
 template <typename T, int BM, int BN, int WM, int WN, bool UT, int KC, bool NLOOP, bool SA = false, bool RUNS = false, bool BKN = false>
-__global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(const GatherParams p) {
+__device__ __forceinline__ void gather_gemm_dma_body(const GatherParams& p, const BlockId blk, f4* lds_a0, f4* lds_a1, f4* lds_b0,
+                                                     f4* lds_b1) {
     static_assert(!BKN || (sizeof(T) == 4 && KC == 8 && !NLOOP && (BN == 64 || BN == 32)), "filter in place: fp32 slab tiles");
     // 4 waves, or 8 for the widest bf16 tiles (256 x 128 and 256 x 256: one workgroup per CU)
     constexpr int NW = (BM / WM) * (BN / WN);
@@ -219,11 +222,6 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
     constexpr int TM = WM / 32;
     constexpr int TN = WN / 32;
 
-    __shared__ f4 lds_a0[BM * KC];
-    __shared__ f4 lds_a1[BM * KC];
-    __shared__ f4 lds_b0[BN * KC];
-    __shared__ f4 lds_b1[BN * KC];
-
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -232,7 +230,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
     const int wm0 = (wave % (BM / WM)) * WM;
     const int wn0 = (wave / (BM / WM)) * WN;
     const int ntile = (p.N + BN - 1) / BN;
-    const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
+    const int lid = xcd_contiguous_id(blk.x, blk.gx);
     // (one n tile: no division; the compiler divides scalars by way of the vector unit's reciprocal, some 20
     // vector instructions that a workgroup starting next to busy ones waits for one by one)
     const int mt = (NLOOP || ntile == 1) ? lid : lid / ntile;
@@ -240,7 +238,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
     int n0 = (NLOOP || ntile == 1) ? 0 : (lid - mt * ntile) * BN;
 
     // The bias is fetched first: its latency passes behind the row decode.
-    const int split = (int)blockIdx.y;
+    const int split = blk.y;
     f4 bv[TN][4];
     load_bias<TN>(p, split == 0 ? p.bias : nullptr, bv, n0 + wn0, lh);
 
@@ -624,6 +622,15 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(co
     if constexpr (RUNS && TN == 1) store_tile_lines<TM, TN>(p, p.out + (size_t)split * p.M * p.N, acc, m0 + wm0, n0 + wn0, l32, lh, p.M);
     else if constexpr (RUNS) store_tile_runs<TM, TN>(p, p.out + (size_t)split * p.M * p.N, acc, m0 + wm0, n0 + wn0, l32, lh, p.M);
     else store_tile<TM, TN>(p, p.out + (size_t)split * p.M * p.N, acc, m0 + wm0, n0 + wn0, l32, lh);
+}
+
+template <typename T, int BM, int BN, int WM, int WN, bool UT, int KC, bool NLOOP, bool SA = false, bool RUNS = false, bool BKN = false>
+__global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gather_gemm_dma(const GatherParams p) {
+    __shared__ f4 lds_a0[BM * KC];
+    __shared__ f4 lds_a1[BM * KC];
+    __shared__ f4 lds_b0[BN * KC];
+    __shared__ f4 lds_b1[BN * KC];
+    gather_gemm_dma_body<T, BM, BN, WM, WN, UT, KC, NLOOP, SA, RUNS, BKN>(p, launch_block(), lds_a0, lds_a1, lds_b0, lds_b1);
 }
 
 // ------------------------------------------------------------------------------
@@ -1662,12 +1669,12 @@ static __global__ __launch_bounds__(kThreads) void direct_fprop_smallc(const Dir
 
 // NG = groups of 4 output channels per lane, 1 or 2.  With 2 a lane does the work of two neighbouring lanes of the
 // one-group form and adds their sums as the first xor-shuffle of that form would: same bits, half the address work.
+// (the body takes the workgroup's number and the filter's place in LDS as arguments: see BlockId)
 template <typename T, int FH, int FW, int C, int NG = 1>
-static __global__ __launch_bounds__(kThreads) void direct_dgrad_smallc(const DirectParams p) {
-    extern __shared__ __attribute__((aligned(16))) float wl[];
+static __device__ __forceinline__ void direct_dgrad_body(const DirectParams& p, const unsigned block, float* wl) {
     direct_load_filter<T>(p, wl);
     const T* __restrict__ dy = static_cast<const T*>(p.a);
-    const int g = (int)(blockIdx.x * kThreads + threadIdx.x);
+    const int g = (int)(block * kThreads + threadIdx.x);
     const int m = g >> p.q_shift;                            // a pixel's lanes sit in one wave: q_shift <= 6
     const int q = g & ((1 << p.q_shift) - 1);
     unsigned s_, rem, i, j;
@@ -1728,6 +1735,12 @@ static __global__ __launch_bounds__(kThreads) void direct_dgrad_smallc(const Dir
         for (int c = 0; c < C; ++c)
             if (q == c) p.out[(size_t)m * C + c] = sum[c];
     }
+}
+
+template <typename T, int FH, int FW, int C, int NG = 1>
+static __global__ __launch_bounds__(kThreads) void direct_dgrad_smallc(const DirectParams p) {
+    extern __shared__ __attribute__((aligned(16))) float wl[];
+    direct_dgrad_body<T, FH, FW, C, NG>(p, blockIdx.x, wl);
 }
 
 // The shapes the direct kernels take; everything else goes to the gather kernels.

@@ -51,7 +51,7 @@ bool tuning_set(const char* name, int value) {
         {"gather_pairs", &Tuning::gather_pairs},
         {"gather_runs", &Tuning::gather_runs},   {"narrow", &Tuning::narrow},   {"gather_bkn", &Tuning::gather_bkn},
         {"wgrad_br", &Tuning::wgrad_br},         {"wgrad_rounds", &Tuning::wgrad_rounds},
-        {"wgrad_swap", &Tuning::wgrad_swap},
+        {"wgrad_swap", &Tuning::wgrad_swap},     {"pair_bwd", &Tuning::pair_bwd},
     };
     for (const Field& f : fields)
         if (strcmp(f.name, name) == 0) {
@@ -85,10 +85,14 @@ void tuning_parse(const char* spec, const char** bad) {
 static WorkspaceLedger g_ws;                            // the scratch workspace and who may still use old ones
 static bool recording_open() { return g_ws.recording_open; }
 
+static int64_t g_ws_prefix = 0;
+void workspace_prefix(int64_t bytes) { g_ws_prefix = bytes > 0 ? round_up(bytes, 256) : 0; }
+void* workspace_base() { return g_ws.cur; }
+
 int workspace(int64_t bytes, void** out) {
     hipError_t err = hipSuccess;
     const WorkspaceLedger::Result r = g_ws.acquire(
-        bytes, out,
+        bytes + g_ws_prefix, out,
         [&](int64_t want) -> void* {
             void* p = nullptr;
             err = hipMalloc(&p, (size_t)want);
@@ -101,7 +105,8 @@ int workspace(int64_t bytes, void** out) {
         return fail(AETH_E_STATE, "the workspace would have to grow while a step is being recorded: run the step once first");
     if (r == WorkspaceLedger::kAllocFailed)
         return fail(err == hipErrorOutOfMemory ? AETH_E_NOMEM : AETH_E_HIP, "workspace: hipMalloc(%lld bytes) -> %s",
-                    (long long)WorkspaceLedger::grown_size(bytes), hipGetErrorString(err));
+                    (long long)WorkspaceLedger::grown_size(bytes + g_ws_prefix), hipGetErrorString(err));
+    *out = static_cast<char*>(*out) + g_ws_prefix;
     return AETH_OK;
 }
 

@@ -34,6 +34,7 @@ struct Tuning {
     int wgrad_br = -1;       // slab height of the 192-wide form: 32 or 16
     int wgrad_swap = -1;     // fp32 1x1 wgrad on few input channels with the operands swapped: 0 never, 1 wherever it applies
     int wgrad_rounds = -1;   // rounds of resident workgroups the splits are sized for: 1 to 4
+    int pair_bwd = -1;       // 0: the backward entry points launch a layer's wgrad and dgrad one after the other
 };
 
 Tuning& tuning();

@@ -2,6 +2,7 @@
 #pragma once
 #include "wgrad_kernels.h"
 #include "narrow_kernels.h"
+#include "pair_launch.h"
 #include "sample_runs.h"
 #include "tuning.h"
 
@@ -264,6 +265,28 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     p.db_out = single ? dbias : nullptr;
     p.kt = kt; p.nt = nt;
     dim3 grid(kt * nt * splits);
+    const int n = (int)(kd + (dbias ? p.db_len : 0));
+    const bool r4 = kd % 4 == 0 && D % 4 == 0 && p.db_len % 4 == 0 && (reinterpret_cast<uintptr_t>(dw) & 15) == 0 &&
+                    (dbias == nullptr || (reinterpret_cast<uintptr_t>(dbias) & 15) == 0);
+    if constexpr (sizeof(T) == 4) {
+        // An entry point that also computes this layer's input gradient is collecting the launches (pair_launch.h): the
+        // two fp32 LDS-direct forms with 32-row slabs wait for the dgrad launch to share a grid with.
+        PairCtl& pc = pair_ctl();
+        if (pc.armed && pc.wgrad_kind == kHeldNone && dma && !swapped && (p.cw != 6 || br == 32) && (single || r4)) {
+            pc.wgrad_kind = p.cw == 6 ? kHeldWgrad192 : kHeldWgrad128;
+            pc.wgrad_blocks = grid.x;
+            pc.wgrad_in_ws = !single;
+            held_wgrad_params() = p;
+            pc.wgrad_sum = HeldSum();
+            if (!single) {
+                pc.wgrad_sum.on = 1;
+                pc.wgrad_sum.out = dw; pc.wgrad_sum.dbias = dbias;
+                pc.wgrad_sum.n_out = (int)kd; pc.wgrad_sum.n = n; pc.wgrad_sum.stride = (int)(kd + p.db_len); pc.wgrad_sum.splits = splits;
+                workspace_prefix((int64_t)splits * (kd + p.db_len) * (int64_t)sizeof(float));
+            }
+            return AETH_OK;
+        }
+    }
     if (wide_k) hipLaunchKernelGGL((wgrad_gemm_dma_bf16w<4, 4>), grid, dim3(512), 0, c.stream, p);
     else if (wide_nb == 4) hipLaunchKernelGGL((wgrad_gemm_dma_bf16w<2, 4>), grid, dim3(kThreads), 0, c.stream, p);
     else if (wide_nb == 2) hipLaunchKernelGGL((wgrad_gemm_dma_bf16w<2, 2>), grid, dim3(kThreads), 0, c.stream, p);
@@ -277,9 +300,6 @@ int conv_wgrad_impl(const char* fn, const T* x, const T* dy, float* dw, float* d
     else hipLaunchKernelGGL((wgrad_gemm<T, 1, 1>), grid, dim3(kThreads), 0, c.stream, p);
     AETH_LAUNCH_CHECK();
     if (single) return AETH_OK;
-    const int n = (int)(kd + (dbias ? p.db_len : 0));
-    const bool r4 = kd % 4 == 0 && D % 4 == 0 && p.db_len % 4 == 0 && (reinterpret_cast<uintptr_t>(dw) & 15) == 0 &&
-                    (dbias == nullptr || (reinterpret_cast<uintptr_t>(dbias) & 15) == 0);
     const int tr = swapped ? D : 0;                      // the partials hold dw^T in rows of D (the caller's C) floats
     if (r4)
         hipLaunchKernelGGL(reduce_splits4, dim3(cdiv(n, 64)), dim3(kThreads), 0, c.stream, (const float*)ws, dw, dbias,

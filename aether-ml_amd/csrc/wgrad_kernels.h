@@ -264,7 +264,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_gemm(const WgradParams p) {
 // ------------------------------------------------------------------------------
 template <int CW, int BR = kWgBR>                        // BR rows of m per slab: 32, or 16 (CW == 6 only)
 static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, float* lds_a0, float* lds_a1, float* lds_y0,
-                                                       float* lds_y1) {
+                                                       float* lds_y1, const BlockId blk) {
     static_assert(BR == 32 || (BR == 16 && CW == 6), "slab heights");
     constexpr int RW = BR / 4;                           // slab rows a wave loads
     constexpr int YL = BR / 16;                          // dy loads per wave per slab (4 rows x 16 chunks each)
@@ -292,7 +292,7 @@ static __device__ __forceinline__ void wgrad_dma_body(const WgradParams& p, floa
     const int nt = wave & 1;                             // n half of this wave
     const int mh = wave >> 1;                            // parity of the m pairs it multiplies
 
-    const int lid = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
+    const int lid = xcd_contiguous_id(blk.x, blk.gx);
     const int tiles = p.kt * p.nt;
     const int split = lid / tiles;
     const int tile = lid - split * tiles;
@@ -563,9 +563,9 @@ static __global__ __launch_bounds__(kThreads, 3) void wgrad_gemm_dma(const Wgrad
     // (measured on K = 576: 722 MB fetched with a fast last tile, 445 MB with an even pace
     // at 1.5 % more time for its padded MFMAs).
     // p.cw (workgroup-uniform): 1 for channel counts that are not multiples of 4
-    if (p.cw == 1) wgrad_dma_body<1>(p, lds_a0, lds_a1, lds_y0, lds_y1);
-    else if (p.cw == 2) wgrad_dma_body<2>(p, lds_a0, lds_a1, lds_y0, lds_y1);
-    else wgrad_dma_body<4>(p, lds_a0, lds_a1, lds_y0, lds_y1);
+    if (p.cw == 1) wgrad_dma_body<1>(p, lds_a0, lds_a1, lds_y0, lds_y1, launch_block());
+    else if (p.cw == 2) wgrad_dma_body<2>(p, lds_a0, lds_a1, lds_y0, lds_y1, launch_block());
+    else wgrad_dma_body<4>(p, lds_a0, lds_a1, lds_y0, lds_y1, launch_block());
 }
 
 // The 192-wide k tile: 64 KB of LDS, two workgroups per CU.
@@ -574,7 +574,7 @@ static __global__ __launch_bounds__(kThreads, 2) void wgrad_gemm_dma192(const Wg
     __shared__ float lds_a1[kWgBR * 192];
     __shared__ float lds_y0[kWgBR * kWgBN];
     __shared__ float lds_y1[kWgBR * kWgBN];
-    wgrad_dma_body<6>(p, lds_a0, lds_a1, lds_y0, lds_y1);
+    wgrad_dma_body<6>(p, lds_a0, lds_a1, lds_y0, lds_y1, launch_block());
 }
 
 // The same with 16-row slabs: 32 KB of LDS and half the per-load state, so that three
@@ -584,7 +584,7 @@ static __global__ __launch_bounds__(kThreads, 3) void wgrad_gemm_dma192h(const W
     __shared__ float lds_a1[16 * 192];
     __shared__ float lds_y0[16 * kWgBN];
     __shared__ float lds_y1[16 * kWgBN];
-    wgrad_dma_body<6, 16>(p, lds_a0, lds_a1, lds_y0, lds_y1);
+    wgrad_dma_body<6, 16>(p, lds_a0, lds_a1, lds_y0, lds_y1, launch_block());
 }
 
 // ------------------------------------------------------------------------------

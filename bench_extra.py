@@ -123,7 +123,9 @@ def build_cnn(aether):
     return m
 
 
-def train_step(steps, warmup):
+def train_step(steps, warmup, eager_only=False):
+    """`eager_only`: no recorded steps and no Model.train loops (a kernel trace of the step: the launches of an eager step
+    are those a recording replays)."""
     import aether
     from aether import _lib
     np.random.seed(0)
@@ -146,6 +148,8 @@ def train_step(steps, warmup):
 
     np.random.seed(0)
     med, loss = timed(build_cnn(aether))
+    if eager_only:
+        return {"ms_per_step_median": med * 1e3, "images_per_sec": 128.0 / med, "batch": 128, "last_loss": loss}
     np.random.seed(0)
     recorded = build_cnn(aether)
     recorded.record_steps(True)
@@ -343,7 +347,7 @@ if __name__ == "__main__":
     elif "--layers" in sys.argv:
         print(json.dumps(layer_kernels(20, 5), indent=1))
     elif "--train-only" in sys.argv:
-        print(json.dumps(train_step(50, 10), indent=1))
+        print(json.dumps(train_step(50, 10, eager_only="--eager" in sys.argv), indent=1))
     elif "--shape" in sys.argv:
         # one shape of the list only, e.g. --shape cfg4_1x1_64_to256 (for profiler runs)
         print(json.dumps(conv_table(20, 2, only=sys.argv[sys.argv.index("--shape") + 1]), indent=1))

@@ -107,6 +107,15 @@ int aeth_conv_wgrad_f32(const float* x, const float* dy, float* dw, float* dbias
                         int S, int H, int W, int C, int D,
                         int fH, int fW, int sH, int sW, int pH, int pW);
 
+/* Conv_Layer.backward :122-153 in one call: the wgrad and the dgrad above, bit for bit.  The two
+ * products do not depend on each other, and where neither fills the GPU (the layers of a small
+ * network: unit stride, a few hundred workgroups each) they go out as ONE launch whose
+ * workgroups are shared between them, and their split sums as one more; everywhere else the
+ * call is the two calls above in a row.  dbias may be NULL. */
+int aeth_conv_bwd_f32(const float* x, const float* dy, const float* w, float* dw, float* dbias, float* dx,
+                      int S, int H, int W, int C, int D,
+                      int fH, int fW, int sH, int sW, int pH, int pW);
+
 /* aeth_conv_fprop_f32 for callers that cannot allocate (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
  * reference.  Same arguments, same kernels, bit-identical results; the packed filter and
@@ -158,7 +167,8 @@ int aeth_dense_wgrad_f32(const float* x, const float* dy, float* dw, float* dbia
  * regulariser terms stay with the caller) and, with act_in / act_dx not NULL, the backward
  * pass of the activation IN FRONT of the layer on the way: act_dx = act_in < 0 ? alpha * dx
  * : dx (act_in = that activation's input).  A layer of at most 16 outputs on at most 1024
- * rows goes out as one launch. */
+ * rows goes out as one launch; a wider layer on a small batch shares one launch between its
+ * weight gradient and its input gradient, as aeth_conv_bwd_f32 does. */
 int aeth_dense_fprop_act_f32(const float* x, const float* w, const float* bias, float* y, float* act_y,
                              float alpha, int M, int n_in, int n_out);
 int aeth_dense_bwd_f32(const float* x, const float* dy, const float* w, float* dw, float* dbias, float* dx,
