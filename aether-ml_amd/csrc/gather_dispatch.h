@@ -34,6 +34,66 @@ static inline bool run_stores(const GatherParams& gp) {
     return v > 0 || gp.out_bytes >= (64u << 20);
 }
 
+// The classes of a strided fp32 dgrad: while armed, a class whose launch is the 128 x 64 slab kernel with scalar addressing
+// and an unsplit K is collected here instead of going out, and conv_dgrad_impl launches what it has collected as one grid.
+struct ClassHold {
+    bool armed = false;
+    int count = 0;
+    bool runs[kMaxClasses];
+    unsigned blocks[kMaxClasses];
+    GatherParams gp[kMaxClasses];
+};
+static inline ClassHold& class_hold() {
+    static ClassHold h;
+    return h;
+}
+static inline bool hold_class(const GatherParams& gp, const dim3& grid, bool runs) {
+    ClassHold& h = class_hold();
+    if (!h.armed || h.count >= kMaxClasses || grid.y != 1 || gp.split_slabs != 0) return false;
+    h.runs[h.count] = runs;
+    h.blocks[h.count] = grid.x;
+    h.gp[h.count] = gp;
+    ++h.count;
+    return true;
+}
+// Launches what was collected: one grid when every class of the dgrad was collected with the same store form, else the
+// collected ones one by one (the others have gone out already; the classes write disjoint pixels of dx).
+static inline void flush_classes(int nclass, hipStream_t st) {
+    ClassHold& h = class_hold();
+    h.armed = false;
+    bool same = h.count == nclass && h.count > 1;
+    for (int i = 1; i < h.count; ++i) same = same && h.runs[i] == h.runs[0];
+    if (!same) {
+        for (int i = 0; i < h.count; ++i) {
+            if (h.runs[i]) hipLaunchKernelGGL((gather_gemm_dma<float, 128, 64, 32, 64, true, 8, false, true, true>), dim3(h.blocks[i]), dim3(kThreads), 0, st, h.gp[i]);
+            else hipLaunchKernelGGL((gather_gemm_dma<float, 128, 64, 32, 64, true, 8, false, true>), dim3(h.blocks[i]), dim3(kThreads), 0, st, h.gp[i]);
+        }
+        h.count = 0;
+        return;
+    }
+    int order[kMaxClasses];                                  // most taps first
+    for (int i = 0; i < h.count; ++i) {
+        int j = i;
+        for (; j > 0 && h.gp[order[j - 1]].K < h.gp[i].K; --j) order[j] = order[j - 1];
+        order[j] = i;
+    }
+    GatherClasses gc;
+    ClassGrid cg;
+    unsigned total = 0;
+    for (int i = 0; i < kMaxClasses; ++i) {
+        cg.start[i] = total;
+        cg.blocks[i] = 0;
+        if (i >= h.count) continue;
+        gc.cls[i] = h.gp[order[i]];
+        cg.blocks[i] = h.blocks[order[i]];
+        total += (unsigned)round_up(cg.blocks[i], kXcds);
+    }
+    gc.ncls = h.count;
+    if (h.runs[0]) hipLaunchKernelGGL(gather_classes_f32<true>, dim3(total), dim3(kThreads), 0, st, gc, cg);
+    else hipLaunchKernelGGL(gather_classes_f32<false>, dim3(total), dim3(kThreads), 0, st, gc, cg);
+    h.count = 0;
+}
+
 // A dgrad launch of one of the two slab-kernel forms that small layers get joins the wgrad launch that is being held
 // for it (pair_launch.h) instead of going out on its own.
 // Launches of at most 4 workgroups per CU: a pair has room for 2 per CU (the LDS of the larger body), which a launch that
@@ -90,6 +150,9 @@ static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
                     hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, true, false, true>), grid, dim3(kThreads), 0, st, gp);
                     return;
                 }
+            }
+            if constexpr (BM == 128 && BN == 64 && WM == 32 && WN == 64 && KC == 8) {
+                if (hold_class(gp, grid, runs)) return;
             }
             if constexpr (WN == 64 || WN == 32) {
                 if (runs) {
@@ -884,11 +947,23 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
     rc = workspace(total_bytes > 0 ? total_bytes : 256, &ws);
     if (rc) return rc;
     int64_t off = 0;
+    // fp32, 2 to 4 classes: the classes that the 128 x 64 slab kernel takes are collected and go out as one grid
+    // (tuning: gather_merge = 0 keeps one launch per class)
+    const bool collect = sizeof(T) == 4 && sets.size() >= 2 && (int)sets.size() <= kMaxClasses && tuning().gather_merge != 0;
+    if (collect) {
+        class_hold().count = 0;
+        class_hold().armed = true;
+    }
     for (auto& gs : sets) {
         rc = run_gather<T>(gs, (char*)ws, off, D % Elem<T>::CE == 0);
-        if (rc) return rc;
+        if (rc) break;
         off += gs.bt_bytes + gs.part_bytes;
     }
+    if (collect) {
+        flush_classes((int)sets.size(), ctx().stream);
+        if (rc == AETH_OK) AETH_LAUNCH_CHECK();
+    }
+    if (rc) return rc;
     if (h_lim < H || w_lim < W) {
         ZeroStripParams zp;
         zp.dx = dx; zp.S = S; zp.H = H; zp.W = W; zp.C = C; zp.h0 = h_lim; zp.w0 = w_lim;

@@ -446,6 +446,37 @@ def test_strided_dgrad_with_clipped_class_grids(case, tune):
     assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
 
 
+# Strided fp32 dgrad whose classes all take the 128 x 64 slab kernel (64 input channels and more, many pixels; the
+# gather_bm switch lets small inputs reach it): the classes go out as ONE grid, most taps first.  With gather_merge at 0
+# every class is a launch of its own; same bits either way.  S, H, W, C, D, fH, fW, sH, sW, padding
+MERGED_CLASS_CASES = [
+    (6, 13, 13, 64, 64, 3, 3, 2, 2, "valid"),     # 4 classes of 4, 2, 2 and 1 taps, clipped to different pixel grids
+    (4, 12, 14, 128, 96, 3, 3, 2, 2, "same"),     # two n tiles per class
+    (5, 9, 16, 64, 32, 3, 3, 1, 2, "same"),       # stride (1, 2): 2 classes
+    (3, 11, 11, 72, 64, 5, 5, 2, 2, "same"),      # 72 input channels: a ragged n tile; 9, 6, 6 and 4 taps
+    (2, 12, 12, 64, 64, 3, 3, 3, 3, "valid"),     # 9 classes: more than one grid takes, one launch each
+    (4, 10, 10, 64, 40, 2, 2, 2, 2, "valid"),     # one tap per class; 40 output channels: slabs that are not whole
+]
+
+
+@pytest.mark.parametrize("case", MERGED_CLASS_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_strided_dgrad_with_its_classes_in_one_launch(case, tune):
+    from tests import abi
+    x, w, b, dy = _case(case, 23)
+    stride, pad = (case[7], case[8]), case[9]
+    want = O.conv_dgrad(dy, w, x.shape[1:3], stride, pad, dtype=np.float64)
+    tune(gather_bm=128, gather_split=0)
+    dx = abi.dgrad(dy, w, x.shape, stride, pad)
+    abi.close(dx, want)
+    tune(gather_runs=1)                                  # the tiles stored as runs of contiguous channels
+    dx_runs = abi.dgrad(dy, w, x.shape, stride, pad)
+    assert np.array_equal(dx, dx_runs)
+    tune(gather_merge=0)
+    assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
+    tune(gather_runs=0)
+    assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
+
+
 # fp32 wgrad of a unit-stride filter of at most 9 taps on 64 input channels and at most 64 output
 # channels, on rows of 28, 32, 56 or 64 output pixels: one persistent workgroup per CU keeps the whole
 # K x N result in registers (12 multiplying waves of three 32 x 32 blocks) and a loading wave brings one
