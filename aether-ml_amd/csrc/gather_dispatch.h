@@ -34,14 +34,16 @@ static inline bool run_stores(const GatherParams& gp) {
     return v > 0 || gp.out_bytes >= (64u << 20);
 }
 
-// The classes of a strided fp32 dgrad: while armed, a class whose launch is the 128 x 64 slab kernel with scalar addressing
-// and an unsplit K is collected here instead of going out, and conv_dgrad_impl launches what it has collected as one grid.
+// The problems of a strided fp32 dgrad: while armed, a problem whose launch is the 128 x 64 slab kernel with scalar addressing
+// and an unsplit K is collected here instead of going out, and conv_dgrad_impl launches what it has collected in grids of up to
+// kMaxClassesF32 problems.
+constexpr int kMaxHeldClasses = 16;
 struct ClassHold {
     bool armed = false;
     int count = 0;
-    bool runs[kMaxClasses];
-    unsigned blocks[kMaxClasses];
-    GatherParams gp[kMaxClasses];
+    bool runs[kMaxHeldClasses];
+    unsigned blocks[kMaxHeldClasses];
+    GatherParams gp[kMaxHeldClasses];
 };
 static inline ClassHold& class_hold() {
     static ClassHold h;
@@ -49,19 +51,20 @@ static inline ClassHold& class_hold() {
 }
 static inline bool hold_class(const GatherParams& gp, const dim3& grid, bool runs) {
     ClassHold& h = class_hold();
-    if (!h.armed || h.count >= kMaxClasses || grid.y != 1 || gp.split_slabs != 0) return false;
+    if (!h.armed || h.count >= kMaxHeldClasses || grid.y != 1 || gp.split_slabs != 0) return false;
     h.runs[h.count] = runs;
     h.blocks[h.count] = grid.x;
     h.gp[h.count] = gp;
     ++h.count;
     return true;
 }
-// Launches what was collected: one grid when every class of the dgrad was collected with the same store form, else the
-// collected ones one by one (the others have gone out already; the classes write disjoint pixels of dx).
-static inline void flush_classes(int nclass, hipStream_t st) {
+// Launches what was collected: shared grids, the problems with the most taps first, when all problems of the dgrad were collected
+// with the same store form; else the collected ones one by one (the others have gone out already; the problems write
+// disjoint pixels of dx).
+static inline void flush_classes(int nsets, hipStream_t st) {
     ClassHold& h = class_hold();
     h.armed = false;
-    bool same = h.count == nclass && h.count > 1;
+    bool same = h.count == nsets && h.count > 1;
     for (int i = 1; i < h.count; ++i) same = same && h.runs[i] == h.runs[0];
     if (!same) {
         for (int i = 0; i < h.count; ++i) {
@@ -71,26 +74,28 @@ static inline void flush_classes(int nclass, hipStream_t st) {
         h.count = 0;
         return;
     }
-    int order[kMaxClasses];                                  // most taps first
+    int order[kMaxHeldClasses];                              // most taps first
     for (int i = 0; i < h.count; ++i) {
         int j = i;
         for (; j > 0 && h.gp[order[j - 1]].K < h.gp[i].K; --j) order[j] = order[j - 1];
         order[j] = i;
     }
-    GatherClasses gc;
-    ClassGrid cg;
-    unsigned total = 0;
-    for (int i = 0; i < kMaxClasses; ++i) {
-        cg.start[i] = total;
-        cg.blocks[i] = 0;
-        if (i >= h.count) continue;
-        gc.cls[i] = h.gp[order[i]];
-        cg.blocks[i] = h.blocks[order[i]];
-        total += (unsigned)round_up(cg.blocks[i], kXcds);
+    for (int first = 0; first < h.count; first += kMaxClassesF32) {
+        GatherClassesF32 gc;
+        ClassGrid cg;
+        unsigned total = 0;
+        gc.ncls = std::min(kMaxClassesF32, h.count - first);
+        for (int i = 0; i < kMaxClassesF32; ++i) {
+            cg.start[i] = total;
+            cg.blocks[i] = 0;
+            if (i >= gc.ncls) continue;
+            gc.cls[i] = h.gp[order[first + i]];
+            cg.blocks[i] = h.blocks[order[first + i]];
+            total += (unsigned)round_up(cg.blocks[i], kXcds);
+        }
+        if (h.runs[0]) hipLaunchKernelGGL(gather_classes_f32<true>, dim3(total), dim3(kThreads), 0, st, gc, cg);
+        else hipLaunchKernelGGL(gather_classes_f32<false>, dim3(total), dim3(kThreads), 0, st, gc, cg);
     }
-    gc.ncls = h.count;
-    if (h.runs[0]) hipLaunchKernelGGL(gather_classes_f32<true>, dim3(total), dim3(kThreads), 0, st, gc, cg);
-    else hipLaunchKernelGGL(gather_classes_f32<false>, dim3(total), dim3(kThreads), 0, st, gc, cg);
     h.count = 0;
 }
 
@@ -207,6 +212,13 @@ static void launch_gather_cfg(const GatherParams& gp, bool vec, bool kc4, hipStr
 
 static inline int gather_bn(int N) { return N <= 32 ? 32 : 64; }
 
+// Set while the problems of one strided fp32 dgrad are planned and launched so that all of them, the border strips
+// included, take the 128-row slab kernel with an unsplit K and can share one grid (conv_dgrad_impl).
+static inline bool& uniform_class_tiles() {
+    static bool on = false;
+    return on;
+}
+
 // Tile height.  The LDS-direct kernel keeps two slabs per operand in LDS, so a
 // 128-row tile (48 KB) lets three workgroups share a CU where a 256-row tile
 // (80 KB) allows one or two; measured on the 56x56x64 shape, 128 rows is 11 %
@@ -223,6 +235,7 @@ static inline int gather_bm(int M, int N, int cus, bool dma, int elem_bytes = 4)
         const int v = tuning().gather_bm;
         if (v == 256 || v == 128 || (v == 64 && bn == 64)) return v;
     }
+    if (uniform_class_tiles() && elem_bytes == 4) return 128;
     const int ntiles = cdiv(N, bn);
     const int want = elem_bytes == 2 ? cus : 2 * cus;   // bf16: the taller tile pays off from one tile per CU on
     const int cands[3] = {256, 128, 64};
@@ -494,6 +507,7 @@ static void plan_split(GatherSetup& gs, bool vec, int cus) {
     if (!dma || !g.dense_out || g.N % 4 != 0 || ob >= lim || (reinterpret_cast<uintptr_t>(g.out) & 15) != 0) return;
     if (tuning().gather_kc != -1) return;                    // the tuning switch changes the slab depth
     if (tuning().gather_split == 0) return;                  // lets small inputs reach the kernels of large ones
+    if (uniform_class_tiles()) return;
     const int bn = gather_bn(g.N), bm = gather_bm(g.M, g.N, cus, true, (int)sizeof(T));
     const int64_t tiles = (int64_t)cdiv(g.M, bm) * cdiv(g.N, bn);
     const int nslabs = g.Kpad / Elem<T>::BK;
@@ -768,6 +782,27 @@ int conv_fprop_impl(const char* fn, const T* x, const T* w, const float* bias, f
     return run_gather<T>(gs, (char*)ws, 0, C % Elem<T>::CE == 0);
 }
 
+// Rows (or columns) [r0, r1) of a dgrad class and the taps [t0, t1) of the class that fall inside dy for all of them.
+struct TapSpan {
+    int r0, r1, t0, t1;
+};
+// Class row r reads dy row r + off + t under tap t (0 <= t < taps), which exists for 0 <= r + off + t < len.  Returns the
+// maximal runs of rows with the same range of existing taps (`split`), or one span with all taps.
+static inline std::vector<TapSpan> tap_spans(int rows, int off, int taps, int len, bool split) {
+    std::vector<TapSpan> out;
+    if (!split || taps <= 0) {
+        out.push_back(TapSpan{0, rows, 0, taps > 0 ? taps : 0});
+        return out;
+    }
+    for (int r = 0; r < rows; ++r) {
+        const int lo = std::min(taps, std::max(0, -(r + off)));
+        const int hi = std::max(lo, std::min(taps, len - (r + off)));
+        if (!out.empty() && out.back().t0 == lo && out.back().t1 == hi) out.back().r1 = r + 1;
+        else out.push_back(TapSpan{r, r + 1, lo, hi});
+    }
+    return out;
+}
+
 // dgrad: for input row i the contributing taps are x with (i + pH - x) % sH == 0 and
 // 0 <= (i + pH - x)/sH < Ho.  Rows are split by a = i % sH; inside a class the taps
 // are x_t = xmax - sH*t (xmax = largest x < fH with x == (a+pH) mod sH), and the
@@ -830,9 +865,13 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
     }
     std::vector<GatherSetup> sets;
     int64_t total_bytes = 0;
-    auto build_sets = [&](int hl, int wl) {
+    // `borders`: a class is cut into the runs of rows and columns that see the same taps inside dy (first rows, interior,
+    // last rows), each a problem of its own with only those taps, so that no tile multiplies a tap that lies outside.
+    int64_t taps_whole = 0, taps_inside = 0;                 // tap-pixels multiplied per sample without and with the cut
+    auto build_sets = [&](int hl, int wl, bool borders = false) {
         sets.clear();
         total_bytes = 0;
+        taps_whole = taps_inside = 0;
         for (int a = 0; a < sH; ++a) {
             if (a >= H) continue;
             int ra = (a + pH) % sH;
@@ -847,26 +886,35 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
                 int ymax = rb + (Tw - 1) * sW;
                 int offw = Tw > 0 ? (b + pW - ymax) / sW : 0;
                 int Wg = (std::min(W, std::max(wl, b + 1)) - b + sW - 1) / sW;
-                GatherSetup gs;
-                GatherParams& g = gs.gp;
-                g.src = dy; g.bias = nullptr; g.out = dx;
-                g.S = S; g.Hs = Ho; g.Ws = Wo; g.Cs = D;
-                g.Hg = Hg; g.Wg = Wg; g.M = S * Hg * Wg; g.N = C;
-                g.K = Th * Tw * D;
-                g.Kpad = (int)round_up(g.K, BK);
-                g.Tw = Tw; g.sh = 1; g.sw = 1; g.rh0 = offh; g.rw0 = offw;
-                g.Hof = H; g.Wof = W; g.oh0 = a; g.ow0 = b; g.ohs = sH; g.ows = sW;
-                g.dense_out = (nclass == 1);
-                set_out_divs(g);
-                PackParams& pk = gs.pp;
-                pk.w = w; pk.fW = fW; pk.C = C; pk.D = D; pk.Tw = Tw > 0 ? Tw : 1; pk.Ck = D; pk.w_elems = (int64_t)fH * fW * C * D;
-                pk.xa = xmax; pk.xs = -sH; pk.ya = ymax; pk.ys = -sW; pk.transposed = 1;
-                pk.N = C; pk.K = g.K; pk.Npad = (int)round_up(C, 64); pk.Kpad = g.Kpad;
-                gs.bt_bytes = round_up((int64_t)pk.Npad * pk.Kpad * sizeof(T), 256);
-                g.split_slabs = 0;
-                plan_split<T>(gs, D % Elem<T>::CE == 0, ctx().prop.multiProcessorCount);
-                total_bytes += gs.bt_bytes + gs.part_bytes;
-                sets.push_back(gs);
+                taps_whole += (int64_t)Hg * Wg * Th * Tw;
+                const bool cut = borders && Th > 0 && Tw > 0;
+                for (const TapSpan& rs : tap_spans(Hg, offh, Th, Ho, cut))
+                    for (const TapSpan& cs : tap_spans(Wg, offw, Tw, Wo, cut)) {
+                        const int th = rs.t1 - rs.t0, tw = cs.t1 - cs.t0;     // taps of this part (the whole class: Th, Tw)
+                        const int hg = rs.r1 - rs.r0, wg = cs.r1 - cs.r0;
+                        taps_inside += (int64_t)hg * wg * th * tw;
+                        GatherSetup gs;
+                        GatherParams& g = gs.gp;
+                        g.src = dy; g.bias = nullptr; g.out = dx;
+                        g.S = S; g.Hs = Ho; g.Ws = Wo; g.Cs = D;
+                        g.Hg = hg; g.Wg = wg; g.M = S * hg * wg; g.N = C;
+                        g.K = th * tw * D;
+                        g.Kpad = (int)round_up(g.K, BK);
+                        // part row r' is class row r' + r0 and its tap t' is class tap t' + t0: dy row r' + (offh + r0 + t0) + t'
+                        g.Tw = tw; g.sh = 1; g.sw = 1; g.rh0 = offh + rs.r0 + rs.t0; g.rw0 = offw + cs.r0 + cs.t0;
+                        g.Hof = H; g.Wof = W; g.oh0 = a + sH * rs.r0; g.ow0 = b + sW * cs.r0; g.ohs = sH; g.ows = sW;
+                        g.dense_out = (nclass == 1);
+                        set_out_divs(g);
+                        PackParams& pk = gs.pp;
+                        pk.w = w; pk.fW = fW; pk.C = C; pk.D = D; pk.Tw = tw > 0 ? tw : 1; pk.Ck = D; pk.w_elems = (int64_t)fH * fW * C * D;
+                        pk.xa = xmax - sH * rs.t0; pk.xs = -sH; pk.ya = ymax - sW * cs.t0; pk.ys = -sW; pk.transposed = 1;
+                        pk.N = C; pk.K = g.K; pk.Npad = (int)round_up(C, 64); pk.Kpad = g.Kpad;
+                        gs.bt_bytes = round_up((int64_t)pk.Npad * pk.Kpad * sizeof(T), 256);
+                        g.split_slabs = 0;
+                        plan_split<T>(gs, D % Elem<T>::CE == 0, ctx().prop.multiProcessorCount);
+                        total_bytes += gs.bt_bytes + gs.part_bytes;
+                        sets.push_back(gs);
+                    }
             }
         }
     };
@@ -943,13 +991,36 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
         }
     }
     build_sets(h_lim, w_lim);
+    // fp32, strided: the problems that the 128 x 64 slab kernel takes are collected and go out as one grid (tuning: gather_merge
+    // = 0 keeps one launch each).  Where every class is large enough for that kernel (or tuning: gather_border = 1), the classes
+    // are first cut along their borders into parts that see the same taps inside dy, all of them on 128-row tiles, if that
+    // takes at least 3 % off the taps multiplied and leaves at most kMaxHeldClasses problems (tuning: gather_border = 0 never).
+    bool collect = false, borders = false;
+    if constexpr (sizeof(T) == 4) {
+        collect = nclass >= 2 && sets.size() >= 2 && (int)sets.size() <= kMaxHeldClasses && tuning().gather_merge != 0;
+        const int v = tuning().gather_border;
+        if (collect && v != 0 && D % Elem<T>::BK == 0) {
+            bool large = gather_bn(C) == 64;
+            for (const GatherSetup& gs : sets)
+                large = large && gs.nsplit == 1 && gs.gp.M > 0 && gather_bm(gs.gp.M, C, ctx().prop.multiProcessorCount, true) == 128;
+            if (large || v > 0) {
+                uniform_class_tiles() = true;
+                build_sets(h_lim, w_lim, true);
+                borders = (int)sets.size() <= kMaxHeldClasses && (v > 0 || taps_inside * 100 <= taps_whole * 97);
+                if (!borders) {
+                    uniform_class_tiles() = false;
+                    build_sets(h_lim, w_lim);
+                }
+            }
+        }
+    }
     void* ws;
     rc = workspace(total_bytes > 0 ? total_bytes : 256, &ws);
-    if (rc) return rc;
+    if (rc) {
+        uniform_class_tiles() = false;
+        return rc;
+    }
     int64_t off = 0;
-    // fp32, 2 to 4 classes: the classes that the 128 x 64 slab kernel takes are collected and go out as one grid
-    // (tuning: gather_merge = 0 keeps one launch per class)
-    const bool collect = sizeof(T) == 4 && sets.size() >= 2 && (int)sets.size() <= kMaxClasses && tuning().gather_merge != 0;
     if (collect) {
         class_hold().count = 0;
         class_hold().armed = true;
@@ -959,6 +1030,7 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
         if (rc) break;
         off += gs.bt_bytes + gs.part_bytes;
     }
+    uniform_class_tiles() = false;
     if (collect) {
         flush_classes((int)sets.size(), ctx().stream);
         if (rc == AETH_OK) AETH_LAUNCH_CHECK();

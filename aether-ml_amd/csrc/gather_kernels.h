@@ -906,36 +906,39 @@ struct GatherClasses {
     GatherParams cls[kMaxClasses];
     int ncls;
 };
-// fp32: the classes of a strided dgrad whose launches would all be the 128 x 64 slab kernel, in ONE launch.  Class c owns
-// the workgroups [start[c], start[c] + blocks[c]); every start is a multiple of the XCD count, so that a workgroup sits on
-// the XCD it would sit on in a launch of its class alone, and the workgroups that pad a class do nothing.  The host puts
-// the classes with the most taps first: the short ones fill the tail of the long ones, where four launches leave the
-// GPU part empty four times.
+// fp32: the problems of a strided dgrad (its classes, or the parts the classes are cut into along their borders) whose
+// launches would all be the 128 x 64 slab kernel, in ONE launch.  Problem c owns the workgroups [start[c], start[c] +
+// blocks[c]); every start is a multiple of the XCD count, so that a workgroup sits on the XCD it would sit on in a launch of
+// its problem alone, and the workgroups that pad a problem do nothing.  The host puts the problems with the most taps first:
+// the short ones fill the tail of the long ones, where a launch each leaves the GPU part empty every time.
+constexpr int kMaxClassesF32 = 8;
+struct GatherClassesF32 {
+    GatherParams cls[kMaxClassesF32];     // (the first kernel argument: the kernel reads it from the argument segment)
+    int ncls;
+};
 struct ClassGrid {
-    unsigned start[kMaxClasses];
-    unsigned blocks[kMaxClasses];
+    unsigned start[kMaxClassesF32];
+    unsigned blocks[kMaxClassesF32];
 };
 template <bool RUNS>
-static __global__ __launch_bounds__(kThreads) void gather_classes_f32(const GatherClasses q, const ClassGrid cg) {
+static __global__ __launch_bounds__(kThreads) void gather_classes_f32(const GatherClassesF32 q, const ClassGrid cg) {
     __shared__ f4 lds_a0[128 * 8];
     __shared__ f4 lds_a1[128 * 8];
     __shared__ f4 lds_b0[64 * 8];
     __shared__ f4 lds_b1[64 * 8];
     const unsigned b = blockIdx.x;
     int c = 0;
-#pragma unroll
-    for (int i = 1; i < kMaxClasses; ++i)
-        if (i < q.ncls && b >= cg.start[i]) c = i;
     unsigned start = cg.start[0], blocks = cg.blocks[0];
 #pragma unroll
-    for (int i = 1; i < kMaxClasses; ++i)
-        if (c == i) {
+    for (int i = 1; i < kMaxClassesF32; ++i)
+        if (i < q.ncls && b >= cg.start[i]) {
+            c = i;
             start = cg.start[i];
             blocks = cg.blocks[i];
         }
     const unsigned idx = b - start;
     if (idx >= blocks) return;
-    // The class's parameters are read where the launch put them, in the kernel argument segment (`q` is the first argument):
+    // The problem's parameters are read where the launch put them, in the kernel argument segment (`q` is the first argument):
     // scalar loads at a wave-uniform address.  Indexing the by-value copy with a run-time index would go through per-lane memory.
     typedef __attribute__((address_space(4))) const GatherParams* const_params_t;
     const_params_t args = (const_params_t)__builtin_amdgcn_kernarg_segment_ptr();

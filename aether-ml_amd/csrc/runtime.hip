@@ -51,7 +51,7 @@ bool tuning_set(const char* name, int value) {
         {"gather_pairs", &Tuning::gather_pairs},
         {"gather_runs", &Tuning::gather_runs},   {"narrow", &Tuning::narrow},   {"gather_bkn", &Tuning::gather_bkn},
         {"wgrad_br", &Tuning::wgrad_br},         {"wgrad_rounds", &Tuning::wgrad_rounds},
-        {"wgrad_swap", &Tuning::wgrad_swap},     {"pair_bwd", &Tuning::pair_bwd},
+        {"wgrad_swap", &Tuning::wgrad_swap},     {"pair_bwd", &Tuning::pair_bwd},     {"gather_border", &Tuning::gather_border},
     };
     for (const Field& f : fields)
         if (strcmp(f.name, name) == 0) {

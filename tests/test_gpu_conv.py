@@ -477,6 +477,42 @@ def test_strided_dgrad_with_its_classes_in_one_launch(case, tune):
     assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
 
 
+# The classes of a strided fp32 dgrad cut along their borders: the first and last rows and columns of a class see fewer of
+# its taps inside dy than the interior does, and a tile that mixes them multiplies the missing taps as zeros.  Cut into the
+# runs of rows and columns that see the same taps, every part is a problem with only those taps; all parts take 128-row tiles
+# and go out in grids of up to 8 problems.  The library does this for layers whose classes are large; the gather_border switch
+# lets small inputs reach it.  The sums run over the same taps in the same order: same values as the uncut classes.
+BORDER_CASES = [
+    (6, 28, 28, 64, 64, 3, 3, 2, 2, "valid"),     # the stride-2 benchmark layer's geometry: 16 parts (9 + 3 + 3 + 1)
+    (4, 28, 28, 64, 96, 3, 3, 2, 2, "same"),      # padding 1: other classes lose their taps at the other end
+    (3, 17, 15, 96, 64, 5, 5, 2, 2, "same"),      # 5x5: up to 3 taps per dimension and class, two border rows at each end
+    (3, 12, 16, 64, 32, 3, 3, 1, 2, "same"),      # stride (1, 2): 2 classes, rows cut as well as columns
+    (2, 14, 13, 64, 32, 2, 2, 3, 3, "valid"),     # filter smaller than the stride: classes without taps
+    (2, 9, 9, 72, 64, 7, 7, 2, 2, "same"),        # more parts than one dgrad may hold: the classes stay whole
+    (5, 10, 10, 24, 64, 3, 3, 2, 2, "same"),      # 24 input channels: 32-wide tiles, a launch per part
+    (3, 11, 11, 64, 40, 3, 3, 2, 2, "same"),      # 40 output channels: not whole slabs, the classes stay whole
+]
+
+
+@pytest.mark.parametrize("case", BORDER_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_strided_dgrad_cut_along_the_borders_of_its_classes(case, tune):
+    from tests import abi
+    x, w, b, dy = _case(case, 24)
+    stride, pad = (case[7], case[8]), case[9]
+    want = O.conv_dgrad(dy, w, x.shape[1:3], stride, pad, dtype=np.float64)
+    tune(gather_border=0, gather_bm=128, gather_split=0)  # the same tiles and an unsplit K for the classes left whole
+    whole = abi.dgrad(dy, w, x.shape, stride, pad)
+    abi.close(whole, want)
+    tune(gather_border=1)
+    cut = abi.dgrad(dy, w, x.shape, stride, pad)          # the output buffer starts as NaN: every element must be written
+    abi.close(cut, want)
+    assert np.array_equal(whole, cut)
+    tune(gather_merge=0)                                  # a launch per part
+    assert np.array_equal(cut, abi.dgrad(dy, w, x.shape, stride, pad))
+    tune(gather_merge=-1, gather_runs=1)
+    assert np.array_equal(cut, abi.dgrad(dy, w, x.shape, stride, pad))
+
+
 # fp32 wgrad of a unit-stride filter of at most 9 taps on 64 input channels and at most 64 output
 # channels, on rows of 28, 32, 56 or 64 output pixels: one persistent workgroup per CU keeps the whole
 # K x N result in registers (12 multiplying waves of three 32 x 32 blocks) and a loading wave brings one
