@@ -903,7 +903,7 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
                         // part row r' is class row r' + r0 and its tap t' is class tap t' + t0: dy row r' + (offh + r0 + t0) + t'
                         g.Tw = tw; g.sh = 1; g.sw = 1; g.rh0 = offh + rs.r0 + rs.t0; g.rw0 = offw + cs.r0 + cs.t0;
                         g.Hof = H; g.Wof = W; g.oh0 = a + sH * rs.r0; g.ow0 = b + sW * cs.r0; g.ohs = sH; g.ows = sW;
-                        g.dense_out = (nclass == 1);
+                        g.dense_out = (nclass == 1 && !cut);
                         set_out_divs(g);
                         PackParams& pk = gs.pp;
                         pk.w = w; pk.fW = fW; pk.C = C; pk.D = D; pk.Tw = tw > 0 ? tw : 1; pk.Ck = D; pk.w_elems = (int64_t)fH * fW * C * D;
@@ -991,28 +991,32 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
         }
     }
     build_sets(h_lim, w_lim);
-    // fp32, strided: the problems that the 128 x 64 slab kernel takes are collected and go out as one grid (tuning: gather_merge
-    // = 0 keeps one launch each).  Where every class is large enough for that kernel (or tuning: gather_border = 1), the classes
-    // are first cut along their borders into parts that see the same taps inside dy, all of them on 128-row tiles, if that
-    // takes at least 3 % off the taps multiplied and leaves at most kMaxHeldClasses problems (tuning: gather_border = 0 never).
-    bool collect = false, borders = false;
+    // fp32: where every class is large enough for the 128 x 64 slab kernel (or tuning: gather_border = 1), the classes are cut
+    // along their borders into parts that see the same taps inside dy, all of them on 128-row tiles, if that takes at least 3 %
+    // off the taps multiplied (3x3 "same" at unit stride: 4.7 % on 28x28 images, 2.4 % on 56x56, where the cut measured 0.432 ms
+    // against 0.438; the stride-2 28x28 layer: 10.5 %) and leaves at most kMaxHeldClasses problems (tuning: gather_border = 0 never).  The problems of a
+    // strided or cut dgrad that the 128 x 64 slab kernel takes are collected and go out in shared grids (tuning: gather_merge = 0
+    // keeps a launch each).
+    bool collect = false;
     if constexpr (sizeof(T) == 4) {
-        collect = nclass >= 2 && sets.size() >= 2 && (int)sets.size() <= kMaxHeldClasses && tuning().gather_merge != 0;
         const int v = tuning().gather_border;
-        if (collect && v != 0 && D % Elem<T>::BK == 0) {
+        const bool merge = tuning().gather_merge != 0 && (int)sets.size() <= kMaxHeldClasses;
+        bool borders = false;
+        if (merge && v != 0 && D % Elem<T>::BK == 0) {
             bool large = gather_bn(C) == 64;
             for (const GatherSetup& gs : sets)
                 large = large && gs.nsplit == 1 && gs.gp.M > 0 && gather_bm(gs.gp.M, C, ctx().prop.multiProcessorCount, true) == 128;
             if (large || v > 0) {
                 uniform_class_tiles() = true;
                 build_sets(h_lim, w_lim, true);
-                borders = (int)sets.size() <= kMaxHeldClasses && (v > 0 || taps_inside * 100 <= taps_whole * 97);
+                borders = sets.size() >= 2 && (int)sets.size() <= kMaxHeldClasses && (v > 0 || taps_inside * 100 <= taps_whole * 97);
                 if (!borders) {
                     uniform_class_tiles() = false;
                     build_sets(h_lim, w_lim);
                 }
             }
         }
+        collect = merge && sets.size() >= 2 && (nclass >= 2 || borders);
     }
     void* ws;
     rc = workspace(total_bytes > 0 ? total_bytes : 256, &ws);

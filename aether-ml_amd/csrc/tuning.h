@@ -20,7 +20,7 @@ struct Tuning {
     int gather_direct_b = -1; // 0: dgrad always packs its filter (no reads from w itself)
     int gather_clip = -1;    // 0: strided dgrad multiplies its classes' full pixel grids (no zeroed strips)
     int gather_merge = -1;   // 0: a strided dgrad launches its classes one by one
-    int gather_border = -1;  // fp32 strided dgrad cut into border strips and interiors: 0 never, 1 wherever the stride is not 1
+    int gather_border = -1;  // fp32 dgrad classes cut into border strips and interiors: 0 never, 1 also for small inputs
     int gather_pairs = -1;   // 0: the merged launch keeps one class per workgroup
     int gather_bkn = -1;     // 0: fp32 fprop always packs its filter
     int narrow = -1;         // 0: products with at most 16 output channels go to the slab kernels too

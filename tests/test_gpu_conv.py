@@ -477,7 +477,7 @@ def test_strided_dgrad_with_its_classes_in_one_launch(case, tune):
     assert np.array_equal(dx, abi.dgrad(dy, w, x.shape, stride, pad))
 
 
-# The classes of a strided fp32 dgrad cut along their borders: the first and last rows and columns of a class see fewer of
+# The classes of an fp32 dgrad cut along their borders: the first and last rows and columns of a class see fewer of
 # its taps inside dy than the interior does, and a tile that mixes them multiplies the missing taps as zeros.  Cut into the
 # runs of rows and columns that see the same taps, every part is a problem with only those taps; all parts take 128-row tiles
 # and go out in grids of up to 8 problems.  The library does this for layers whose classes are large; the gather_border switch
@@ -491,11 +491,14 @@ BORDER_CASES = [
     (2, 9, 9, 72, 64, 7, 7, 2, 2, "same"),        # more parts than one dgrad may hold: the classes stay whole
     (5, 10, 10, 24, 64, 3, 3, 2, 2, "same"),      # 24 input channels: 32-wide tiles, a launch per part
     (3, 11, 11, 64, 40, 3, 3, 2, 2, "same"),      # 40 output channels: not whole slabs, the classes stay whole
+    (3, 14, 14, 64, 64, 3, 3, 1, 1, "same"),      # unit stride: one class, 9 parts (interior, 4 edges, 4 corners)
+    (2, 12, 10, 128, 32, 5, 3, 1, 1, "same"),     # 5x3 at unit stride: 5 row parts x 3 column parts
+    (2, 12, 12, 64, 64, 3, 3, 1, 1, "valid"),     # no padding: every tap inside, the class stays whole
 ]
 
 
 @pytest.mark.parametrize("case", BORDER_CASES, ids=lambda c: "x".join(str(v) for v in c))
-def test_strided_dgrad_cut_along_the_borders_of_its_classes(case, tune):
+def test_dgrad_cut_along_the_borders_of_its_classes(case, tune):
     from tests import abi
     x, w, b, dy = _case(case, 24)
     stride, pad = (case[7], case[8]), case[9]
