@@ -207,6 +207,27 @@ def test_random_geometries(case):
     abi.close(db, O.conv_dbias(dy, dtype=np.float64), rms_scaled=True)
 
 
+@pytest.mark.parametrize("case", _random_cases(40, 20250911), ids=lambda c: "x".join(str(v) for v in c))
+def test_random_geometries_through_the_backward_call_and_with_cut_classes(case, tune):
+    """aeth_conv_bwd_f32 gives the bits of the wgrad and the dgrad call whatever the geometry selects; a dgrad whose classes are
+    cut along their borders (forced here: the library cuts large layers only) gives the values of the uncut one."""
+    from tests import abi
+    from tests.test_gpu_pair import conv_bwd
+    S, H, W, C, D, fH, fW, sH, sW, pad = case
+    x, w, b, dy = _case(case, 12)
+    dw0, db0 = abi.wgrad(x, dy, w.shape, (sH, sW), pad)
+    dx0 = abi.dgrad(dy, w, x.shape, (sH, sW), pad)
+    dw1, db1, dx1 = conv_bwd(x, dy, w, (sH, sW), pad)
+    assert np.array_equal(dw0, dw1) and np.array_equal(db0, db1) and np.array_equal(dx0, dx1)
+    tune(gather_border=1)
+    cut = abi.dgrad(dy, w, x.shape, (sH, sW), pad)
+    abi.close(cut, O.conv_dgrad(dy, w, (H, W), (sH, sW), pad, dtype=np.float64))
+    tune(gather_split=0)
+    cut2 = abi.dgrad(dy, w, x.shape, (sH, sW), pad)
+    tune(gather_border=0, gather_bm=128)
+    assert np.array_equal(cut2, abi.dgrad(dy, w, x.shape, (sH, sW), pad))
+
+
 # The mode in which one workgroup keeps its rows of x in LDS and walks all n tiles is chosen
 # for 128-row tiles only, which the library takes from about 800 000 output pixels on; the
 # tuning switch forces that tile height so that small inputs reach the same code.
