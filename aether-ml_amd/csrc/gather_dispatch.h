@@ -2,6 +2,7 @@
 // entry points' shared implementation.
 #pragma once
 #include "gather_kernels.h"
+#include "dgrad_parts.h"
 #include "narrow_kernels.h"
 #include "pair_launch.h"
 #include "sample_runs.h"
@@ -782,27 +783,6 @@ int conv_fprop_impl(const char* fn, const T* x, const T* w, const float* bias, f
     return run_gather<T>(gs, (char*)ws, 0, C % Elem<T>::CE == 0);
 }
 
-// Rows (or columns) [r0, r1) of a dgrad class and the taps [t0, t1) of the class that fall inside dy for all of them.
-struct TapSpan {
-    int r0, r1, t0, t1;
-};
-// Class row r reads dy row r + off + t under tap t (0 <= t < taps), which exists for 0 <= r + off + t < len.  Returns the
-// maximal runs of rows with the same range of existing taps (`split`), or one span with all taps.
-static inline std::vector<TapSpan> tap_spans(int rows, int off, int taps, int len, bool split) {
-    std::vector<TapSpan> out;
-    if (!split || taps <= 0) {
-        out.push_back(TapSpan{0, rows, 0, taps > 0 ? taps : 0});
-        return out;
-    }
-    for (int r = 0; r < rows; ++r) {
-        const int lo = std::min(taps, std::max(0, -(r + off)));
-        const int hi = std::max(lo, std::min(taps, len - (r + off)));
-        if (!out.empty() && out.back().t0 == lo && out.back().t1 == hi) out.back().r1 = r + 1;
-        else out.push_back(TapSpan{r, r + 1, lo, hi});
-    }
-    return out;
-}
-
 // dgrad: for input row i the contributing taps are x with (i + pH - x) % sH == 0 and
 // 0 <= (i + pH - x)/sH < Ho.  Rows are split by a = i % sH; inside a class the taps
 // are x_t = xmax - sH*t (xmax = largest x < fH with x == (a+pH) mod sH), and the
@@ -865,57 +845,35 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
     }
     std::vector<GatherSetup> sets;
     int64_t total_bytes = 0;
-    // `borders`: a class is cut into the runs of rows and columns that see the same taps inside dy (first rows, interior,
-    // last rows), each a problem of its own with only those taps, so that no tile multiplies a tap that lies outside.
+    // The problems of the dgrad (dgrad_parts.h); `borders`: the classes cut along their borders.
     int64_t taps_whole = 0, taps_inside = 0;                 // tap-pixels multiplied per sample without and with the cut
     auto build_sets = [&](int hl, int wl, bool borders = false) {
         sets.clear();
         total_bytes = 0;
-        taps_whole = taps_inside = 0;
-        for (int a = 0; a < sH; ++a) {
-            if (a >= H) continue;
-            int ra = (a + pH) % sH;
-            int Th = ra < fH ? (fH - 1 - ra) / sH + 1 : 0;
-            int xmax = ra + (Th - 1) * sH;
-            int offh = Th > 0 ? (a + pH - xmax) / sH : 0;   // exact: (a+pH-xmax) is a multiple of sH
-            int Hg = (std::min(H, std::max(hl, a + 1)) - a + sH - 1) / sH;      // class rows i = a + sH i' below hl (at least one)
-            for (int b = 0; b < sW; ++b) {
-                if (b >= W) continue;
-                int rb = (b + pW) % sW;
-                int Tw = rb < fW ? (fW - 1 - rb) / sW + 1 : 0;
-                int ymax = rb + (Tw - 1) * sW;
-                int offw = Tw > 0 ? (b + pW - ymax) / sW : 0;
-                int Wg = (std::min(W, std::max(wl, b + 1)) - b + sW - 1) / sW;
-                taps_whole += (int64_t)Hg * Wg * Th * Tw;
-                const bool cut = borders && Th > 0 && Tw > 0;
-                for (const TapSpan& rs : tap_spans(Hg, offh, Th, Ho, cut))
-                    for (const TapSpan& cs : tap_spans(Wg, offw, Tw, Wo, cut)) {
-                        const int th = rs.t1 - rs.t0, tw = cs.t1 - cs.t0;     // taps of this part (the whole class: Th, Tw)
-                        const int hg = rs.r1 - rs.r0, wg = cs.r1 - cs.r0;
-                        taps_inside += (int64_t)hg * wg * th * tw;
-                        GatherSetup gs;
-                        GatherParams& g = gs.gp;
-                        g.src = dy; g.bias = nullptr; g.out = dx;
-                        g.S = S; g.Hs = Ho; g.Ws = Wo; g.Cs = D;
-                        g.Hg = hg; g.Wg = wg; g.M = S * hg * wg; g.N = C;
-                        g.K = th * tw * D;
-                        g.Kpad = (int)round_up(g.K, BK);
-                        // part row r' is class row r' + r0 and its tap t' is class tap t' + t0: dy row r' + (offh + r0 + t0) + t'
-                        g.Tw = tw; g.sh = 1; g.sw = 1; g.rh0 = offh + rs.r0 + rs.t0; g.rw0 = offw + cs.r0 + cs.t0;
-                        g.Hof = H; g.Wof = W; g.oh0 = a + sH * rs.r0; g.ow0 = b + sW * cs.r0; g.ohs = sH; g.ows = sW;
-                        g.dense_out = (nclass == 1 && !cut);
-                        set_out_divs(g);
-                        PackParams& pk = gs.pp;
-                        pk.w = w; pk.fW = fW; pk.C = C; pk.D = D; pk.Tw = tw > 0 ? tw : 1; pk.Ck = D; pk.w_elems = (int64_t)fH * fW * C * D;
-                        pk.xa = xmax - sH * rs.t0; pk.xs = -sH; pk.ya = ymax - sW * cs.t0; pk.ys = -sW; pk.transposed = 1;
-                        pk.N = C; pk.K = g.K; pk.Npad = (int)round_up(C, 64); pk.Kpad = g.Kpad;
-                        gs.bt_bytes = round_up((int64_t)pk.Npad * pk.Kpad * sizeof(T), 256);
-                        g.split_slabs = 0;
-                        plan_split<T>(gs, D % Elem<T>::CE == 0, ctx().prop.multiProcessorCount);
-                        total_bytes += gs.bt_bytes + gs.part_bytes;
-                        sets.push_back(gs);
-                    }
-            }
+        const DgradPlan plan = plan_dgrad_parts(H, W, Ho, Wo, fH, fW, sH, sW, pH, pW, hl, wl, borders);
+        taps_whole = plan.taps_whole;
+        taps_inside = plan.taps_parts;
+        for (const DgradPart& part : plan.parts) {
+            GatherSetup gs;
+            GatherParams& g = gs.gp;
+            g.src = dy; g.bias = nullptr; g.out = dx;
+            g.S = S; g.Hs = Ho; g.Ws = Wo; g.Cs = D;
+            g.Hg = part.Hg; g.Wg = part.Wg; g.M = S * part.Hg * part.Wg; g.N = C;
+            g.K = part.Th * part.Tw * D;
+            g.Kpad = (int)round_up(g.K, BK);
+            g.Tw = part.Tw; g.sh = 1; g.sw = 1; g.rh0 = part.rh0; g.rw0 = part.rw0;
+            g.Hof = H; g.Wof = W; g.oh0 = part.oh0; g.ow0 = part.ow0; g.ohs = sH; g.ows = sW;
+            g.dense_out = (nclass == 1 && !part.cut);
+            set_out_divs(g);
+            PackParams& pk = gs.pp;
+            pk.w = w; pk.fW = fW; pk.C = C; pk.D = D; pk.Tw = part.Tw > 0 ? part.Tw : 1; pk.Ck = D; pk.w_elems = (int64_t)fH * fW * C * D;
+            pk.xa = part.xa; pk.xs = -sH; pk.ya = part.ya; pk.ys = -sW; pk.transposed = 1;
+            pk.N = C; pk.K = g.K; pk.Npad = (int)round_up(C, 64); pk.Kpad = g.Kpad;
+            gs.bt_bytes = round_up((int64_t)pk.Npad * pk.Kpad * sizeof(T), 256);
+            g.split_slabs = 0;
+            plan_split<T>(gs, D % Elem<T>::CE == 0, ctx().prop.multiProcessorCount);
+            total_bytes += gs.bt_bytes + gs.part_bytes;
+            sets.push_back(gs);
         }
     };
     // bf16, 2 or 4 classes with the same pixel grid, each of them a problem for gather_halo_bf16 with the same
