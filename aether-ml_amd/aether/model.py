@@ -148,8 +148,8 @@ class Model:
             print(f' epoch: {epoch}')
             self.loss.new_pass()
             self.accuracy.new_pass()
-            # Replayed steps (record_steps) are read one step late: the host queues step k + 1 while step k runs
-            # and takes step k's loss and predictions afterwards; sums and printed lines are those of the plain loop.
+            # Steps are read one step late: the host queues step k + 1 while step k runs and takes step k's loss and
+            # predictions afterwards; sums and printed lines are those of a loop that reads every step at once.
             waiting = []                                     # (step, function that reads its scalars)
 
             def report(step, loss, data_loss, regularization_loss, accuracy, lr):
@@ -165,13 +165,14 @@ class Model:
                 for step, rows in enumerate(spans):
                     batch_X, batch_y = _rows(X, rows), _rows(y, rows)
                     finish = self._recorded_step(batch_X, batch_y, later=True) if self.recording_active else None
-                    if finish is not None:
+                    if finish is None:
+                        finish = self._eager_step(batch_X, batch_y, later=True)
+                    if callable(finish):
                         waiting.append((step, finish))
                         drain(1)
                         continue
                     drain(0)                                 # results enter the sums in the order of the steps
-                    loss, data_loss, regularization_loss, accuracy = self._eager_step(batch_X, batch_y)
-                    report(step, loss, data_loss, regularization_loss, accuracy, self.optimizer.current_learning_rate)
+                    report(step, *finish, self.optimizer.current_learning_rate)
                 drain(0)
             finally:
                 for _, finish in waiting:                    # (only after an exception: hand the pending copies back)
@@ -296,11 +297,15 @@ class Model:
             predictions = self.output_layer_activation.predictions(rec["output"])
             accuracy = self.accuracy.calculate(predictions, batch_y)
             return data_loss + regularization_loss, data_loss, regularization_loss, accuracy
-        # the step's scalars are copied to the host behind the replay and read when the caller asks for them,
-        # by which time the next replay may be running (Model.train)
-        buf, rows, _ = rec["pending"]
+        return self._read_later(rec["pending"], rec.get("reg_pending"), batch_y)
+
+    def _read_later(self, pending, reg, batch_y):
+        """The step's scalars (per-sample losses with the predictions beside them, the regulariser's sums) are copied to
+        the host behind what the step has queued and read when the caller asks for them, by which time the next step
+        may be running (Model.train).  Returns the function that reads them: (loss, data loss, regularisation loss,
+        accuracy, learning rate of the step)."""
+        buf, rows, _ = pending
         loss_later = buf.get_later()
-        reg = rec.get("reg_pending")
         reg_later = reg[1].get_later() if reg is not None else None
         lr = self.optimizer.current_learning_rate
 
@@ -328,7 +333,9 @@ class Model:
                 return result
         return self._eager_step(batch_X, batch_y)
 
-    def _eager_step(self, batch_X, batch_y):
+    def _eager_step(self, batch_X, batch_y, later=False):
+        """One step launched kernel by kernel.  With `later` (and a loss that can be queued): a function that reads the
+        step's scalars when called, instead of the scalars."""
         # The loss kernel is queued here and read after backward and the update have been
         # queued too, so the device never idles while the host prepares the backward pass.
         # A regulariser's sums are queued here as well: they see the weights before the update,
@@ -347,6 +354,8 @@ class Model:
         for layer in self.trainable_layers:
             self.optimizer.update_parameters(layer)
         self.optimizer.post_update_parameters()
+        if later and pending is not None:
+            return self._read_later(pending, reg_pending, batch_y)
         if pending is not None:
             data_loss = self.loss.finish(pending)
             regularization_loss = self.loss.regularization_finish(reg_pending)

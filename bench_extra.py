@@ -180,8 +180,8 @@ def train_step(steps, warmup, eager_only=False):
             "train_loop": {"ms_per_step": loop * 1e3, "images_per_sec": 128.0 / loop,
                            "recorded_ms_per_step": loop_rec * 1e3, "recorded_images_per_sec": 128.0 / loop_rec,
                            "note": "Model.train(X, y, epochs=3, batch_size=128, print_every=100) on 8192 images resident in HBM: "
-                                   "wall time of the call per step; with record_steps the host reads a step's loss and "
-                                   "predictions while the next step runs"},
+                                   "wall time of the call per step; the host reads a step's loss and predictions while the "
+                                   "next step runs, with steps launched kernel by kernel and with replayed ones"},
             "recorded_steps": {"ms_per_step_median": med_rec * 1e3, "images_per_sec": 128.0 / med_rec,
                                "last_loss": loss_rec,
                                "note": "Model.record_steps(True): the step replayed from a HIP graph, one host call"},

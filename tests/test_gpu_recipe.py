@@ -176,29 +176,33 @@ def test_cifar1_recipe_recorded_steps_draw_the_same_masks_as_eager_steps():
     assert all(np.array_equal(a, b) for a, b in zip(params_e, params_r))
 
 
-def test_train_reads_replayed_steps_one_step_late_and_prints_the_same_lines(capsys):
-    """Model.train on a recorded model queues step k + 1 before it reads step k's loss and predictions.  The printed
-    lines (every second step and the last of an epoch, the summary, the validation line), the accumulated sums
-    and the parameters are those of the plain loop; the last batch of an epoch is ragged (another shape: it runs
-    normally in the first epoch, is recorded in the second and replayed in the third)."""
+def test_train_reads_steps_one_step_late_and_prints_the_same_lines(capsys):
+    """Model.train queues step k + 1 before it reads step k's loss and predictions, with steps launched kernel by kernel
+    and with replayed ones.  The printed lines (every second step and the last of an epoch, the summary, the validation
+    line), the accumulated sums and the parameters are those of a loop that reads every step at once; the last batch of
+    an epoch is ragged (another shape: with recorded steps it runs normally in the first epoch, is recorded in the second
+    and replayed in the third)."""
     import aether
     rng = np.random.RandomState(31)
     X = rng.rand(150, 32, 32, 3).astype(np.float32)
     y = rng.randint(0, 10, 150)
     outs, params = [], []
-    for record in (False, True):
+    for mode in ("at once", "late", "recorded"):
         np.random.seed(17)
         model = cifar1_model(aether)
-        model.record_steps(record)
+        model.record_steps(mode == "recorded")
+        if mode == "at once":                                # every step's scalars read before the next step is queued
+            plain = model._eager_step
+            model._eager_step = lambda bx, by, later=False: plain(bx, by)
         np.random.seed(18)                                   # the dropout masks' random stream
         model.train(X, y, epochs=3, batch_size=32, print_every=2, validation_data=(X[:40], y[:40]))
         outs.append(capsys.readouterr().out)
         params.append([np.asarray(p) for layer in model.trainable_layers for p in layer.get_parameters()])
-        if record:
+        if mode == "recorded":
             assert len([r for r in model._recordings.values() if r.get("graph")]) == 2
-    assert outs[0] == outs[1]
+    assert outs[0] == outs[1] == outs[2]
     assert outs[0].count("epoch: ") == 3 + 3 * 3             # the epoch headers and steps 0, 2, 4 of each
-    assert all(np.array_equal(a, b) for a, b in zip(*params))
+    assert all(np.array_equal(a, b) and np.array_equal(a, c) for a, b, c in zip(*params))
 
 
 def test_two_part_copies_to_the_host():
