@@ -56,9 +56,9 @@ int aeth_device_info(char* host_buf, int n);
  * kernel with an input smaller than the shapes it is chosen for, or run a problem on a
  * second, independently scheduled kernel.  -1 restores "decide from the shape";
  * host_name == NULL resets every switch.  Names: gather_bm, gather_kc, gather_nloop,
- * gather_halo, gather_split, gather_sa, gather_direct_b, gather_clip, gather_merge, gather_pairs, gather_runs,
- * gather_bkn, gather_wide, gather_res, narrow, dense_res, direct, wgrad_halo, wgrad_wide, wgrad_cw, wgrad_br,
- * wgrad_rounds, wgrad_swap.  May be called before aeth_init.  The
+ * gather_halo, gather_split, gather_sa, gather_direct_b, gather_clip, gather_merge, gather_border, gather_pairs,
+ * gather_runs, gather_bkn, gather_wide, gather_res, narrow, dense_res, direct, wgrad_halo, wgrad_wide, wgrad_cw,
+ * wgrad_br, wgrad_rounds, wgrad_swap, pair_bwd.  May be called before aeth_init.  The
  * same switches can be given once through the environment variable AETHER_TUNE
  * ("name=value,name=value"), read by aeth_init; the library reads no other variable. */
 int aeth_debug_set(const char* host_name, int value);

@@ -143,7 +143,7 @@ def test_debug_switches_are_known_by_name(lib):
     an unknown name is refused with a message that names it."""
     for name in (b"gather_bm", b"gather_kc", b"gather_nloop", b"gather_halo", b"gather_split", b"gather_sa",
                  b"gather_direct_b", b"gather_clip", b"gather_merge", b"gather_pairs", b"gather_runs", b"narrow", b"gather_bkn", b"gather_wide", b"gather_res", b"dense_res", b"direct",
-                 b"wgrad_halo", b"wgrad_wide", b"wgrad_cw", b"wgrad_br", b"wgrad_rounds", b"wgrad_swap"):
+                 b"wgrad_halo", b"wgrad_wide", b"wgrad_cw", b"wgrad_br", b"wgrad_rounds", b"wgrad_swap", b"gather_border", b"pair_bwd"):
         assert lib.aeth_debug_set(name, 1) == 0, name
         assert lib.aeth_debug_set(name, -1) == 0, name
     assert lib.aeth_debug_set(None, 0) == 0
