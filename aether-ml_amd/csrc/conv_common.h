@@ -93,7 +93,8 @@ struct GatherParams {
     // already contiguous in k = d; the slab of tap (th, tw), channel offset c0 starts at element
     // ((bd_xa + bd_xs th) bd_fw + bd_ya + bd_ys tw) * bd_tap_elems + c0 of row 0: no packing launch.
     int bt_ld, bt_direct;
-    int bt_kn;           // fp32 fprop: bt is the filter itself as a [K][N] matrix (row k = (tap, c), bt_ld = D floats apart)
+    int bt_kn;           // fp32 fprop: bt is the filter itself as a [K][N] matrix (row k = (tap, c), bt_ld = D floats apart);
+                         // 2: the problem is a part of an fprop with the taps (bd_xa + th, bd_ya + tw) of a filter bd_fw taps wide
     int bd_xa, bd_xs, bd_ya, bd_ys, bd_fw, bd_tap_elems;
     // gather_halo_bf16: columns and rows of the padded source image, 256-row tiles per image (0: tiles
     // run over image boundaries)

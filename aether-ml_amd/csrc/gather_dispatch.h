@@ -43,6 +43,7 @@ struct ClassHold {
     bool armed = false;
     int count = 0;
     bool runs[kMaxHeldClasses];
+    bool bkn[kMaxHeldClasses];             // the problem reads the filter as the [K][N] operand (fprop)
     unsigned blocks[kMaxHeldClasses];
     GatherParams gp[kMaxHeldClasses];
 };
@@ -50,10 +51,11 @@ static inline ClassHold& class_hold() {
     static ClassHold h;
     return h;
 }
-static inline bool hold_class(const GatherParams& gp, const dim3& grid, bool runs) {
+static inline bool hold_class(const GatherParams& gp, const dim3& grid, bool runs, bool bkn = false) {
     ClassHold& h = class_hold();
     if (!h.armed || h.count >= kMaxHeldClasses || grid.y != 1 || gp.split_slabs != 0) return false;
     h.runs[h.count] = runs;
+    h.bkn[h.count] = bkn;
     h.blocks[h.count] = grid.x;
     h.gp[h.count] = gp;
     ++h.count;
@@ -66,11 +68,14 @@ static inline void flush_classes(int nsets, hipStream_t st) {
     ClassHold& h = class_hold();
     h.armed = false;
     bool same = h.count == nsets && h.count > 1;
-    for (int i = 1; i < h.count; ++i) same = same && h.runs[i] == h.runs[0];
+    for (int i = 1; i < h.count; ++i) same = same && h.runs[i] == h.runs[0] && h.bkn[i] == h.bkn[0];
     if (!same) {
         for (int i = 0; i < h.count; ++i) {
-            if (h.runs[i]) hipLaunchKernelGGL((gather_gemm_dma<float, 128, 64, 32, 64, true, 8, false, true, true>), dim3(h.blocks[i]), dim3(kThreads), 0, st, h.gp[i]);
-            else hipLaunchKernelGGL((gather_gemm_dma<float, 128, 64, 32, 64, true, 8, false, true>), dim3(h.blocks[i]), dim3(kThreads), 0, st, h.gp[i]);
+            const dim3 g(h.blocks[i]), b(kThreads);
+            if (h.bkn[i] && h.runs[i]) hipLaunchKernelGGL((gather_gemm_dma<float, 128, 64, 32, 64, true, 8, false, true, true, true>), g, b, 0, st, h.gp[i]);
+            else if (h.bkn[i]) hipLaunchKernelGGL((gather_gemm_dma<float, 128, 64, 32, 64, true, 8, false, true, false, true>), g, b, 0, st, h.gp[i]);
+            else if (h.runs[i]) hipLaunchKernelGGL((gather_gemm_dma<float, 128, 64, 32, 64, true, 8, false, true, true>), g, b, 0, st, h.gp[i]);
+            else hipLaunchKernelGGL((gather_gemm_dma<float, 128, 64, 32, 64, true, 8, false, true>), g, b, 0, st, h.gp[i]);
         }
         h.count = 0;
         return;
@@ -94,8 +99,10 @@ static inline void flush_classes(int nsets, hipStream_t st) {
             cg.blocks[i] = h.blocks[order[first + i]];
             total += (unsigned)round_up(cg.blocks[i], kXcds);
         }
-        if (h.runs[0]) hipLaunchKernelGGL(gather_classes_f32<true>, dim3(total), dim3(kThreads), 0, st, gc, cg);
-        else hipLaunchKernelGGL(gather_classes_f32<false>, dim3(total), dim3(kThreads), 0, st, gc, cg);
+        if (h.bkn[0] && h.runs[0]) hipLaunchKernelGGL((gather_classes_f32<true, true>), dim3(total), dim3(kThreads), 0, st, gc, cg);
+        else if (h.bkn[0]) hipLaunchKernelGGL((gather_classes_f32<false, true>), dim3(total), dim3(kThreads), 0, st, gc, cg);
+        else if (h.runs[0]) hipLaunchKernelGGL((gather_classes_f32<true, false>), dim3(total), dim3(kThreads), 0, st, gc, cg);
+        else hipLaunchKernelGGL((gather_classes_f32<false, false>), dim3(total), dim3(kThreads), 0, st, gc, cg);
     }
     h.count = 0;
 }
@@ -147,6 +154,9 @@ static void launch_gather_dma(const GatherParams& gp, hipStream_t st) {
             if constexpr (WN == 64 || WN == 32) runs = gp.split_slabs == 0 && run_stores(gp);
             if constexpr (KC == 8) {
                 if (gp.bt_kn) {
+                    if constexpr (BM == 128 && BN == 64 && WM == 32 && WN == 64) {
+                        if (hold_class(gp, grid, runs, true)) return;
+                    }
                     if constexpr (WN == 64 || WN == 32) {
                         if (runs) {
                             hipLaunchKernelGGL((gather_gemm_dma<T, BM, BN, WM, WN, true, KC, false, true, true, true>), grid, dim3(kThreads), 0, st, gp);
@@ -411,6 +421,7 @@ struct GatherSetup {
     int nsplit = 1;          // > 1: split K, partial products behind the packed filter in the workspace
     int64_t part_bytes = 0;
     struct ActOut* act = nullptr;   // fprop: the activation behind the layer, written by the split reduction where there is one
+    bool kn_part = false;    // a part of an fprop: its taps are the filter's taps (pp.xa + th, pp.ya + tw)
 };
 
 // The output of the ReLU / leaky ReLU that follows a dense layer, for the split reduction to write on the way
@@ -581,7 +592,8 @@ static int choose_b_operand(GatherSetup& gs, bool vec, int min_slabs = 3) {
             gs.gp.bt = pk.w;
             gs.gp.bt_bytes = (unsigned)(pk.w_elems * 4);
             gs.gp.bt_ld = pk.D;
-            gs.gp.bt_kn = 1;
+            gs.gp.bt_kn = gs.kn_part ? 2 : 1;
+            gs.gp.bd_xa = pk.xa; gs.gp.bd_ya = pk.ya; gs.gp.bd_fw = pk.fW;
             return 0;
         }
     }
@@ -769,6 +781,67 @@ int conv_fprop_impl(const char* fn, const T* x, const T* w, const float* bias, f
     g.split_slabs = 0;
     gs.act = act;
     plan_split<T>(gs, C % Elem<T>::CE == 0, ctx().prop.multiProcessorCount);
+    if constexpr (sizeof(T) == 4) {
+        // A padded fprop at unit stride that is large enough for the 128 x 64 slab kernel (or tuning: gather_border = 1) is cut
+        // into the runs of output rows and columns that see the same taps inside x (interior, edges, corners: nine parts for
+        // 3x3 "same"), each a problem with only those taps, all in one grid: no tile multiplies a tap that lies in the padding.
+        // Taken from 2 % of the taps on (56x56 images: 2.4 %); the filter is read in place by every part.
+        const int v = tuning().gather_border;
+        const int cus = ctx().prop.multiProcessorCount;
+        const bool large = gs.nsplit == 1 && gather_bn(D) == 64 && g.M > 0 && gather_bm(g.M, D, cus, true) == 128;
+        if (sH == 1 && sW == 1 && (pH > 0 || pW > 0) && fixed_scratch == nullptr && act == nullptr && v != 0 &&
+            tuning().gather_merge != 0 && C % BK == 0 && (large || v > 0)) {
+            const std::vector<TapSpan> rows = tap_spans(Ho, -pH, fH, H, true), cols = tap_spans(Wo, -pW, fW, W, true);
+            int64_t inside = 0;
+            for (const TapSpan& rs : rows)
+                for (const TapSpan& cs : cols) inside += (int64_t)(rs.r1 - rs.r0) * (cs.r1 - cs.r0) * (rs.t1 - rs.t0) * (cs.t1 - cs.t0);
+            const int64_t whole = (int64_t)Ho * Wo * fH * fW;
+            const size_t nparts = rows.size() * cols.size();
+            if (nparts >= 2 && nparts <= (size_t)kMaxHeldClasses && (v > 0 || inside * 100 <= whole * 98)) {
+                std::vector<GatherSetup> parts;
+                int64_t total = 0;
+                uniform_class_tiles() = true;
+                for (const TapSpan& rs : rows)
+                    for (const TapSpan& cs : cols) {
+                        GatherSetup ps = gs;
+                        GatherParams& q = ps.gp;
+                        const int th = rs.t1 - rs.t0, tw = cs.t1 - cs.t0;
+                        q.Hg = rs.r1 - rs.r0; q.Wg = cs.r1 - cs.r0; q.M = S * q.Hg * q.Wg;
+                        q.K = th * tw * C;
+                        q.Kpad = (int)round_up(q.K, BK);
+                        // part row r is output row r + r0 and its tap t is filter row t + t0: x row r + (r0 + t0 - pH) + t
+                        q.Tw = tw; q.rh0 = -pH + rs.r0 + rs.t0; q.rw0 = -pW + cs.r0 + cs.t0;
+                        q.oh0 = rs.r0; q.ow0 = cs.r0; q.dense_out = 0;
+                        set_out_divs(q);
+                        PackParams& pq = ps.pp;
+                        pq.Tw = tw > 0 ? tw : 1; pq.xa = rs.t0; pq.ya = cs.t0; pq.K = q.K; pq.Kpad = q.Kpad;
+                        ps.bt_bytes = (int64_t)pq.Npad * pq.Kpad * sizeof(T);
+                        ps.kn_part = true;
+                        ps.nsplit = 1; ps.part_bytes = 0; q.split_slabs = 0;
+                        total += round_up(ps.bt_bytes, 256);
+                        parts.push_back(ps);
+                    }
+                void* ws;
+                rc = workspace(total > 0 ? total : 256, &ws);
+                if (rc) {
+                    uniform_class_tiles() = false;
+                    return rc;
+                }
+                class_hold().count = 0;
+                class_hold().armed = true;
+                int64_t off = 0;
+                for (GatherSetup& ps : parts) {
+                    rc = run_gather<T>(ps, (char*)ws, off, true);
+                    if (rc) break;
+                    off += round_up(ps.bt_bytes, 256);
+                }
+                uniform_class_tiles() = false;
+                flush_classes((int)parts.size(), ctx().stream);
+                if (rc == AETH_OK) AETH_LAUNCH_CHECK();
+                return rc;
+            }
+        }
+    }
     void* ws;
     const int64_t need = round_up(gs.bt_bytes, 256) + gs.part_bytes;
     if (fixed_scratch != nullptr) {
@@ -967,7 +1040,7 @@ int conv_dgrad_impl(const char* fn, const T* dy, const T* w, float* dx,
             if (large || v > 0) {
                 uniform_class_tiles() = true;
                 build_sets(h_lim, w_lim, true);
-                borders = sets.size() >= 2 && (int)sets.size() <= kMaxHeldClasses && (v > 0 || taps_inside * 100 <= taps_whole * 97);
+                borders = sets.size() >= 2 && (int)sets.size() <= kMaxHeldClasses && (v > 0 || taps_inside * 100 <= taps_whole * 98);
                 if (!borders) {
                     uniform_class_tiles() = false;
                     build_sets(h_lim, w_lim);

@@ -356,6 +356,8 @@ __device__ __forceinline__ void gather_gemm_dma_body(const GatherParams& p, cons
             if (!BKN && p.bt_direct)                     // the filter itself: tap (th, tw) of this class, channels c0..
                 b_k_bytes = (unsigned)(((p.bd_xa + p.bd_xs * (int)th) * p.bd_fw + p.bd_ya + p.bd_ys * (int)tw) * p.bd_tap_elems +
                                        (int)c0) * (unsigned)sizeof(T);
+            if (BKN && p.bt_kn == 2)                     // a part of an fprop: its tap (th, tw) is the filter's tap (bd_xa + th, bd_ya + tw)
+                b_k_bytes = (unsigned)(((p.bd_xa + (int)th) * p.bd_fw + p.bd_ya + (int)tw) * p.Cs + (int)c0) * (unsigned)p.bt_ld * 4u;
             if constexpr (SA) cur_mask = (unsigned)__builtin_amdgcn_ballot_w64(((aux_row >> ut_tap) & 1u) != 0u);
             return;
         }
@@ -906,12 +908,12 @@ struct GatherClasses {
     GatherParams cls[kMaxClasses];
     int ncls;
 };
-// fp32: the problems of a strided dgrad (its classes, or the parts the classes are cut into along their borders) whose
-// launches would all be the 128 x 64 slab kernel, in ONE launch.  Problem c owns the workgroups [start[c], start[c] +
+// fp32: the problems of a dgrad or an fprop (stride classes, or the parts that classes and fprops are cut into along their
+// borders) whose launches would all be the 128 x 64 slab kernel, in ONE launch.  Problem c owns the workgroups [start[c], start[c] +
 // blocks[c]); every start is a multiple of the XCD count, so that a workgroup sits on the XCD it would sit on in a launch of
 // its problem alone, and the workgroups that pad a problem do nothing.  The host puts the problems with the most taps first:
 // the short ones fill the tail of the long ones, where a launch each leaves the GPU part empty every time.
-constexpr int kMaxClassesF32 = 8;
+constexpr int kMaxClassesF32 = 9;            // (the nine parts of a 3x3 "same" convolution at unit stride: one launch)
 struct GatherClassesF32 {
     GatherParams cls[kMaxClassesF32];     // (the first kernel argument: the kernel reads it from the argument segment)
     int ncls;
@@ -920,7 +922,7 @@ struct ClassGrid {
     unsigned start[kMaxClassesF32];
     unsigned blocks[kMaxClassesF32];
 };
-template <bool RUNS>
+template <bool RUNS, bool BKN = false>
 static __global__ __launch_bounds__(kThreads) void gather_classes_f32(const GatherClassesF32 q, const ClassGrid cg) {
     __shared__ f4 lds_a0[128 * 8];
     __shared__ f4 lds_a1[128 * 8];
@@ -944,7 +946,8 @@ static __global__ __launch_bounds__(kThreads) void gather_classes_f32(const Gath
     const_params_t args = (const_params_t)__builtin_amdgcn_kernarg_segment_ptr();
     GatherParams p = q.cls[0];
     __builtin_memcpy(&p, (const void*)(args + c), sizeof(p));
-    gather_gemm_dma_body<float, 128, 64, 32, 64, true, 8, false, true, RUNS>(p, BlockId{(int)idx, 0, (int)blocks}, lds_a0, lds_a1, lds_b0, lds_b1);
+    gather_gemm_dma_body<float, 128, 64, 32, 64, true, 8, false, true, RUNS, BKN>(p, BlockId{(int)idx, 0, (int)blocks}, lds_a0, lds_a1, lds_b0,
+                                                                                  lds_b1);
 }
 
 template <int STAGES, bool LINES = false>

@@ -220,14 +220,15 @@ def main():
         in_step[name] = {"ms": ms, "tflops": fl / (ms * 1e-3) / 1e12,
                          "frac_fp32_mfma_peak": fl / (ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS}
 
-    # The dominant kernel is the one with the largest share of the step: gather_gemm_dma runs twice per step (fprop
-    # and dgrad, both reading the filter in place: no packing launch), wgrad_halo_f32 once (its interval also holds
-    # the reduction of its split sums, a few us).  `achieved` = algorithmic flops per launch / the kernel's average
-    # duration inside the timed steps.  The slowest direction is reported beside it.
+    # The dominant kernel is the one with the largest share of the step: gather_classes_f32 runs twice per step (fprop
+    # and dgrad, each cut into the nine parts that see the same taps inside the image, the parts in one launch whose
+    # workgroups run the body of gather_gemm_dma; both read the filter in place: no packing launch), wgrad_halo_f32
+    # once (its interval also holds the reduction of its split sums, a few us).  `achieved` = algorithmic flops per
+    # launch / the kernel's average duration inside the timed steps.  The slowest direction is reported beside it.
     gather_ms = 0.5 * (in_step["fprop"]["ms"] + in_step["dgrad"]["ms"])
-    share = {"gather_gemm_dma": 2 * gather_ms, "wgrad_halo_f32": in_step["wgrad"]["ms"]}
+    share = {"gather_classes_f32": 2 * gather_ms, "wgrad_halo_f32": in_step["wgrad"]["ms"]}
     kernel = max(share, key=share.get)
-    kernel_ms = gather_ms if kernel == "gather_gemm_dma" else in_step["wgrad"]["ms"]
+    kernel_ms = gather_ms if kernel == "gather_classes_f32" else in_step["wgrad"]["ms"]
     achieved = fl / (kernel_ms * 1e-3) / 1e12
     slowest = min(in_step, key=lambda k: in_step[k]["tflops"])
     traffic, traffic_source = counter_traffic(kernel)

@@ -537,6 +537,43 @@ def test_dgrad_cut_along_the_borders_of_its_classes(case, tune):
     assert np.array_equal(cut, abi.dgrad(dy, w, x.shape, stride, pad))
 
 
+# The same cut for a padded fp32 fprop at unit stride: the output's first and last rows and columns see fewer taps inside x.
+# Every part reads the filter in place as the [K][N] operand, at the rows of its own taps.  S, H, W, C, D, fH, fW, sH, sW, padding
+FPROP_BORDER_CASES = [
+    (3, 14, 14, 64, 64, 3, 3, 1, 1, "same"),      # nine parts: interior, four edges, four corners
+    (2, 56, 56, 64, 64, 3, 3, 1, 1, "same"),      # the headline layer's geometry
+    (2, 12, 10, 32, 128, 5, 3, 1, 1, "same"),     # 5x3: five row parts x three column parts, two n tiles
+    (2, 9, 9, 64, 64, 7, 7, 1, 1, "same"),        # more parts than one call may hold: the fprop stays whole
+    (3, 11, 13, 96, 96, 3, 3, 1, 1, "same"),      # 96 output channels: not whole n tiles, every part packs its taps
+    (2, 12, 12, 64, 64, 3, 3, 1, 1, "valid"),     # no padding: nothing to cut
+    (2, 10, 10, 24, 64, 3, 3, 1, 1, "same"),      # 24 input channels: slabs that are not whole, the fprop stays whole
+    (2, 16, 16, 64, 64, 2, 2, 1, 1, "same"),      # even filter: "same" pads nothing here (P = 0)
+]
+
+
+@pytest.mark.parametrize("case", FPROP_BORDER_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_fprop_cut_along_the_borders_of_the_output(case, tune):
+    from tests import abi
+    x, w, b, dy = _case(case, 25)
+    stride, pad = (case[7], case[8]), case[9]
+    want = O.conv_fprop(x, w, b, stride, pad, dtype=np.float64)
+    tune(gather_border=0, gather_bm=128, gather_split=0)
+    whole = abi.fprop(x, w, b, stride, pad)
+    abi.close(whole, want)
+    tune(gather_border=1)
+    cut = abi.fprop(x, w, b, stride, pad)                 # the output buffer starts as NaN: every element must be written
+    abi.close(cut, want)
+    assert np.array_equal(whole, cut)
+    tune(gather_merge=0)                                  # nothing is cut without the shared launch
+    assert np.array_equal(cut, abi.fprop(x, w, b, stride, pad))
+    tune(gather_merge=-1, gather_runs=1)
+    assert np.array_equal(cut, abi.fprop(x, w, b, stride, pad))
+    tune(gather_bkn=0)                                    # the parts pack their taps instead of reading the filter in place
+    assert np.array_equal(cut, abi.fprop(x, w, b, stride, pad))
+    nb = abi.fprop(x, w, None, stride, pad)               # no bias
+    abi.close(nb, O.conv_fprop(x, w, np.zeros_like(b), stride, pad, dtype=np.float64))
+
+
 # fp32 wgrad of a unit-stride filter of at most 9 taps on 64 input channels and at most 64 output
 # channels, on rows of 28, 32, 56 or 64 output pixels: one persistent workgroup per CU keeps the whole
 # K x N result in registers (12 multiplying waves of three 32 x 32 blocks) and a loading wave brings one
