@@ -1,4 +1,4 @@
-// The problems a dgrad is made of.
+// The problems a dgrad is made of, and the parts of a padded fprop.
 //
 // dx[i][j] gets a contribution of filter tap (x, y) from dy[(i + pH - x) / sH][(j + pW - y) / sW] where the divisions are
 // exact and the result lies inside dy.  Input rows are taken in classes a = i % sH (i = a + sH i'): a class sees only the
@@ -89,6 +89,40 @@ static inline DgradPlan plan_dgrad_parts(int H, int W, int Ho, int Wo, int fH, i
                 }
         }
     }
+    return plan;
+}
+
+// A padded fprop at unit stride cut the same way: part pixel (r, c), 0 <= r < Hg, 0 <= c < Wg, is output pixel (oh0 + r,
+// ow0 + c); its tap (t, u), 0 <= t < Th, 0 <= u < Tw, is filter tap (xa + t, ya + u) and reads x pixel (r + rh0 + t, c + rw0 + u),
+// which lies inside x for every pixel and tap of the part.
+struct FpropPart {
+    int Hg, Wg, Th, Tw;
+    int rh0, rw0;
+    int oh0, ow0;
+    int xa, ya;
+};
+
+struct FpropPlan {
+    std::vector<FpropPart> parts;
+    int64_t taps_whole = 0;     // tap-pixels per sample of the whole problem: Ho * Wo * fH * fW
+    int64_t taps_parts = 0;     // ... that the parts multiply
+};
+
+static inline FpropPlan plan_fprop_parts(int H, int W, int Ho, int Wo, int fH, int fW, int pH, int pW) {
+    FpropPlan plan;
+    plan.taps_whole = (int64_t)Ho * Wo * fH * fW;
+    // output row r reads x row r - pH + t under filter row t
+    for (const TapSpan& rs : tap_spans(Ho, -pH, fH, H, true))
+        for (const TapSpan& cs : tap_spans(Wo, -pW, fW, W, true)) {
+            FpropPart p;
+            p.Hg = rs.r1 - rs.r0; p.Wg = cs.r1 - cs.r0;
+            p.Th = rs.t1 - rs.t0; p.Tw = cs.t1 - cs.t0;
+            p.rh0 = -pH + rs.r0 + rs.t0; p.rw0 = -pW + cs.r0 + cs.t0;
+            p.oh0 = rs.r0; p.ow0 = cs.r0;
+            p.xa = rs.t0; p.ya = cs.t0;
+            plan.taps_parts += (int64_t)p.Hg * p.Wg * p.Th * p.Tw;
+            plan.parts.push_back(p);
+        }
     return plan;
 }
 

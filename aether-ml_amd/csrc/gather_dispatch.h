@@ -791,36 +791,29 @@ int conv_fprop_impl(const char* fn, const T* x, const T* w, const float* bias, f
         const bool large = gs.nsplit == 1 && gather_bn(D) == 64 && g.M > 0 && gather_bm(g.M, D, cus, true) == 128;
         if (sH == 1 && sW == 1 && (pH > 0 || pW > 0) && fixed_scratch == nullptr && act == nullptr && v != 0 &&
             tuning().gather_merge != 0 && C % BK == 0 && (large || v > 0)) {
-            const std::vector<TapSpan> rows = tap_spans(Ho, -pH, fH, H, true), cols = tap_spans(Wo, -pW, fW, W, true);
-            int64_t inside = 0;
-            for (const TapSpan& rs : rows)
-                for (const TapSpan& cs : cols) inside += (int64_t)(rs.r1 - rs.r0) * (cs.r1 - cs.r0) * (rs.t1 - rs.t0) * (cs.t1 - cs.t0);
-            const int64_t whole = (int64_t)Ho * Wo * fH * fW;
-            const size_t nparts = rows.size() * cols.size();
-            if (nparts >= 2 && nparts <= (size_t)kMaxHeldClasses && (v > 0 || inside * 100 <= whole * 98)) {
+            const FpropPlan plan = plan_fprop_parts(H, W, Ho, Wo, fH, fW, pH, pW);
+            const size_t nparts = plan.parts.size();
+            if (nparts >= 2 && nparts <= (size_t)kMaxHeldClasses && (v > 0 || plan.taps_parts * 100 <= plan.taps_whole * 98)) {
                 std::vector<GatherSetup> parts;
                 int64_t total = 0;
                 uniform_class_tiles() = true;
-                for (const TapSpan& rs : rows)
-                    for (const TapSpan& cs : cols) {
-                        GatherSetup ps = gs;
-                        GatherParams& q = ps.gp;
-                        const int th = rs.t1 - rs.t0, tw = cs.t1 - cs.t0;
-                        q.Hg = rs.r1 - rs.r0; q.Wg = cs.r1 - cs.r0; q.M = S * q.Hg * q.Wg;
-                        q.K = th * tw * C;
-                        q.Kpad = (int)round_up(q.K, BK);
-                        // part row r is output row r + r0 and its tap t is filter row t + t0: x row r + (r0 + t0 - pH) + t
-                        q.Tw = tw; q.rh0 = -pH + rs.r0 + rs.t0; q.rw0 = -pW + cs.r0 + cs.t0;
-                        q.oh0 = rs.r0; q.ow0 = cs.r0; q.dense_out = 0;
-                        set_out_divs(q);
-                        PackParams& pq = ps.pp;
-                        pq.Tw = tw > 0 ? tw : 1; pq.xa = rs.t0; pq.ya = cs.t0; pq.K = q.K; pq.Kpad = q.Kpad;
-                        ps.bt_bytes = (int64_t)pq.Npad * pq.Kpad * sizeof(T);
-                        ps.kn_part = true;
-                        ps.nsplit = 1; ps.part_bytes = 0; q.split_slabs = 0;
-                        total += round_up(ps.bt_bytes, 256);
-                        parts.push_back(ps);
-                    }
+                for (const FpropPart& part : plan.parts) {
+                    GatherSetup ps = gs;
+                    GatherParams& q = ps.gp;
+                    q.Hg = part.Hg; q.Wg = part.Wg; q.M = S * q.Hg * q.Wg;
+                    q.K = part.Th * part.Tw * C;
+                    q.Kpad = (int)round_up(q.K, BK);
+                    q.Tw = part.Tw; q.rh0 = part.rh0; q.rw0 = part.rw0;
+                    q.oh0 = part.oh0; q.ow0 = part.ow0; q.dense_out = 0;
+                    set_out_divs(q);
+                    PackParams& pq = ps.pp;
+                    pq.Tw = part.Tw > 0 ? part.Tw : 1; pq.xa = part.xa; pq.ya = part.ya; pq.K = q.K; pq.Kpad = q.Kpad;
+                    ps.bt_bytes = (int64_t)pq.Npad * pq.Kpad * sizeof(T);
+                    ps.kn_part = true;
+                    ps.nsplit = 1; ps.part_bytes = 0; q.split_slabs = 0;
+                    total += round_up(ps.bt_bytes, 256);
+                    parts.push_back(ps);
+                }
                 void* ws;
                 rc = workspace(total > 0 ? total : 256, &ws);
                 if (rc) {

@@ -87,8 +87,58 @@ static int check(const char* name, int H, int W, int fH, int fW, int sH, int sW,
     return 0;
 }
 
+// The parts of a padded fprop at unit stride (Conv_Layer.forward, CNN_classes_cupy.py:92-116): y[r][c] takes filter tap (x, y) from
+// the image pixel (r + x - pH, c + y - pW) when that lies inside the image.  The parts must list every such (r, c, x, y) exactly
+// once with that pixel, no tap outside the image, and every output pixel exactly once.
+static int check_fprop(const char* name, int H, int W, int fH, int fW, int pH, int pW) {
+    const int Ho = H + 2 * pH - fH + 1, Wo = W + 2 * pW - fW + 1;
+    const FpropPlan plan = plan_fprop_parts(H, W, Ho, Wo, fH, fW, pH, pW);
+    std::set<std::tuple<int, int, int, int>> got;
+    std::map<std::pair<int, int>, int> pixels;
+    for (const FpropPart& p : plan.parts) {
+        if (p.Hg < 1 || p.Wg < 1 || p.Th < 0 || p.Tw < 0) { printf("FAIL %s: empty part\n", name); return 1; }
+        for (int r = 0; r < p.Hg; ++r)
+            for (int c = 0; c < p.Wg; ++c) {
+                const int orow = p.oh0 + r, ocol = p.ow0 + c;
+                if (orow < 0 || orow >= Ho || ocol < 0 || ocol >= Wo) { printf("FAIL %s: pixel outside y\n", name); return 1; }
+                ++pixels[std::make_pair(orow, ocol)];
+                for (int t = 0; t < p.Th; ++t)
+                    for (int u = 0; u < p.Tw; ++u) {
+                        const int x = p.xa + t, y = p.ya + u;
+                        const int i = r + p.rh0 + t, j = c + p.rw0 + u;
+                        if (x < 0 || x >= fH || y < 0 || y >= fW) { printf("FAIL %s: tap outside the filter\n", name); return 1; }
+                        if (i < 0 || i >= H || j < 0 || j >= W) { printf("FAIL %s: a part multiplies a tap in the padding\n", name); return 1; }
+                        if (i != orow + x - pH || j != ocol + y - pW) { printf("FAIL %s: (%d, %d) tap (%d, %d) reads x (%d, %d)\n", name, orow, ocol, x, y, i, j); return 1; }
+                        if (!got.insert(std::make_tuple(orow, ocol, x, y)).second) { printf("FAIL %s: listed twice\n", name); return 1; }
+                    }
+            }
+    }
+    int64_t want = 0;
+    for (int r = 0; r < Ho; ++r)
+        for (int c = 0; c < Wo; ++c) {
+            if (pixels[std::make_pair(r, c)] != 1) { printf("FAIL %s: y (%d, %d) written %d times\n", name, r, c, pixels[std::make_pair(r, c)]); return 1; }
+            for (int x = 0; x < fH; ++x)
+                for (int y = 0; y < fW; ++y) {
+                    const int i = r + x - pH, j = c + y - pW;
+                    if (i >= 0 && i < H && j >= 0 && j < W) ++want;
+                }
+        }
+    if ((int64_t)got.size() != want || plan.taps_parts != want || plan.taps_whole != (int64_t)Ho * Wo * fH * fW) {
+        printf("FAIL %s: %zu contributions listed, %lld exist\n", name, got.size(), (long long)want);
+        return 1;
+    }
+    printf("ok %s\n", name);
+    return 0;
+}
+
 int main() {
     int bad = 0;
+    bad += check_fprop("fprop_same_56x56_3x3", 56, 56, 3, 3, 1, 1);                   // the headline layer: nine parts
+    bad += check_fprop("fprop_same_12x10_5x3", 12, 10, 5, 3, 2, 1);
+    bad += check_fprop("fprop_same_9x9_7x7", 9, 9, 7, 7, 3, 3);
+    bad += check_fprop("fprop_valid_12x12_3x3", 12, 12, 3, 3, 0, 0);                  // one part
+    bad += check_fprop("fprop_pad3_6x6_3x3", 6, 6, 3, 3, 3, 3);                       // more padding than the filter needs: rows without taps
+    bad += check_fprop("fprop_rows_only_8x20_3x1", 8, 20, 3, 1, 1, 0);
     bad += check("stride2_valid_28x28_3x3", 28, 28, 3, 3, 2, 2, 0, 0, true);        // the benchmark layer: 16 parts, a clipped row and column
     bad += check("stride2_same_28x28_3x3", 28, 28, 3, 3, 2, 2, 1, 1, true);
     bad += check("unit_stride_same_56x56_3x3", 56, 56, 3, 3, 1, 1, 1, 1, true);     // 9 parts

@@ -34,12 +34,13 @@ def test_sample_runs_cover_the_batch_below_the_descriptor_limit(tmp_path):
 
 def test_dgrad_parts_list_every_contribution_once(tmp_path):
     """aether-ml_amd/csrc/dgrad_parts.h: the problems a dgrad is made of (stride classes, and their parts when the classes
-    are cut along their borders).  tests/cpu/dgrad_parts_check.cpp enumerates, for 14 geometries, every (dx pixel, filter
-    tap) pair of every problem and compares with the definition of the input gradient (CNN_classes_cupy.py:136-153)."""
+    are cut along their borders) and the parts of a padded fprop.  tests/cpu/dgrad_parts_check.cpp enumerates, for 14 + 6
+    geometries, every (pixel, filter tap) pair of every problem and compares with the definitions of the input gradient
+    (CNN_classes_cupy.py:136-153) and of the forward pass (:92-116)."""
     exe = str(tmp_path / "dgrad_parts_check")
     src = os.path.join(ROOT, "tests", "cpu", "dgrad_parts_check.cpp")
     inc = os.path.join(ROOT, "aether-ml_amd", "csrc")
     subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-Werror", "-I", inc, src, "-o", exe], check=True)
     r = subprocess.run([exe], capture_output=True, text=True)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert len([line for line in r.stdout.splitlines() if line.startswith("ok ")]) == 14
+    assert len([line for line in r.stdout.splitlines() if line.startswith("ok ")]) == 20
