@@ -501,7 +501,7 @@ def test_strided_dgrad_with_its_classes_in_one_launch(case, tune):
 # The classes of an fp32 dgrad cut along their borders: the first and last rows and columns of a class see fewer of
 # its taps inside dy than the interior does, and a tile that mixes them multiplies the missing taps as zeros.  Cut into the
 # runs of rows and columns that see the same taps, every part is a problem with only those taps; all parts take 128-row tiles
-# and go out in grids of up to 8 problems.  The library does this for layers whose classes are large; the gather_border switch
+# and go out in grids of up to 9 problems.  The library does this for layers whose classes are large; the gather_border switch
 # lets small inputs reach it.  The sums run over the same taps in the same order: same values as the uncut classes.
 BORDER_CASES = [
     (6, 28, 28, 64, 64, 3, 3, 2, 2, "valid"),     # the stride-2 benchmark layer's geometry: 16 parts (9 + 3 + 3 + 1)
