@@ -255,15 +255,19 @@ def test_load_parameters_accepts_cupy_wrapped_float64_checkpoints(tmp_path):
     abi.close(got, want, rtol=1e-3)
 
 
-def test_recorded_steps_equal_eager_steps():
+@pytest.mark.parametrize("switches", [{}, {"gather_border": 1}], ids=["as the shapes decide", "fprop and dgrad cut along their borders"])
+def test_recorded_steps_equal_eager_steps(switches, tune):
     """Model.record_steps: a step replayed from a HIP graph must give what the same
     step gives when every kernel is launched from Python.  Same kernels in the same
     order, so the comparison is exact.  The replays are interleaved with eager work
     of the same model (an evaluation, a step of another batch shape, a
     synchronisation), every replay is checked, and learning-rate decay is on so that
-    the step state kept on the device matters."""
+    the step state kept on the device matters.  Second run: the convolutions' forward
+    and input-gradient products cut into their border parts, nine problems per launch
+    (what large layers get), so that these launches are recorded and replayed too."""
     import aether
     from aether import _lib
+    tune(**switches)
 
     def make():
         np.random.seed(3)
