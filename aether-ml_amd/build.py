@@ -14,14 +14,18 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIBDIR = os.path.join(HERE, "aether", "lib")
 LIB = os.path.join(LIBDIR, "libaether_hip.so")
-SOURCES = ["runtime.hip", "gather_f32.hip", "gather_bf16.hip", "wgrad_f32.hip", "wgrad_bf16.hip", "pair_f32.hip", "layers.hip"]
+SOURCES = ["runtime.hip", "gather_f32.hip", "gather_bf16.hip", "gather_res9_bf16.hip", "wgrad_f32.hip", "wgrad_bf16.hip", "pair_f32.hip",
+           "layers.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wno-unused-command-line-argument",
 ]
+# MFMA results in the ordinary registers: what the kernels that hold a tile's accumulators next to their operands want.  Not
+# for the kernel that fills all 512 registers of a lane and needs the accumulation registers for accumulators and filter.
+VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form"]
+AGPR_SOURCES = {"gather_res9_bf16.hip"}
 
 
 def _headers():
@@ -42,7 +46,7 @@ def _compile(src, force):
     obj = os.path.join(OBJ, src.replace(".hip", ".o"))
     path = os.path.join(CSRC, src)
     if force or _stale(obj, [path] + _headers()):
-        cmd = [HIPCC] + FLAGS + ["-c", path, "-o", obj]
+        cmd = [HIPCC] + FLAGS + ([] if src in AGPR_SOURCES else VGPR_FORM) + ["-c", path, "-o", obj]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
@@ -52,7 +56,7 @@ def _compile(src, force):
 def build(force=False):
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(LIBDIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=7) as ex:
+    with ThreadPoolExecutor(max_workers=8) as ex:
         objs = list(ex.map(lambda s: _compile(s, force), SOURCES))
     if force or _stale(LIB, objs):
         cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs

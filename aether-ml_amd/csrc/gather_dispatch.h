@@ -317,7 +317,7 @@ static bool plan_halo(GatherParams& gp, bool dma, int* mtiles, int* stages, int 
 // gather_halo_res_bf16 applies to unit-stride gathers of 2 to 9 taps over one 64-channel block
 // with N in one tile, when 224-row tiles are whole rows of one image (Wg divides 224, at most
 // 15 % of empty rows in an image's last tile), a tile's rows and its halo fit a halo buffer and
-// there are at least 4 tiles per CU to walk (tuning: gather_res = 1 drops the last condition,
+// there are at least 4 tiles per CU to walk (tuning: gather_res = 1 or 2 drops the last condition,
 // 0 turns the kernel off).
 static bool plan_halo_res(GatherParams& gp, bool dma, int cus, int* mtiles) {
     if (!dma || gp.sh != 1 || gp.sw != 1 || gp.Cs != 64 || gp.K != gp.Kpad || gp.split_slabs != 0) return false;
@@ -600,6 +600,9 @@ static int choose_b_operand(GatherSetup& gs, bool vec, int min_slabs = 3) {
     return pk.Npad * pk.Kpad;
 }
 
+// (gather_res9_bf16.hip)
+void launch_halo_res9_bf16(const GatherParams& p, const PackParams& pk, int mtiles, unsigned grid, hipStream_t stream);
+
 template <typename T>
 static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
     Context& c = ctx();
@@ -611,6 +614,13 @@ static int run_gather(GatherSetup& gs, char* ws, int64_t ws_off, bool vec) {
         const bool dma = vec && hp.src_bytes != 0 && gs.pp.w_elems * 2 < ((int64_t)1 << 31) && gs.pp.N % 2 == 0;
         if (gs.nsplit == 1 && hp.M > 0 && plan_halo_res(hp, dma, c.prop.multiProcessorCount, &mtiles)) {
             const dim3 rgrid((unsigned)std::min(mtiles, c.prop.multiProcessorCount));
+            // 3 x 3 taps onto rows stored one after the other: the filter lives in registers (tuning: gather_res = 2 keeps
+            // it in LDS)
+            if (hp.Th == 3 && hp.Tw == 3 && hp.dense_out && run_stores(hp) && tuning().gather_res != 2) {
+                launch_halo_res9_bf16(hp, gs.pp, mtiles, rgrid.x, c.stream);
+                AETH_LAUNCH_CHECK();
+                return AETH_OK;
+            }
             // tiles stored as runs of 256 contiguous bytes per pixel (tuning: gather_runs = 0 keeps the 16-byte pieces)
             if (run_stores(hp))
                 hipLaunchKernelGGL(gather_halo_res_bf16<true>, rgrid, dim3(kResThreads), 0, c.stream, hp, gs.pp, mtiles);

@@ -26,7 +26,7 @@ struct Tuning {
     int narrow = -1;         // 0: products with at most 16 output channels go to the slab kernels too
     int gather_runs = -1;    // tiles stored as runs of contiguous channels (non-temporal): 0 never, 1 always (default: from 64 MB of output on)
     int gather_wide = -1;    // bf16 8-wave tiles: 0 never, 1 also for few tiles
-    int gather_res = -1;     // gather_halo_res_bf16: 0 off, 1 also for few tiles
+    int gather_res = -1;     // gather_halo_res_bf16 / gather_halo_res9_bf16: 0 off, 1 also for few tiles, 2 the same with the filter in LDS for 3 x 3 taps too
     int dense_res = -1;      // dense_res_f32: 0 off, 1 also for few tiles
     int direct = -1;         // 0: no direct kernels for 1 to 3 input channels; 2: 4 output channels per lane in them
     int wgrad_halo = -1;     // wgrad_halo_f32 / _bf16: 0 off, 1 also for few slabs

@@ -209,8 +209,9 @@ def test_bf16_random_geometries_without_split_k(case, tune):
 
 # A filter of at most 9 taps on 64 channels and at most 64 output channels stays in LDS whole: one
 # persistent workgroup per CU, one wave fetching the source pixels of the next 224-row tile while
-# seven multiply the current one.  Tiles are whole image rows (the width divides 224).  The library
-# takes that kernel from 4 tiles per CU on; the gather_res switch lets small inputs reach it.
+# seven multiply the current one.  Tiles are whole image rows (the width divides 224).  A 3 x 3 filter
+# whose output rows lie one after the other goes into the registers of four waves instead.  The library
+# takes these kernels from 4 tiles per CU on; the gather_res switch lets small inputs reach them.
 RES_CASES = [
     (2, 56, 56, 64, 64, 3, 3, 1, 1, "same"),      # the 56x56x64 layer: 14 tiles of 4 image rows per image
     (3, 28, 28, 64, 64, 3, 3, 1, 1, "same"),      # 784 pixels per image: the fourth tile is half empty
@@ -238,6 +239,9 @@ def test_bf16_fprop_dgrad_with_the_filter_resident_in_lds(case, tune):
     abi.close(abi.fprop_bf16(x, w, None, stride, pad), O.conv_fprop(xr, wr, None, stride, pad, dtype=np.float64))
     dx = abi.dgrad_bf16(dy, w, x.shape, stride, pad)
     abi.close(dx, O.conv_dgrad(dyr, wr, x.shape[1:3], stride, pad, dtype=np.float64))
+    tune(gather_res=2)                            # 3 x 3 taps too with the filter in LDS, not in registers: same bits
+    assert np.array_equal(got, abi.fprop_bf16(x, w, b, stride, pad))
+    assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
     tune(gather_runs=0)                           # tiles stored as 16-byte pieces (the filter as the MFMAs' first operand): same bits
     assert np.array_equal(got, abi.fprop_bf16(x, w, b, stride, pad))
     assert np.array_equal(dx, abi.dgrad_bf16(dy, w, x.shape, stride, pad))
