@@ -20,6 +20,8 @@ namespace aeth {
 // a tap are issued during the tap before it, across the halves too.
 // Output rows are stored at out + m N (the host checks dense_out) as runs of 256 contiguous bytes per
 // pixel, as in the RUNS form of gather_halo_res_bf16; the filter takes the same way into LDS first.
+// What is left of a launch's time is the memory taking the fp32 output: on [256,56,56,64] -> 64 the
+// launch moves 309 MB in 68 us where a copy of that size takes 59, and a build without the stores 55.
 // ------------------------------------------------------------------------------
 static __global__ __launch_bounds__(256, 1) void gather_halo_res9_bf16(const GatherParams p, const PackParams pk, const int mtiles) {
     constexpr int BM = kResBM, BN = 64, TN = 2, KC = 8, NW = 4, NL = kResSlots / 8 / NW, WR = BM / NW, NT = 9, FW = 3;
