@@ -250,6 +250,46 @@ def test_bf16_fprop_dgrad_with_the_filter_resident_in_lds(case, tune):
     abi.close(abi.fprop_bf16(x, w, b, stride, pad), got, rtol=1e-5, atol=1e-5)
 
 
+def test_bf16_register_filter_kernel_replayed_from_a_graph(tune):
+    """The 3 x 3 kernel that keeps its filter in registers, recorded between aeth_graph_begin and aeth_graph_end (fprop and
+    dgrad of one layer: nothing runs) and replayed three times with new inputs and eager work in between: every replay
+    gives the bits of the eager calls."""
+    import ctypes as C
+    from aether import _lib
+    from aether.tensor import DeviceTensor
+    from tests import abi
+    tune(gather_split=0, gather_runs=1, gather_res=1)
+    lib = _lib.lib()
+    rng = np.random.default_rng(23)
+    xshape, wshape = (3, 28, 28, 64), (3, 3, 64, 64)
+    dims, yshape = abi.conv_dims(xshape, wshape, (1, 1), "same")
+    w = (rng.standard_normal(wshape) * 0.1).astype(np.float32)
+    b = rng.standard_normal(64).astype(np.float32)
+    wd, bd = abi.to_bf16_device(w), DeviceTensor.from_numpy(b, np.float32)
+    x16, dy16 = DeviceTensor(xshape, np.uint16), DeviceTensor(yshape, np.uint16)
+    y, dx = DeviceTensor.full(yshape, np.nan), DeviceTensor.full(xshape, np.nan)
+    _lib.check(lib.aeth_graph_begin())
+    rc1 = lib.aeth_conv_fprop_bf16(x16.ptr, wd.ptr, bd.ptr, y.ptr, *dims)
+    rc2 = lib.aeth_conv_dgrad_bf16(dy16.ptr, wd.ptr, dx.ptr, *dims)
+    handle = C.c_void_p()
+    rc_end = lib.aeth_graph_end(C.byref(handle))
+    _lib.check(rc1), _lib.check(rc2), _lib.check(rc_end)
+    assert np.all(np.isnan(y.get())) and np.all(np.isnan(dx.get()))           # recorded, not run
+    try:
+        for rep in range(3):
+            x = rng.standard_normal(xshape).astype(np.float32)
+            dy = rng.standard_normal(yshape).astype(np.float32)
+            for src, dst in ((x, x16), (dy, dy16)):
+                f = DeviceTensor.from_numpy(src, np.float32)
+                _lib.check(lib.aeth_cast_f32_to_bf16(f.ptr, dst.ptr, f.size))
+            _lib.check(lib.aeth_graph_launch(handle))
+            got_y, got_dx = y.get(), dx.get()
+            assert np.array_equal(got_y, abi.fprop_bf16(x, w, b, (1, 1), "same")), rep      # eager work between the replays
+            assert np.array_equal(got_dx, abi.dgrad_bf16(dy, w, xshape, (1, 1), "same")), rep
+    finally:
+        _lib.check(lib.aeth_graph_destroy(handle))
+
+
 # bf16 launches outside the halo kernels (strides, 1x1, more than 64 channels in) with more than 64 output
 # channels use tiles of 256 x 128 or 256 x 256 on 8 waves.  The library takes them from 2 tiles per CU on;
 # the gather_wide switch lets small inputs reach them, at 0 it gives the 4-wave tiles: the same sums in the same order.
